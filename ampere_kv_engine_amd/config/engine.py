@@ -1,0 +1,34 @@
+"""Sizes of the engine itself (not of the model): cache pool, batch limits, arithmetic.
+
+The reference fixes these as module constants and constructor arguments (`PAGED_BLOCK_SIZE = 16`,
+ampere_kv/runner.py:19; `blocks_per_layer`, `max_batch`, `prefill_chunk_size`, ampere_kv/scheduler.py:44-45).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+DTYPES = ("bfloat16", "float32")
+
+
+@dataclass(frozen=True)
+class EngineConfig:
+    dtype: str = "bfloat16"          # "bfloat16": serving kernels; "float32": every tensor and product in 32-bit
+    page_size: int = 16              # tokens per cache page
+    num_pages: int = 1024            # pages of every cache group's pool
+    max_seqs: int = 64               # per-request state slots = most live requests
+    max_batched_tokens: int = 2048   # most tokens one step may carry
+    max_seq_len: int = 8192          # longest sequence a request may reach (block-table width, rotary table)
+    device: str = "cuda:0"
+
+    def __post_init__(self):
+        if self.dtype not in DTYPES:
+            raise ValueError(f"dtype must be one of {DTYPES}, got {self.dtype!r}")
+        for name in ("page_size", "num_pages", "max_seqs", "max_batched_tokens", "max_seq_len"):
+            value = getattr(self, name)
+            if not isinstance(value, int) or value <= 0:
+                raise ValueError(f"{name} must be a positive integer, got {value!r}")
+
+    @property
+    def max_pages_per_seq(self) -> int:
+        return (self.max_seq_len + self.page_size - 1) // self.page_size

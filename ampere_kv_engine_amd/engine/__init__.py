@@ -1,0 +1,5 @@
+from .batch import Arena, BatchBuilder, PagedMeta, StepContext, StepEntry
+from .model import Model, expected_tensors
+from .engine import Engine
+
+__all__ = ["Arena", "BatchBuilder", "PagedMeta", "StepContext", "StepEntry", "Model", "expected_tensors", "Engine"]

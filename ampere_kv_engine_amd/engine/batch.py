@@ -1,0 +1,236 @@
+"""One step's batch: (request, its next tokens) for any mix of prompt portions and single decoded tokens,
+flattened to `tokens` rows, plus everything kernels need to find each token's request, position and pages.
+
+The reference builds three different inputs for its three forward functions and uploads block tables once
+per layer (ampere_kv/runner.py:205-215, :227-229; ampere_kv/scheduler.py:133-139).  Here one batch layout
+serves every step and all of its integer metadata reaches the device in one copy.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Sequence as Seq
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager, Sequence
+
+
+@dataclass
+class StepEntry:
+    """A request's share of a step: its next `tokens` and `want`, the places among them whose logits are
+    asked for."""
+    seq: Sequence
+    tokens: Seq[int]
+    want: Seq[int] = ()
+
+
+@dataclass
+class PagedMeta:
+    """Per cache group: where each new token's key/value goes and where each request's pages are."""
+    block_table: torch.Tensor     # int32 [seqs, width]; RELEASED (-1) or stale entries are never read
+    slot_map: torch.Tensor        # int32 [tokens]: page * page_size + offset of the token's own slot
+    width: int
+    window: int | None
+
+
+class Arena:
+    """Bump allocator for a step's activations.  Chunks are kept between steps, so after the first step
+    of a given size no device memory is allocated and addresses repeat from step to step."""
+
+    ALIGN = 256
+
+    def __init__(self, device, chunk_bytes: int = 64 << 20):
+        self.device = device
+        self.chunk_bytes = chunk_bytes
+        self.chunks: list[torch.Tensor] = []
+        self.chunk_index = 0
+        self.offset = 0
+
+    def reset(self) -> None:
+        self.chunk_index = 0
+        self.offset = 0
+
+    def take(self, shape, dtype: torch.dtype) -> torch.Tensor:
+        count = 1
+        for s in shape:
+            count *= int(s)
+        nbytes = max(count * torch.empty((), dtype=dtype).element_size(), 1)
+        nbytes = (nbytes + self.ALIGN - 1) // self.ALIGN * self.ALIGN
+        while True:
+            if self.chunk_index >= len(self.chunks):
+                self.chunks.append(torch.empty(max(nbytes, self.chunk_bytes), dtype=torch.uint8, device=self.device))
+            chunk = self.chunks[self.chunk_index]
+            if self.offset + nbytes <= chunk.numel():
+                raw = chunk[self.offset:self.offset + count * torch.empty((), dtype=dtype).element_size()]
+                self.offset += nbytes
+                return raw.view(dtype).view(*shape)
+            self.chunk_index += 1
+            self.offset = 0
+
+
+@dataclass
+class StepContext:
+    """What every part sees of the step."""
+    num_tokens: int
+    num_seqs: int
+    num_decode_seqs: int           # the first `num_decode_seqs` requests bring exactly one token each
+    token_ids: torch.Tensor        # int32 [tokens]
+    positions: torch.Tensor        # int32 [tokens], absolute
+    seq_of_token: torch.Tensor     # int32 [tokens], row of the step's request list
+    q_start: torch.Tensor          # int32 [seqs + 1], first token row of each request
+    seq_lens: torch.Tensor         # int32 [seqs], tokens the request holds after this step
+    seq_slots: torch.Tensor        # int32 [seqs], per-request state slot
+    logit_rows: torch.Tensor       # int32 [wanted], token rows whose logits are asked for
+    paged: list[PagedMeta]
+    arena: Arena
+    # host copies for parts that loop on the host (and for sizing launches without a device read)
+    host_q_start: list[int] = field(default_factory=list)
+    host_seq_lens: list[int] = field(default_factory=list)
+    host_seq_slots: list[int] = field(default_factory=list)
+    max_seq_len: int = 0           # longest request of the step, after the step
+    max_new_tokens: int = 0        # longest portion of the step
+    arenas: tuple = ()             # two arenas used by alternate layers (a layer's output outlives its own arena's reset)
+    stream_buffer: torch.Tensor | None = None   # float32 [max tokens, hidden]: the residual sum
+
+
+class BatchBuilder:
+    """Turns entries into a `StepContext`: registers the new tokens with the cache manager (which hands out
+    pages), lays the tokens out with single-token requests first, and uploads the metadata in one copy."""
+
+    def __init__(self, cache: CacheManager, device, max_batched_tokens: int, max_seqs: int, max_pages_per_seq: int):
+        self.cache = cache
+        self.device = torch.device(device)
+        self.max_tokens, self.max_seqs, self.max_width = max_batched_tokens, max_seqs, max_pages_per_seq
+        groups = len(cache.groups)
+        capacity = (3 * self.max_tokens + 3 * self.max_seqs + 1 + self.max_tokens
+                    + groups * (self.max_tokens + self.max_seqs * self.max_width))
+        pin = self.device.type == "cuda"
+        # Two pinned staging buffers in turn: the copy of one step may still be in flight while the host
+        # lays out the next, so a buffer is written again only after the copy that read it has finished.
+        self._hosts = [torch.empty(capacity, dtype=torch.int32, pin_memory=pin) for _ in range(2)]
+        self._copied = [torch.cuda.Event() if pin else None for _ in range(2)]
+        self._turn = 0
+        self._device = torch.empty(capacity, dtype=torch.int32, device=self.device)
+        self.arenas = (Arena(self.device), Arena(self.device))
+
+    def build(self, entries: list[StepEntry]) -> tuple[StepContext, list[int]]:
+        """Returns the context and, for every entry in the caller's order, the offset of its first wanted
+        row in the logits the step returns."""
+        if not entries:
+            raise ValueError("a step needs at least one entry")
+        if len(entries) > self.max_seqs:
+            raise ValueError(f"{len(entries)} requests in one step; the engine was built for {self.max_seqs}")
+        if len({id(e.seq) for e in entries}) != len(entries):
+            raise ValueError("a request appears twice in one step")
+        total = sum(len(e.tokens) for e in entries)
+        if total > self.max_tokens:
+            raise ValueError(f"{total} tokens in one step; the engine was built for {self.max_tokens}")
+        for e in entries:
+            if len(e.tokens) == 0:
+                raise ValueError(f"request {e.seq.request_id!r} brings no tokens")
+            for place in e.want:
+                if not 0 <= place < len(e.tokens):
+                    raise ValueError(f"request {e.seq.request_id!r} wants place {place} of {len(e.tokens)} tokens")
+            if e.seq.length + len(e.tokens) > self.max_width * self.cache.page_size:
+                raise ValueError(f"request {e.seq.request_id!r} would reach {e.seq.length + len(e.tokens)} tokens; "
+                                 f"the engine was built for {self.max_width * self.cache.page_size}")
+        # all-or-nothing over the whole step: check every request before registering any
+        self._check_pages(entries)
+        order = sorted(range(len(entries)), key=lambda i: (len(entries[i].tokens) != 1, i))
+        ordered = [entries[i] for i in order]
+        num_decode = sum(1 for e in ordered if len(e.tokens) == 1)
+        starts = [self.cache.reserve(e.seq, len(e.tokens)) for e in ordered]
+
+        n, r = total, len(ordered)
+        width = max(max((len(t.pages) for t in e.seq.tables), default=1) for e in ordered)
+        width = max(width, 1)
+        self._turn ^= 1
+        if self._copied[self._turn] is not None:
+            self._copied[self._turn].synchronize()
+        host_tensor = self._hosts[self._turn]
+        host = host_tensor.numpy()
+        cursor = 0
+
+        def region(count):
+            nonlocal cursor
+            view = host[cursor:cursor + count]
+            span = (cursor, cursor + count)
+            cursor += count
+            return view, span
+
+        token_ids, s_ids = region(n)
+        positions, s_pos = region(n)
+        seq_of_token, s_sot = region(n)
+        q_start, s_qs = region(r + 1)
+        seq_lens, s_sl = region(r)
+        seq_slots, s_ss = region(r)
+        wanted = sum(len(e.want) for e in entries)
+        logit_rows, s_lr = region(wanted)
+        group_spans = []
+        for g in self.cache.groups:
+            slot_map, s_sm = region(n)
+            table, s_bt = region(r * width)
+            group_spans.append((slot_map, s_sm, table.reshape(r, width), s_bt))
+
+        row = 0
+        first_row_of = [0] * len(entries)
+        for index, (e, start) in enumerate(zip(ordered, starts)):
+            count = len(e.tokens)
+            token_ids[row:row + count] = np.asarray(e.tokens, dtype=np.int64)
+            positions[row:row + count] = np.arange(start, start + count)
+            seq_of_token[row:row + count] = index
+            q_start[index] = row
+            seq_lens[index] = start + count
+            seq_slots[index] = e.seq.slot
+            first_row_of[order[index]] = row
+            for g, (slot_map, _, table, _) in zip(self.cache.groups, group_spans):
+                pages = e.seq.tables[g.index].pages
+                table[index, :len(pages)] = pages
+                table[index, len(pages):] = -1
+                pos = np.arange(start, start + count)
+                page_of = np.asarray(pages, dtype=np.int64)[pos // self.cache.page_size]
+                slot_map[row:row + count] = page_of * self.cache.page_size + pos % self.cache.page_size
+            row += count
+        # wanted rows in the caller's order of entries and places, whatever the layout above
+        want_cursor = 0
+        first_wanted_of = []
+        for e, first_row in zip(entries, first_row_of):
+            first_wanted_of.append(want_cursor)
+            for place in e.want:
+                logit_rows[want_cursor] = first_row + place
+                want_cursor += 1
+        q_start[r] = row
+
+        self._device[:cursor].copy_(host_tensor[:cursor], non_blocking=True)
+        if self._copied[self._turn] is not None:
+            self._copied[self._turn].record()
+        dev = lambda span: self._device[span[0]:span[1]]
+        paged = [PagedMeta(block_table=dev(s_bt).view(r, width), slot_map=dev(s_sm), width=width,
+                           window=g.need.window)
+                 for g, (_, s_sm, _, s_bt) in zip(self.cache.groups, group_spans)]
+        for arena in self.arenas:
+            arena.reset()
+        ctx = StepContext(
+            num_tokens=n, num_seqs=r, num_decode_seqs=num_decode, token_ids=dev(s_ids), positions=dev(s_pos),
+            seq_of_token=dev(s_sot), q_start=dev(s_qs), seq_lens=dev(s_sl), seq_slots=dev(s_ss),
+            logit_rows=dev(s_lr), paged=paged, arena=self.arenas[0],
+            host_q_start=[int(x) for x in q_start[:r + 1]], host_seq_lens=[int(x) for x in seq_lens[:r]],
+            host_seq_slots=[int(x) for x in seq_slots[:r]],
+            max_seq_len=int(seq_lens[:r].max()), max_new_tokens=max(len(e.tokens) for e in ordered),
+            arenas=self.arenas,
+        )
+        return ctx, first_wanted_of
+
+    def _check_pages(self, entries: list[StepEntry]) -> None:
+        from ..cache.pages import PagePoolExhausted
+        for g in self.cache.groups:
+            available = g.allocator.num_free
+            for e in entries:
+                table = e.seq.tables[g.index]
+                required = (table.length + len(e.tokens) + self.cache.page_size - 1) // self.cache.page_size
+                available += table._passed_pages(table.length) - max(0, required - len(table.pages))
+            if available < 0:
+                raise PagePoolExhausted(f"the step needs {-available} more page(s) than the pool of cache group "
+                                        f"{g.index} has free; no token of the step was registered")

@@ -1,0 +1,47 @@
+"""A weight matrix [out, in] used as y = x W^T (ampere_kv/runner.py:64).  Several matrices that read the
+same input may be stacked along `out` at load; a row of W keeps its own reduction, so stacking changes no
+value."""
+
+from __future__ import annotations
+
+import torch
+
+from ..weights.spec import MATRIX, TensorSpec
+from .base import Part
+
+
+class Linear(Part):
+    def __init__(self, runtime, in_features: int, out_features: list[int], names: list[str], role: str = MATRIX):
+        self.rt = runtime
+        self.in_features = in_features
+        self.out_features = list(out_features)
+        self.names = list(names)
+        self.role = role
+        self.weight: torch.Tensor | None = None
+
+    @property
+    def total_out(self) -> int:
+        return sum(self.out_features)
+
+    def tensors(self, prefix: str):
+        return [TensorSpec(prefix + name, (out, self.in_features), self.role)
+                for name, out in zip(self.names, self.out_features)]
+
+    def load(self, fetch, prefix: str):
+        pieces = [fetch(spec) for spec in self.tensors(prefix)]
+        dtypes = {p.dtype for p in pieces}
+        if len(dtypes) != 1:
+            raise ValueError(f"matrices stacked into one product are stored in different dtypes: "
+                             f"{[prefix + n for n in self.names]} -> {sorted(map(str, dtypes))}")
+        self.weight = pieces[0].contiguous() if len(pieces) == 1 else torch.cat(pieces, dim=0).contiguous()
+
+    def adopt(self, weight: torch.Tensor):
+        """Use an already loaded matrix (a head tied to the embedding)."""
+        self.weight = weight
+
+    def weight_bytes(self):
+        return self.weight.numel() * self.weight.element_size()
+
+    def forward(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        self.rt.kernels.linear(x, self.weight, out)
+        return out

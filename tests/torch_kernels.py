@@ -1,0 +1,134 @@
+"""A test double for the engine's kernel set, written with plain torch operations.
+
+It exists so that the host side of the engine (batch layout, block tables, page reuse, scheduling, replay)
+can be exercised where there is no GPU.  It is handed to `Engine(..., kernels=TorchKernels())` by tests only;
+the product never constructs it and has no fallback to it.  Each method states the contract of the HIP
+kernel of the same name; the GPU tests hold the HIP kernels to these same contracts.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+
+def _round(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    return x.to(dtype)
+
+
+class TorchKernels:
+    name = "torch-double"
+
+    def check_attention_sizes(self, q_heads, kv_heads, head_dim, page_size):
+        if q_heads % kv_heads:
+            raise ValueError("q_heads must be a multiple of kv_heads")
+
+    # ---- token-wise ------------------------------------------------------------------------------------
+    def embed(self, ids, table, out):
+        out.copy_(table[ids.long()].float())
+
+    def add_rmsnorm(self, stream, delta, weight, eps, out):
+        if delta is not None:
+            stream += delta.float()
+        normed = stream * torch.rsqrt((stream * stream).mean(-1, keepdim=True) + eps)
+        out.copy_(_round(_round(normed, out.dtype).float() * weight, out.dtype))
+
+    def rmsnorm(self, x, weight, eps, out):
+        xf = x.float()
+        normed = xf * torch.rsqrt((xf * xf).mean(-1, keepdim=True) + eps)
+        out.copy_(_round(_round(normed, out.dtype).float() * weight, out.dtype))
+
+    def rmsnorm_heads(self, x, weight, eps, out):
+        self.rmsnorm(x, weight, eps, out)
+
+    def copy_heads(self, x, out):
+        out.copy_(x)
+
+    def gather_rows(self, stream, pending, rows, out):
+        picked = stream[rows.long()]
+        if pending is not None:
+            picked = picked + pending[rows.long()].float()
+        out.copy_(picked)
+
+    def linear(self, x, weight, out):
+        out.copy_((x.float() @ weight.float().T).to(out.dtype))
+
+    def swiglu(self, gate_up, out):
+        inter = out.shape[-1]
+        g, u = gate_up[:, :inter].float(), gate_up[:, inter:].float()
+        out.copy_((g * torch.sigmoid(g) * u).to(out.dtype))
+
+    # ---- position ----------------------------------------------------------------------------------------
+    def rope_table(self, inv_freq, table):
+        positions = torch.arange(table.shape[0], dtype=torch.float32, device=table.device)
+        angles = positions[:, None] * inv_freq[None, :].float()
+        table[..., 0] = angles.cos()
+        table[..., 1] = angles.sin()
+
+    def _rotate(self, x, positions, table):
+        half = x.shape[-1] // 2
+        cs = table[positions.long()]                      # [N, d/2, 2]
+        cos, sin = cs[:, None, :, 0], cs[:, None, :, 1]
+        lo, hi = x[..., :half].float(), x[..., half:].float()
+        return torch.cat((lo * cos - hi * sin, hi * cos + lo * sin), dim=-1)
+
+    def rope(self, x, positions, table):
+        x.copy_(self._rotate(x, positions, table).to(x.dtype))
+
+    # ---- cache ---------------------------------------------------------------------------------------------
+    def kv_write(self, k, v, slot_map, k_pages, v_pages):
+        pages, kv_heads, page_size, d = k_pages.shape
+        slots = slot_map.long()
+        k_pages[slots // page_size, :, slots % page_size] = k
+        v_pages[slots // page_size, :, slots % page_size] = v
+
+    def qk_norm_rope_write(self, qkv, q_weight, k_weight, eps, table, positions, slot_map, k_pages, v_pages,
+                           q_out, q_heads, kv_heads, head_dim):
+        n = qkv.shape[0]
+        q_size, kv_size = q_heads * head_dim, kv_heads * head_dim
+        q = qkv[:, :q_size].reshape(n, q_heads, head_dim).float()
+        k = qkv[:, q_size:q_size + kv_size].reshape(n, kv_heads, head_dim).float()
+        v = qkv[:, q_size + kv_size:].reshape(n, kv_heads, head_dim)
+        dtype = qkv.dtype
+        if q_weight is not None:
+            q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + eps)
+            q = _round(q, dtype).float() * q_weight
+            k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + eps)
+            k = _round(k, dtype).float() * k_weight
+        if table is not None:
+            q = self._rotate(_round(q, dtype), positions, table)
+            k = self._rotate(_round(k, dtype), positions, table)
+        q_out.copy_(q.reshape(n, q_size).to(dtype))
+        if slot_map is not None:
+            self.kv_write(k.to(dtype), v, slot_map, k_pages, v_pages)
+
+    def attention(self, q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out):
+        page_size = k_pages.shape[2]
+        group = q_heads // kv_heads
+        table = meta.block_table.cpu()
+        for r in range(ctx.num_seqs):
+            first, last = ctx.host_q_start[r], ctx.host_q_start[r + 1]
+            length = ctx.host_seq_lens[r]
+            history = length - (last - first)
+            lowest = 0 if window is None else max(0, history - window + 1)
+            key_pos = torch.arange(lowest, length)
+            pages = table[r][key_pos // page_size].long()
+            assert (pages >= 0).all(), "attention would read a page that was given back"
+            keys = k_pages[pages, :, key_pos % page_size].float()        # [S, kv_heads, d]
+            values = v_pages[pages, :, key_pos % page_size].float()
+            qs = q[first:last].reshape(last - first, q_heads, head_dim).float()
+            keys = keys.repeat_interleave(group, dim=1)
+            values = values.repeat_interleave(group, dim=1)
+            scores = torch.einsum("ihd,jhd->hij", qs, keys) * scale
+            q_pos = history + torch.arange(last - first)
+            visible = key_pos[None, :] <= q_pos[:, None]
+            if window is not None:
+                visible &= key_pos[None, :] > q_pos[:, None] - window
+            scores = scores.masked_fill(~visible[None], -math.inf)
+            merged = torch.einsum("hij,jhd->ihd", scores.softmax(-1), values)
+            out[first:last] = merged.reshape(last - first, q_heads * head_dim).to(out.dtype)
+
+    # ---- sampling -----------------------------------------------------------------------------------------
+    def argmax(self, logits, out):
+        out.copy_(logits.argmax(dim=-1).to(out.dtype))
