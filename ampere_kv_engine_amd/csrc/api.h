@@ -1,0 +1,39 @@
+// C entry points of the kernel library.  Every function enqueues on `stream` and returns 0, a hipError_t of the
+// launch, -1 for an unknown dtype code or -2 for sizes the kernel does not take.  dtype codes: 0 float32,
+// 1 bfloat16.  Pointers are device pointers; shapes are checked by the caller on the host.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+extern "C" {
+
+int akv_embed(const int* ids, const void* table, int table_dtype, float* out, int tokens, int hidden, int vocab,
+              hipStream_t stream);
+int akv_add_rmsnorm(float* stream_buf, const void* delta, const float* weight, float eps, void* out, int dtype,
+                    int tokens, int hidden, hipStream_t stream);
+int akv_rmsnorm_rows(const void* x, long token_stride, const float* weight, float eps, void* out, int dtype,
+                     long tokens, int heads, int width, hipStream_t stream);
+int akv_copy_rows(const void* x, long token_stride, void* out, int dtype, long tokens, int heads, int width,
+                  hipStream_t stream);
+int akv_gather_rows(const float* stream_buf, const void* pending, int dtype, const int* rows, float* out, int wanted,
+                    int hidden, int tokens, hipStream_t stream);
+int akv_swiglu(const void* gate_up, void* out, int dtype, long tokens, int inter, hipStream_t stream);
+int akv_rope_table(const float* inv_freq, float* table, int positions, int half, hipStream_t stream);
+int akv_rope(void* x, int dtype, const int* positions, const float* table, long tokens, int heads, int dim,
+             int table_positions, hipStream_t stream);
+int akv_kv_write(const void* k, long k_stride, const void* v, long v_stride, const int* slot_map, void* k_pages,
+                 void* v_pages, int dtype, long tokens, int kv_heads, int dim, int page_size, long num_pages,
+                 hipStream_t stream);
+int akv_qk_norm_rope_write(const void* qkv, const float* q_weight, const float* k_weight, float eps,
+                           const float* table, int table_positions, const int* positions, const int* slot_map,
+                           void* k_pages, void* v_pages, void* q_out, int dtype, long tokens, int q_heads,
+                           int kv_heads, int dim, int page_size, long num_pages, hipStream_t stream);
+int akv_linear_tiled(const void* x, int x_dtype, const void* w, int w_dtype, void* y, int y_dtype, int rows, int outs,
+                     int k, hipStream_t stream);
+int akv_attention_rows(const void* q, const void* k_pages, const void* v_pages, const int* seq_of_token,
+                       const int* positions, const int* block_table, int table_width, void* out, int dtype,
+                       long tokens, int q_heads, int kv_heads, int dim, int page_size, long num_pages, float scale,
+                       int window, hipStream_t stream);
+int akv_sample(const float* logits, const float* temperature, const unsigned long long* seeds,
+               const unsigned int* draws, int* out, int rows, int vocab, hipStream_t stream);
+}

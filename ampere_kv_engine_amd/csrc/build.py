@@ -1,0 +1,119 @@
+"""Compile the HIP sources of this folder for gfx950 into one shared library, in-tree.
+
+`build()` always compiles.  `ensure_built()` compiles only when no library matching the current sources is
+there (a fresh checkout's first call), printing a line per file so that a waiting user sees progress.  The
+library is plain C ABI (`api.h`), loaded with ctypes; nothing here depends on a Python extension toolchain,
+a home directory or a network.
+"""
+
+from __future__ import annotations
+
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import time
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SOURCES = ("elementwise.hip", "gemm.hip", "attention.hip", "sampling.hip")
+HEADERS = ("common.h", "api.h")
+LIBRARY = "libakv_kernels.so"
+ARCH = "gfx950"
+# packed-fp32 instructions are switched off for all device code of this library
+FLAGS = ("-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
+         "-packed-fp32-ops", "-Wno-unused-command-line-argument")
+
+
+def _hipcc() -> str:
+    for candidate in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if candidate and os.path.exists(candidate):
+            return candidate
+    raise RuntimeError("hipcc was not found (looked at $HIPCC, PATH and /opt/rocm/bin): the HIP kernels cannot be "
+                       "built, and the engine has no other way to compute")
+
+
+def source_stamp() -> str:
+    digest = hashlib.sha256()
+    for name in SOURCES + HEADERS:
+        with open(os.path.join(HERE, name), "rb") as handle:
+            digest.update(name.encode() + b"\0" + handle.read())
+    digest.update(" ".join(FLAGS).encode())
+    return digest.hexdigest()
+
+
+def _build_dir() -> str:
+    """`_build/` beside the sources; a per-user temporary folder when the tree cannot be written."""
+    local = os.path.join(HERE, "_build")
+    try:
+        os.makedirs(local, exist_ok=True)
+        probe = os.path.join(local, f".probe{os.getpid()}")
+        with open(probe, "w"):
+            pass
+        os.remove(probe)
+        return local
+    except OSError:
+        fallback = os.path.join(tempfile.gettempdir(), f"akv_build_{os.getuid()}_{source_stamp()[:12]}")
+        os.makedirs(fallback, exist_ok=True)
+        return fallback
+
+
+def library_path() -> str | None:
+    """The built library matching the current sources, or None."""
+    stamp = source_stamp()
+    for folder in (os.path.join(HERE, "_build"),
+                   os.path.join(tempfile.gettempdir(), f"akv_build_{os.getuid()}_{stamp[:12]}")):
+        lib, mark = os.path.join(folder, LIBRARY), os.path.join(folder, "stamp")
+        if os.path.exists(lib) and os.path.exists(mark):
+            with open(mark) as handle:
+                if handle.read().strip() == stamp:
+                    return lib
+    return None
+
+
+def _log(message: str) -> None:
+    print(f"[akv build] {message}", file=sys.stderr, flush=True)
+
+
+def build(verbose: bool = True) -> str:
+    """Compile every source and link the library; returns its path."""
+    hipcc = _hipcc()
+    out_dir = _build_dir()
+    started = time.time()
+    if verbose:
+        _log(f"compiling {len(SOURCES)} HIP sources for {ARCH} into {out_dir}")
+
+    def compile_one(name: str) -> str:
+        obj = os.path.join(out_dir, name.replace(".hip", ".o"))
+        cmd = [hipcc, *FLAGS, "-c", os.path.join(HERE, name), "-o", obj]
+        result = subprocess.run(cmd, capture_output=True, text=True)
+        if result.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {name}:\n{result.stderr}")
+        if verbose:
+            _log(f"compiled {name} ({time.time() - started:.0f} s)")
+        return obj
+
+    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
+        objects = list(pool.map(compile_one, SOURCES))
+    lib = os.path.join(out_dir, LIBRARY)
+    partial = lib + f".{os.getpid()}.tmp"
+    result = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objects, "-o", partial],
+                            capture_output=True, text=True)
+    if result.returncode != 0:
+        raise RuntimeError(f"linking {LIBRARY} failed:\n{result.stderr}")
+    os.replace(partial, lib)
+    with open(os.path.join(out_dir, "stamp"), "w") as handle:
+        handle.write(source_stamp())
+    if verbose:
+        _log(f"linked {lib} ({time.time() - started:.0f} s)")
+    return lib
+
+
+def ensure_built(verbose: bool = True) -> str:
+    return library_path() or build(verbose)
+
+
+if __name__ == "__main__":
+    print(build())

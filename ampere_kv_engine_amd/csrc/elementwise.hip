@@ -1,0 +1,342 @@
+// Token-wise kernels: embedding gather, RMSNorm (alone, with the residual add, per head), rotary encoding,
+// cache write, the fused q/k-norm + rotation + cache write, SwiGLU, row gather.
+// Statistics, angles and the residual sum are float32 whatever the activation type T is.
+
+#include "common.h"
+#include "api.h"
+
+using namespace akv;
+
+namespace {
+
+// ---- embedding: out[n, :] = table[ids[n], :] widened to float32 (no scaling) ------------------------------
+template <typename T>
+__global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out,
+                             int hidden, int vocab) {
+  const int n = blockIdx.x;
+  const int id = ids[n];
+  float* dst = out + static_cast<size_t>(n) * hidden;
+  if (id < 0 || id >= vocab) {  // never read outside the table; a poisoned row shows the fault downstream
+    for (int d = threadIdx.x; d < hidden; d += blockDim.x) dst[d] = __uint_as_float(0x7fc00000u);
+    return;
+  }
+  const T* src = table + static_cast<size_t>(id) * hidden;
+  for (int d = threadIdx.x; d < hidden; d += blockDim.x) dst[d] = to_float(src[d]);
+}
+
+// ---- residual add + RMSNorm: stream += delta (float32); out = T( T(stream * rsqrt(mean^2 + eps)) * w ) ----
+template <typename T>
+__global__ void add_rmsnorm_kernel(float* __restrict__ stream, const T* __restrict__ delta,
+                                   const float* __restrict__ weight, float eps, T* __restrict__ out, int hidden) {
+  __shared__ float scratch[16];
+  const size_t base = static_cast<size_t>(blockIdx.x) * hidden;
+  float* s = stream + base;
+  float acc = 0.f;
+  if (delta != nullptr) {
+    const T* d = delta + base;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      const float v = s[i] + to_float(d[i]);
+      s[i] = v;
+      acc += v * v;
+    }
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      const float v = s[i];
+      acc += v * v;
+    }
+  }
+  const float total = block_sum(acc, scratch);
+  const float scale = rsqrtf(total / static_cast<float>(hidden) + eps);
+  T* o = out + base;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = from_float<T>(rounded<T>(s[i] * scale) * weight[i]);
+}
+
+// ---- RMSNorm of rows [tokens, heads, width]: one wave per (token, head); input may be a strided view -------
+template <typename T>
+__global__ void rmsnorm_rows_kernel(const T* __restrict__ x, long token_stride, const float* __restrict__ weight,
+                                    float eps, T* __restrict__ out, long rows, int heads, int width) {
+  const long row = static_cast<long>(blockIdx.x) * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (row >= rows) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  const T* src = x + (row / heads) * token_stride + (row % heads) * static_cast<long>(width);
+  T* dst = out + row * width;
+  float acc = 0.f;
+  for (int i = lane; i < width; i += kWave) {
+    const float v = to_float(src[i]);
+    acc += v * v;
+  }
+  const float scale = rsqrtf(wave_sum(acc) / static_cast<float>(width) + eps);
+  for (int i = lane; i < width; i += kWave) dst[i] = from_float<T>(rounded<T>(to_float(src[i]) * scale) * weight[i]);
+}
+
+template <typename T>
+__global__ void copy_rows_kernel(const T* __restrict__ x, long token_stride, T* __restrict__ out, long rows,
+                                 int heads, int width) {
+  const long row = static_cast<long>(blockIdx.x) * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (row >= rows) return;
+  const T* src = x + (row / heads) * token_stride + (row % heads) * static_cast<long>(width);
+  for (int i = threadIdx.x & (kWave - 1); i < width; i += kWave) out[row * width + i] = src[i];
+}
+
+// ---- out[m, :] = stream[rows[m], :] (+ pending[rows[m], :]) in float32 ---------------------------------------
+template <typename T>
+__global__ void gather_rows_kernel(const float* __restrict__ stream, const T* __restrict__ pending,
+                                   const int* __restrict__ rows, float* __restrict__ out, int hidden, int tokens) {
+  const int row = rows[blockIdx.x];
+  float* dst = out + static_cast<size_t>(blockIdx.x) * hidden;
+  if (row < 0 || row >= tokens) {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = __uint_as_float(0x7fc00000u);
+    return;
+  }
+  const size_t base = static_cast<size_t>(row) * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x)
+    dst[i] = stream[base + i] + (pending != nullptr ? to_float(pending[base + i]) : 0.f);
+}
+
+// ---- SwiGLU: out[n, i] = silu(gate_up[n, i]) * gate_up[n, inter + i] ----------------------------------------
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, long tokens, int inter) {
+  const long index = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (index >= tokens * inter) return;
+  const long n = index / inter;
+  const int i = static_cast<int>(index % inter);
+  const float g = to_float(gate_up[n * 2 * inter + i]);
+  const float u = to_float(gate_up[n * 2 * inter + inter + i]);
+  out[index] = from_float<T>(g / (1.f + expf(-g)) * u);
+}
+
+// ---- rotary table: table[p, j] = (cos, sin)(p * inv_freq[j]) in float32 --------------------------------------
+__global__ void rope_table_kernel(const float* __restrict__ inv_freq, float* __restrict__ table, int positions,
+                                  int half) {
+  const long index = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (index >= static_cast<long>(positions) * half) return;
+  const float angle = static_cast<float>(index / half) * inv_freq[index % half];
+  float s, c;
+  sincosf(angle, &s, &c);
+  table[2 * index] = c;
+  table[2 * index + 1] = s;
+}
+
+// ---- rotation in place of x [tokens, heads, dim]: pairs (j, j + dim/2) ----------------------------------------
+template <typename T>
+__global__ void rope_kernel(T* __restrict__ x, const int* __restrict__ positions, const float* __restrict__ table,
+                            long tokens, int heads, int dim, int table_positions) {
+  const int half = dim / 2;
+  const long index = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (index >= tokens * heads * half) return;
+  const int j = static_cast<int>(index % half);
+  const long row = index / half;  // token * heads + head
+  const int pos = positions[row / heads];
+  T* p = x + row * dim;
+  if (pos < 0 || pos >= table_positions) {
+    p[j] = from_float<T>(__uint_as_float(0x7fc00000u));
+    p[j + half] = from_float<T>(__uint_as_float(0x7fc00000u));
+    return;
+  }
+  const float c = table[(static_cast<long>(pos) * half + j) * 2], s = table[(static_cast<long>(pos) * half + j) * 2 + 1];
+  const float lo = to_float(p[j]), hi = to_float(p[j + half]);
+  p[j] = from_float<T>(lo * c - hi * s);
+  p[j + half] = from_float<T>(hi * c + lo * s);
+}
+
+// ---- cache write: pages [num_pages, kv_heads, page_size, dim]; slot = page * page_size + offset -----------------
+template <typename T>
+__global__ void kv_write_kernel(const T* __restrict__ k, long k_stride, const T* __restrict__ v, long v_stride,
+                                const int* __restrict__ slot_map, T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                long tokens, int kv_heads, int dim, int page_size, long num_slots) {
+  const long row = static_cast<long>(blockIdx.x) * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (row >= tokens * kv_heads) return;
+  const long n = row / kv_heads;
+  const int h = static_cast<int>(row % kv_heads);
+  const long slot = slot_map[n];
+  if (slot < 0 || slot >= num_slots) return;  // host checks the map; never write outside the pool
+  const long dst = ((slot / page_size * kv_heads + h) * page_size + slot % page_size) * dim;
+  const T* ks = k + n * k_stride + static_cast<long>(h) * dim;
+  const T* vs = v + n * v_stride + static_cast<long>(h) * dim;
+  for (int i = threadIdx.x & (kWave - 1); i < dim; i += kWave) {
+    k_pages[dst + i] = ks[i];
+    v_pages[dst + i] = vs[i];
+  }
+}
+
+// ---- fused: per-head RMSNorm of q and k, rotation of q and k, q out, k and v into the token's cache slot -------
+// One wave per (token, head) over the q_heads + 2 * kv_heads heads of a qkv row.  Any of the three steps can be
+// switched off: q_weight/k_weight null (no norm), table null (no rotation), slot_map null (no cache write).
+template <typename T>
+__global__ void qk_norm_rope_write_kernel(const T* __restrict__ qkv, const float* __restrict__ q_weight,
+                                          const float* __restrict__ k_weight, float eps,
+                                          const float* __restrict__ table, int table_positions,
+                                          const int* __restrict__ positions, const int* __restrict__ slot_map,
+                                          T* __restrict__ k_pages, T* __restrict__ v_pages, T* __restrict__ q_out,
+                                          long tokens, int q_heads, int kv_heads, int dim, int page_size,
+                                          long num_slots) {
+  extern __shared__ float lds[];
+  const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const int heads = q_heads + 2 * kv_heads;
+  const long row = static_cast<long>(blockIdx.x) * waves + wave;
+  if (row >= tokens * heads) return;
+  const long n = row / heads;
+  const int h = static_cast<int>(row % heads);
+  const T* src = qkv + row * dim;  // a qkv row is heads * dim wide, so (n, h) starts at row * dim
+  float* mine = lds + wave * dim;
+
+  T* dst;  // where this head's result goes
+  if (h < q_heads) {
+    dst = q_out + (n * q_heads + h) * dim;
+  } else {
+    if (slot_map == nullptr) return;
+    const long slot = slot_map[n];
+    if (slot < 0 || slot >= num_slots) return;
+    const int kvh = (h - q_heads) % kv_heads;
+    const long at = ((slot / page_size * kv_heads + kvh) * page_size + slot % page_size) * dim;
+    if (h >= q_heads + kv_heads) {  // value: copied as it is
+      for (int i = lane; i < dim; i += kWave) v_pages[at + i] = src[i];
+      return;
+    }
+    dst = k_pages + at;
+  }
+
+  const float* weight = h < q_heads ? q_weight : k_weight;
+  float scale = 1.f;
+  if (weight != nullptr) {
+    float acc = 0.f;
+    for (int i = lane; i < dim; i += kWave) {
+      const float v = to_float(src[i]);
+      acc += v * v;
+    }
+    scale = rsqrtf(wave_sum(acc) / static_cast<float>(dim) + eps);
+  }
+  if (table == nullptr) {
+    for (int i = lane; i < dim; i += kWave) {
+      const float v = to_float(src[i]);
+      dst[i] = weight != nullptr ? from_float<T>(rounded<T>(v * scale) * weight[i]) : src[i];
+    }
+    return;
+  }
+  for (int i = lane; i < dim; i += kWave) {
+    const float v = to_float(src[i]);
+    mine[i] = weight != nullptr ? rounded<T>(rounded<T>(v * scale) * weight[i]) : v;
+  }
+  // the wave's own writes to its LDS row must be visible to its other lanes before the pairs are read
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const int half = dim / 2;
+  const int pos = positions[n];
+  const bool bad = pos < 0 || pos >= table_positions;
+  for (int j = lane; j < half; j += kWave) {
+    if (bad) {
+      dst[j] = from_float<T>(__uint_as_float(0x7fc00000u));
+      dst[j + half] = from_float<T>(__uint_as_float(0x7fc00000u));
+      continue;
+    }
+    const float c = table[(static_cast<long>(pos) * half + j) * 2], s = table[(static_cast<long>(pos) * half + j) * 2 + 1];
+    const float lo = mine[j], hi = mine[j + half];
+    dst[j] = from_float<T>(lo * c - hi * s);
+    dst[j + half] = from_float<T>(hi * c + lo * s);
+  }
+}
+
+inline unsigned blocks_for(long items, int per_block) { return static_cast<unsigned>((items + per_block - 1) / per_block); }
+
+}  // namespace
+
+extern "C" {
+
+int akv_embed(const int* ids, const void* table, int table_dtype, float* out, int tokens, int hidden, int vocab,
+              hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  AKV_DISPATCH(table_dtype, T,
+               embed_kernel<T><<<tokens, 256, 0, stream>>>(ids, static_cast<const T*>(table), out, hidden, vocab));
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_add_rmsnorm(float* stream_buf, const void* delta, const float* weight, float eps, void* out, int dtype,
+                    int tokens, int hidden, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  AKV_DISPATCH(dtype, T,
+               add_rmsnorm_kernel<T><<<tokens, 256, 0, stream>>>(stream_buf, static_cast<const T*>(delta), weight, eps,
+                                                                 static_cast<T*>(out), hidden));
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_rmsnorm_rows(const void* x, long token_stride, const float* weight, float eps, void* out, int dtype,
+                     long tokens, int heads, int width, hipStream_t stream) {
+  const long rows = tokens * heads;
+  if (rows <= 0) return 0;
+  AKV_DISPATCH(dtype, T,
+               rmsnorm_rows_kernel<T><<<blocks_for(rows, 4), 256, 0, stream>>>(
+                   static_cast<const T*>(x), token_stride, weight, eps, static_cast<T*>(out), rows, heads, width));
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_copy_rows(const void* x, long token_stride, void* out, int dtype, long tokens, int heads, int width,
+                  hipStream_t stream) {
+  const long rows = tokens * heads;
+  if (rows <= 0) return 0;
+  AKV_DISPATCH(dtype, T,
+               copy_rows_kernel<T><<<blocks_for(rows, 4), 256, 0, stream>>>(static_cast<const T*>(x), token_stride,
+                                                                            static_cast<T*>(out), rows, heads, width));
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_gather_rows(const float* stream_buf, const void* pending, int dtype, const int* rows, float* out, int wanted,
+                    int hidden, int tokens, hipStream_t stream) {
+  if (wanted <= 0) return 0;
+  AKV_DISPATCH(dtype, T,
+               gather_rows_kernel<T><<<wanted, 256, 0, stream>>>(stream_buf, static_cast<const T*>(pending), rows, out,
+                                                                 hidden, tokens));
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_swiglu(const void* gate_up, void* out, int dtype, long tokens, int inter, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  AKV_DISPATCH(dtype, T,
+               swiglu_kernel<T><<<blocks_for(tokens * inter, 256), 256, 0, stream>>>(
+                   static_cast<const T*>(gate_up), static_cast<T*>(out), tokens, inter));
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_rope_table(const float* inv_freq, float* table, int positions, int half, hipStream_t stream) {
+  rope_table_kernel<<<blocks_for(static_cast<long>(positions) * half, 256), 256, 0, stream>>>(inv_freq, table,
+                                                                                              positions, half);
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_rope(void* x, int dtype, const int* positions, const float* table, long tokens, int heads, int dim,
+             int table_positions, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  AKV_DISPATCH(dtype, T,
+               rope_kernel<T><<<blocks_for(tokens * heads * (dim / 2), 256), 256, 0, stream>>>(
+                   static_cast<T*>(x), positions, table, tokens, heads, dim, table_positions));
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_kv_write(const void* k, long k_stride, const void* v, long v_stride, const int* slot_map, void* k_pages,
+                 void* v_pages, int dtype, long tokens, int kv_heads, int dim, int page_size, long num_pages,
+                 hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  AKV_DISPATCH(dtype, T,
+               kv_write_kernel<T><<<blocks_for(tokens * kv_heads, 4), 256, 0, stream>>>(
+                   static_cast<const T*>(k), k_stride, static_cast<const T*>(v), v_stride, slot_map,
+                   static_cast<T*>(k_pages), static_cast<T*>(v_pages), tokens, kv_heads, dim, page_size,
+                   num_pages * page_size));
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_qk_norm_rope_write(const void* qkv, const float* q_weight, const float* k_weight, float eps,
+                           const float* table, int table_positions, const int* positions, const int* slot_map,
+                           void* k_pages, void* v_pages, void* q_out, int dtype, long tokens, int q_heads,
+                           int kv_heads, int dim, int page_size, long num_pages, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  const long rows = tokens * (q_heads + 2 * kv_heads);
+  const size_t lds = 4 * static_cast<size_t>(dim) * sizeof(float);
+  AKV_DISPATCH(dtype, T,
+               qk_norm_rope_write_kernel<T><<<blocks_for(rows, 4), 256, lds, stream>>>(
+                   static_cast<const T*>(qkv), q_weight, k_weight, eps, table, table_positions, positions, slot_map,
+                   static_cast<T*>(k_pages), static_cast<T*>(v_pages), static_cast<T*>(q_out), tokens, q_heads,
+                   kv_heads, dim, page_size, num_pages * page_size));
+  return AKV_LAUNCH_STATUS();
+}
+
+}  // extern "C"

@@ -1,0 +1,78 @@
+// Choosing the next token from float32 logits.
+//   temperature == 0: the largest logit, ties to the lowest id (the reference's argmax, ampere_kv/runner.py:346).
+//   temperature  > 0: a draw from softmax(logits / temperature) by the Gumbel-max rule:
+//                     argmax_i( logits[i] / temperature - log(-log(u_i)) ), u_i uniform in (0, 1).
+// u_i comes from Philox-4x32-10 keyed by the request's seed with counter (i, draw number), so a request's draws
+// depend on its own seed and draw count only, never on the batch it shares a step with.
+
+#include "common.h"
+#include "api.h"
+
+using namespace akv;
+
+namespace {
+
+__device__ __forceinline__ uint32_t philox_first(uint32_t c0, uint32_t c1, uint32_t k0, uint32_t k1) {
+  uint32_t c2 = 0u, c3 = 0u;
+#pragma unroll
+  for (int round = 0; round < 10; ++round) {
+    const uint64_t p0 = static_cast<uint64_t>(0xD2511F53u) * c0;
+    const uint64_t p1 = static_cast<uint64_t>(0xCD9E8D57u) * c2;
+    const uint32_t n0 = static_cast<uint32_t>(p1 >> 32) ^ c1 ^ k0;
+    const uint32_t n1 = static_cast<uint32_t>(p1);
+    const uint32_t n2 = static_cast<uint32_t>(p0 >> 32) ^ c3 ^ k1;
+    const uint32_t n3 = static_cast<uint32_t>(p0);
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  return c0;
+}
+
+__global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ logits,
+                                                      const float* __restrict__ temperature,
+                                                      const unsigned long long* __restrict__ seeds,
+                                                      const unsigned int* __restrict__ draws, int* __restrict__ out,
+                                                      int vocab) {
+  __shared__ float best_value[16];
+  __shared__ int best_index[16];
+  const int row = blockIdx.x;
+  const float* x = logits + static_cast<size_t>(row) * vocab;
+  const float t = temperature != nullptr ? temperature[row] : 0.f;
+  const uint32_t k0 = t > 0.f ? static_cast<uint32_t>(seeds[row]) : 0u;
+  const uint32_t k1 = t > 0.f ? static_cast<uint32_t>(seeds[row] >> 32) : 0u;
+  const uint32_t draw = t > 0.f ? draws[row] : 0u;
+  float value = -INFINITY;
+  int index = vocab;  // "none yet"; any real index is lower
+  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+    float score = x[i];
+    if (t > 0.f) {
+      const uint32_t bits = philox_first(static_cast<uint32_t>(i), draw, k0, k1);
+      const float u = (static_cast<float>(bits >> 8) + 0.5f) * 0x1p-24f;
+      score = score / t - logf(-logf(u));
+    }
+    if (score > value) { value = score; index = i; }  // ascending i per thread: the first maximum stays
+  }
+  for (int offset = kWave / 2; offset > 0; offset >>= 1) {
+    const float other_value = __shfl_xor(value, offset, kWave);
+    const int other_index = __shfl_xor(index, offset, kWave);
+    if (other_value > value || (other_value == value && other_index < index)) { value = other_value; index = other_index; }
+  }
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  if (lane == 0) { best_value[wave] = value; best_index[wave] = index; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < blockDim.x / kWave; ++w)
+      if (best_value[w] > value || (best_value[w] == value && best_index[w] < index)) { value = best_value[w]; index = best_index[w]; }
+    out[row] = index < vocab ? index : 0;
+  }
+}
+
+}  // namespace
+
+extern "C" int akv_sample(const float* logits, const float* temperature, const unsigned long long* seeds,
+                          const unsigned int* draws, int* out, int rows, int vocab, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  sample_kernel<<<rows, 1024, 0, stream>>>(logits, temperature, seeds, draws, out, vocab);
+  return AKV_LAUNCH_STATUS();
+}

@@ -29,6 +29,8 @@ class Engine:
         was never built), and its absence is an error, never a fallback."""
         self.spec, self.config = spec, engine_config
         self.device = torch.device(engine_config.device)
+        if self.device.type == "cuda" and self.device.index is None:
+            self.device = torch.device("cuda", 0)
         self.dtype = _TORCH_DTYPE[engine_config.dtype]
         if kernels is None:
             from ..kernels.hip import HipKernels

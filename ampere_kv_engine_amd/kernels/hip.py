@@ -1,0 +1,259 @@
+"""The engine's kernel set: thin, checking wrappers over the HIP library (`csrc/api.h`) loaded with ctypes.
+
+Every method checks on the host that shapes, dtypes, contiguity and devices are what its kernel and grid assume
+before anything is launched, because a kernel reading outside its operands can take the whole GPU down.  There is
+no other implementation behind these methods: if the library cannot be built or loaded, construction fails.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from ..csrc.build import ensure_built
+
+_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+MAX_HEAD_DIM = 256
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise KernelError(f"kernels take float32 or bfloat16 tensors, got {t.dtype}") from None
+
+
+def _ptr(t: torch.Tensor | None):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+class HipKernels:
+    name = "hip-gfx950"
+
+    def __init__(self, device: torch.device | str = "cuda:0"):
+        self.device = torch.device(device)
+        if self.device.type == "cuda" and self.device.index is None:
+            self.device = torch.device("cuda", 0)
+        if self.device.type != "cuda":
+            raise KernelError(f"the HIP kernels run on a GPU; device {self.device} is not one")
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible: the engine computes with HIP kernels only and has no CPU path")
+        path = ensure_built()
+        try:
+            self.lib = ctypes.CDLL(path)
+        except OSError as error:
+            raise KernelError(f"the kernel library {path} could not be loaded: {error}") from error
+        self.library_path = path
+        for name in ("akv_embed", "akv_add_rmsnorm", "akv_rmsnorm_rows", "akv_copy_rows", "akv_gather_rows",
+                     "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
+                     "akv_linear_tiled", "akv_attention_rows", "akv_sample"):
+            getattr(self.lib, name).restype = ctypes.c_int
+
+    # ---- helpers -----------------------------------------------------------------------------------------
+    def _stream(self):
+        return ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def _check(self, status: int, what: str) -> None:
+        if status == 0:
+            return
+        if status == -1:
+            raise KernelError(f"{what}: dtype not supported by the kernel")
+        if status == -2:
+            raise KernelError(f"{what}: sizes not supported by the kernel")
+        raise KernelError(f"{what}: launch failed with HIP error {status}")
+
+    def _dense(self, t: torch.Tensor, name: str, dtype: torch.dtype | None = None, shape: tuple | None = None):
+        if not isinstance(t, torch.Tensor) or t.device != self.device:
+            raise KernelError(f"{name} must be a tensor on {self.device}, got {getattr(t, 'device', type(t))}")
+        if not t.is_contiguous():
+            raise KernelError(f"{name} must be contiguous")
+        if dtype is not None and t.dtype != dtype:
+            raise KernelError(f"{name} must be {dtype}, got {t.dtype}")
+        if shape is not None and tuple(t.shape) != tuple(shape):
+            raise KernelError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+        return t
+
+    def check_attention_sizes(self, q_heads: int, kv_heads: int, head_dim: int, page_size: int) -> None:
+        if head_dim % 16 or not 16 <= head_dim <= MAX_HEAD_DIM:
+            raise KernelError(f"head_dim {head_dim} is not supported: the attention kernels take multiples of 16 "
+                              f"from 16 to {MAX_HEAD_DIM}")
+        if q_heads % kv_heads:
+            raise KernelError(f"q_heads {q_heads} is not a multiple of kv_heads {kv_heads}")
+        if page_size <= 0:
+            raise KernelError(f"page_size {page_size} must be positive")
+
+    # ---- token-wise --------------------------------------------------------------------------------------
+    def embed(self, ids, table, out):
+        tokens = ids.shape[0]
+        self._dense(ids, "ids", torch.int32, (tokens,))
+        self._dense(table, "table")
+        vocab, hidden = table.shape
+        self._dense(out, "out", torch.float32, (tokens, hidden))
+        self._check(self.lib.akv_embed(_ptr(ids), _ptr(table), _code(table), _ptr(out), tokens, hidden, vocab,
+                                       self._stream()), "embed")
+
+    def add_rmsnorm(self, stream, delta, weight, eps, out):
+        tokens, hidden = stream.shape
+        self._dense(stream, "stream", torch.float32)
+        self._dense(weight, "weight", torch.float32, (hidden,))
+        self._dense(out, "out", None, (tokens, hidden))
+        if delta is not None:
+            self._dense(delta, "delta", out.dtype, (tokens, hidden))
+        self._check(self.lib.akv_add_rmsnorm(_ptr(stream), _ptr(delta), _ptr(weight), ctypes.c_float(eps), _ptr(out),
+                                             _code(out), tokens, hidden, self._stream()), "add_rmsnorm")
+
+    def _rows_view(self, x, name):
+        """x [tokens, heads, width] whose last two axes are dense; returns (tokens, heads, width, token_stride)."""
+        if x.dim() != 3 or x.stride(2) != 1 or x.stride(1) != x.shape[2] or x.device != self.device:
+            raise KernelError(f"{name} must be [tokens, heads, width] on {self.device} with dense heads, got shape "
+                              f"{tuple(x.shape)} strides {x.stride()}")
+        return x.shape[0], x.shape[1], x.shape[2], x.stride(0)
+
+    def rmsnorm(self, x, weight, eps, out):
+        rows, width = x.shape
+        self._dense(x, "x")
+        self._dense(weight, "weight", torch.float32, (width,))
+        self._dense(out, "out", x.dtype, (rows, width))
+        self._check(self.lib.akv_rmsnorm_rows(_ptr(x), ctypes.c_long(width), _ptr(weight), ctypes.c_float(eps),
+                                              _ptr(out), _code(x), ctypes.c_long(rows), 1, width, self._stream()),
+                    "rmsnorm")
+
+    def rmsnorm_heads(self, x, weight, eps, out):
+        tokens, heads, width, stride = self._rows_view(x, "x")
+        self._dense(weight, "weight", torch.float32, (width,))
+        self._dense(out, "out", x.dtype, (tokens, heads, width))
+        self._check(self.lib.akv_rmsnorm_rows(_ptr(x), ctypes.c_long(stride), _ptr(weight), ctypes.c_float(eps),
+                                              _ptr(out), _code(x), ctypes.c_long(tokens), heads, width,
+                                              self._stream()), "rmsnorm_heads")
+
+    def copy_heads(self, x, out):
+        tokens, heads, width, stride = self._rows_view(x, "x")
+        self._dense(out, "out", x.dtype, (tokens, heads, width))
+        self._check(self.lib.akv_copy_rows(_ptr(x), ctypes.c_long(stride), _ptr(out), _code(x), ctypes.c_long(tokens),
+                                           heads, width, self._stream()), "copy_heads")
+
+    def gather_rows(self, stream, pending, rows, out):
+        tokens, hidden = stream.shape
+        wanted = rows.shape[0]
+        self._dense(stream, "stream", torch.float32)
+        self._dense(rows, "rows", torch.int32, (wanted,))
+        self._dense(out, "out", torch.float32, (wanted, hidden))
+        code = 0
+        if pending is not None:
+            self._dense(pending, "pending", None, (tokens, hidden))
+            code = _code(pending)
+        self._check(self.lib.akv_gather_rows(_ptr(stream), _ptr(pending), code, _ptr(rows), _ptr(out), wanted, hidden,
+                                             tokens, self._stream()), "gather_rows")
+
+    def linear(self, x, weight, out):
+        rows, k = x.shape
+        outs = weight.shape[0]
+        self._dense(x, "x")
+        self._dense(weight, "weight", None, (outs, k))
+        self._dense(out, "out", None, (rows, outs))
+        self._check(self.lib.akv_linear_tiled(_ptr(x), _code(x), _ptr(weight), _code(weight), _ptr(out), _code(out),
+                                              rows, outs, k, self._stream()), "linear")
+
+    def swiglu(self, gate_up, out):
+        tokens, inter = out.shape
+        self._dense(gate_up, "gate_up", out.dtype, (tokens, 2 * inter))
+        self._dense(out, "out")
+        self._check(self.lib.akv_swiglu(_ptr(gate_up), _ptr(out), _code(out), ctypes.c_long(tokens), inter,
+                                        self._stream()), "swiglu")
+
+    # ---- position ----------------------------------------------------------------------------------------
+    def rope_table(self, inv_freq, table):
+        positions, half, two = table.shape
+        self._dense(inv_freq, "inv_freq", torch.float32, (half,))
+        self._dense(table, "table", torch.float32, (positions, half, 2))
+        self._check(self.lib.akv_rope_table(_ptr(inv_freq), _ptr(table), positions, half, self._stream()), "rope_table")
+
+    def rope(self, x, positions, table):
+        tokens, heads, dim = x.shape
+        self._dense(x, "x")
+        self._dense(positions, "positions", torch.int32, (tokens,))
+        self._dense(table, "table", torch.float32, (table.shape[0], dim // 2, 2))
+        if dim % 2:
+            raise KernelError("rotary head width must be even")
+        self._check(self.lib.akv_rope(_ptr(x), _code(x), _ptr(positions), _ptr(table), ctypes.c_long(tokens), heads,
+                                      dim, table.shape[0], self._stream()), "rope")
+
+    # ---- cache -------------------------------------------------------------------------------------------
+    def _pages(self, k_pages, v_pages, kv_heads, dim, dtype):
+        self._dense(k_pages, "k_pages", dtype)
+        self._dense(v_pages, "v_pages", dtype, tuple(k_pages.shape))
+        if k_pages.dim() != 4 or k_pages.shape[1] != kv_heads or k_pages.shape[3] != dim:
+            raise KernelError(f"pages must be [pages, {kv_heads}, page_size, {dim}], got {tuple(k_pages.shape)}")
+        return k_pages.shape[0], k_pages.shape[2]
+
+    def kv_write(self, k, v, slot_map, k_pages, v_pages):
+        tokens, kv_heads, dim, k_stride = self._rows_view(k, "k")
+        tv, hv, dv, v_stride = self._rows_view(v, "v")
+        if (tv, hv, dv) != (tokens, kv_heads, dim) or v.dtype != k.dtype:
+            raise KernelError("k and v must agree in shape and dtype")
+        num_pages, page_size = self._pages(k_pages, v_pages, kv_heads, dim, k.dtype)
+        self._dense(slot_map, "slot_map", torch.int32, (tokens,))
+        self._check(self.lib.akv_kv_write(_ptr(k), ctypes.c_long(k_stride), _ptr(v), ctypes.c_long(v_stride),
+                                          _ptr(slot_map), _ptr(k_pages), _ptr(v_pages), _code(k),
+                                          ctypes.c_long(tokens), kv_heads, dim, page_size, ctypes.c_long(num_pages),
+                                          self._stream()), "kv_write")
+
+    def qk_norm_rope_write(self, qkv, q_weight, k_weight, eps, table, positions, slot_map, k_pages, v_pages, q_out,
+                           q_heads, kv_heads, head_dim):
+        tokens = qkv.shape[0]
+        self._dense(qkv, "qkv", None, (tokens, (q_heads + 2 * kv_heads) * head_dim))
+        self._dense(q_out, "q_out", qkv.dtype, (tokens, q_heads * head_dim))
+        if (q_weight is None) != (k_weight is None):
+            raise KernelError("q and k are normed together or not at all")
+        if q_weight is not None:
+            self._dense(q_weight, "q_weight", torch.float32, (head_dim,))
+            self._dense(k_weight, "k_weight", torch.float32, (head_dim,))
+        table_positions = 0
+        if table is not None:
+            self._dense(table, "table", torch.float32, (table.shape[0], head_dim // 2, 2))
+            table_positions = table.shape[0]
+        self._dense(positions, "positions", torch.int32, (tokens,))
+        num_pages, page_size = self._pages(k_pages, v_pages, kv_heads, head_dim, qkv.dtype)
+        if slot_map is not None:
+            self._dense(slot_map, "slot_map", torch.int32, (tokens,))
+        self._check(self.lib.akv_qk_norm_rope_write(
+            _ptr(qkv), _ptr(q_weight), _ptr(k_weight), ctypes.c_float(eps), _ptr(table), table_positions,
+            _ptr(positions), _ptr(slot_map), _ptr(k_pages), _ptr(v_pages), _ptr(q_out), _code(qkv),
+            ctypes.c_long(tokens), q_heads, kv_heads, head_dim, page_size, ctypes.c_long(num_pages), self._stream()),
+            "qk_norm_rope_write")
+
+    def attention(self, q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out):
+        tokens = q.shape[0]
+        self._dense(q, "q", None, (tokens, q_heads * head_dim))
+        self._dense(out, "out", q.dtype, (tokens, q_heads * head_dim))
+        num_pages, page_size = self._pages(k_pages, v_pages, kv_heads, head_dim, q.dtype)
+        self._dense(ctx.seq_of_token, "seq_of_token", torch.int32, (tokens,))
+        self._dense(ctx.positions, "positions", torch.int32, (tokens,))
+        self._dense(meta.block_table, "block_table", torch.int32, (ctx.num_seqs, meta.width))
+        if ctx.max_seq_len > meta.width * page_size:
+            raise KernelError(f"a request of {ctx.max_seq_len} tokens does not fit a block table of {meta.width} pages")
+        self._check(self.lib.akv_attention_rows(
+            _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(ctx.seq_of_token), _ptr(ctx.positions),
+            _ptr(meta.block_table), meta.width, _ptr(out), _code(q), ctypes.c_long(tokens), q_heads, kv_heads,
+            head_dim, page_size, ctypes.c_long(num_pages), ctypes.c_float(scale),
+            int(window) if window is not None else 0, self._stream()), "attention")
+
+    # ---- sampling ----------------------------------------------------------------------------------------
+    def sample(self, logits, temperature, seeds, draws, out):
+        rows, vocab = logits.shape
+        self._dense(logits, "logits", torch.float32)
+        self._dense(out, "out", torch.int32, (rows,))
+        if temperature is not None:
+            self._dense(temperature, "temperature", torch.float32, (rows,))
+            self._dense(seeds, "seeds", torch.int64, (rows,))
+            self._dense(draws, "draws", torch.int32, (rows,))
+        self._check(self.lib.akv_sample(_ptr(logits), _ptr(temperature), _ptr(seeds), _ptr(draws), _ptr(out), rows,
+                                        vocab, self._stream()), "sample")
+
+    def argmax(self, logits, out):
+        self.sample(logits, None, None, None, out)

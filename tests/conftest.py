@@ -1,0 +1,44 @@
+import os
+import sys
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+for path in (ROOT, os.path.dirname(os.path.abspath(__file__))):
+    if path not in sys.path:
+        sys.path.insert(0, path)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs an MI355X (run with -m gpu on the GPU box)")
+
+
+# The two tiny configurations differ in every size and option: layers, width, heads and groups (grouped vs one
+# kv head), head size (q width equal / unequal to the hidden width), feed-forward width and vocabulary (powers of
+# two vs neither), rotary base, norm eps, tied vs separate head, page size.
+TINY_A = dict(architectures=["Qwen3ForCausalLM"], vocab_size=256, hidden_size=64, num_hidden_layers=2,
+              num_attention_heads=4, num_key_value_heads=2, head_dim=16, intermediate_size=128, rope_theta=10000.0,
+              rms_norm_eps=1e-6, tie_word_embeddings=True, hidden_act="silu")
+TINY_B = dict(architectures=["Qwen3ForCausalLM"], vocab_size=379, hidden_size=96, num_hidden_layers=3,
+              num_attention_heads=6, num_key_value_heads=1, head_dim=32, intermediate_size=200, rope_theta=1000000.0,
+              rms_norm_eps=1e-5, tie_word_embeddings=False, hidden_act="silu")
+TINY = {"A": (TINY_A, 0, 16), "B": (TINY_B, 1, 8)}   # config, weight seed, page size
+
+
+@pytest.fixture(scope="session")
+def model_folders(tmp_path_factory):
+    """Model folders of the tiny configurations, written once per session into a temporary place."""
+    from ampere_kv_engine_amd.config import Qwen3Config
+    from ampere_kv_engine_amd.weights import write_random_model
+    folders = {}
+    for name, (raw, seed, _page) in TINY.items():
+        folder = str(tmp_path_factory.mktemp(f"tiny_{name}"))
+        write_random_model(folder, Qwen3Config.from_dict(raw), seed)
+        folders[name] = folder
+    return folders
+
+
+def random_ids(vocab: int, count: int, seed: int) -> list[int]:
+    generator = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (count,), generator=generator).tolist()

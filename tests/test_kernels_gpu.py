@@ -1,0 +1,362 @@
+"""Each HIP kernel alone against its plain reference (`torch_kernels.TorchKernels`, float32 torch arithmetic),
+at sizes other than the engine's: widths and vocabularies that are no power of two, head sizes 16..256, one and
+several kv heads, page sizes 4..32."""
+
+import math
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from torch_kernels import TorchKernels
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from ampere_kv_engine_amd.kernels.hip import HipKernels
+    return HipKernels("cuda:0")
+
+
+@pytest.fixture(scope="module")
+def ref():
+    return TorchKernels()
+
+
+def tol(dtype):
+    return dict(rtol=2e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=1.6e-2, atol=1e-3)
+
+
+def rand(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed(hip, ref, dtype):
+    table = rand(379, 96, dtype=dtype, seed=1)
+    ids = torch.tensor([0, 378, 5, 5, 17], dtype=torch.int32)
+    want = torch.empty(5, 96)
+    ref.embed(ids, table, want)
+    got = torch.empty(5, 96, device="cuda")
+    hip.embed(ids.cuda(), table.cuda(), got)
+    torch.testing.assert_close(got.cpu(), want, rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden", [96, 1000, 4096])
+def test_add_rmsnorm(hip, ref, dtype, hidden):
+    stream = rand(7, hidden, seed=2, scale=3.0)
+    delta = rand(7, hidden, dtype=dtype, seed=3)
+    weight = 1 + rand(hidden, seed=4, scale=0.1)
+    for d in (delta, None):
+        s_ref, s_hip = stream.clone(), stream.clone().cuda()
+        want = torch.empty(7, hidden, dtype=dtype)
+        ref.add_rmsnorm(s_ref, d, weight, 1e-5, want)
+        got = torch.empty(7, hidden, dtype=dtype, device="cuda")
+        hip.add_rmsnorm(s_hip, d.cuda() if d is not None else None, weight.cuda(), 1e-5, got)
+        torch.testing.assert_close(s_hip.cpu(), s_ref, rtol=0, atol=0)          # the residual sum itself
+        torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_heads_and_copy(hip, ref, dtype):
+    tokens, heads, width = 5, 3, 48
+    wide = rand(tokens, 7 * width, dtype=dtype, seed=5)
+    view = wide[:, 2 * width:5 * width].unflatten(1, (heads, width))           # a strided view, as inside qkv
+    weight = 1 + rand(width, seed=6, scale=0.1)
+    want = torch.empty(tokens, heads, width, dtype=dtype)
+    ref.rmsnorm_heads(view, weight, 1e-6, want)
+    got = torch.empty(tokens, heads, width, dtype=dtype, device="cuda")
+    hip.rmsnorm_heads(wide.cuda()[:, 2 * width:5 * width].unflatten(1, (heads, width)), weight.cuda(), 1e-6, got)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dtype))
+    copied = torch.empty(tokens, heads, width, dtype=dtype, device="cuda")
+    hip.copy_heads(wide.cuda()[:, 2 * width:5 * width].unflatten(1, (heads, width)), copied)
+    torch.testing.assert_close(copied.cpu(), view.contiguous(), rtol=0, atol=0)
+    flat = rand(11, 200, dtype=dtype, seed=7)
+    w2 = 1 + rand(200, seed=8, scale=0.1)
+    want2 = torch.empty_like(flat)
+    ref.rmsnorm(flat, w2, 1e-5, want2)
+    got2 = torch.empty(11, 200, dtype=dtype, device="cuda")
+    hip.rmsnorm(flat.cuda(), w2.cuda(), 1e-5, got2)
+    torch.testing.assert_close(got2.cpu().float(), want2.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gather_rows(hip, ref, dtype):
+    stream, pending = rand(9, 96, seed=9), rand(9, 96, dtype=dtype, seed=10)
+    rows = torch.tensor([8, 0, 3, 3], dtype=torch.int32)
+    for p in (pending, None):
+        want = torch.empty(4, 96)
+        ref.gather_rows(stream, p, rows, want)
+        got = torch.empty(4, 96, device="cuda")
+        hip.gather_rows(stream.cuda(), p.cuda() if p is not None else None, rows.cuda(), got)
+        torch.testing.assert_close(got.cpu(), want, rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("x_dtype,w_dtype,y_dtype", [
+    (torch.float32, torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16, torch.bfloat16),
+    (torch.bfloat16, torch.bfloat16, torch.float32), (torch.float32, torch.bfloat16, torch.float32),
+    (torch.bfloat16, torch.float32, torch.bfloat16)])
+@pytest.mark.parametrize("rows,outs,k", [(1, 379, 96), (5, 64, 200), (70, 130, 33), (129, 257, 1000)])
+def test_linear(hip, ref, x_dtype, w_dtype, y_dtype, rows, outs, k):
+    x, w = rand(rows, k, dtype=x_dtype, seed=11), rand(outs, k, dtype=w_dtype, seed=12, scale=0.05)
+    want = torch.empty(rows, outs, dtype=y_dtype)
+    ref.linear(x, w, want)
+    got = torch.empty(rows, outs, dtype=y_dtype, device="cuda")
+    hip.linear(x.cuda(), w.cuda(), got)
+    t = dict(rtol=1e-4, atol=1e-5) if y_dtype == torch.float32 else tol(torch.bfloat16)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **t)
+
+
+def test_linear_rows_do_not_depend_on_the_batch(hip):
+    """Float32: a row's result is bit-identical whether it is computed alone or among others."""
+    x, w = rand(67, 300, seed=13).cuda(), rand(150, 300, seed=14).cuda()
+    whole = torch.empty(67, 150, device="cuda")
+    hip.linear(x, w, whole)
+    for row in (0, 1, 63, 64, 66):
+        alone = torch.empty(1, 150, device="cuda")
+        hip.linear(x[row:row + 1].contiguous(), w, alone)
+        assert torch.equal(alone[0], whole[row])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu(hip, ref, dtype):
+    gate_up = rand(6, 2 * 200, dtype=dtype, seed=15, scale=2.0)
+    want = torch.empty(6, 200, dtype=dtype)
+    ref.swiglu(gate_up, want)
+    got = torch.empty(6, 200, dtype=dtype, device="cuda")
+    hip.swiglu(gate_up.cuda(), got)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dim,theta", [(16, 1e4), (32, 1e6), (128, 1e6), (80, 5e5)])
+def test_rope_table_and_rope(hip, ref, dim, theta):
+    exponent = torch.arange(0, dim, 2, dtype=torch.int64).float() / dim
+    inv_freq = 1.0 / (theta ** exponent)
+    want = torch.empty(9000, dim // 2, 2)
+    ref.rope_table(inv_freq, want)
+    got = torch.empty(9000, dim // 2, 2, device="cuda")
+    hip.rope_table(inv_freq.cuda(), got)
+    torch.testing.assert_close(got.cpu(), want, rtol=0, atol=2e-6)       # sin/cos of angles up to 9000 rad
+    for dtype in DTYPES:
+        x = rand(5, 3, dim, dtype=dtype, seed=16)
+        positions = torch.tensor([0, 1, 17, 4095, 8999], dtype=torch.int32)
+        x_ref, x_hip = x.clone(), x.clone().cuda()
+        ref.rope(x_ref, positions, want)
+        hip.rope(x_hip, positions.cuda(), got)
+        torch.testing.assert_close(x_hip.cpu().float(), x_ref.float(), **tol(dtype))
+        torch.testing.assert_close(x_hip.cpu()[0], x[0], rtol=0, atol=0)          # position 0 leaves x as it is
+
+
+def _pages(num_pages, kv_heads, page_size, dim, dtype):
+    k = torch.full((num_pages, kv_heads, page_size, dim), float("nan"), dtype=dtype)
+    return k, k.clone()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("q_heads,kv_heads,dim,page_size", [(4, 2, 16, 16), (6, 1, 32, 8), (8, 8, 128, 4), (5, 5, 80, 32),
+                                                             (2, 1, 256, 16)])
+@pytest.mark.parametrize("normed,rotated,written", [(True, True, True), (False, True, True), (True, False, True),
+                                                    (True, True, False)])
+def test_qk_norm_rope_write(hip, ref, dtype, q_heads, kv_heads, dim, page_size, normed, rotated, written):
+    tokens, num_pages = 7, 6
+    qkv = rand(tokens, (q_heads + 2 * kv_heads) * dim, dtype=dtype, seed=17)
+    qw, kw = (1 + rand(dim, seed=18, scale=0.1), 1 + rand(dim, seed=19, scale=0.1)) if normed else (None, None)
+    exponent = torch.arange(0, dim, 2, dtype=torch.int64).float() / dim
+    table = torch.empty(300, dim // 2, 2)
+    ref.rope_table(1.0 / (1e4 ** exponent), table)
+    positions = torch.tensor([0, 1, 2, 100, 101, 299, 7], dtype=torch.int32)
+    # slots in reversed page order, crossing a page edge, leaving the others untouched
+    slots = torch.tensor([5 * page_size + page_size - 1, 4 * page_size, 4 * page_size + 1, 2 * page_size + 3 % page_size,
+                          1 * page_size, 0, 3 * page_size + page_size - 1], dtype=torch.int32)
+    k_ref, v_ref = _pages(num_pages, kv_heads, page_size, dim, dtype)
+    q_ref = torch.empty(tokens, q_heads * dim, dtype=dtype)
+    ref.qk_norm_rope_write(qkv, qw, kw, 1e-6, table if rotated else None, positions, slots if written else None,
+                           k_ref, v_ref, q_ref, q_heads, kv_heads, dim)
+    k_hip, v_hip = (t.cuda() for t in _pages(num_pages, kv_heads, page_size, dim, dtype))
+    q_hip = torch.empty(tokens, q_heads * dim, dtype=dtype, device="cuda")
+    cu = lambda t: t.cuda() if t is not None else None
+    hip.qk_norm_rope_write(qkv.cuda(), cu(qw), cu(kw), 1e-6, cu(table) if rotated else None, positions.cuda(),
+                           slots.cuda() if written else None, k_hip, v_hip, q_hip, q_heads, kv_heads, dim)
+    torch.testing.assert_close(q_hip.cpu().float(), q_ref.float(), **tol(dtype))
+    torch.testing.assert_close(k_hip.cpu().float(), k_ref.float(), equal_nan=True, **tol(dtype))
+    torch.testing.assert_close(v_hip.cpu().float(), v_ref.float(), equal_nan=True, rtol=0, atol=0)   # v: bitwise copy
+    assert torch.isnan(k_hip.cpu().float()).sum() == torch.isnan(k_ref.float()).sum()   # nothing else was written
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_kv_write(hip, ref, dtype):
+    tokens, kv_heads, dim, page_size = 5, 3, 48, 8
+    k = rand(tokens, kv_heads, dim, dtype=dtype, seed=20)
+    wide = rand(tokens, 5 * kv_heads * dim, dtype=dtype, seed=21)
+    v = wide[:, kv_heads * dim:2 * kv_heads * dim].unflatten(1, (kv_heads, dim))
+    slots = torch.tensor([15, 16, 0, 31, 9], dtype=torch.int32)
+    k_ref, v_ref = _pages(4, kv_heads, page_size, dim, dtype)
+    ref.kv_write(k, v, slots, k_ref, v_ref)
+    k_hip, v_hip = (t.cuda() for t in _pages(4, kv_heads, page_size, dim, dtype))
+    hip.kv_write(k.cuda(), wide.cuda()[:, kv_heads * dim:2 * kv_heads * dim].unflatten(1, (kv_heads, dim)), slots.cuda(),
+                 k_hip, v_hip)
+    torch.testing.assert_close(k_hip.cpu().float(), k_ref.float(), equal_nan=True, rtol=0, atol=0)
+    torch.testing.assert_close(v_hip.cpu().float(), v_ref.float(), equal_nan=True, rtol=0, atol=0)
+
+
+def _attention_case(dtype, q_heads, kv_heads, dim, page_size, portions, window, seed, spike=None):
+    """`portions` = [(history, new tokens)] per request.  Pages are handed out in a scrambled order; pages a
+    window has passed and table padding hold -1; unwritten slots hold NaN."""
+    g = torch.Generator().manual_seed(seed)
+    lengths = [h + n for h, n in portions]
+    pages_of = [math.ceil(l / page_size) for l in lengths]
+    num_pages = sum(pages_of) + 3
+    order = torch.randperm(num_pages, generator=g).tolist()
+    k_pages, v_pages = _pages(num_pages, kv_heads, page_size, dim, dtype)
+    width = max(pages_of) + 1
+    table = torch.full((len(portions), width), -1, dtype=torch.int32)
+    keys, values = [], []
+    cursor = 0
+    for r, length in enumerate(lengths):
+        k = torch.randn(length, kv_heads, dim, generator=g).to(dtype)
+        v = torch.randn(length, kv_heads, dim, generator=g).to(dtype)
+        if spike is not None and r == spike[0]:
+            k[spike[1]] *= 6.0       # one far key stands out of hundreds
+        keys.append(k)
+        values.append(v)
+        history = portions[r][0]
+        lowest = 0 if window is None else max(0, history - window + 1)
+        for p in range(pages_of[r]):
+            page = order[cursor]
+            cursor += 1
+            if (p + 1) * page_size <= lowest:
+                continue               # wholly passed by the window: given back, entry stays -1
+            table[r, p] = page
+            lo, hi = p * page_size, min((p + 1) * page_size, length)
+            k_pages[page, :, :hi - lo] = k[lo:hi].transpose(0, 1)
+            v_pages[page, :, :hi - lo] = v[lo:hi].transpose(0, 1)
+    tokens = sum(n for _, n in portions)
+    q = torch.randn(tokens, q_heads * dim, generator=g).to(dtype)
+    if spike is not None:
+        r, at = spike
+        first = sum(n for _, n in portions[:r])
+        q[first:first + portions[r][1]] = (keys[r][at].float().repeat(q_heads // kv_heads, 1).reshape(-1) * 2.0).to(dtype)
+    q_start = [0]
+    for _, n in portions:
+        q_start.append(q_start[-1] + n)
+    positions = torch.cat([torch.arange(h, h + n) for h, n in portions]).int()
+    seq_of_token = torch.cat([torch.full((n,), r) for r, (_, n) in enumerate(portions)]).int()
+    ctx = SimpleNamespace(num_seqs=len(portions), num_tokens=tokens, host_q_start=q_start, host_seq_lens=lengths,
+                          positions=positions, seq_of_token=seq_of_token, max_seq_len=max(lengths),
+                          num_decode_seqs=0, max_new_tokens=max(n for _, n in portions))
+    meta = SimpleNamespace(block_table=table, width=width, window=window)
+    return q, k_pages, v_pages, ctx, meta, keys, values
+
+
+def _to_cuda(ctx, meta):
+    c = SimpleNamespace(**vars(ctx))
+    c.positions, c.seq_of_token = ctx.positions.cuda(), ctx.seq_of_token.cuda()
+    m = SimpleNamespace(**vars(meta))
+    m.block_table = meta.block_table.cuda()
+    return c, m
+
+
+ATTENTION_SIZES = [(4, 2, 16, 16), (6, 1, 32, 8), (8, 2, 128, 16), (5, 5, 80, 4), (3, 1, 256, 32)]
+PORTIONS = [[(0, 1)], [(0, 33)], [(64, 1), (17, 1), (0, 1)], [(5, 7), (63, 2), (130, 1), (0, 70)]]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("q_heads,kv_heads,dim,page_size", ATTENTION_SIZES)
+@pytest.mark.parametrize("portions", PORTIONS)
+@pytest.mark.parametrize("window", [None, 24])
+def test_attention(hip, ref, dtype, q_heads, kv_heads, dim, page_size, portions, window):
+    q, k_pages, v_pages, ctx, meta, _, _ = _attention_case(dtype, q_heads, kv_heads, dim, page_size, portions, window, 22)
+    want = torch.empty_like(q)
+    ref.attention(q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, dim, dim ** -0.5, window, want)
+    cctx, cmeta = _to_cuda(ctx, meta)
+    got = torch.empty_like(q, device="cuda")
+    hip.attention(q.cuda(), k_pages.cuda(), v_pages.cuda(), cctx, cmeta, q_heads, kv_heads, dim, dim ** -0.5, window, got)
+    assert not torch.isnan(got).any()
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_finds_a_far_key(hip, ref, dtype):
+    """One key among a thousand matches the query: the output must be (nearly) that key's value."""
+    portions = [(1000, 1), (900, 3)]
+    for spike in ((0, 3), (1, 517)):
+        q, k_pages, v_pages, ctx, meta, keys, values = _attention_case(dtype, 4, 2, 64, 16, portions, None, 23, spike)
+        cctx, cmeta = _to_cuda(ctx, meta)
+        got = torch.empty_like(q, device="cuda")
+        hip.attention(q.cuda(), k_pages.cuda(), v_pages.cuda(), cctx, cmeta, 4, 2, 64, 64 ** -0.5, None, got)
+        want = torch.empty_like(q)
+        ref.attention(q, k_pages, v_pages, ctx, meta, 4, 2, 64, 64 ** -0.5, None, want)
+        torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dtype))
+        r, at = spike
+        first = ctx.host_q_start[r]
+        picked = got.cpu().float()[first].reshape(4, 64)
+        torch.testing.assert_close(picked[0], values[r][at, 0].float(), rtol=0.05, atol=0.05)
+        torch.testing.assert_close(picked[3], values[r][at, 1].float(), rtol=0.05, atol=0.05)
+
+
+def _philox_first(c0, c1, k0, k1):
+    import numpy as np
+    c0, c1 = np.asarray(c0, dtype=np.uint64), np.uint64(c1)
+    c2, c3 = np.zeros_like(c0), np.zeros_like(c0)
+    c1 = np.full_like(c0, c1)
+    k0, k1 = np.uint64(k0), np.uint64(k1)
+    mask = np.uint64(0xFFFFFFFF)
+    for _ in range(10):
+        p0, p1 = np.uint64(0xD2511F53) * c0, np.uint64(0xCD9E8D57) * c2
+        c0, c1, c2, c3 = ((p1 >> np.uint64(32)) ^ c1 ^ k0) & mask, p1 & mask, ((p0 >> np.uint64(32)) ^ c3 ^ k1) & mask, p0 & mask
+        k0, k1 = (k0 + np.uint64(0x9E3779B9)) & mask, (k1 + np.uint64(0xBB67AE85)) & mask
+    return c0
+
+
+def test_sample(hip):
+    import numpy as np
+    vocab = 1531
+    logits = rand(6, vocab, seed=24, scale=2.0)
+    logits[1, 100] = logits[1, 900] = 50.0                                  # a tie: the lowest id wins
+    logits[5] = logits[2]
+    temperature = torch.tensor([0.0, 0.0, 0.7, 0.7, 1.3, 0.7])
+    seeds = torch.tensor([1, 2, 3, 3, (5 << 33) + 9, 3], dtype=torch.int64)
+    draws = torch.tensor([0, 0, 0, 1, 7, 0], dtype=torch.int32)
+    out = torch.empty(6, dtype=torch.int32, device="cuda")
+    hip.sample(logits.cuda(), temperature.cuda(), seeds.cuda(), draws.cuda(), out)
+    out = out.cpu().tolist()
+    assert out[0] == int(logits[0].argmax()) and out[1] == 100
+    assert out[2] == out[5]                                                   # same seed and draw: same token
+    for row in (2, 3, 4):
+        bits = _philox_first(np.arange(vocab), int(draws[row]), int(seeds[row]) & 0xFFFFFFFF, int(seeds[row]) >> 32)
+        u = ((bits >> np.uint64(8)).astype(np.float64) + 0.5) * 2.0 ** -24
+        scores = logits[row].double().numpy() / float(temperature[row]) - np.log(-np.log(u))
+        assert scores[out[row]] >= scores.max() - 1e-4
+    greedy = torch.empty(6, dtype=torch.int32, device="cuda")
+    hip.argmax(logits.cuda(), greedy)
+    assert greedy.cpu().tolist() == [int(r.argmax()) if i != 1 else 100 for i, r in enumerate(logits)]
+
+
+def test_sampling_follows_the_distribution(hip):
+    probs = torch.tensor([0.5, 0.25, 0.125, 0.125])
+    rows = 4000
+    logits = probs.log().repeat(rows, 1).cuda()
+    out = torch.empty(rows, dtype=torch.int32, device="cuda")
+    hip.sample(logits, torch.ones(rows, device="cuda"), torch.full((rows,), 11, dtype=torch.int64, device="cuda"),
+               torch.arange(rows, dtype=torch.int32, device="cuda"), out)
+    freq = torch.bincount(out.cpu().long(), minlength=4).float() / rows
+    assert (freq - probs).abs().max() < 0.03
+
+
+def test_sizes_are_refused_not_miscomputed(hip):
+    from ampere_kv_engine_amd.kernels.hip import KernelError
+    with pytest.raises(KernelError):
+        hip.check_attention_sizes(4, 2, 24, 16)
+    with pytest.raises(KernelError):
+        hip.check_attention_sizes(4, 3, 32, 16)
+    with pytest.raises(KernelError):
+        hip.check_attention_sizes(4, 2, 512, 16)
+    with pytest.raises(KernelError):
+        hip.linear(torch.zeros(2, 3), torch.zeros(4, 3, device="cuda"), torch.zeros(2, 4, device="cuda"))
+    with pytest.raises(KernelError):
+        hip.linear(torch.zeros(2, 3, device="cuda"), torch.zeros(4, 5, device="cuda"), torch.zeros(2, 4, device="cuda"))
