@@ -38,8 +38,9 @@ class Attention(Part):
         self.k_norm = build_part("norm", norm_spec, runtime) if norm_spec is not None else None
         self.position = build_part("position", spec["position"], runtime)
         # One fused kernel does norm, rotation and the cache write when the parts are the kinds it knows.
-        self.fused = (isinstance(self.position, (RotaryHalf, NoPosition))
-                      and (self.q_norm is None or isinstance(self.q_norm, RMSNorm)))
+        # (exact types: a subclass may compute something else)
+        self.fused = (type(self.position) in (RotaryHalf, NoPosition)
+                      and (self.q_norm is None or type(self.q_norm) is RMSNorm))
         runtime.kernels.check_attention_sizes(self.q_heads, self.kv_heads, self.head_dim, runtime.page_size)
 
     # ---- weights ----------------------------------------------------------------------------------

@@ -1,0 +1,59 @@
+"""Choosing next tokens from a step's logits.
+
+The reference samples greedily only (`logits.argmax()`, ampere_kv/runner.py:346; ampere_kv/scheduler.py:142).
+Here a request has a temperature: 0 is that same argmax (ties to the lowest id), above 0 a draw from
+softmax(logits / temperature).  Draws are numbered per request and keyed by the request's seed, so what a request
+generates does not depend on which other requests share its steps.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+
+@dataclass
+class SamplingParams:
+    temperature: float = 0.0
+    seed: int = 0
+
+    def __post_init__(self):
+        if self.temperature < 0:
+            raise ValueError(f"temperature must not be negative, got {self.temperature}")
+        if not 0 <= self.seed < 2 ** 63:
+            raise ValueError("seed must fit in 63 bits")
+
+
+class Sampler:
+    def __init__(self, kernels, device, max_rows: int):
+        self.kernels, self.device, self.max_rows = kernels, torch.device(device), max_rows
+        pin = self.device.type == "cuda"
+        self._temperature = torch.empty(max_rows, dtype=torch.float32, device=self.device)
+        self._seeds = torch.empty(max_rows, dtype=torch.int64, device=self.device)
+        self._draws = torch.empty(max_rows, dtype=torch.int32, device=self.device)
+        self._out = torch.empty(max_rows, dtype=torch.int32, device=self.device)
+        self._host_t = torch.empty(max_rows, dtype=torch.float32, pin_memory=pin)
+        self._host_s = torch.empty(max_rows, dtype=torch.int64, pin_memory=pin)
+        self._host_d = torch.empty(max_rows, dtype=torch.int32, pin_memory=pin)
+
+    def sample(self, logits: torch.Tensor, params: list[SamplingParams], draws: list[int]) -> list[int]:
+        """logits float32 [rows, vocab]; `draws[i]` is how many tokens request i has drawn before.  Returns the
+        chosen ids (one device-to-host copy for the whole batch)."""
+        rows = logits.shape[0]
+        if rows != len(params) or rows != len(draws):
+            raise ValueError("one SamplingParams and one draw count per row of logits")
+        if rows > self.max_rows:
+            raise ValueError(f"{rows} rows to sample; the sampler was built for {self.max_rows}")
+        out = self._out[:rows]
+        if all(p.temperature == 0 for p in params):
+            self.kernels.sample(logits, None, None, None, out)
+        else:
+            for i, (p, d) in enumerate(zip(params, draws)):
+                self._host_t[i], self._host_s[i], self._host_d[i] = p.temperature, p.seed, d
+            # the staging tensors are rewritten next call, so these copies must have been read by then
+            self._temperature[:rows].copy_(self._host_t[:rows])
+            self._seeds[:rows].copy_(self._host_s[:rows])
+            self._draws[:rows].copy_(self._host_d[:rows])
+            self.kernels.sample(logits, self._temperature[:rows], self._seeds[:rows], self._draws[:rows], out)
+        return out.tolist()

@@ -1,0 +1,151 @@
+"""The cache manager's bookkeeping: no page lost, held twice or freed twice, under random orders of requests;
+windows give pages back mid-request; slots for per-request state."""
+
+import random
+
+import pytest
+import torch
+
+from ampere_kv_engine_amd.cache import (RELEASED, BlockTable, CacheManager, PageAllocator, PagePoolExhausted,
+                                        SlotsExhausted, SlotTable)
+from ampere_kv_engine_amd.parts.base import PagedKV, SlotState
+
+
+def test_pool_is_a_stack_and_refuses_double_free():
+    pool = PageAllocator(4)
+    assert [pool.allocate() for _ in range(4)] == [0, 1, 2, 3]            # reference: block_pool.py:12-13
+    with pytest.raises(PagePoolExhausted):
+        pool.allocate()
+    pool.free(1)
+    pool.free(3)
+    assert pool.allocate() == 3 and pool.allocate() == 1                      # freed pages are reused first, last in first out
+    pool.free(2)
+    with pytest.raises(ValueError):
+        pool.free(2)
+    with pytest.raises(ValueError):
+        pool.free(17)
+
+
+def test_block_table_appends_all_or_nothing_and_locates():
+    pool = PageAllocator(3)
+    table = BlockTable(pool, 4)
+    assert table.append_tokens(4) == 0 and table.pages == (0,)              # length 4 needs one page of 4
+    assert table.append_tokens(1) == 4 and table.pages == (0, 1)            # length 5 needs two
+    assert table.locate(4) == (1, 0) and table.locate(3) == (0, 3)
+    with pytest.raises(ValueError):
+        table.locate(5)                                                       # beyond the registered length
+    with pytest.raises(PagePoolExhausted):
+        table.append_tokens(8)                                                # needs 2 more pages, 1 free: nothing taken
+    assert table.length == 5 and pool.num_free == 1
+    table.release()
+    table.release()                                                           # harmless
+    assert pool.num_free == 3 and table.length == 0
+
+
+def test_window_gives_pages_back_while_the_request_lives():
+    pool = PageAllocator(8)
+    table = BlockTable(pool, 4, window=6)
+    table.append_tokens(16)                     # a whole 16-token portion needs all its keys: 4 pages
+    assert table.num_held == 4
+    table.append_tokens(1)                      # query at 16 reads keys 11..16: pages 0 and 1 (keys 0..7) are passed
+    assert table.pages[:2] == (RELEASED, RELEASED) and table.num_held == 3 and pool.num_free == 5
+    with pytest.raises(ValueError):
+        table.locate(3)
+    assert table.locate(16) == (table.pages[4], 0)
+    for _ in range(40):
+        table.append_tokens(1)
+    assert table.num_held <= 3                  # never more than the window needs
+    table.release()
+    assert pool.num_free == 8
+
+
+def _manager(**kw):
+    needs = {0: PagedKV(2, 16), 1: PagedKV(2, 16), 2: PagedKV(2, 16, window=12), 3: SlotState((3, 5)), 4: None}
+    return CacheManager(needs, page_size=4, num_pages=24, max_seqs=3, dtype=torch.float32, **kw)
+
+
+def test_groups_by_need_and_tensor_shapes():
+    m = _manager()
+    assert [g.layers for g in m.groups] == [[0, 1], [2]]
+    assert m.groups[0].pages.shape == (2, 2, 24, 2, 4, 16) and m.groups[1].pages.shape == (1, 2, 24, 2, 4, 16)
+    assert m.layer_cache[1].k.shape == (24, 2, 4, 16) and m.layer_cache[1].k.data_ptr() == m.groups[0].pages[1, 0].data_ptr()
+    assert m.layer_cache[3].state.shape == (3, 3, 5) and m.layer_cache[4].group is None
+    assert m.bytes_per_token() == (2 * 2 + 2 * 1) * 2 * 16 * 4
+
+
+def test_slots_are_zeroed_when_taken_again():
+    m = _manager()
+    a = m.open("a")
+    m.layer_cache[3].state[a.slot] = 7.0
+    m.close(a)
+    b = m.open("b")
+    assert b.slot == a.slot and float(m.layer_cache[3].state[b.slot].abs().sum()) == 0.0
+    m.open("c"), m.open("d")
+    with pytest.raises(SlotsExhausted):
+        m.open("e")
+    with pytest.raises(ValueError):
+        m.open("c")
+
+
+def test_reserve_is_all_or_nothing_across_groups():
+    m = _manager()
+    a, b = m.open("a"), m.open("b")
+    assert m.reserve(a, 60) == 0               # 15 pages in each group
+    assert m.num_free_pages == [9, 9]
+    with pytest.raises(PagePoolExhausted):
+        m.reserve(b, 40)                       # needs 10 pages
+    assert b.length == 0 and all(t.length == 0 for t in b.tables) and m.num_free_pages == [9, 9]
+    m.close(a)
+    m.close(a)
+    m.close(b)
+    assert m.num_free_pages == [24, 24] and m.slots.num_free == 3
+    with pytest.raises(ValueError):
+        m.reserve(a, 1)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_no_page_lost_held_twice_or_freed_twice_under_random_orders(seed):
+    rng = random.Random(seed)
+    m = _manager(allocate_tensors=False)
+    live, counter = {}, 0
+    for _ in range(600):
+        action = rng.random()
+        if action < 0.25 and m.slots.num_free:
+            counter += 1
+            live[f"r{counter}"] = m.open(f"r{counter}")
+        elif action < 0.85 and live:
+            seq = live[rng.choice(sorted(live))]
+            count = rng.choice((1, 1, 1, 2, 3, 7, 13))
+            before = (seq.length, [t.pages for t in seq.tables], m.num_free_pages)
+            try:
+                m.reserve(seq, count)
+            except PagePoolExhausted:
+                assert (seq.length, [t.pages for t in seq.tables], m.num_free_pages) == before
+        elif live:
+            name = rng.choice(sorted(live))
+            m.close(live.pop(name))
+        # invariants
+        for group in m.groups:
+            held = [p for s in live.values() for p in s.tables[group.index].pages if p != RELEASED]
+            assert len(held) == len(set(held)), "a page is held twice"
+            assert len(held) + group.allocator.num_free == m.num_pages, "a page was lost"
+            assert all(group.allocator.is_held(p) for p in held)
+        for s in live.values():
+            assert all(t.length == s.length for t in s.tables)
+            full, windowed = s.tables
+            assert full.num_held == -(-s.length // 4)
+            assert windowed.num_held <= -(-(12 + 13) // 4) + 1
+        assert len({s.slot for s in live.values()}) == len(live) == m.max_seqs - m.slots.num_free
+    for seq in live.values():
+        m.close(seq)
+    assert m.num_free_pages == [24, 24] and m.slots.num_free == 3
+
+
+def test_slot_table():
+    slots = SlotTable(2)
+    a, b = slots.take(), slots.take()
+    assert (a, b) == (0, 1)
+    slots.give_back(a)
+    with pytest.raises(ValueError):
+        slots.give_back(a)
+    assert slots.take() == a

@@ -1,0 +1,82 @@
+"""Typed configuration from config.json keys, and the architecture registry."""
+
+import json
+
+import pytest
+
+from ampere_kv_engine_amd.config import (ConfigError, EngineConfig, Qwen3Config, known_architectures, load_config,
+                                         register_architecture)
+from conftest import TINY_A, TINY_B
+
+
+def test_reads_every_size_from_the_keys():
+    a, b = Qwen3Config.from_dict(TINY_A), Qwen3Config.from_dict(TINY_B)
+    assert (a.num_hidden_layers, a.hidden_size, a.num_attention_heads, a.num_key_value_heads, a.head_dim) == (2, 64, 4, 2, 16)
+    assert (a.intermediate_size, a.vocab_size, a.rope_theta, a.rms_norm_eps, a.tie_word_embeddings) == (128, 256, 1e4, 1e-6, True)
+    assert (b.q_size, b.kv_size, b.group_size) == (192, 32, 6) and b.q_size != b.hidden_size
+    assert not b.tie_word_embeddings and b.rms_norm_eps == 1e-5 and b.rope_theta == 1e6
+
+
+def test_head_dim_defaults_to_hidden_over_heads_and_kv_heads_to_heads():
+    raw = {k: v for k, v in TINY_A.items() if k not in ("head_dim", "num_key_value_heads")}
+    c = Qwen3Config.from_dict(raw)
+    assert c.head_dim == 16 and c.num_key_value_heads == 4
+
+
+@pytest.mark.parametrize("key", ["vocab_size", "hidden_size", "num_hidden_layers", "num_attention_heads",
+                                 "intermediate_size", "rope_theta", "rms_norm_eps"])
+def test_a_missing_size_is_an_error_not_a_default(key):
+    raw = {k: v for k, v in TINY_B.items() if k != key}
+    with pytest.raises(ConfigError, match=key):
+        Qwen3Config.from_dict(raw)
+
+
+@pytest.mark.parametrize("change,match", [
+    ({"hidden_act": "gelu"}, "hidden_act"), ({"use_sliding_window": True, "sliding_window": 128}, "sliding"),
+    ({"rope_scaling": {"type": "yarn"}}, "rope_scaling"), ({"attention_bias": True}, "attention_bias"),
+    ({"num_key_value_heads": 4}, "multiple"), ({"head_dim": 31}, "odd"), ({"vocab_size": -1}, "vocab_size"),
+    ({"num_hidden_layers": 2.5}, "num_hidden_layers"), ({"rope_theta": 0}, "rope_theta")])
+def test_unsupported_options_are_refused(change, match):
+    with pytest.raises(ConfigError, match=match):
+        Qwen3Config.from_dict({**TINY_B, **change})
+
+
+def test_round_trip_through_config_json(tmp_path):
+    c = Qwen3Config.from_dict({**TINY_B, "eos_token_id": [7, 9]})
+    (tmp_path / "config.json").write_text(json.dumps(c.to_dict()))
+    again = load_config(str(tmp_path))
+    assert again == c and again.eos_token_ids == (7, 9)
+    (tmp_path / "generation_config.json").write_text(json.dumps({"eos_token_id": 3}))
+    assert load_config(str(tmp_path)).eos_token_ids == (3,)
+
+
+def test_registry_chooses_by_architecture_name(tmp_path):
+    assert "Qwen3ForCausalLM" in known_architectures()
+    (tmp_path / "config.json").write_text(json.dumps({**TINY_A, "architectures": ["NoSuchModel"]}))
+    with pytest.raises(ConfigError, match="NoSuchModel.*Qwen3ForCausalLM"):
+        load_config(str(tmp_path))
+    (tmp_path / "config.json").write_text(json.dumps({k: v for k, v in TINY_A.items() if k != "architectures"}))
+    with pytest.raises(ConfigError, match="architectures"):
+        load_config(str(tmp_path))
+    with pytest.raises(ValueError, match="already registered"):
+        register_architecture("Qwen3ForCausalLM", Qwen3Config)
+
+
+def test_model_spec_carries_sizes_layer_by_layer():
+    spec = Qwen3Config.from_dict(TINY_B).to_model_spec()
+    assert len(spec.layers) == 3 and [e.layer for e in spec.run_order] == [0, 1, 2]
+    mixer = spec.layers[1].mixer
+    assert mixer.kind == "attention" and mixer["q_heads"] == 6 and mixer["kv_heads"] == 1 and mixer["head_dim"] == 32
+    assert mixer["position"].kind == "rope_half" and mixer["position"]["theta"] == 1e6
+    assert mixer["qk_norm"]["eps"] == 1e-5 and mixer["scale"] == 32 ** -0.5
+    assert spec.layers[2].feed_forward["intermediate_size"] == 200 and spec.layers[2].prefix == "model.layers.2."
+    assert spec.head["tied_to"] is None
+    assert Qwen3Config.from_dict(TINY_A).to_model_spec().head["tied_to"] == "model.embed_tokens.weight"
+
+
+def test_engine_config_checks_its_numbers():
+    with pytest.raises(ValueError):
+        EngineConfig(dtype="float16")
+    with pytest.raises(ValueError):
+        EngineConfig(page_size=0)
+    assert EngineConfig(page_size=16, max_seq_len=100).max_pages_per_seq == 7

@@ -8,7 +8,7 @@ from types import SimpleNamespace
 import pytest
 import torch
 
-from torch_kernels import TorchKernels
+from torch_kernels import TorchKernels, philox_first
 
 pytestmark = pytest.mark.gpu
 
@@ -299,20 +299,6 @@ def test_attention_finds_a_far_key(hip, ref, dtype):
         torch.testing.assert_close(picked[3], values[r][at, 1].float(), rtol=0.05, atol=0.05)
 
 
-def _philox_first(c0, c1, k0, k1):
-    import numpy as np
-    c0, c1 = np.asarray(c0, dtype=np.uint64), np.uint64(c1)
-    c2, c3 = np.zeros_like(c0), np.zeros_like(c0)
-    c1 = np.full_like(c0, c1)
-    k0, k1 = np.uint64(k0), np.uint64(k1)
-    mask = np.uint64(0xFFFFFFFF)
-    for _ in range(10):
-        p0, p1 = np.uint64(0xD2511F53) * c0, np.uint64(0xCD9E8D57) * c2
-        c0, c1, c2, c3 = ((p1 >> np.uint64(32)) ^ c1 ^ k0) & mask, p1 & mask, ((p0 >> np.uint64(32)) ^ c3 ^ k1) & mask, p0 & mask
-        k0, k1 = (k0 + np.uint64(0x9E3779B9)) & mask, (k1 + np.uint64(0xBB67AE85)) & mask
-    return c0
-
-
 def test_sample(hip):
     import numpy as np
     vocab = 1531
@@ -328,7 +314,7 @@ def test_sample(hip):
     assert out[0] == int(logits[0].argmax()) and out[1] == 100
     assert out[2] == out[5]                                                   # same seed and draw: same token
     for row in (2, 3, 4):
-        bits = _philox_first(np.arange(vocab), int(draws[row]), int(seeds[row]) & 0xFFFFFFFF, int(seeds[row]) >> 32)
+        bits = philox_first(np.arange(vocab), int(draws[row]), int(seeds[row]) & 0xFFFFFFFF, int(seeds[row]) >> 32)
         u = ((bits >> np.uint64(8)).astype(np.float64) + 0.5) * 2.0 ** -24
         scores = logits[row].double().numpy() / float(temperature[row]) - np.log(-np.log(u))
         assert scores[out[row]] >= scores.max() - 1e-4

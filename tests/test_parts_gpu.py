@@ -1,0 +1,246 @@
+"""Each part alone on the GPU against the plain function of the same part, at sizes that are not the tiny
+models'; and the entry points: greedy generation through `generate_tokens`, the scheduler and the command line."""
+
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from ampere_kv_engine_amd.cache import CacheManager
+from ampere_kv_engine_amd.config import EngineConfig, part
+from ampere_kv_engine_amd.engine import BatchBuilder, Engine, StepEntry
+from ampere_kv_engine_amd.engine.generate import generate_tokens
+from ampere_kv_engine_amd.engine.scheduler import Scheduler
+from ampere_kv_engine_amd.parts import Runtime, build_part
+from conftest import ROOT, TINY, random_ids
+from plain import qwen3_plain as P
+
+pytestmark = pytest.mark.gpu
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def runtime(dtype, page_size=8, max_seq_len=256):
+    from ampere_kv_engine_amd.kernels.hip import HipKernels
+    return Runtime(kernels=HipKernels("cuda:0"), dtype=dtype, device=torch.device("cuda:0"), max_seq_len=max_seq_len,
+                   page_size=page_size)
+
+
+def tol(dtype, scale=1.0):
+    return dict(rtol=1e-4, atol=1e-5 * scale) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2 * scale)
+
+
+def loader(weights, dtype):
+    """fetch(spec) for parts: random values per tensor name, rounded to bfloat16 so both dtypes see the same."""
+    def fetch(spec):
+        if spec.name not in weights:
+            g = torch.Generator().manual_seed(abs(hash(spec.name)) % (2 ** 31))
+            base = torch.randn(spec.shape, generator=g)
+            weights[spec.name] = (1 + 0.1 * base if spec.role == "norm" else 0.05 * base).bfloat16().float()
+        return weights[spec.name].to(dtype).cuda()
+    return fetch
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_part(dtype):
+    rt = runtime(dtype)
+    norm = build_part("norm", part("rmsnorm", size=200, eps=1e-5), rt)
+    weights = {}
+    norm.load(loader(weights, dtype), "n.weight")
+    x = torch.randn(9, 200).to(dtype)
+    out = torch.empty(9, 200, dtype=dtype, device="cuda")
+    norm.forward(x.cuda(), out)
+    want = P.rms_norm(x.float(), weights["n.weight"], 1e-5)
+    torch.testing.assert_close(out.cpu().float(), want, **tol(dtype))
+    stream, delta = torch.randn(9, 200), torch.randn(9, 200).to(dtype)
+    s = stream.clone().cuda()
+    norm.forward_residual(s, delta.cuda(), out)
+    torch.testing.assert_close(s.cpu(), stream + delta.float(), rtol=0, atol=0)
+    torch.testing.assert_close(out.cpu().float(), P.rms_norm(stream + delta.float(), weights["n.weight"], 1e-5), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rotary_part(dtype):
+    rt = runtime(dtype, max_seq_len=5000)
+    rope = build_part("position", part("rope_half", head_dim=48, theta=5e5), rt)
+    x = torch.randn(6, 5, 48).to(dtype)
+    positions = torch.tensor([0, 1, 2, 77, 4095, 4999], dtype=torch.int32)
+    got = rope.apply(x.clone().cuda(), positions.cuda()).cpu().float()
+    want = P.rope(x.float(), positions, P.rope_inverse_frequencies(48, 5e5))
+    torch.testing.assert_close(got, want, **tol(dtype))
+    assert torch.equal(rope.inv_freq.cpu(), P.rope_inverse_frequencies(48, 5e5))
+
+
+def step_context(rt, needs, portions, page_size, num_pages=64):
+    """A cache manager and the context of one step in which request i brings `portions[i]` tokens."""
+    cache = CacheManager(needs, page_size=page_size, num_pages=num_pages, max_seqs=len(portions), dtype=rt.dtype,
+                         device=rt.device)
+    builder = BatchBuilder(cache, rt.device, 256, len(portions), 32)
+    seqs = [cache.open(f"r{i}") for i in range(len(portions))]
+    return cache, builder, seqs
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("q_heads,kv_heads,head_dim,window", [(6, 2, 48, None), (4, 4, 16, None), (8, 1, 64, 9)])
+def test_attention_mixer_alone(dtype, q_heads, kv_heads, head_dim, window):
+    """Two requests, each fed in two steps (so the second step reads the cache the first one wrote), against the
+    plain mixer on the whole sequences."""
+    hidden, page_size = 80, 8
+    rt = runtime(dtype, page_size)
+    spec = part("attention", hidden_size=hidden, q_heads=q_heads, kv_heads=kv_heads, head_dim=head_dim, window=window,
+                qk_norm=part("rmsnorm", size=head_dim, eps=1e-6), position=part("rope_half", head_dim=head_dim, theta=1e4),
+                scale=head_dim ** -0.5, name="attn")
+    mixer = build_part("mixer", spec, rt)
+    weights = {}
+    mixer.load(loader(weights, dtype), "L.")
+    cache, builder, seqs = step_context(rt, {0: mixer.cache_request()}, [0, 0], page_size)
+    xs = [torch.randn(21, hidden).to(dtype), torch.randn(13, hidden).to(dtype)]
+    outs = [[], []]
+    cuts = [[(0, 10), (10, 21)], [(0, 12), (12, 13)]]
+    for step in range(2):
+        entries = [StepEntry(seqs[i], [0] * (cuts[i][step][1] - cuts[i][step][0]), []) for i in range(2)]
+        ctx, _ = builder.build(entries)
+        order = sorted(range(2), key=lambda i: (cuts[i][step][1] - cuts[i][step][0] != 1, i))
+        x = torch.cat([xs[i][cuts[i][step][0]:cuts[i][step][1]] for i in order]).cuda()
+        y = mixer.forward(x, ctx, cache.layer_cache[0]).cpu().float()
+        row = 0
+        for i in order:
+            n = cuts[i][step][1] - cuts[i][step][0]
+            outs[i].append(y[row:row + n])
+            row += n
+    names = {"q_proj": "L.attn.q_proj.weight", "k_proj": "L.attn.k_proj.weight", "v_proj": "L.attn.v_proj.weight",
+             "o_proj": "L.attn.o_proj.weight", "q_norm": "L.attn.q_norm.weight", "k_norm": "L.attn.k_norm.weight"}
+    w = {k: weights[v] for k, v in names.items()}
+    for i in range(2):
+        want = P.attention_mixer(xs[i].float(), torch.arange(xs[i].shape[0]), w, q_heads=q_heads, kv_heads=kv_heads,
+                                 head_dim=head_dim, eps=1e-6, inv_freq=P.rope_inverse_frequencies(head_dim, 1e4),
+                                 window=window)
+        torch.testing.assert_close(torch.cat(outs[i]), want, **tol(dtype, float(want.abs().max())))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_mixer_through_the_parts_own_entry_points(dtype):
+    """A position kind the fused kernel does not know sends the mixer through norm, position and cache-write one
+    by one; with the same rotation behind it the result must equal the fused path's."""
+    from ampere_kv_engine_amd.parts import RotaryHalf, register_part
+
+    class OtherRotary(RotaryHalf):
+        pass
+
+    register_part("position", "rope_half_unfused", OtherRotary, replace=True)
+    hidden, page_size, results = 64, 8, []
+    x = torch.randn(19, hidden).to(dtype)
+    for kind in ("rope_half", "rope_half_unfused"):
+        rt = runtime(dtype, page_size)
+        spec = part("attention", hidden_size=hidden, q_heads=4, kv_heads=2, head_dim=32, window=None,
+                    qk_norm=part("rmsnorm", size=32, eps=1e-6), position=part(kind, head_dim=32, theta=1e4),
+                    scale=32 ** -0.5, name="attn")
+        mixer = build_part("mixer", spec, rt)
+        assert mixer.fused == (kind == "rope_half")
+        mixer.load(loader({}, dtype), "L.")
+        cache, builder, seqs = step_context(rt, {0: mixer.cache_request()}, [0], page_size)
+        ctx, _ = builder.build([StepEntry(seqs[0], [0] * 19, [])])
+        results.append(mixer.forward(x.cuda(), ctx, cache.layer_cache[0]).cpu().float())
+    torch.testing.assert_close(results[0], results[1], **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu_part(dtype):
+    rt = runtime(dtype)
+    ff = build_part("feed_forward", part("swiglu", hidden_size=72, intermediate_size=200, name="mlp"), rt)
+    weights = {}
+    ff.load(loader(weights, dtype), "L.")
+    cache, builder, seqs = step_context(rt, {0: None}, [0], 8)
+    ctx, _ = builder.build([StepEntry(seqs[0], [0] * 11, [])])
+    x = torch.randn(11, 72).to(dtype)
+    got = ff.forward(x.cuda(), ctx).cpu().float()
+    want = P.swiglu_feed_forward(x.float(), weights["L.mlp.gate_proj.weight"], weights["L.mlp.up_proj.weight"],
+                                 weights["L.mlp.down_proj.weight"])
+    torch.testing.assert_close(got, want, **tol(dtype, float(want.abs().max())))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_block_alone(dtype):
+    hidden, heads, kv, d, page_size = 64, 4, 2, 16, 8
+    rt = runtime(dtype, page_size)
+    norm = part("rmsnorm", size=hidden, eps=1e-5)
+    mixer = build_part("mixer", part("attention", hidden_size=hidden, q_heads=heads, kv_heads=kv, head_dim=d, window=None,
+                                     qk_norm=part("rmsnorm", size=d, eps=1e-5),
+                                     position=part("rope_half", head_dim=d, theta=1e4), scale=d ** -0.5,
+                                     name="self_attn"), rt)
+    ff = build_part("feed_forward", part("swiglu", hidden_size=hidden, intermediate_size=96, name="mlp"), rt)
+    block = build_part("block", part("prenorm", hidden_size=hidden, norm=norm), rt, mixer=mixer, feed_forward=ff)
+    weights = {}
+    block.load(loader(weights, dtype), "L.")
+    cache, builder, seqs = step_context(rt, {0: mixer.cache_request()}, [0], page_size)
+    ctx, _ = builder.build([StepEntry(seqs[0], [0] * 17, [])])
+    ctx.arena = ctx.arenas[0]
+    h0 = torch.randn(17, hidden)
+    stream = h0.clone().cuda()
+    pending = block.forward(stream, None, ctx, cache.layer_cache[0])
+    got = stream.cpu() + pending.cpu().float()
+    short = {k.split(".")[-2]: v for k, v in weights.items()}
+    want = P.decoder_block(h0, torch.arange(17), short, q_heads=heads, kv_heads=kv, head_dim=d, eps=1e-5,
+                           inv_freq=P.rope_inverse_frequencies(d, 1e4))
+    torch.testing.assert_close(got, want, **tol(dtype, float(want.abs().max())))
+
+
+# ---- entry points ---------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_through_the_entry_points(name, model_folders):
+    raw, _, page = TINY[name]
+    folder = model_folders[name]
+    plain = P.PlainQwen3(folder)
+    prompts = [random_ids(raw["vocab_size"], n, seed=70 + i) for i, n in enumerate((5, 17, 33))]
+    want = [plain.greedy(p, 8) for p in prompts]
+    config = EngineConfig(dtype="float32", page_size=page, num_pages=24, max_seqs=4, max_batched_tokens=64,
+                          max_seq_len=128, device="cuda:0")
+    engine = Engine.from_folder(folder, config)
+    assert [generate_tokens(engine, p, max_new_tokens=8, ignore_eos=True) for p in prompts] == want
+    scheduler = Scheduler(engine, prefill_chunk_size=7)
+    requests = [scheduler.submit(f"r{i}", p, 8, ignore_eos=True) for i, p in enumerate(prompts)]
+    scheduler.run_until_idle()
+    assert [r.output_ids for r in requests] == want
+    assert engine.cache.num_free_pages == [24] and "libakv_kernels" in engine.kernels.library_path
+    bf = Engine.from_folder(folder, EngineConfig(**{**config.__dict__, "dtype": "bfloat16"}))
+    for p, w in zip(prompts, want):                       # bfloat16: the first token agrees, most of the rest too
+        got = generate_tokens(bf, p, max_new_tokens=8, ignore_eos=True)
+        assert got[0] == w[0] and sum(a == b for a, b in zip(got, w)) >= 6
+
+
+def test_temperature_sampling_does_not_depend_on_the_batch(model_folders):
+    raw, _, page = TINY["B"]
+    config = EngineConfig(dtype="float32", page_size=page, num_pages=40, max_seqs=4, max_batched_tokens=32,
+                          max_seq_len=128, device="cuda:0")
+    engine = Engine.from_folder(model_folders["B"], config)
+    prompts = [random_ids(379, n, seed=80 + i) for i, n in enumerate((1, 9, 24, 40))]
+    alone = [generate_tokens(engine, p, max_new_tokens=10, ignore_eos=True, temperature=0.7, seed=5 + i)
+             for i, p in enumerate(prompts)]
+    scheduler = Scheduler(engine, prefill_chunk_size=7)
+    requests = [scheduler.submit(f"r{i}", p, 10, ignore_eos=True, temperature=0.7, seed=5 + i)
+                for i, p in enumerate(prompts)]
+    scheduler.run_until_idle()
+    assert [r.output_ids for r in requests] == alone and scheduler.mixed_rounds > 0
+    assert len({tuple(a) for a in alone}) == 4
+
+
+def test_command_line(model_folders):
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    prompt = random_ids(256, 17, seed=71)
+    want = P.PlainQwen3(model_folders["A"]).greedy(prompt, 6)
+    run = lambda *args, **kw: subprocess.run([sys.executable, "-m", "ampere_kv_engine_amd.runner", *args], env=env,
+                                             capture_output=True, text=True, timeout=300, **kw)
+    result = run("--model", model_folders["A"], "--mode", "generate", "--cache", "paged", "--dtype", "float32",
+                 "--max-new-tokens", "6", "--ignore-eos", input=" ".join(map(str, prompt)) + "\n")
+    assert result.returncode == 0, result.stderr[-2000:]
+    assert f"generated_token_ids = {want}" in result.stdout
+    result = run("--model", model_folders["A"], "--mode", "check", "--max-new-tokens", "6", "--ignore-eos",
+                 "--prompt-ids", ",".join(map(str, prompt)))
+    assert result.returncode == 0 and "check: 6 steps" in result.stdout, result.stderr[-2000:]
+    result = run("--model", model_folders["A"], "--mode", "benchmark", "--repeats", "2", "--max-new-tokens", "6",
+                 "--prompt-len", "20")
+    assert result.returncode == 0 and '"tpot_ms"' in result.stdout, result.stderr[-2000:]
+    result = run("--model", model_folders["A"], "--mode", "generate", "--cache", "contiguous", "--prompt-ids", "1")
+    assert result.returncode != 0

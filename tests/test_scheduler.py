@@ -1,0 +1,193 @@
+"""The scheduler's decisions, with the torch test double in place of the kernels (float32, on the host):
+admission against the page budget, portions under the token budget, the lifecycle, stops, what is given back."""
+
+import pytest
+import torch
+
+from ampere_kv_engine_amd.config import EngineConfig
+from ampere_kv_engine_amd.engine import Engine
+from ampere_kv_engine_amd.engine.generate import generate_tokens
+from ampere_kv_engine_amd.engine.scheduler import (FINISHED, PREFILLING, RUNNING, STOP_CANCELLED, STOP_EOS,
+                                                   STOP_EXPIRED, STOP_LIMIT, WAITING, Scheduler)
+from conftest import TINY, random_ids
+from plain.qwen3_plain import PlainQwen3
+from torch_kernels import TorchKernels
+
+
+def make_engine(folder, page_size, num_pages, max_seqs=4, max_tokens=64):
+    config = EngineConfig(dtype="float32", page_size=page_size, num_pages=num_pages, max_seqs=max_seqs,
+                          max_batched_tokens=max_tokens, max_seq_len=256, device="cpu")
+    return Engine.from_folder(folder, config, kernels=TorchKernels())
+
+
+def drive(scheduler, limit=500):
+    finished, log = [], []
+    for _ in range(limit):
+        if scheduler.idle:
+            break
+        done, sizes = scheduler.step()
+        finished += done
+        log.append((sizes, list(scheduler.last_portions), len(scheduler.waiting)))
+    assert scheduler.idle
+    return finished, log
+
+
+def alone(folder, page_size, prompt, new_tokens, **kw):
+    engine = make_engine(folder, page_size, 64)
+    return generate_tokens(engine, prompt, max_new_tokens=new_tokens, ignore_eos=True, **kw)
+
+
+def test_generate_equals_plain_greedy(model_folders):
+    """tiny-A workload: prompts of 5, 17 and 33 tokens, 8 greedy tokens each."""
+    raw, _, page = TINY["A"]
+    plain = PlainQwen3(model_folders["A"])
+    for i, length in enumerate((5, 17, 33)):
+        prompt = random_ids(raw["vocab_size"], length, seed=40 + i)
+        timings = {}
+        got = generate_tokens(make_engine(model_folders["A"], page, 8), prompt, max_new_tokens=8, ignore_eos=True,
+                              timings=timings)
+        assert got == plain.greedy(prompt, 8)
+        assert {"ttft_ms", "tpot_ms", "total_ms", "output_tokens_per_s", "kv_data_bytes", "capacity"} <= set(timings)
+        assert timings["kv_data_bytes"] == (length + 7) * 2 * 2 * 2 * 16 * 4      # final length P+N-1: last token not cached
+
+
+def test_interleaved_requests_equal_each_alone_and_everything_is_given_back(model_folders):
+    """tiny-B workload: prompts 1, 9, 24, 40; temperature 0.7 seeded; 10 tokens each; portions of 7 mixed with decodes."""
+    raw, _, page = TINY["B"]
+    folder = model_folders["B"]
+    prompts = [random_ids(raw["vocab_size"], n, seed=50 + i) for i, n in enumerate((1, 9, 24, 40))]
+    want = [alone(folder, page, p, 10, temperature=0.7, seed=90 + i) for i, p in enumerate(prompts)]
+    engine = make_engine(folder, page, num_pages=14, max_tokens=24)                # budgets 2+3+5+7 = 17 > 14: someone waits
+    scheduler = Scheduler(engine, prefill_chunk_size=7)
+    requests = [scheduler.submit(f"r{i}", p, 10, ignore_eos=True, temperature=0.7, seed=90 + i)
+                for i, p in enumerate(prompts)]
+    finished, log = drive(scheduler)
+    assert [r.output_ids for r in requests] == want
+    assert {r.request_id for r in finished} == {"r0", "r1", "r2", "r3"} and all(r.status == FINISHED for r in requests)
+    assert all(r.stop_reason == STOP_LIMIT for r in requests)
+    assert max(w for _, _, w in log) > 0, "nobody ever waited: the pool was not small enough to test admission"
+    assert any(sizes and portions for sizes, portions, _ in log), "no round mixed decodes with a portion"
+    assert all(sum(portions) + sum(sizes) <= 24 for sizes, portions, _ in log)
+    assert all(p <= 7 for _, portions, _ in log for p in portions)
+    assert scheduler.reserved_pages == [0] and engine.cache.num_free_pages == [14]
+    assert engine.cache.slots.num_free == 4 and scheduler.mixed_rounds > 0
+    different = alone(folder, page, prompts[3], 10, temperature=0.7, seed=1234)
+    assert different != want[3], "the seed does not reach the sampler"
+
+
+def test_mixed_and_separate_rounds_choose_the_same_tokens(model_folders):
+    raw, _, page = TINY["A"]
+    folder = model_folders["A"]
+    prompts = [random_ids(raw["vocab_size"], n, seed=60 + i) for i, n in enumerate((5, 17, 33, 20))]
+    outputs = []
+    for mixed in (True, False):
+        scheduler = Scheduler(make_engine(folder, page, 32), prefill_chunk_size=8, mixed=mixed)
+        requests = [scheduler.submit(f"r{i}", p, 8, ignore_eos=True) for i, p in enumerate(prompts)]
+        drive(scheduler)
+        outputs.append([r.output_ids for r in requests])
+        assert (scheduler.mixed_rounds > 0) == mixed
+    assert outputs[0] == outputs[1]
+    plain = PlainQwen3(folder)
+    assert outputs[0] == [plain.greedy(p, 8) for p in prompts]
+
+
+def test_first_token_comes_from_the_last_portion_and_no_decode_in_that_round(model_folders):
+    raw, _, page = TINY["A"]
+    scheduler = Scheduler(make_engine(model_folders["A"], page, 32), prefill_chunk_size=16)
+    short = scheduler.submit("short", random_ids(256, 3, 1), 12, ignore_eos=True)
+    scheduler.step()
+    assert short.status == RUNNING and len(short.output_ids) == 1
+    long = scheduler.submit("long", random_ids(256, 40, 2), 4, ignore_eos=True)
+    for expected_progress in (16, 32):                       # two middle portions: no token for the long request
+        scheduler.step()
+        assert long.status == PREFILLING and long.prefilled == expected_progress and not long.output_ids
+    produced = len(short.output_ids)
+    assert produced == 3                                      # the short one decoded in every one of those rounds
+    scheduler.step()
+    assert long.status == RUNNING and len(long.output_ids) == 1 and long.prefilled == 40   # first token, not yet decoded
+    scheduler.step()
+    assert len(long.output_ids) == 2 and long.prefilled == 41
+
+
+def test_eos_stops_and_the_final_token_is_not_cached(model_folders):
+    raw, _, page = TINY["A"]
+    engine = make_engine(model_folders["A"], page, 32)
+    prompt = random_ids(256, 9, 3)
+    sampling = dict(temperature=3.0, seed=7)                # a hot draw, so that the six tokens differ
+    free_run = generate_tokens(engine, prompt, max_new_tokens=6, ignore_eos=True, **sampling)
+    assert free_run[2] not in free_run[:2], "test premise: the third token must be new"
+    engine.spec = type(engine.spec)(**{**engine.spec.__dict__, "eos_token_ids": (free_run[2],)})
+    scheduler = Scheduler(engine)
+    stopping = scheduler.submit("s", prompt, 6, **sampling)
+    ignoring = scheduler.submit("i", prompt, 6, ignore_eos=True, **sampling)
+    drive(scheduler)
+    assert stopping.output_ids == free_run[:3] and stopping.stop_reason == STOP_EOS
+    assert ignoring.output_ids == free_run and ignoring.stop_reason == STOP_LIMIT
+    assert stopping.cached_tokens == 9 + 3 - 1 and ignoring.cached_tokens == 9 + 6 - 1
+    assert generate_tokens(engine, prompt, max_new_tokens=6, **sampling) == free_run[:3]
+
+
+def test_admission_is_first_come_and_by_reserved_budget(model_folders):
+    raw, _, page = TINY["A"]                                            # page 16
+    engine = make_engine(model_folders["A"], page, num_pages=8)
+    scheduler = Scheduler(engine)
+    with pytest.raises(ValueError, match="exceeds the pool"):
+        scheduler.submit("huge", random_ids(256, 100, 1), 40)           # (100+40+16)//16 = 9 pages > 8
+    with pytest.raises(ValueError):
+        scheduler.submit("empty", [], 4)
+    with pytest.raises(ValueError):
+        scheduler.submit("nothing", [1], 0)
+    with pytest.raises(ValueError):
+        scheduler.submit("vocabulary", [256], 1)
+    first = scheduler.submit("first", random_ids(256, 40, 2), 30, ignore_eos=True)     # (40+30+16)//16 = 5 pages
+    second = scheduler.submit("second", random_ids(256, 40, 3), 20, ignore_eos=True)   # 4 pages: 5+4 > 8, waits
+    third = scheduler.submit("third", random_ids(256, 3, 4), 2, ignore_eos=True)       # 1 page: would fit, but is behind
+    scheduler.step()
+    assert first.status == RUNNING and second.status == WAITING and third.status == WAITING
+    assert scheduler.reserved_pages == [5] and engine.cache.num_free_pages == [8 - 3]   # reserved 5, really held 3
+    finished, log = drive(scheduler)
+    order = [r.request_id for r in finished]
+    assert order.index("first") < order.index("second") and set(order) == {"first", "second", "third"}
+    assert scheduler.reserved_pages == [0] and engine.cache.num_free_pages == [8]
+
+
+def test_cancel_and_deadline_in_every_state(model_folders):
+    raw, _, page = TINY["A"]
+    now = [100.0]
+    engine = make_engine(model_folders["A"], page, num_pages=10, max_seqs=3)
+    scheduler = Scheduler(engine, prefill_chunk_size=8, clock=lambda: now[0])
+    running = scheduler.submit("running", random_ids(256, 4, 1), 50, ignore_eos=True)
+    neighbour = scheduler.submit("neighbour", random_ids(256, 6, 2), 12, ignore_eos=True)
+    scheduler.step()
+    prefilling = scheduler.submit("prefilling", random_ids(256, 30, 3), 5, ignore_eos=True, deadline=50.0)  # already past
+    waiting = scheduler.submit("waiting", random_ids(256, 30, 4), 40, ignore_eos=True)
+    late = scheduler.submit("late", random_ids(256, 3, 5), 3, ignore_eos=True, deadline=103.0)
+    done, _ = scheduler.step()
+    assert [r.request_id for r in done] == ["prefilling"] and prefilling.stop_reason == STOP_EXPIRED
+    assert prefilling.status == FINISHED and not prefilling.output_ids
+    scheduler.cancel(running)
+    scheduler.cancel(running)                                # twice is harmless
+    scheduler.cancel(waiting)
+    before = len(running.output_ids)
+    done, _ = scheduler.step()
+    assert {r.request_id for r in done} == {"running", "waiting"}
+    assert running.stop_reason == waiting.stop_reason == STOP_CANCELLED and len(running.output_ids) == before
+    scheduler.cancel(running)                                # finished: left alone
+    assert running.stop_reason == STOP_CANCELLED
+    now[0] = 104.0
+    done, _ = scheduler.step()
+    assert "late" in {r.request_id for r in done} and late.stop_reason == STOP_EXPIRED
+    finished, _ = drive(scheduler)
+    assert neighbour.output_ids == alone(model_folders["A"], page, neighbour.input_ids, 12)
+    assert scheduler.reserved_pages == [0] and engine.cache.num_free_pages == [10] and engine.cache.slots.num_free == 3
+
+
+def test_scheduler_arguments():
+    class FakeEngine:
+        config = EngineConfig(max_seqs=4, max_batched_tokens=16, device="cpu")
+    with pytest.raises(ValueError):
+        Scheduler(FakeEngine(), max_batch=5)
+    with pytest.raises(ValueError):
+        Scheduler(FakeEngine(), prefill_chunk_size=-1)
+    with pytest.raises(ValueError):
+        Scheduler(FakeEngine(), max_batched_tokens=2)

@@ -10,6 +10,7 @@ from __future__ import annotations
 
 import math
 
+import numpy as np
 import torch
 
 
@@ -130,5 +131,34 @@ class TorchKernels:
             out[first:last] = merged.reshape(last - first, q_heads * head_dim).to(out.dtype)
 
     # ---- sampling -----------------------------------------------------------------------------------------
+    def sample(self, logits, temperature, seeds, draws, out):
+        """temperature 0: the largest logit, ties to the lowest id.  Otherwise the Gumbel-max draw
+        argmax(logits / t - log(-log(u))), u from Philox-4x32-10 keyed by the seed with counter (id, draw)."""
+        for row in range(logits.shape[0]):
+            t = float(temperature[row]) if temperature is not None else 0.0
+            scores = logits[row].double()
+            if t > 0:
+                seed = int(seeds[row])
+                bits = philox_first(np.arange(logits.shape[1]), int(draws[row]), seed & 0xFFFFFFFF, seed >> 32)
+                u = ((bits >> np.uint64(8)).astype(np.float64) + 0.5) * 2.0 ** -24
+                scores = scores / t - torch.from_numpy(np.log(-np.log(u)))
+            best = scores.max()
+            out[row] = int((scores == best).nonzero()[0])
+
     def argmax(self, logits, out):
-        out.copy_(logits.argmax(dim=-1).to(out.dtype))
+        self.sample(logits, None, None, None, out)
+
+
+def philox_first(c0, c1, k0, k1):
+    """First output word of Philox-4x32-10 for counters (c0, c1, 0, 0) and key (k0, k1); c0 may be an array."""
+    c0 = np.asarray(c0, dtype=np.uint64)
+    c1 = np.full_like(c0, np.uint64(c1))
+    c2, c3 = np.zeros_like(c0), np.zeros_like(c0)
+    k0, k1 = np.uint64(k0), np.uint64(k1)
+    mask = np.uint64(0xFFFFFFFF)
+    for _ in range(10):
+        p0, p1 = np.uint64(0xD2511F53) * c0, np.uint64(0xCD9E8D57) * c2
+        c0, c1, c2, c3 = (((p1 >> np.uint64(32)) ^ c1 ^ k0) & mask, p1 & mask,
+                          ((p0 >> np.uint64(32)) ^ c3 ^ k1) & mask, p0 & mask)
+        k0, k1 = (k0 + np.uint64(0x9E3779B9)) & mask, (k1 + np.uint64(0xBB67AE85)) & mask
+    return c0
