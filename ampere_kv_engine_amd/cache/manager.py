@@ -4,8 +4,10 @@ group, and slots for per-request state of fixed size.
 The reference keeps one pool and one tensor pair per layer and lets every request hold one table per layer
 that all grow in lock-step (ampere_kv/scheduler.py:63-69, ampere_kv/paged_cache.py:10-62).  Here layers whose
 mixers ask for the same thing (`PagedKV(kv_heads, head_dim, window)`) form a group with ONE pool, ONE table
-per request and one tensor `[layers, 2, pages, kv_heads, page_size, head_dim]`, so a page id is valid for
-every layer of its group.  Groups with a window give pages back while the request lives.  Mixers that ask
+per request and one tensor `[layers, 2, pages, kv_heads, page_size * head_dim]`, so a page id is valid for
+every layer of its group.  Within a page, keys lie `[page_size, head_dim]` and values `[head_dim, page_size]`:
+scores contract over head_dim and the weighted sum over keys, and each reaches the matrix cores with its
+contracted axis contiguous.  Groups with a window give pages back while the request lives.  Mixers that ask
 for `SlotState` get a tensor `[slots, *shape]` per layer, zeroed when a request takes the slot.
 
 Everything here except the tensors is host bookkeeping and runs without a GPU (`allocate_tensors=False`).
@@ -29,7 +31,7 @@ class PagedGroup:
     layers: list[int]                 # cache-layer ids, in the order of the tensor's first axis
     allocator: PageAllocator
     page_size: int
-    pages: torch.Tensor | None = None  # [len(layers), 2, num_pages, kv_heads, page_size, head_dim]
+    pages: torch.Tensor | None = None  # [len(layers), 2, num_pages, kv_heads, page_size * head_dim]
 
     def bytes_per_token(self, element_size: int) -> int:
         return 2 * len(self.layers) * self.need.kv_heads * self.need.head_dim * element_size
@@ -40,7 +42,7 @@ class LayerCache:
     """What one cache layer's mixer sees: its group id and its own key and value pages, or its state."""
     group: int | None = None
     k: torch.Tensor | None = None      # [num_pages, kv_heads, page_size, head_dim]
-    v: torch.Tensor | None = None
+    v: torch.Tensor | None = None      # [num_pages, kv_heads, head_dim, page_size]
     state: torch.Tensor | None = None  # [slots, *shape]
 
 
@@ -76,12 +78,14 @@ class CacheManager:
                 by_need[need].layers.append(layer)
         for group in self.groups:
             if allocate_tensors:
-                group.pages = torch.empty((len(group.layers), 2, num_pages, group.need.kv_heads, page_size,
-                                           group.need.head_dim), dtype=dtype, device=device)
+                group.pages = torch.empty((len(group.layers), 2, num_pages, group.need.kv_heads,
+                                           page_size * group.need.head_dim), dtype=dtype, device=device)
             for row, layer in enumerate(group.layers):
                 view = LayerCache(group=group.index)
                 if group.pages is not None:
-                    view.k, view.v = group.pages[row, 0], group.pages[row, 1]
+                    heads, dim = group.need.kv_heads, group.need.head_dim
+                    view.k = group.pages[row, 0].view(num_pages, heads, page_size, dim)
+                    view.v = group.pages[row, 1].view(num_pages, heads, dim, page_size)
                 self.layer_cache[layer] = view
         for layer in sorted(needs):
             need = needs[layer]
@@ -176,5 +180,5 @@ class CacheManager:
             if page < 0:
                 continue
             keys.append(view.k[page, :, offset])
-            values.append(view.v[page, :, offset])
+            values.append(view.v[page, :, :, offset])
         return torch.stack(keys), torch.stack(values)

@@ -59,12 +59,11 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(
       if (page < 0 || page >= num_pages) {
         s = __uint_as_float(0x7fc00000u);  // a page that is not the request's: poison, never read
       } else {
-        const long at = ((page * kv_heads + kvh) * page_size + j % page_size) * dim;
-        const T* kp = k_pages + at;
+        const T* kp = k_pages + ((page * kv_heads + kvh) * page_size + j % page_size) * dim;
         float dot = 0.f;
         for (int i = 0; i < dim; ++i) dot = fmaf(qs[i], to_float(kp[i]), dot);
         s = dot * scale;
-        value_at = at;
+        value_at = (page * kv_heads + kvh) * dim * page_size + j % page_size;  // values are [dim, page_size]
       }
     }
     const float m_new = fmaxf(m, wave_max(s));
@@ -84,7 +83,7 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(
 #pragma unroll
       for (int c = 0; c < kMaxDimRegs; ++c) {
         const int i = lane + c * kWave;
-        if (i < dim) acc[c] = fmaf(pj, to_float(v_pages[at + i]), acc[c]);
+        if (i < dim) acc[c] = fmaf(pj, to_float(v_pages[at + static_cast<long>(i) * page_size]), acc[c]);
       }
     }
     wave_sync_lds();

@@ -18,7 +18,7 @@ import time
 from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCES = ("elementwise.hip", "gemm.hip", "attention.hip", "sampling.hip")
+SOURCES = ("elementwise.hip", "gemm.hip", "gemm_mfma.hip", "attention.hip", "sampling.hip")
 HEADERS = ("common.h", "api.h")
 LIBRARY = "libakv_kernels.so"
 ARCH = "gfx950"

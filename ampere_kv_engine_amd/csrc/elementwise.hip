@@ -139,7 +139,10 @@ __global__ void rope_kernel(T* __restrict__ x, const int* __restrict__ positions
   p[j + half] = from_float<T>(hi * c + lo * s);
 }
 
-// ---- cache write: pages [num_pages, kv_heads, page_size, dim]; slot = page * page_size + offset -----------------
+// ---- cache write; slot = page * page_size + offset -----------------------------------------------------------
+// Key pages are [num_pages, kv_heads, page_size, dim] (a key's dims are contiguous: the score product runs over
+// them); value pages are [num_pages, kv_heads, dim, page_size] (a dim's keys are contiguous: the weighted sum runs
+// over keys), so that both reach the matrix cores without a transposition.
 template <typename T>
 __global__ void kv_write_kernel(const T* __restrict__ k, long k_stride, const T* __restrict__ v, long v_stride,
                                 const int* __restrict__ slot_map, T* __restrict__ k_pages, T* __restrict__ v_pages,
@@ -150,12 +153,14 @@ __global__ void kv_write_kernel(const T* __restrict__ k, long k_stride, const T*
   const int h = static_cast<int>(row % kv_heads);
   const long slot = slot_map[n];
   if (slot < 0 || slot >= num_slots) return;  // host checks the map; never write outside the pool
-  const long dst = ((slot / page_size * kv_heads + h) * page_size + slot % page_size) * dim;
+  const long page = slot / page_size, offset = slot % page_size;
+  const long k_at = ((page * kv_heads + h) * page_size + offset) * dim;
+  const long v_at = (page * kv_heads + h) * dim * page_size + offset;
   const T* ks = k + n * k_stride + static_cast<long>(h) * dim;
   const T* vs = v + n * v_stride + static_cast<long>(h) * dim;
   for (int i = threadIdx.x & (kWave - 1); i < dim; i += kWave) {
-    k_pages[dst + i] = ks[i];
-    v_pages[dst + i] = vs[i];
+    k_pages[k_at + i] = ks[i];
+    v_pages[v_at + static_cast<long>(i) * page_size] = vs[i];
   }
 }
 
@@ -188,12 +193,13 @@ __global__ void qk_norm_rope_write_kernel(const T* __restrict__ qkv, const float
     const long slot = slot_map[n];
     if (slot < 0 || slot >= num_slots) return;
     const int kvh = (h - q_heads) % kv_heads;
-    const long at = ((slot / page_size * kv_heads + kvh) * page_size + slot % page_size) * dim;
-    if (h >= q_heads + kv_heads) {  // value: copied as it is
-      for (int i = lane; i < dim; i += kWave) v_pages[at + i] = src[i];
+    const long page = slot / page_size, offset = slot % page_size;
+    if (h >= q_heads + kv_heads) {  // value: copied as it is, into the [dim, page_size] layout
+      const long at = (page * kv_heads + kvh) * dim * page_size + offset;
+      for (int i = lane; i < dim; i += kWave) v_pages[at + static_cast<long>(i) * page_size] = src[i];
       return;
     }
-    dst = k_pages + at;
+    dst = k_pages + ((page * kv_heads + kvh) * page_size + offset) * dim;
   }
 
   const float* weight = h < q_heads ? q_weight : k_weight;

@@ -1,0 +1,246 @@
+// bfloat16 matrix products y = x W^T on the matrix cores (v_mfma_f32_16x16x32_bf16), float32 accumulation.
+//
+// W is not read row-major.  At load time it is packed into tiles of 16 output rows x 32 k, 1 KB each, stored
+// [row_tile][k_tile][lane][8]: lane l of a wave holds row l % 16, k = (l / 16) * 8 .. + 8 of the tile, which is
+// exactly the MFMA's A operand.  One global_load_dwordx4 per lane then brings a whole tile as 1 KB of consecutive
+// bytes, and a wave that walks along k streams one contiguous region of memory - what HBM likes best.  Rows and k
+// beyond the matrix are zero in the packing.
+//
+//   linear_skinny  rows <= 64 (decode): every wave streams its own tiles once; the few activations come from
+//                  cache; k is split over the waves of a block and summed through LDS in a fixed order.
+//   linear_wide    rows  > 64 (prefill): 128 x 128 output tiles per block, activations staged through LDS,
+//                  weights straight from the packed layout into the A operand.
+// In both, a row of x meets the weights in the same k order whatever else is in the batch.
+
+#include "common.h"
+#include "api.h"
+
+using namespace akv;
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float floatx4;
+
+__device__ __forceinline__ floatx4 mfma16(uint4 a, uint4 b, floatx4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+template <typename TY> __device__ __forceinline__ void store4(TY* p, floatx4 v);
+template <> __device__ __forceinline__ void store4<float>(float* p, floatx4 v) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, floatx4 v) {
+  uint2 packed;
+  packed.x = bf16_bits(v[0]) | (static_cast<uint32_t>(bf16_bits(v[1])) << 16);
+  packed.y = bf16_bits(v[2]) | (static_cast<uint32_t>(bf16_bits(v[3])) << 16);
+  *reinterpret_cast<uint2*>(p) = packed;
+}
+
+// Lane (r = l % 16, g = l / 16) owns outputs [feature0 + g * 4 + i][token r] of a 16 x 16 tile.
+template <typename TY>
+__device__ __forceinline__ void store_tile(TY* y, floatx4 acc, int token, int feature, int rows, int outs) {
+  if (token >= rows) return;
+  TY* dst = y + static_cast<size_t>(token) * outs + feature;
+  if (feature + 3 < outs && (outs & 3) == 0) {
+    store4<TY>(dst, acc);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (feature + i < outs) dst[i] = from_float<TY>(acc[i]);
+  }
+}
+
+// ---- rows <= 16 * MT --------------------------------------------------------------------------------------------
+constexpr int kUnroll = 8;  // weight tiles in flight per wave
+
+template <int MT, typename TY>
+__global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __restrict__ x, const uint4* __restrict__ wp,
+                                                            TY* __restrict__ y, int rows, int outs, int k,
+                                                            int k_tiles, int n_tiles, int k_split) {
+  extern __shared__ float red[];  // [wave][MT][4][64]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int row_tile = blockIdx.x * (waves / k_split) + wave / k_split;
+  const int part = wave % k_split;
+  const int per_part = (k_tiles + k_split - 1) / k_split;
+  const int kt0 = part * per_part, kt1 = min(k_tiles, kt0 + per_part);
+  floatx4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  if (row_tile < n_tiles) {
+    const uint4* wt = wp + static_cast<size_t>(row_tile) * k_tiles * 64 + lane;
+    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+    for (int kt = kt0; kt < kt1; kt += kUnroll) {
+      uint4 a[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) a[u] = (kt + u < kt1) ? wt[static_cast<size_t>(kt + u) * 64] : zero;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const int token = mt * 16 + r;
+        uint4 b[kUnroll];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+          const int at = (kt + u) * 32 + g * 8;
+          b[u] = (kt + u < kt1 && token < rows && at < k)
+                     ? *reinterpret_cast<const uint4*>(x + static_cast<size_t>(token) * k + at) : zero;
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) acc[mt] = mfma16(a[u], b[u], acc[mt]);
+      }
+    }
+  }
+  if (k_split > 1) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) red[((wave * MT + mt) * 4 + i) * 64 + lane] = acc[mt][i];
+    __syncthreads();
+    if (part != 0) return;
+    for (int other = 1; other < k_split; ++other)  // fixed order: part 0 + part 1 + ...
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[mt][i] += red[(((wave + other) * MT + mt) * 4 + i) * 64 + lane];
+  }
+  if (row_tile >= n_tiles) return;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) store_tile<TY>(y, acc[mt], mt * 16 + r, row_tile * 16 + g * 4, rows, outs);
+}
+
+template <int MT, typename TY>
+int launch_skinny(const void* x, const void* wp, void* y, int rows, int outs, int k, int k_tiles, int n_tiles,
+                  hipStream_t stream) {
+  // enough waves to keep every CU's memory pipe full: split k over the waves of a block when there are few row tiles
+  int k_split = 1;
+  while (k_split < 8 && n_tiles * k_split < 2048 && k_tiles / (k_split * 2) >= 4) k_split *= 2;
+  const int waves = k_split == 8 ? 8 : 4;
+  const int tiles_per_block = waves / k_split;
+  const int blocks = (n_tiles + tiles_per_block - 1) / tiles_per_block;
+  const size_t lds = k_split > 1 ? static_cast<size_t>(waves) * MT * 4 * 64 * sizeof(float) : 0;
+  linear_skinny_kernel<MT, TY><<<blocks, waves * 64, lds, stream>>>(
+      static_cast<const bf16_t*>(x), static_cast<const uint4*>(wp), static_cast<TY*>(y), rows, outs, k, k_tiles,
+      n_tiles, k_split);
+  return AKV_LAUNCH_STATUS();
+}
+
+template <typename TY>
+int dispatch_skinny(const void* x, const void* wp, void* y, int rows, int outs, int k, int k_tiles, int n_tiles,
+                    hipStream_t stream) {
+  switch ((rows + 15) / 16) {
+    case 1: return launch_skinny<1, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+    case 2: return launch_skinny<2, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+    case 3: return launch_skinny<3, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+    case 4: return launch_skinny<4, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+    default: return -2;
+  }
+}
+
+// ---- rows > 64 ----------------------------------------------------------------------------------------------------
+// Block: 256 threads = 2 x 2 waves; block tile 128 tokens x 128 features; wave tile 64 x 64 = 4 x 4 MFMA tiles.
+// Per stage of 64 k: activations [128 tokens][64 k] go through LDS laid out [k chunk of 8][token][8] so that a
+// wave's B-operand read (16 consecutive tokens of one chunk) is 256 consecutive bytes; weights come from the packed
+// layout directly into registers.
+constexpr int kWideM = 128, kWideN = 128, kWideK = 64;
+
+template <typename TY>
+__global__ __launch_bounds__(256) void linear_wide_kernel(const bf16_t* __restrict__ x, const uint4* __restrict__ wp,
+                                                          TY* __restrict__ y, int rows, int outs, int k, int k_tiles,
+                                                          int n_tiles) {
+  __shared__ uint4 xs[2][kWideK / 8][kWideM];  // 2 stages x 8 chunks x 128 tokens x 16 B = 32 KB
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int wave_m = wave & 1, wave_n = wave >> 1;
+  const int token0 = blockIdx.y * kWideM, tile0 = blockIdx.x * (kWideN / 16) + wave_n * 4;
+  const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+  const int stages = (k_tiles + 1) / 2;
+
+  floatx4 acc[4][4];  // [feature tile][token tile]
+#pragma unroll
+  for (int n = 0; n < 4; ++n)
+#pragma unroll
+    for (int m = 0; m < 4; ++m) acc[n][m] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  // each thread moves 4 chunks of 16 B per stage: chunk c = e % 8 of token e / 8 (8 consecutive threads = 128 B of a row)
+  uint4 moving[4];
+  auto fetch = [&](int stage) {
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int e = p * 256 + threadIdx.x;
+      const int token = token0 + e / 8, at = stage * kWideK + (e % 8) * 8;
+      moving[p] = (token < rows && at < k) ? *reinterpret_cast<const uint4*>(x + static_cast<size_t>(token) * k + at) : zero;
+    }
+  };
+  auto stash = [&](int buffer) {
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int e = p * 256 + threadIdx.x;
+      xs[buffer][e % 8][e / 8] = moving[p];
+    }
+  };
+  uint4 a[2][4];  // weights of the stage's two k-tiles, 4 feature tiles
+  auto weights = [&](int stage) {
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+#pragma unroll
+      for (int n = 0; n < 4; ++n) {
+        const int kt = stage * 2 + half, tile = tile0 + n;
+        a[half][n] = (kt < k_tiles && tile < n_tiles) ? wp[(static_cast<size_t>(tile) * k_tiles + kt) * 64 + lane] : zero;
+      }
+  };
+
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  for (int stage = 0; stage < stages; ++stage) {
+    const int buffer = stage & 1;
+    weights(stage);
+    if (stage + 1 < stages) fetch(stage + 1);
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      uint4 b[4];
+#pragma unroll
+      for (int m = 0; m < 4; ++m) b[m] = xs[buffer][half * 4 + g][wave_m * 64 + m * 16 + r];
+#pragma unroll
+      for (int n = 0; n < 4; ++n)
+#pragma unroll
+        for (int m = 0; m < 4; ++m) acc[n][m] = mfma16(a[half][n], b[m], acc[n][m]);
+    }
+    if (stage + 1 < stages) stash(buffer ^ 1);
+    __syncthreads();
+  }
+#pragma unroll
+  for (int n = 0; n < 4; ++n)
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+      store_tile<TY>(y, acc[n][m], token0 + wave_m * 64 + m * 16 + r, (tile0 + n) * 16 + g * 4, rows, outs);
+}
+
+template <typename TY>
+int launch_wide(const void* x, const void* wp, void* y, int rows, int outs, int k, int k_tiles, int n_tiles,
+                hipStream_t stream) {
+  dim3 grid((n_tiles * 16 + kWideN - 1) / kWideN, (rows + kWideM - 1) / kWideM);
+  if (grid.y > 65535) return -2;
+  linear_wide_kernel<TY><<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<const uint4*>(wp),
+                                                    static_cast<TY*>(y), rows, outs, k, k_tiles, n_tiles);
+  return AKV_LAUNCH_STATUS();
+}
+
+}  // namespace
+
+// x [rows, k] bfloat16 row-major; wp the packed weight of `n_tiles` x `k_tiles` tiles; y [rows, outs] bfloat16 or
+// float32.  k must be a multiple of 8 (a lane's 16-byte read of x must lie inside or outside the row as a whole).
+extern "C" int akv_linear_packed(const void* x, const void* wp, void* y, int y_dtype, int rows, int outs, int k,
+                                 int n_tiles, int k_tiles, hipStream_t stream) {
+  if (rows <= 0 || outs <= 0) return 0;
+  if ((k & 7) != 0 || n_tiles * 16 < outs || k_tiles * 32 < k) return -2;
+  if (rows <= 64) {
+    if (y_dtype == kF32) return dispatch_skinny<float>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+    if (y_dtype == kBF16) return dispatch_skinny<bf16_t>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+    return -1;
+  }
+  if (y_dtype == kF32) return launch_wide<float>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+  if (y_dtype == kBF16) return launch_wide<bf16_t>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+  return -1;
+}

@@ -21,6 +21,28 @@ class KernelError(RuntimeError):
     pass
 
 
+class PackedWeight:
+    """A bfloat16 matrix [outs, k] re-laid for the matrix cores: tiles of 16 rows x 32 k, 1 KB each, stored
+    [row tile][k tile][lane][8] with lane = (k chunk of 8) * 16 + row; rows and k beyond the matrix are zero."""
+
+    def __init__(self, matrix: torch.Tensor):
+        outs, k = matrix.shape
+        self.outs, self.k = outs, k
+        self.n_tiles, self.k_tiles = (outs + 15) // 16, (k + 31) // 32
+        padded = matrix
+        if outs % 16 or k % 32:
+            padded = torch.zeros((self.n_tiles * 16, self.k_tiles * 32), dtype=matrix.dtype, device=matrix.device)
+            padded[:outs, :k] = matrix
+        self.data = (padded.view(self.n_tiles, 16, self.k_tiles, 4, 8).permute(0, 2, 3, 1, 4).contiguous()
+                     .view(self.n_tiles, self.k_tiles, 512))
+        self.dtype, self.device, self.shape = matrix.dtype, matrix.device, (outs, k)
+
+    def unpack(self) -> torch.Tensor:
+        """The matrix back in row-major order (for checks)."""
+        full = self.data.view(self.n_tiles, self.k_tiles, 4, 16, 8).permute(0, 3, 1, 2, 4)
+        return full.reshape(self.n_tiles * 16, self.k_tiles * 32)[:self.outs, :self.k].contiguous()
+
+
 def _code(t: torch.Tensor) -> int:
     try:
         return _DTYPE_CODE[t.dtype]
@@ -51,7 +73,7 @@ class HipKernels:
         self.library_path = path
         for name in ("akv_embed", "akv_add_rmsnorm", "akv_rmsnorm_rows", "akv_copy_rows", "akv_gather_rows",
                      "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
-                     "akv_linear_tiled", "akv_attention_rows", "akv_sample"):
+                     "akv_linear_tiled", "akv_linear_packed", "akv_attention_rows", "akv_sample"):
             getattr(self.lib, name).restype = ctypes.c_int
 
     # ---- helpers -----------------------------------------------------------------------------------------
@@ -150,7 +172,22 @@ class HipKernels:
         self._check(self.lib.akv_gather_rows(_ptr(stream), _ptr(pending), code, _ptr(rows), _ptr(out), wanted, hidden,
                                              tokens, self._stream()), "gather_rows")
 
+    def prepare_linear(self, matrix: torch.Tensor):
+        """bfloat16 matrices whose k is a multiple of 8 are packed for the MFMA kernels; others stay row-major and
+        go through the plain tiled kernel."""
+        if matrix.dtype == torch.bfloat16 and matrix.shape[1] % 8 == 0:
+            return PackedWeight(matrix)
+        return matrix
+
     def linear(self, x, weight, out):
+        if isinstance(weight, PackedWeight):
+            rows, k = x.shape
+            self._dense(x, "x", torch.bfloat16, (rows, weight.k))
+            self._dense(out, "out", None, (rows, weight.outs))
+            self._dense(weight.data, "packed weight", torch.bfloat16)
+            self._check(self.lib.akv_linear_packed(_ptr(x), _ptr(weight.data), _ptr(out), _code(out), rows, weight.outs,
+                                                   weight.k, weight.n_tiles, weight.k_tiles, self._stream()), "linear")
+            return
         rows, k = x.shape
         outs = weight.shape[0]
         self._dense(x, "x")
@@ -186,10 +223,11 @@ class HipKernels:
     # ---- cache -------------------------------------------------------------------------------------------
     def _pages(self, k_pages, v_pages, kv_heads, dim, dtype):
         self._dense(k_pages, "k_pages", dtype)
-        self._dense(v_pages, "v_pages", dtype, tuple(k_pages.shape))
         if k_pages.dim() != 4 or k_pages.shape[1] != kv_heads or k_pages.shape[3] != dim:
-            raise KernelError(f"pages must be [pages, {kv_heads}, page_size, {dim}], got {tuple(k_pages.shape)}")
-        return k_pages.shape[0], k_pages.shape[2]
+            raise KernelError(f"key pages must be [pages, {kv_heads}, page_size, {dim}], got {tuple(k_pages.shape)}")
+        num_pages, page_size = k_pages.shape[0], k_pages.shape[2]
+        self._dense(v_pages, "v_pages", dtype, (num_pages, kv_heads, dim, page_size))
+        return num_pages, page_size
 
     def kv_write(self, k, v, slot_map, k_pages, v_pages):
         tokens, kv_heads, dim, k_stride = self._rows_view(k, "k")

@@ -17,7 +17,8 @@ class Linear(Part):
         self.out_features = list(out_features)
         self.names = list(names)
         self.role = role
-        self.weight: torch.Tensor | None = None
+        self.weight = None          # what the kernels read: the matrix, or the kernel set's packing of it
+        self._bytes = 0
 
     @property
     def total_out(self) -> int:
@@ -33,14 +34,19 @@ class Linear(Part):
         if len(dtypes) != 1:
             raise ValueError(f"matrices stacked into one product are stored in different dtypes: "
                              f"{[prefix + n for n in self.names]} -> {sorted(map(str, dtypes))}")
-        self.weight = pieces[0].contiguous() if len(pieces) == 1 else torch.cat(pieces, dim=0).contiguous()
+        self._adopt(pieces[0].contiguous() if len(pieces) == 1 else torch.cat(pieces, dim=0).contiguous())
 
     def adopt(self, weight: torch.Tensor):
         """Use an already loaded matrix (a head tied to the embedding)."""
-        self.weight = weight
+        self._adopt(weight)
+
+    def _adopt(self, matrix: torch.Tensor):
+        self._bytes = matrix.numel() * matrix.element_size()
+        # the kernel set may re-lay the matrix for its matrix cores; the row-major original is then let go
+        self.weight = self.rt.kernels.prepare_linear(matrix)
 
     def weight_bytes(self):
-        return self.weight.numel() * self.weight.element_size()
+        return self._bytes
 
     def forward(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         self.rt.kernels.linear(x, self.weight, out)

@@ -1,0 +1,155 @@
+"""Decode and prefill throughput of the engine at Qwen3-8B layer sizes with random bfloat16 weights on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--context S] [--layers L]
+
+A "step" is one decode step of the whole batch: every live request feeds its last token through the engine's
+step function and the sampler chooses the next one (greedy), exactly as generation does.  The requests' caches
+are brought to the context length beforehand (pages filled with random keys and values: what they hold does
+not change the time a step takes).  One JSON line is printed:
+  value     decoded tokens per second at the default batch
+  prefill   one request's 2,048-token prompt fed whole: tokens/s, ms, and flops / time / bf16 MFMA peak
+  roofline  bytes a decode step has to read (every weight once + the live requests' cache) / its time / HBM peak
+  points    decoded tokens per second at batch 1 and 64
+Peaks are MI355X's published ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# BASELINE.json configs[2]: Qwen3-8B layer sizes, page size 16, context 8,192, prefill of 2,048 tokens
+QWEN3_8B = dict(architectures=["Qwen3ForCausalLM"], num_hidden_layers=36, hidden_size=4096, num_attention_heads=32,
+                num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=151936, rope_theta=1000000.0,
+                rms_norm_eps=1e-6, tie_word_embeddings=False, hidden_act="silu")
+PAGE_SIZE, CONTEXT, PREFILL_TOKENS = 16, 8192, 2048
+HBM_PEAK_GBS, BF16_PEAK_FLOPS = 8000.0, 2.5e15
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=64)
+    parser.add_argument("--warmup", type=int, default=8)
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--context", type=int, default=CONTEXT)
+    parser.add_argument("--layers", type=int, default=QWEN3_8B["num_hidden_layers"],
+                        help="fewer layers than the configuration has, where memory or time needs it")
+    parser.add_argument("--points", default="1,64", help="further batch sizes to time (comma separated, '' for none)")
+    parser.add_argument("--no-prefill", action="store_true")
+    args = parser.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this engine has no multi-GPU path, run it with --gpus 1")
+        return 2
+
+    import torch
+    from ampere_kv_engine_amd.config import EngineConfig, Qwen3Config
+    from ampere_kv_engine_amd.engine import Engine, StepEntry
+    from ampere_kv_engine_amd.sampling import Sampler, SamplingParams
+
+    points = [int(p) for p in args.points.split(",") if p]
+    max_batch = max([args.batch] + points)
+    raw = dict(QWEN3_8B, num_hidden_layers=args.layers)
+    config = Qwen3Config.from_dict(raw)
+    tokens_per_request = args.context + args.warmup + args.steps + 1
+    pages = max_batch * ((tokens_per_request + PAGE_SIZE - 1) // PAGE_SIZE) + PREFILL_TOKENS // PAGE_SIZE + 2
+    engine_config = EngineConfig(dtype="bfloat16", page_size=PAGE_SIZE, num_pages=pages, max_seqs=max_batch,
+                                 max_batched_tokens=PREFILL_TOKENS, max_seq_len=tokens_per_request + PAGE_SIZE,
+                                 device="cuda:0")
+    engine = Engine.from_random(config, seed=0, engine_config=engine_config)
+    for group in engine.cache.groups:       # any finite keys and values: their content does not change the timing
+        group.pages.normal_(0.0, 0.5)
+    sampler = Sampler(engine.kernels, engine.device, max_batch)
+    generator = torch.Generator().manual_seed(0)
+    sync = lambda: torch.cuda.synchronize(engine.device)
+
+    def decode(batch: int, steps: int, warmup: int) -> float:
+        """Seconds for `steps` decode steps of `batch` requests whose caches hold `context` tokens."""
+        seqs = [engine.open(f"b{batch}_{i}") for i in range(batch)]
+        for seq in seqs:
+            engine.cache.reserve(seq, args.context - 1)
+        tokens = torch.randint(0, config.vocab_size, (batch,), generator=generator).tolist()
+        greedy, draws = [SamplingParams() for _ in range(batch)], [0] * batch
+
+        def one_step():
+            nonlocal tokens
+            logits = engine.step([StepEntry(seq, [token], [0]) for seq, token in zip(seqs, tokens)])
+            tokens = sampler.sample(logits, greedy, draws)
+
+        for _ in range(warmup):
+            one_step()
+        sync()
+        started = time.perf_counter()
+        for _ in range(steps):
+            one_step()
+        sync()
+        elapsed = time.perf_counter() - started
+        for seq in seqs:
+            engine.close(seq)
+        assert engine.cache.num_free_pages == [pages]
+        return elapsed
+
+    def prefill(repeats: int = 3) -> float:
+        """Median seconds to feed one 2,048-token prompt whole and choose its first token."""
+        prompt = torch.randint(0, config.vocab_size, (PREFILL_TOKENS,), generator=generator).tolist()
+        samples = []
+        for run in range(repeats + 1):
+            seq = engine.open(f"prefill{run}")
+            sync()
+            started = time.perf_counter()
+            logits = engine.step([StepEntry(seq, prompt, [PREFILL_TOKENS - 1])])
+            sampler.sample(logits, [SamplingParams()], [0])
+            sync()
+            if run:                          # the first run warms up
+                samples.append(time.perf_counter() - started)
+            engine.close(seq)
+        return sorted(samples)[len(samples) // 2]
+
+    elapsed = decode(args.batch, args.steps, args.warmup)
+    ms_per_step = elapsed / args.steps * 1000
+    value = args.batch * args.steps / elapsed
+    weight_bytes = engine.model.weight_bytes_per_step()
+    kv_bytes = args.batch * (args.context + args.warmup + args.steps // 2) * engine.cache.bytes_per_token()
+    achieved = (weight_bytes + kv_bytes) / (ms_per_step / 1000) / 1e9
+    record = {
+        "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2,048 tokens (Qwen3-8B bf16)",
+        "value": round(value, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic: random-init weights N(0, 0.02), uniform random token ids, random cache",
+        "config": {"model": "Qwen3-8B layer sizes", "global_batch": args.batch, "seq_len": args.context,
+                   "parallelism": "single GPU", "layers": args.layers, "layers_of_config": QWEN3_8B["num_hidden_layers"],
+                   "hidden": config.hidden_size, "q_heads": config.num_attention_heads,
+                   "kv_heads": config.num_key_value_heads, "head_dim": config.head_dim,
+                   "intermediate": config.intermediate_size, "vocab": config.vocab_size, "page_size": PAGE_SIZE,
+                   "prefill_tokens": PREFILL_TOKENS, "rope_theta": config.rope_theta, "rms_norm_eps": config.rms_norm_eps,
+                   "tied_embeddings": config.tie_word_embeddings},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+    }
+    if points:
+        record["points"] = {}
+        for batch in points:
+            steps = max(8, args.steps // 2) if batch > args.batch else args.steps
+            seconds = decode(batch, steps, max(2, args.warmup // 2))
+            record["points"][f"decode_b{batch}"] = round(batch * steps / seconds, 2)
+    if not args.no_prefill:
+        seconds = prefill()
+        layer_params = sum(engine.model.blocks[e.layer].mixer.weight_bytes() + engine.model.blocks[e.layer].feed_forward.weight_bytes()
+                           for e in engine.spec.run_order) / 2
+        flops = 2 * PREFILL_TOKENS * layer_params                              # the layers' matrix products
+        flops += 2 * PREFILL_TOKENS * PREFILL_TOKENS * config.q_size * args.layers   # causal attention (QK^T and PV halves)
+        flops += 2 * config.vocab_size * config.hidden_size                     # the head on the one wanted row
+        record["prefill"] = {"value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS,
+                             "ms": round(seconds * 1000, 3), "frac": round(flops / seconds / BF16_PEAK_FLOPS, 4)}
+    print(json.dumps(record))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -67,8 +67,9 @@ def _manager(**kw):
 def test_groups_by_need_and_tensor_shapes():
     m = _manager()
     assert [g.layers for g in m.groups] == [[0, 1], [2]]
-    assert m.groups[0].pages.shape == (2, 2, 24, 2, 4, 16) and m.groups[1].pages.shape == (1, 2, 24, 2, 4, 16)
+    assert m.groups[0].pages.shape == (2, 2, 24, 2, 4 * 16) and m.groups[1].pages.shape == (1, 2, 24, 2, 4 * 16)
     assert m.layer_cache[1].k.shape == (24, 2, 4, 16) and m.layer_cache[1].k.data_ptr() == m.groups[0].pages[1, 0].data_ptr()
+    assert m.layer_cache[1].v.shape == (24, 2, 16, 4) and m.layer_cache[1].v.data_ptr() == m.groups[0].pages[1, 1].data_ptr()
     assert m.layer_cache[3].state.shape == (3, 3, 5) and m.layer_cache[4].group is None
     assert m.bytes_per_token() == (2 * 2 + 2 * 1) * 2 * 16 * 4
 

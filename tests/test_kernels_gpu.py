@@ -112,6 +112,43 @@ def test_linear(hip, ref, x_dtype, w_dtype, y_dtype, rows, outs, k):
     torch.testing.assert_close(got.cpu().float(), want.float(), **t)
 
 
+@pytest.mark.parametrize("y_dtype", DTYPES)
+@pytest.mark.parametrize("rows", [1, 5, 16, 17, 33, 64, 65, 130, 300])
+@pytest.mark.parametrize("outs,k", [(379, 96), (64, 4096), (200, 200), (8192, 256), (1040, 1000)])
+def test_linear_packed(hip, ref, y_dtype, rows, outs, k):
+    """bfloat16 weights packed for the matrix cores: few rows (k split over waves), many rows (LDS-staged tiles),
+    sizes that are no multiple of the 16 x 32 tile."""
+    from ampere_kv_engine_amd.kernels.hip import PackedWeight
+    x = rand(rows, k, dtype=torch.bfloat16, seed=31)
+    w = rand(outs, k, dtype=torch.bfloat16, seed=32, scale=0.05)
+    packed = hip.prepare_linear(w.cuda())
+    assert isinstance(packed, PackedWeight) and torch.equal(packed.unpack().cpu(), w)
+    want = torch.empty(rows, outs, dtype=y_dtype)
+    ref.linear(x, w, want)
+    got = torch.full((rows, outs), float("nan"), dtype=y_dtype, device="cuda")
+    hip.linear(x.cuda(), packed, got)
+    t = dict(rtol=2e-4, atol=2e-5 * k ** 0.5) if y_dtype == torch.float32 else tol(torch.bfloat16)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **t)
+
+
+def test_linear_packed_rows_do_not_depend_on_the_batch(hip):
+    """A row's result is bit-identical alone and among up to 64 rows (one kernel), and among more (the other)."""
+    x = rand(200, 512, dtype=torch.bfloat16, seed=33).cuda()
+    packed = hip.prepare_linear(rand(300, 512, dtype=torch.bfloat16, seed=34).cuda())
+    for count in (40, 200):
+        whole = torch.empty(count, 300, device="cuda")
+        hip.linear(x[:count].contiguous(), packed, whole)
+        for first, n in ((0, 1), (17, 3), (39, 1)) if count == 40 else ((0, 70), (100, 100)):
+            part = torch.empty(n, 300, device="cuda")
+            hip.linear(x[first:first + n].contiguous(), packed, part)
+            assert torch.equal(part, whole[first:first + n])
+
+
+def test_linear_keeps_other_weights_row_major(hip):
+    assert isinstance(hip.prepare_linear(torch.zeros(4, 12, dtype=torch.bfloat16, device="cuda")), torch.Tensor)   # k % 8
+    assert isinstance(hip.prepare_linear(torch.zeros(4, 16, device="cuda")), torch.Tensor)                         # float32
+
+
 def test_linear_rows_do_not_depend_on_the_batch(hip):
     """Float32: a row's result is bit-identical whether it is computed alone or among others."""
     x, w = rand(67, 300, seed=13).cuda(), rand(150, 300, seed=14).cuda()
@@ -153,8 +190,9 @@ def test_rope_table_and_rope(hip, ref, dim, theta):
 
 
 def _pages(num_pages, kv_heads, page_size, dim, dtype):
+    """Key pages [pages, kv_heads, page_size, dim] and value pages [pages, kv_heads, dim, page_size], NaN-filled."""
     k = torch.full((num_pages, kv_heads, page_size, dim), float("nan"), dtype=dtype)
-    return k, k.clone()
+    return k, torch.full((num_pages, kv_heads, dim, page_size), float("nan"), dtype=dtype)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -234,7 +272,7 @@ def _attention_case(dtype, q_heads, kv_heads, dim, page_size, portions, window, 
             table[r, p] = page
             lo, hi = p * page_size, min((p + 1) * page_size, length)
             k_pages[page, :, :hi - lo] = k[lo:hi].transpose(0, 1)
-            v_pages[page, :, :hi - lo] = v[lo:hi].transpose(0, 1)
+            v_pages[page, :, :, :hi - lo] = v[lo:hi].permute(1, 2, 0)
     tokens = sum(n for _, n in portions)
     q = torch.randn(tokens, q_heads * dim, generator=g).to(dtype)
     if spike is not None:

@@ -52,6 +52,9 @@ class TorchKernels:
             picked = picked + pending[rows.long()].float()
         out.copy_(picked)
 
+    def prepare_linear(self, matrix):
+        return matrix
+
     def linear(self, x, weight, out):
         out.copy_((x.float() @ weight.float().T).to(out.dtype))
 
@@ -81,8 +84,8 @@ class TorchKernels:
     def kv_write(self, k, v, slot_map, k_pages, v_pages):
         pages, kv_heads, page_size, d = k_pages.shape
         slots = slot_map.long()
-        k_pages[slots // page_size, :, slots % page_size] = k
-        v_pages[slots // page_size, :, slots % page_size] = v
+        k_pages[slots // page_size, :, slots % page_size] = k          # keys   [pages, kv_heads, page_size, d]
+        v_pages[slots // page_size, :, :, slots % page_size] = v       # values [pages, kv_heads, d, page_size]
 
     def qk_norm_rope_write(self, qkv, q_weight, k_weight, eps, table, positions, slot_map, k_pages, v_pages,
                            q_out, q_heads, kv_heads, head_dim):
@@ -117,7 +120,7 @@ class TorchKernels:
             pages = table[r][key_pos // page_size].long()
             assert (pages >= 0).all(), "attention would read a page that was given back"
             keys = k_pages[pages, :, key_pos % page_size].float()        # [S, kv_heads, d]
-            values = v_pages[pages, :, key_pos % page_size].float()
+            values = v_pages[pages, :, :, key_pos % page_size].float()
             qs = q[first:last].reshape(last - first, q_heads, head_dim).float()
             keys = keys.repeat_interleave(group, dim=1)
             values = values.repeat_interleave(group, dim=1)
