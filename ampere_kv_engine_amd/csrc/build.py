@@ -21,6 +21,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ("elementwise.hip", "gemm.hip", "gemm_mfma.hip", "attention.hip", "sampling.hip")
 HEADERS = ("common.h", "api.h")
 LIBRARY = "libakv_kernels.so"
+ATTENTION_SOURCE = "attention_mfma.hip"        # compiled once per head size, into its own small library
+DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 128, 256)
 ARCH = "gfx950"
 # packed-fp32 instructions are switched off for all device code of this library
 FLAGS = ("-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
@@ -35,9 +37,9 @@ def _hipcc() -> str:
                        "built, and the engine has no other way to compute")
 
 
-def source_stamp() -> str:
+def source_stamp(sources=None) -> str:
     digest = hashlib.sha256()
-    for name in SOURCES + HEADERS:
+    for name in (SOURCES if sources is None else tuple(sources)) + HEADERS:
         with open(os.path.join(HERE, name), "rb") as handle:
             digest.update(name.encode() + b"\0" + handle.read())
     digest.update(" ".join(FLAGS).encode())
@@ -115,5 +117,59 @@ def ensure_built(verbose: bool = True) -> str:
     return library_path() or build(verbose)
 
 
+# ---- the attention kernels, one library per head size ------------------------------------------------------------
+
+def _attention_names(head_dim: int) -> tuple[str, str]:
+    return f"libakv_attention_d{head_dim}.so", f"stamp_attention_d{head_dim}"
+
+
+def attention_library_path(head_dim: int) -> str | None:
+    stamp = source_stamp((ATTENTION_SOURCE,))
+    lib_name, mark_name = _attention_names(head_dim)
+    for folder in (os.path.join(HERE, "_build"),
+                   os.path.join(tempfile.gettempdir(), f"akv_build_{os.getuid()}_{source_stamp()[:12]}")):
+        lib, mark = os.path.join(folder, lib_name), os.path.join(folder, mark_name)
+        if os.path.exists(lib) and os.path.exists(mark):
+            with open(mark) as handle:
+                if handle.read().strip() == stamp:
+                    return lib
+    return None
+
+
+def build_attention(head_dim: int, verbose: bool = True) -> str:
+    if head_dim % 16 or not 16 <= head_dim <= 256:
+        raise ValueError(f"the attention kernels take head sizes that are multiples of 16 up to 256, not {head_dim}")
+    hipcc = _hipcc()
+    out_dir = _build_dir()
+    started = time.time()
+    lib_name, mark_name = _attention_names(head_dim)
+    lib = os.path.join(out_dir, lib_name)
+    partial = lib + f".{os.getpid()}.tmp"
+    if verbose:
+        _log(f"compiling {ATTENTION_SOURCE} for head size {head_dim}")
+    cmd = [hipcc, *FLAGS, f"-DAKV_HEAD_DIM={head_dim}", "-shared", os.path.join(HERE, ATTENTION_SOURCE), "-o", partial]
+    result = subprocess.run(cmd, capture_output=True, text=True)
+    if result.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {ATTENTION_SOURCE} (head size {head_dim}):\n{result.stderr}")
+    os.replace(partial, lib)
+    with open(os.path.join(out_dir, mark_name), "w") as handle:
+        handle.write(source_stamp((ATTENTION_SOURCE,)))
+    if verbose:
+        _log(f"built {lib} ({time.time() - started:.0f} s)")
+    return lib
+
+
+def ensure_attention(head_dim: int, verbose: bool = True) -> str:
+    return attention_library_path(head_dim) or build_attention(head_dim, verbose)
+
+
+def build_all(head_dims=DEFAULT_HEAD_DIMS, verbose: bool = True) -> list[str]:
+    """The kernel library and the attention libraries of the usual head sizes."""
+    paths = [build(verbose)]
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        paths += list(pool.map(lambda d: build_attention(d, verbose), head_dims))
+    return paths
+
+
 if __name__ == "__main__":
-    print(build())
+    print("\n".join(build_all()))

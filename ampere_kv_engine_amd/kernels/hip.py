@@ -11,7 +11,7 @@ import ctypes
 
 import torch
 
-from ..csrc.build import ensure_built
+from ..csrc.build import ensure_attention, ensure_built
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 MAX_HEAD_DIM = 256
@@ -71,6 +71,7 @@ class HipKernels:
         except OSError as error:
             raise KernelError(f"the kernel library {path} could not be loaded: {error}") from error
         self.library_path = path
+        self._attention_entry = {}      # head size -> entry point of that head size's attention library
         for name in ("akv_embed", "akv_add_rmsnorm", "akv_rmsnorm_rows", "akv_copy_rows", "akv_gather_rows",
                      "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
                      "akv_linear_tiled", "akv_linear_packed", "akv_attention_rows", "akv_sample"):
@@ -265,16 +266,70 @@ class HipKernels:
             ctypes.c_long(tokens), q_heads, kv_heads, head_dim, page_size, ctypes.c_long(num_pages), self._stream()),
             "qk_norm_rope_write")
 
+    def _attention_mfma_entry(self, head_dim: int):
+        if head_dim not in self._attention_entry:
+            path = ensure_attention(head_dim)
+            try:
+                lib = ctypes.CDLL(path)
+            except OSError as error:
+                raise KernelError(f"the attention library {path} could not be loaded: {error}") from error
+            entry = getattr(lib, f"akv_attention_mfma_d{head_dim}")
+            entry.restype = ctypes.c_int
+            self._attention_entry[head_dim] = entry
+        return self._attention_entry[head_dim]
+
+    def _attention_mfma(self, q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out,
+                        page_size, num_pages, seq_first, seq_count, nq, split):
+        """Requests seq_first .. seq_first + seq_count - 1 of the step on the MFMA kernel, in tiles of 16 * nq
+        (token, head-of-group) columns; `split` cuts the keys over several waves (decode)."""
+        group = q_heads // kv_heads
+        heads_per_tile = min(group, 16 * nq)
+        head_groups = (group + heads_per_tile - 1) // heads_per_tile
+        tokens_per_tile = (16 * nq) // heads_per_tile
+        starts = ctx.host_q_start
+        tiles = sum((starts[r + 1] - starts[r] + tokens_per_tile - 1) // tokens_per_tile
+                    for r in range(seq_first, seq_first + seq_count))
+        num_splits, seg_keys, partial = 1, 0, None
+        if split:
+            longest = max(ctx.host_seq_lens[seq_first:seq_first + seq_count])
+            pairs = tiles * kv_heads * head_groups
+            num_splits = max(1, min((4096 + pairs - 1) // pairs, (longest + 127) // 128))
+            seg_keys = ((longest + num_splits - 1) // num_splits + 31) // 32 * 32
+            num_splits = (longest + seg_keys - 1) // seg_keys
+            if num_splits > 1:
+                count = tiles * kv_heads * head_groups * num_splits * 16 * nq * (head_dim + 4)
+                arena = getattr(ctx, "arena", None)
+                partial = (arena.take((count,), torch.float32) if arena is not None
+                           else torch.empty(count, dtype=torch.float32, device=self.device))
+        self._check(self._attention_mfma_entry(head_dim)(
+            _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial), _ptr(ctx.q_start), _ptr(ctx.seq_lens),
+            _ptr(meta.block_table), meta.width, seq_first, seq_count, tiles, nq, q_heads, kv_heads, heads_per_tile,
+            head_groups, tokens_per_tile, page_size, ctypes.c_long(num_pages), ctypes.c_float(scale),
+            int(window) if window is not None else 0, seg_keys, num_splits, self._stream()), "attention")
+
     def attention(self, q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out):
         tokens = q.shape[0]
         self._dense(q, "q", None, (tokens, q_heads * head_dim))
         self._dense(out, "out", q.dtype, (tokens, q_heads * head_dim))
         num_pages, page_size = self._pages(k_pages, v_pages, kv_heads, head_dim, q.dtype)
-        self._dense(ctx.seq_of_token, "seq_of_token", torch.int32, (tokens,))
-        self._dense(ctx.positions, "positions", torch.int32, (tokens,))
         self._dense(meta.block_table, "block_table", torch.int32, (ctx.num_seqs, meta.width))
         if ctx.max_seq_len > meta.width * page_size:
             raise KernelError(f"a request of {ctx.max_seq_len} tokens does not fit a block table of {meta.width} pages")
+        if q.dtype == torch.bfloat16 and page_size % 4 == 0:
+            self._dense(ctx.q_start, "q_start", torch.int32, (ctx.num_seqs + 1,))
+            self._dense(ctx.seq_lens, "seq_lens", torch.int32, (ctx.num_seqs,))
+            if ctx.host_q_start[ctx.num_seqs] != tokens or len(ctx.host_seq_lens) != ctx.num_seqs:
+                raise KernelError("the step's request boundaries do not match its tokens")
+            common = (q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out, page_size,
+                      num_pages)
+            decodes = ctx.num_decode_seqs
+            if decodes:      # single tokens against long histories: one small tile each, keys split over waves
+                self._attention_mfma(*common, 0, decodes, 1, True)
+            if ctx.num_seqs > decodes:
+                self._attention_mfma(*common, decodes, ctx.num_seqs - decodes, 4 if head_dim <= 128 else 2, False)
+            return
+        self._dense(ctx.seq_of_token, "seq_of_token", torch.int32, (tokens,))
+        self._dense(ctx.positions, "positions", torch.int32, (tokens,))
         self._check(self.lib.akv_attention_rows(
             _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(ctx.seq_of_token), _ptr(ctx.positions),
             _ptr(meta.block_table), meta.width, _ptr(out), _code(q), ctypes.c_long(tokens), q_heads, kv_heads,

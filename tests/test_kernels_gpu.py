@@ -30,6 +30,13 @@ def tol(dtype):
     return dict(rtol=2e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=1.6e-2, atol=1e-3)
 
 
+def attention_tol(dtype):
+    """bfloat16: the reference's own bound for its paged attention against float32 attention
+    (ampere_kv/scheduler.py:410, ampere_kv/paged_decode.py:62-81: rtol 0.01, atol 0.002); softmax weights enter the
+    weighted sum rounded to bfloat16, which alone moves an output by up to ~2^-9 of the values' size."""
+    return dict(rtol=2e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=0.01, atol=0.002)
+
+
 def rand(*shape, dtype=torch.float32, seed=0, scale=1.0):
     g = torch.Generator().manual_seed(seed)
     return (torch.randn(*shape, generator=g) * scale).to(dtype)
@@ -294,6 +301,8 @@ def _attention_case(dtype, q_heads, kv_heads, dim, page_size, portions, window, 
 def _to_cuda(ctx, meta):
     c = SimpleNamespace(**vars(ctx))
     c.positions, c.seq_of_token = ctx.positions.cuda(), ctx.seq_of_token.cuda()
+    c.q_start = torch.tensor(ctx.host_q_start, dtype=torch.int32, device="cuda")
+    c.seq_lens = torch.tensor(ctx.host_seq_lens, dtype=torch.int32, device="cuda")
     m = SimpleNamespace(**vars(meta))
     m.block_table = meta.block_table.cuda()
     return c, m
@@ -315,7 +324,52 @@ def test_attention(hip, ref, dtype, q_heads, kv_heads, dim, page_size, portions,
     got = torch.empty_like(q, device="cuda")
     hip.attention(q.cuda(), k_pages.cuda(), v_pages.cuda(), cctx, cmeta, q_heads, kv_heads, dim, dim ** -0.5, window, got)
     assert not torch.isnan(got).any()
-    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dtype))
+    torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(dtype))
+
+
+@pytest.mark.parametrize("q_heads,kv_heads,dim,page_size", ATTENTION_SIZES + [(32, 8, 128, 16), (40, 2, 64, 8)])
+@pytest.mark.parametrize("histories", [[0], [64, 17, 0], [1500, 2, 700, 255], [4000] * 9])
+@pytest.mark.parametrize("window", [None, 100])
+def test_attention_decode_batch(hip, ref, q_heads, kv_heads, dim, page_size, histories, window):
+    """Single tokens of several requests (the split-key path of the bfloat16 kernel), histories from nothing to
+    thousands of keys, more heads per group than one tile holds."""
+    portions = [(h, 1) for h in histories]
+    q, k_pages, v_pages, ctx, meta, _, _ = _attention_case(torch.bfloat16, q_heads, kv_heads, dim, page_size, portions,
+                                                           window, 25)
+    ctx.num_decode_seqs = len(portions)
+    want = torch.empty_like(q)
+    ref.attention(q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, dim, dim ** -0.5, window, want)
+    cctx, cmeta = _to_cuda(ctx, meta)
+    got = torch.empty_like(q, device="cuda")
+    hip.attention(q.cuda(), k_pages.cuda(), v_pages.cuda(), cctx, cmeta, q_heads, kv_heads, dim, dim ** -0.5, window, got)
+    assert not torch.isnan(got).any()
+    torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(torch.bfloat16))
+
+
+def test_attention_decodes_beside_portions(hip, ref):
+    """A mixed step: three single tokens first, then two portions; both launches write their own rows only."""
+    portions = [(300, 1), (15, 1), (0, 1), (40, 37), (0, 130)]
+    q, k_pages, v_pages, ctx, meta, _, _ = _attention_case(torch.bfloat16, 8, 2, 128, 16, portions, None, 26)
+    ctx.num_decode_seqs = 3
+    want = torch.empty_like(q)
+    ref.attention(q, k_pages, v_pages, ctx, meta, 8, 2, 128, 128 ** -0.5, None, want)
+    cctx, cmeta = _to_cuda(ctx, meta)
+    got = torch.full_like(q, float("nan"), device="cuda")
+    hip.attention(q.cuda(), k_pages.cuda(), v_pages.cuda(), cctx, cmeta, 8, 2, 128, 128 ** -0.5, None, got)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(torch.bfloat16))
+
+
+def test_attention_poisons_a_foreign_page(hip):
+    """A table entry inside a request's length that is no page of the pool gives NaN, not a read outside the pool."""
+    portions = [(40, 1), (40, 5)]
+    q, k_pages, v_pages, ctx, meta, _, _ = _attention_case(torch.bfloat16, 4, 2, 64, 16, portions, None, 27)
+    ctx.num_decode_seqs = 1
+    meta.block_table[0, 1] = -1
+    meta.block_table[1, 0] = 10 ** 6
+    cctx, cmeta = _to_cuda(ctx, meta)
+    got = torch.zeros_like(q, device="cuda")
+    hip.attention(q.cuda(), k_pages.cuda(), v_pages.cuda(), cctx, cmeta, 4, 2, 64, 64 ** -0.5, None, got)
+    assert torch.isnan(got).all()
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -324,12 +378,13 @@ def test_attention_finds_a_far_key(hip, ref, dtype):
     portions = [(1000, 1), (900, 3)]
     for spike in ((0, 3), (1, 517)):
         q, k_pages, v_pages, ctx, meta, keys, values = _attention_case(dtype, 4, 2, 64, 16, portions, None, 23, spike)
+        ctx.num_decode_seqs = 1            # the first request brings one token
         cctx, cmeta = _to_cuda(ctx, meta)
         got = torch.empty_like(q, device="cuda")
         hip.attention(q.cuda(), k_pages.cuda(), v_pages.cuda(), cctx, cmeta, 4, 2, 64, 64 ** -0.5, None, got)
         want = torch.empty_like(q)
         ref.attention(q, k_pages, v_pages, ctx, meta, 4, 2, 64, 64 ** -0.5, None, want)
-        torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dtype))
+        torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(dtype))
         r, at = spike
         first = ctx.host_q_start[r]
         picked = got.cpu().float()[first].reshape(4, 64)
