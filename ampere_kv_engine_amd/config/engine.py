@@ -20,6 +20,7 @@ class EngineConfig:
     max_batched_tokens: int = 2048   # most tokens one step may carry
     max_seq_len: int = 8192          # longest sequence a request may reach (block-table width, rotary table)
     device: str = "cuda:0"
+    decode_graphs: bool = True       # replay a recorded HIP graph for steps in which every request brings one token
 
     def __post_init__(self):
         if self.dtype not in DTYPES:

@@ -13,6 +13,8 @@
 // aligned to absolute positions.  With SPLIT, grid.z cuts the keys into segments whose partial results (maximum,
 // sum, unnormalised output) a second kernel merges: decode has too few (request, head) pairs to fill the GPU otherwise.
 
+#include <type_traits>
+
 #include "common.h"
 #include "api.h"
 
@@ -33,6 +35,8 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
+typedef __attribute__((ext_vector_type(2))) float floatx2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 
 __device__ __forceinline__ floatx4 mfma16(uint4 a, uint4 b, floatx4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
@@ -49,8 +53,9 @@ struct Args {
   const int* block_table;     // [requests, table_width]
   int table_width;
   int seq_first, seq_count;   // the launch covers requests seq_first .. seq_first + seq_count - 1
+  int single_tokens;          // every request of the launch brings exactly one token: tile i is request seq_first + i
   int q_heads, kv_heads, group, heads_per_tile, head_groups, tokens_per_tile;
-  int page_size;
+  int page_shift;             // page_size = 1 << page_shift, at least 4
   long num_pages;
   float scale_log2;           // softmax scale * log2(e)
   int window;                 // 0: none
@@ -59,37 +64,71 @@ struct Args {
 
 // Which request and which of its tiles this block works on.
 struct Tile {
-  int request, first_row, tokens, first_pos, history;
+  int request, first_row, tokens, first_pos;
   bool found;
 };
 
+// Tiles are numbered request by request.  The wave looks at 64 requests at a time: every lane counts the tiles of
+// one request, a prefix sum over the lanes places them, and the lane whose span holds `slot` owns the answer.
 __device__ __forceinline__ Tile find_tile(const Args& a, int slot) {
   Tile t{};
   t.found = false;
-  for (int r = a.seq_first; r < a.seq_first + a.seq_count; ++r) {
-    const int begin = a.q_start[r], count = a.q_start[r + 1] - begin;
+  const int lane = threadIdx.x & 63, end = a.seq_first + a.seq_count;
+  if (a.single_tokens) {
+    if (slot >= a.seq_count) return t;
+    t.request = a.seq_first + slot;
+    t.first_row = a.q_start[t.request];
+    t.tokens = 1;
+    t.first_pos = a.seq_lens[t.request] - 1;
+    t.found = true;
+    return t;
+  }
+  int before = 0;  // tiles of the requests already passed
+  for (int r0 = a.seq_first; r0 < end; r0 += 64) {
+    const int r = r0 + lane;
+    int begin = 0, count = 0;
+    if (r < end) {
+      begin = a.q_start[r];
+      count = a.q_start[r + 1] - begin;
+    }
     const int tiles = (count + a.tokens_per_tile - 1) / a.tokens_per_tile;
-    if (slot < tiles) {
-      t.request = r;
-      t.first_row = begin + slot * a.tokens_per_tile;
-      t.tokens = min(a.tokens_per_tile, count - slot * a.tokens_per_tile);
-      t.history = a.seq_lens[r] - count;
-      t.first_pos = t.history + slot * a.tokens_per_tile;
+    int upto = tiles;  // inclusive prefix sum over the wave
+#pragma unroll
+    for (int step = 1; step < 64; step <<= 1) {
+      const int other = __shfl_up(upto, step, 64);
+      if (lane >= step) upto += other;
+    }
+    const int total = __shfl(upto, 63, 64);
+    if (slot < before + total) {
+      const bool mine = slot >= before + upto - tiles && slot < before + upto;
+      const int owner = __ffsll(static_cast<unsigned long long>(__ballot(mine))) - 1;
+      const int local = slot - (before + __shfl(upto - tiles, owner, 64));
+      const int o_begin = __shfl(begin, owner, 64), o_count = __shfl(count, owner, 64);
+      t.request = r0 + owner;
+      t.first_row = o_begin + local * a.tokens_per_tile;
+      t.tokens = min(a.tokens_per_tile, o_count - local * a.tokens_per_tile);
+      t.first_pos = a.seq_lens[t.request] - o_count + local * a.tokens_per_tile;
       t.found = true;
       return t;
     }
-    slot -= tiles;
+    before += total;
   }
   return t;
 }
 
-template <int NQ, bool SPLIT>
+// Inside a step of 32 keys starting at `base`, MFMA tile j (0 or 1), row rho (0..15) is key
+//     base + (rho / 4) * 8 + j * 4 + rho % 4.
+// With this order the 8 score elements a lane holds (rows 4g .. 4g + 3 of both tiles) are the 8 CONSECUTIVE keys
+// base + 8g .. + 7, so the value operand of lane group g is one 16-byte read of a value page row.
+// PIPE: the next step's keys are fetched while this step computes (costs registers: used where they are there).
+template <int NQ, bool SPLIT, bool PIPE>
 __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
   const int lane = threadIdx.x, r16 = lane & 15, g = lane >> 4;
   const Tile t = find_tile(a, blockIdx.x);
   if (!t.found) return;
   const int kvh = blockIdx.y / a.head_groups, hg = blockIdx.y % a.head_groups;
   const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+  const int page_size = 1 << a.page_shift, page_mask = page_size - 1;
 
   // this lane's columns: one per NQ tile
   bool col_valid[NQ];
@@ -131,108 +170,207 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
   }
   bool poisoned = false;  // a key inside the range lies in a page that is not the request's
   const int* table = a.block_table + static_cast<long>(t.request) * a.table_width;
+  const int key_in_step = (r16 >> 2) * 8 + (r16 & 3);  // + j * 4: this lane's key row of tile j
 
-  for (int base = range_lo & ~31; base <= range_hi; base += 32) {
+  // Addresses are 32-bit byte offsets from the page tensors (the host refuses tensors of 4 GB and more), so that a
+  // load is one instruction on a scalar base and a lane offset instead of 64-bit arithmetic per lane.
+  const char* k_bytes = reinterpret_cast<const char*>(a.k_pages);
+  const char* v_bytes = reinterpret_cast<const char*>(a.v_pages);
+  const uint32_t page_bytes = static_cast<uint32_t>(a.kv_heads) * D * 2u << a.page_shift;  // one page, all kv heads
+  const uint32_t head_bytes = static_cast<uint32_t>(kvh) * D * 2u << a.page_shift;         // this kv head inside a page
+  const uint32_t k_lane = head_bytes + g * 16u;                         // + key row * D * 2 + kt * 64
+  const uint32_t v_lane = head_bytes + (static_cast<uint32_t>(r16) << (a.page_shift + 1));  // + dt * 16 rows + key * 2
+  const uint32_t v_tile = 32u << a.page_shift;                          // 16 value rows
+
+  // Keys of the step at `base` into A operands.  CHECK: the step may reach outside [range_lo, range_hi]; rows outside
+  // are zero and never looked up.
+  auto load_keys = [&](int base, uint4 (&dst)[2][KT], auto check) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int key = base + key_in_step + j * 4;
+      const bool wanted = !decltype(check)::value || (key >= range_lo && key <= range_hi);
+      int page = 0;
+      if (wanted) {
+        page = table[key >> a.page_shift];
+        if (page < 0 || page >= a.num_pages) {
+          poisoned = true;
+          page = 0;
+        }
+      }
+      const uint32_t at = static_cast<uint32_t>(page) * page_bytes + k_lane + static_cast<uint32_t>(key & page_mask) * (D * 2u);
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) {
+        const bool inside = (D % 32 == 0) || kt * 32 + g * 8 < D;
+        dst[j][kt] = (wanted && inside) ? *reinterpret_cast<const uint4*>(k_bytes + at + kt * 64u) : zero;
+      }
+    }
+  };
+  // Values of the step at `base` into A operands: lane (dim row r16 of tile dt, keys base + 8g .. + 7).  CHECK: slots
+  // of keys beyond the range are zeroed (they were never written and may hold anything, NaN included).
+  auto load_values = [&](int base, uint4 (&dst)[DT], auto check) {
+    const int key = base + g * 8;
+    if (!decltype(check)::value && page_size >= 8) {
+      int page = table[key >> a.page_shift];
+      if (page < 0 || page >= a.num_pages) {
+        poisoned = true;
+        page = 0;
+      }
+      const uint32_t at = static_cast<uint32_t>(page) * page_bytes + v_lane + static_cast<uint32_t>(key & page_mask) * 2u;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) dst[dt] = *reinterpret_cast<const uint4*>(v_bytes + at + dt * v_tile);
+      return;
+    }
+    const int live = min(8, range_hi - key + 1);
+    bool have[2] = {false, false};
+    uint32_t at[2] = {0u, 0u};
+    if (live > 0 && key + 7 >= range_lo) {
+      // pages of 8 and more hold the 8 keys together; pages of 4 hold them in two pages
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int first = key + half * 4;
+        if (half == 1 && (page_size >= 8 || live <= 4)) break;
+        if (half == 0 && page_size < 8 && key + 3 < range_lo) continue;
+        const int page = table[first >> a.page_shift];
+        if (page < 0 || page >= a.num_pages) poisoned = true;
+        else {
+          have[half] = true;
+          at[half] = static_cast<uint32_t>(page) * page_bytes + v_lane + static_cast<uint32_t>(first & page_mask) * 2u;
+        }
+      }
+    }
+    uint32_t keep[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) keep[w] = live >= 2 * w + 2 ? 0xffffffffu : (live == 2 * w + 1 ? 0x0000ffffu : 0u);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      uint4 v = zero;
+      if (page_size >= 8) {
+        if (have[0]) v = *reinterpret_cast<const uint4*>(v_bytes + at[0] + dt * v_tile);
+      } else {
+        if (have[0]) {
+          const uint2 h = *reinterpret_cast<const uint2*>(v_bytes + at[0] + dt * v_tile);
+          v.x = h.x;
+          v.y = h.y;
+        }
+        if (have[1]) {
+          const uint2 h = *reinterpret_cast<const uint2*>(v_bytes + at[1] + dt * v_tile);
+          v.z = h.x;
+          v.w = h.y;
+        }
+      }
+      dst[dt] = make_uint4(v.x & keep[0], v.y & keep[1], v.z & keep[2], v.w & keep[3]);
+    }
+  };
+
+  uint4 kreg[2][KT], knext[PIPE ? 2 : 1][PIPE ? KT : 1], vreg[DT];
+  const std::true_type checked{};
+  const std::false_type unchecked{};
+  auto inside = [&](int base) { return base >= range_lo && base + 31 <= range_hi; };
+
+  // One step of 32 keys.  MASK: some column does not see the whole step (diagonal, window, segment edge).
+  auto step = [&](int base, auto mask) {
     // ---- S^T = K . Q^T for two tiles of 16 keys --------------------------------------------------------------
     floatx4 s[NQ][2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int key = base + j * 16 + r16;
-      const bf16_t* kp = nullptr;
-      if (key >= range_lo && key <= range_hi) {
-        const long page = table[key / a.page_size];
-        if (page < 0 || page >= a.num_pages) poisoned = true;
-        else kp = a.k_pages + ((page * a.kv_heads + kvh) * a.page_size + key % a.page_size) * D;
-      }
 #pragma unroll
       for (int nq = 0; nq < NQ; ++nq) s[nq][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int kt = 0; kt < KT; ++kt) {
-        const int dim = kt * 32 + g * 8;
-        const uint4 kreg = (kp != nullptr && dim < D) ? *reinterpret_cast<const uint4*>(kp + dim) : zero;
+      for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-        for (int nq = 0; nq < NQ; ++nq) s[nq][j] = mfma16(kreg, qreg[nq][kt], s[nq][j]);
-      }
+        for (int nq = 0; nq < NQ; ++nq) s[nq][j] = mfma16(kreg[j][kt], qreg[nq][kt], s[nq][j]);
     }
-    // ---- mask, running maximum and sum per column (a column lives in the 4 lanes with the same r16) ---------------
+    // ---- running maximum and sum per column (a column lives in the 4 lanes with the same r16) ---------------------
     uint4 preg[NQ], plow[NQ];  // softmax weights as bfloat16 pairs: rounded value, and what the rounding lost
     float correction[NQ];
+    bool rescale = false;
 #pragma unroll
     for (int nq = 0; nq < NQ; ++nq) {
-      float top = -INFINITY;
+      if (decltype(mask)::value) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int key = base + j * 16 + g * 4 + i;
-          const bool seen = col_valid[nq] && key <= col_pos[nq] && key >= col_low[nq] && key >= range_lo && key <= range_hi;
-          s[nq][j][i] = seen ? s[nq][j][i] * a.scale_log2 : -INFINITY;
-          top = fmaxf(top, s[nq][j][i]);
-        }
+          for (int i = 0; i < 4; ++i) {
+            const int key = base + g * 8 + j * 4 + i;
+            const bool seen = col_valid[nq] && key <= col_pos[nq] && key >= col_low[nq] && key >= range_lo && key <= range_hi;
+            if (!seen) s[nq][j][i] = -INFINITY;
+          }
+      }
+      float top = fmaxf(fmaxf(fmaxf(s[nq][0][0], s[nq][0][1]), fmaxf(s[nq][0][2], s[nq][0][3])),
+                        fmaxf(fmaxf(s[nq][1][0], s[nq][1][1]), fmaxf(s[nq][1][2], s[nq][1][3])));
       top = fmaxf(top, __shfl_xor(top, 16, 64));
       top = fmaxf(top, __shfl_xor(top, 32, 64));
-      const float m_new = fmaxf(m[nq], top);
+      const float m_new = fmaxf(m[nq], top * a.scale_log2);   // the scale is positive: max commutes with it
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;  // nothing seen yet: every weight is 0, no NaN
       correction[nq] = __builtin_amdgcn_exp2f(m[nq] - m_safe);
+      rescale = rescale || correction[nq] != 1.f;
+      floatx2 p[4];
       float sum = 0.f;
-      float p[8];
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          p[j * 4 + i] = __builtin_amdgcn_exp2f(s[nq][j][i] - m_safe);
-          sum += p[j * 4 + i];
-        }
-      sum += __shfl_xor(sum, 16, 64);
-      sum += __shfl_xor(sum, 32, 64);
-      l[nq] = l[nq] * correction[nq] + sum;
-      m[nq] = m_new;
-      // key slots of the second product, for lane group g: keys base + 4g .. + 3, then base + 16 + 4g .. + 3.
-      // A weight enters as two bfloat16 numbers (p = high + low, 16 bits of mantissa together), so that the
-      // weighted sum does not carry the 2^-9 relative error of a single bfloat16.
-      uint32_t high[8], low[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        high[e] = bf16_bits(p[e]);
-        low[e] = bf16_bits(p[e] - __uint_as_float(high[e] << 16));
+      for (int e = 0; e < 4; ++e) {
+        p[e][0] = __builtin_amdgcn_exp2f(fmaf(s[nq][e >> 1][(e & 1) * 2], a.scale_log2, -m_safe));
+        p[e][1] = __builtin_amdgcn_exp2f(fmaf(s[nq][e >> 1][(e & 1) * 2 + 1], a.scale_log2, -m_safe));
+        sum += p[e][0] + p[e][1];
       }
-      preg[nq] = make_uint4(high[0] | (high[1] << 16), high[2] | (high[3] << 16), high[4] | (high[5] << 16), high[6] | (high[7] << 16));
-      plow[nq] = make_uint4(low[0] | (low[1] << 16), low[2] | (low[3] << 16), low[4] | (low[5] << 16), low[6] | (low[7] << 16));
+      l[nq] = l[nq] * correction[nq] + sum;  // this lane's own 8 keys; the 4 lanes of a column are added at the end
+      m[nq] = m_new;
+      // A weight enters the second product as two bfloat16 numbers (p = high + low, 16 bits of mantissa together),
+      // so that the weighted sum does not carry the 2^-9 relative error of a single bfloat16.
+      uint32_t high[4], low[4];
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) o[nq][dt] *= correction[nq];
+      for (int e = 0; e < 4; ++e) {
+        high[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(p[e], bf16x2));
+        const floatx2 rest = {p[e][0] - __uint_as_float(high[e] << 16), p[e][1] - __uint_as_float(high[e] & 0xffff0000u)};
+        low[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(rest, bf16x2));
+      }
+      preg[nq] = make_uint4(high[0], high[1], high[2], high[3]);
+      plow[nq] = make_uint4(low[0], low[1], low[2], low[3]);
+    }
+    if (__any(rescale)) {  // the maxima rarely move after the first steps
+#pragma unroll
+      for (int nq = 0; nq < NQ; ++nq)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o[nq][dt] *= correction[nq];
     }
     // ---- O^T += V^T . P^T -------------------------------------------------------------------------------------------
-    const bf16_t* vp[2];
-    uint32_t keep[2][2];  // masks that zero the slots of keys beyond the range (never written, may hold anything)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int key = base + j * 16 + g * 4;
-      vp[j] = nullptr;
-      const int live = min(4, range_hi - key + 1);  // keys of this group of 4 that exist
-      if (live > 0 && key + 3 >= range_lo) {
-        const long page = table[key / a.page_size];
-        if (page < 0 || page >= a.num_pages) poisoned = true;
-        else vp[j] = a.v_pages + (page * a.kv_heads + kvh) * static_cast<long>(D) * a.page_size + key % a.page_size;
-      }
-      keep[j][0] = live >= 2 ? 0xffffffffu : (live == 1 ? 0x0000ffffu : 0u);
-      keep[j][1] = live >= 4 ? 0xffffffffu : (live == 3 ? 0x0000ffffu : 0u);
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int nq = 0; nq < NQ; ++nq) o[nq][dt] = mfma16(vreg[dt], plow[nq], mfma16(vreg[dt], preg[nq], o[nq][dt]));
+  };
+
+  const int first_base = range_lo & ~31;
+  if (PIPE && first_base <= range_hi) {
+    if (inside(first_base)) load_keys(first_base, kreg, unchecked);
+    else load_keys(first_base, kreg, checked);
+  }
+  for (int base = first_base; base <= range_hi; base += 32) {
+    // memory first: this step's values (needed after the softmax) and the next step's keys (needed next turn)
+    const bool here = inside(base);
+    if (!PIPE) {
+      if (here) load_keys(base, kreg, unchecked);
+      else load_keys(base, kreg, checked);
     }
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      const long row = static_cast<long>(dt * 16 + r16) * a.page_size;
-      uint4 vreg = zero;
-      if (vp[0] != nullptr) {
-        const uint2 v = *reinterpret_cast<const uint2*>(vp[0] + row);
-        vreg.x = v.x & keep[0][0];
-        vreg.y = v.y & keep[0][1];
+    if (here) load_values(base, vreg, unchecked);
+    else load_values(base, vreg, checked);
+    const bool more = PIPE && base + 32 <= range_hi;
+    if constexpr (PIPE) {
+      if (more) {
+        if (inside(base + 32)) load_keys(base + 32, knext, unchecked);
+        else load_keys(base + 32, knext, checked);
       }
-      if (vp[1] != nullptr) {
-        const uint2 v = *reinterpret_cast<const uint2*>(vp[1] + row);
-        vreg.z = v.x & keep[1][0];
-        vreg.w = v.y & keep[1][1];
-      }
+    }
+    // every valid column sees the whole step: below the diagonal, inside window and segment
+    const bool whole = here && base + 31 <= t.first_pos && (a.window == 0 || base >= last_pos - a.window + 1);
+    if (whole) step(base, unchecked);
+    else step(base, checked);
+    if constexpr (PIPE) {
+      if (more) {
 #pragma unroll
-      for (int nq = 0; nq < NQ; ++nq) o[nq][dt] = mfma16(vreg, plow[nq], mfma16(vreg, preg[nq], o[nq][dt]));
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int kt = 0; kt < KT; ++kt) kreg[j][kt] = knext[j][kt];
+      }
     }
   }
 
@@ -241,7 +379,10 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
   poisoned = __any(poisoned);
 #pragma unroll
   for (int nq = 0; nq < NQ; ++nq) {
+    l[nq] += __shfl_xor(l[nq], 16, 64);
+    l[nq] += __shfl_xor(l[nq], 32, 64);
     if (SPLIT) {
+      if (!col_valid[nq]) continue;  // the merge never reads the columns that are no (token, head) of the tile
       const int c = nq * 16 + r16;
       float* dst = a.partial + ((((static_cast<long>(blockIdx.x) * gridDim.y + blockIdx.y) * a.num_splits + blockIdx.z) * (16 * NQ)) + c) * PSTRIDE;
 #pragma unroll
@@ -264,49 +405,54 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
 }
 
 // Merge of the segments' partial results: out = sum_z 2^(m_z - M) O_z / sum_z 2^(m_z - M) l_z, M = max_z m_z
-// (csrc/paged_decode.cu:528-544 of the reference has the same rule in base e).  One wave per (tile, head group);
-// lane = (column, quarter of the dims).
+// (csrc/paged_decode.cu:528-544 of the reference has the same rule in base e).  One wave per (tile, head group,
+// column); a lane owns dims lane, lane + 64, ...; the segments are summed in ascending order.
 template <int NQ>
-__global__ __launch_bounds__(64 * NQ) void attention_merge_kernel(const Args a) {
+__global__ __launch_bounds__(64) void attention_merge_kernel(const Args a) {
   const Tile t = find_tile(a, blockIdx.x);
   if (!t.found) return;
   const int kvh = blockIdx.y / a.head_groups, hg = blockIdx.y % a.head_groups;
-  const int c = threadIdx.x >> 2, quarter = threadIdx.x & 3;  // 16 * NQ columns x 4 lanes
+  const int c = blockIdx.z, lane = threadIdx.x;
   const int token = c / a.heads_per_tile, head_in_group = hg * a.heads_per_tile + c % a.heads_per_tile;
   if (token >= t.tokens || head_in_group >= a.group) return;
   const float* src = a.partial + (((static_cast<long>(blockIdx.x) * gridDim.y + blockIdx.y) * a.num_splits) * (16 * NQ) + c) * PSTRIDE;
   const long split_stride = static_cast<long>(16 * NQ) * PSTRIDE;
   float top = -INFINITY;
-  for (int z = 0; z < a.num_splits; ++z) top = fmaxf(top, src[z * split_stride + D]);  // NaN marks stay NaN below
-  float denom = 0.f;
-  constexpr int PER = D / 4;  // dims per lane
-  float acc[PER];
+  bool poisoned = false;
+  for (int z = 0; z < a.num_splits; ++z) {
+    const float mz = src[z * split_stride + D];
+    poisoned = poisoned || mz != mz;
+    top = fmaxf(top, mz);
+  }
+  constexpr int PER = (D + 63) / 64;
+  float denom = 0.f, acc[PER];
 #pragma unroll
   for (int i = 0; i < PER; ++i) acc[i] = 0.f;
   for (int z = 0; z < a.num_splits; ++z) {
     const float* p = src + z * split_stride;
     const float mz = p[D];
-    const float w = (mz != mz) ? mz : (mz == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mz - top));
-    if (w == 0.f) continue;
+    const float w = mz == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mz - top);
     denom += w * p[D + 1];
 #pragma unroll
-    for (int i = 0; i < PER; ++i) acc[i] += w * p[quarter * PER + i];
+    for (int i = 0; i < PER; ++i)
+      if (lane + i * 64 < D) acc[i] += w * p[lane + i * 64];
   }
-  bf16_t* dst = a.out + (static_cast<long>(t.first_row + token) * a.q_heads + kvh * a.group + head_in_group) * D + quarter * PER;
-  const float inv = 1.f / denom;
+  bf16_t* dst = a.out + (static_cast<long>(t.first_row + token) * a.q_heads + kvh * a.group + head_in_group) * D;
+  const float inv = poisoned ? __uint_as_float(0x7fc00000u) : 1.f / denom;
 #pragma unroll
-  for (int i = 0; i < PER; ++i) dst[i] = from_float<bf16_t>(acc[i] * inv);
+  for (int i = 0; i < PER; ++i)
+    if (lane + i * 64 < D) dst[lane + i * 64] = from_float<bf16_t>(acc[i] * inv);
 }
 
 template <int NQ>
 int launch(const Args& a, int tiles, hipStream_t stream) {
   dim3 grid(tiles, a.kv_heads * a.head_groups, a.num_splits);
   if (a.num_splits > 1) {
-    attention_mfma_kernel<NQ, true><<<grid, 64, 0, stream>>>(a);
-    grid.z = 1;
-    attention_merge_kernel<NQ><<<grid, 64 * NQ, 0, stream>>>(a);
+    attention_mfma_kernel<NQ, true, (NQ < 4)><<<grid, 64, 0, stream>>>(a);
+    grid.z = a.heads_per_tile * a.tokens_per_tile;  // the columns that can be (token, head) pairs
+    attention_merge_kernel<NQ><<<grid, 64, 0, stream>>>(a);
   } else {
-    attention_mfma_kernel<NQ, false><<<grid, 64, 0, stream>>>(a);
+    attention_mfma_kernel<NQ, false, (NQ < 4)><<<grid, 64, 0, stream>>>(a);
   }
   return AKV_LAUNCH_STATUS();
 }
@@ -319,14 +465,18 @@ int launch(const Args& a, int tiles, hipStream_t stream) {
 // Attention of requests seq_first .. seq_first + seq_count - 1 of the step.  `nq` (1, 2 or 4) sets the tile to
 // 16 * nq query columns; `tiles` is the number of tiles over those requests (sum of ceil(tokens / tokens_per_tile));
 // with num_splits > 1 `partial` must hold tiles * kv_heads * head_groups * num_splits * 16 * nq * (D + 4) floats.
+// page_size must be a power of two, at least 4.  `single_tokens` says that every request brings exactly one token.
 extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
     const void* q, const void* k_pages, const void* v_pages, void* out, float* partial, const int* q_start,
     const int* seq_lens, const int* block_table, int table_width, int seq_first, int seq_count, int tiles, int nq,
     int q_heads, int kv_heads, int heads_per_tile, int head_groups, int tokens_per_tile, int page_size, long num_pages,
-    float scale, int window, int seg_keys, int num_splits, hipStream_t stream) {
+    float scale, int window, int seg_keys, int num_splits, int single_tokens, hipStream_t stream) {
   if (tiles <= 0 || seq_count <= 0) return 0;
-  if (page_size % 4 != 0 || q_heads % kv_heads != 0 || heads_per_tile * tokens_per_tile > 16 * nq ||
-      kv_heads * head_groups > 65535 || num_splits > 65535 || num_splits < 1)
+  int page_shift = 0;
+  while ((1 << page_shift) < page_size) ++page_shift;
+  if (page_size < 4 || (1 << page_shift) != page_size || q_heads % kv_heads != 0 ||
+      heads_per_tile * tokens_per_tile > 16 * nq || kv_heads * head_groups > 65535 || num_splits > 65535 ||
+      num_splits < 1 || (single_tokens && tiles != seq_count))
     return -2;
   Args a;
   a.q = static_cast<const bf16_t*>(q);
@@ -346,7 +496,8 @@ extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
   a.heads_per_tile = heads_per_tile;
   a.head_groups = head_groups;
   a.tokens_per_tile = tokens_per_tile;
-  a.page_size = page_size;
+  a.page_shift = page_shift;
+  a.single_tokens = single_tokens;
   a.num_pages = num_pages;
   a.scale_log2 = scale * kLog2e;
   a.window = window;

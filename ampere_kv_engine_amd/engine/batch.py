@@ -115,9 +115,10 @@ class BatchBuilder:
         self._device = torch.empty(capacity, dtype=torch.int32, device=self.device)
         self.arenas = (Arena(self.device), Arena(self.device))
 
-    def build(self, entries: list[StepEntry]) -> tuple[StepContext, list[int]]:
+    def build(self, entries: list[StepEntry], width_multiple: int = 1) -> tuple[StepContext, list[int]]:
         """Returns the context and, for every entry in the caller's order, the offset of its first wanted
-        row in the logits the step returns."""
+        row in the logits the step returns.  The block tables' width is rounded up to `width_multiple` pages:
+        steps of equal shape then lay their metadata out at equal addresses (what a recorded graph needs)."""
         if not entries:
             raise ValueError("a step needs at least one entry")
         if len(entries) > self.max_seqs:
@@ -146,6 +147,7 @@ class BatchBuilder:
         n, r = total, len(ordered)
         width = max(max((len(t.pages) for t in e.seq.tables), default=1) for e in ordered)
         width = max(width, 1)
+        width = min((width + width_multiple - 1) // width_multiple * width_multiple, max(self.max_width, width))
         self._turn ^= 1
         if self._copied[self._turn] is not None:
             self._copied[self._turn].synchronize()

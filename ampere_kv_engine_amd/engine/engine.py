@@ -47,6 +47,9 @@ class Engine:
         self.stream_buffer = torch.empty((engine_config.max_batched_tokens, spec.hidden_size),
                                          dtype=torch.float32, device=self.device)
         self.loaded = False
+        self._graphs: dict[tuple[int, int], tuple] = {}     # (requests, table width) -> recorded decode step
+        self._recordable = (engine_config.decode_graphs and self.device.type == "cuda" and all(
+            part.graph_safe for block in self.model.blocks for part in (block, block.mixer, block.feed_forward)))
 
     # ---- construction -----------------------------------------------------------------------------
     @classmethod
@@ -94,6 +97,47 @@ class Engine:
                 if not 0 <= int(token) < vocab:
                     raise ValueError(f"token id {token} of request {e.seq.request_id!r} is outside the vocabulary "
                                      f"of {vocab}")
+        if self._recordable and all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries):
+            return self._decode_step_recorded(entries)
         ctx, _ = self.builder.build(entries)
         ctx.stream_buffer = self.stream_buffer
         return self.model.forward(ctx, self.cache.layer_cache)
+
+    # ---- decode steps as recorded graphs ----------------------------------------------------------------------
+    GRAPH_WIDTH_MULTIPLE = 64     # block tables of a recorded step are this many pages wide, or a multiple
+
+    def _decode_step_recorded(self, entries: list[StepEntry]) -> torch.Tensor:
+        """A step in which every request brings one token and wants its logits launches the same kernels with the
+        same arguments every time, as long as the number of requests and the width of the block tables stay: only
+        the metadata in the step's device buffer differs.  Such a step is run once as it is, then recorded into a
+        HIP graph, then replayed - which takes the launches' host time out of decoding.  Launch sizes that depend on
+        the requests' lengths are taken from the table width's bound, so one recording serves all lengths under it.
+        The returned logits live in the recording's own buffer: the next replay of it overwrites them."""
+        ctx, _ = self.builder.build(entries, width_multiple=self.GRAPH_WIDTH_MULTIPLE)
+        ctx.stream_buffer = self.stream_buffer
+        width = ctx.paged[0].width if ctx.paged else 0
+        key = (ctx.num_seqs, width)
+        # sizes of launches come from the bound, not from this step's lengths
+        bound = max(width * self.config.page_size, 1)
+        ctx.max_seq_len = bound
+        ctx.host_seq_lens = [bound] * ctx.num_seqs
+        recorded = self._graphs.get(key)
+        if recorded is None:
+            logits = torch.empty((ctx.num_seqs, self.spec.vocab_size), dtype=torch.float32, device=self.device)
+            self.model.forward(ctx, self.cache.layer_cache, logits)        # settles the arenas; also this step's result
+            self._graphs[key] = (None, logits)
+            return logits
+        graph, logits = recorded
+        if graph is None:
+            graph = torch.cuda.CUDAGraph()
+            torch.cuda.synchronize(self.device)
+            with torch.cuda.graph(graph, stream=self._capture_stream()):
+                self.model.forward(ctx, self.cache.layer_cache, logits)
+            self._graphs[key] = (graph, logits)
+        graph.replay()
+        return logits
+
+    def _capture_stream(self):
+        if not hasattr(self, "_side_stream"):
+            self._side_stream = torch.cuda.Stream(self.device)
+        return self._side_stream

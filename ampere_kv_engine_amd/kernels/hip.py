@@ -281,7 +281,8 @@ class HipKernels:
     def _attention_mfma(self, q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out,
                         page_size, num_pages, seq_first, seq_count, nq, split):
         """Requests seq_first .. seq_first + seq_count - 1 of the step on the MFMA kernel, in tiles of 16 * nq
-        (token, head-of-group) columns; `split` cuts the keys over several waves (decode)."""
+        (token, head-of-group) columns; `split` says that each of them brings one token (decode) and cuts the keys
+        over several waves."""
         group = q_heads // kv_heads
         heads_per_tile = min(group, 16 * nq)
         head_groups = (group + heads_per_tile - 1) // heads_per_tile
@@ -305,7 +306,8 @@ class HipKernels:
             _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial), _ptr(ctx.q_start), _ptr(ctx.seq_lens),
             _ptr(meta.block_table), meta.width, seq_first, seq_count, tiles, nq, q_heads, kv_heads, heads_per_tile,
             head_groups, tokens_per_tile, page_size, ctypes.c_long(num_pages), ctypes.c_float(scale),
-            int(window) if window is not None else 0, seg_keys, num_splits, self._stream()), "attention")
+            int(window) if window is not None else 0, seg_keys, num_splits, 1 if split else 0, self._stream()),
+            "attention")
 
     def attention(self, q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out):
         tokens = q.shape[0]
@@ -315,7 +317,8 @@ class HipKernels:
         self._dense(meta.block_table, "block_table", torch.int32, (ctx.num_seqs, meta.width))
         if ctx.max_seq_len > meta.width * page_size:
             raise KernelError(f"a request of {ctx.max_seq_len} tokens does not fit a block table of {meta.width} pages")
-        if q.dtype == torch.bfloat16 and page_size % 4 == 0:
+        small = k_pages.numel() * k_pages.element_size() < 2 ** 32       # the kernel addresses pages with 32 bits
+        if q.dtype == torch.bfloat16 and page_size >= 4 and page_size & (page_size - 1) == 0 and small:
             self._dense(ctx.q_start, "q_start", torch.int32, (ctx.num_seqs + 1,))
             self._dense(ctx.seq_lens, "seq_lens", torch.int32, (ctx.num_seqs,))
             if ctx.host_q_start[ctx.num_seqs] != tokens or len(ctx.host_seq_lens) != ctx.num_seqs:
@@ -326,7 +329,7 @@ class HipKernels:
             if decodes:      # single tokens against long histories: one small tile each, keys split over waves
                 self._attention_mfma(*common, 0, decodes, 1, True)
             if ctx.num_seqs > decodes:
-                self._attention_mfma(*common, decodes, ctx.num_seqs - decodes, 4 if head_dim <= 128 else 2, False)
+                self._attention_mfma(*common, decodes, ctx.num_seqs - decodes, 2 if head_dim <= 128 else 1, False)
             return
         self._dense(ctx.seq_of_token, "seq_of_token", torch.int32, (tokens,))
         self._dense(ctx.positions, "positions", torch.int32, (tokens,))

@@ -16,6 +16,8 @@ from .position import NoPosition, RotaryHalf
 
 
 class Attention(Part):
+    graph_safe = True
+
     def __init__(self, spec, runtime):
         self.rt = runtime
         self.hidden = int(spec["hidden_size"])

@@ -80,6 +80,10 @@ class SlotState:
 class Part:
     """Base of all parts: tensors expected under a name prefix, and their adoption."""
 
+    # True if the part's launches depend on nothing but the step's shape (number of requests and tokens, table
+    # width): everything else it reads on the device.  Only then may a step that runs it be recorded and replayed.
+    graph_safe = False
+
     def tensors(self, prefix: str) -> list[TensorSpec]:
         return []
 

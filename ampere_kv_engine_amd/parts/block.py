@@ -9,6 +9,8 @@ from .base import Part, build_part, register_part
 
 
 class PreNormBlock(Part):
+    graph_safe = True
+
     def __init__(self, spec, runtime, mixer, feed_forward):
         self.rt = runtime
         self.hidden = int(spec["hidden_size"])

@@ -8,6 +8,8 @@ from .linear import Linear
 
 
 class SwiGLU(Part):
+    graph_safe = True
+
     def __init__(self, spec, runtime):
         self.rt = runtime
         self.hidden = int(spec["hidden_size"])

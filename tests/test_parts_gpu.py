@@ -244,3 +244,61 @@ def test_command_line(model_folders):
     assert result.returncode == 0 and '"tpot_ms"' in result.stdout, result.stderr[-2000:]
     result = run("--model", model_folders["A"], "--mode", "generate", "--cache", "contiguous", "--prompt-ids", "1")
     assert result.returncode != 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_recorded_decode_steps_equal_eager_ones(dtype, model_folders):
+    """Decode steps replay a recorded graph.  Every replay is checked against an engine that records nothing, over
+    many steps, with prompts of other requests (eager work) and synchronisations between the replays, with
+    requests joining and leaving (other batch sizes, slots and pages taken again)."""
+    raw, _, page = TINY["B"]
+    folder = model_folders["B"]
+    make = lambda graphs: Engine.from_folder(folder, EngineConfig(
+        dtype=dtype, page_size=page, num_pages=96, max_seqs=4, max_batched_tokens=64, max_seq_len=256, device="cuda:0",
+        decode_graphs=graphs))
+    recorded, eager = make(True), make(False)
+    assert recorded._recordable and not eager._recordable
+    prompts = {name: random_ids(379, n, seed=200 + i) for i, (name, n) in enumerate((("a", 9), ("b", 30), ("c", 3)))}
+    seqs = {}
+
+    def both(build):
+        outs = []
+        for engine in (recorded, eager):
+            out = engine.step(build(seqs.setdefault(id(engine), {}), engine))
+            outs.append(None if out is None else out.clone())
+        if outs[0] is not None:
+            assert torch.equal(outs[0], outs[1])
+        return outs[0]
+
+    def prefill(name):
+        def build(mine, engine):
+            mine[name] = engine.open(name)
+            return [StepEntry(mine[name], prompts[name], [len(prompts[name]) - 1])]
+        return int(both(build)[0].argmax())
+
+    def decode(tokens):
+        def build(mine, engine):
+            return [StepEntry(mine[name], [token], [0]) for name, token in tokens.items()]
+        logits = both(build)
+        return {name: int(row.argmax()) for name, row in zip(tokens, logits)}
+
+    def close(name):
+        for engine in (recorded, eager):
+            engine.close(seqs[id(engine)].pop(name))
+
+    last = {"a": prefill("a"), "b": prefill("b")}
+    for step in range(40):
+        last = decode(last)
+        if step == 5:
+            last["c"] = prefill("c")                  # eager work between replays; then three requests
+        if step == 12:
+            torch.cuda.synchronize()
+            close("a")
+            del last["a"]                             # two again, but other requests than the first two
+        if step == 20:
+            prompts["d"] = random_ids(379, 17, seed=300)
+            last["d"] = prefill("d")                  # takes a's slot and pages
+    assert len(recorded._graphs) >= 2 and all(graph is not None for graph, _ in recorded._graphs.values())
+    for name in list(last):
+        close(name)
+    assert recorded.cache.num_free_pages == eager.cache.num_free_pages == [96]
