@@ -417,26 +417,40 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(const Args a) {
   if (token >= t.tokens || head_in_group >= a.group) return;
   const float* src = a.partial + (((static_cast<long>(blockIdx.x) * gridDim.y + blockIdx.y) * a.num_splits) * (16 * NQ) + c) * PSTRIDE;
   const long split_stride = static_cast<long>(16 * NQ) * PSTRIDE;
+  // first the segments' maxima (a lane per segment), then the weighted sums
   float top = -INFINITY;
   bool poisoned = false;
-  for (int z = 0; z < a.num_splits; ++z) {
-    const float mz = src[z * split_stride + D];
+  for (int z0 = 0; z0 < a.num_splits; z0 += 64) {
+    const int z = z0 + lane;
+    const float mz = z < a.num_splits ? src[z * split_stride + D] : -INFINITY;
     poisoned = poisoned || mz != mz;
     top = fmaxf(top, mz);
   }
+  top = wave_max(top);
+  poisoned = __any(poisoned);
   constexpr int PER = (D + 63) / 64;
   float denom = 0.f, acc[PER];
 #pragma unroll
   for (int i = 0; i < PER; ++i) acc[i] = 0.f;
-  for (int z = 0; z < a.num_splits; ++z) {
-    const float* p = src + z * split_stride;
-    const float mz = p[D];
-    const float w = mz == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mz - top);
-    denom += w * p[D + 1];
+  for (int z0 = 0; z0 < a.num_splits; z0 += 64) {
+    const int z = z0 + lane;
+    float w = 0.f;
+    if (z < a.num_splits) {
+      const float mz = src[z * split_stride + D];
+      w = (mz == -INFINITY || mz != mz) ? 0.f : __builtin_amdgcn_exp2f(mz - top);
+      denom += w * src[z * split_stride + D + 1];
+    }
+    const int count = min(64, a.num_splits - z0);
+#pragma unroll 4
+    for (int zz = 0; zz < count; ++zz) {  // ascending segments: the order of the sum is fixed
+      const float wz = __shfl(w, zz, 64);
+      const float* p = src + (z0 + zz) * split_stride;
 #pragma unroll
-    for (int i = 0; i < PER; ++i)
-      if (lane + i * 64 < D) acc[i] += w * p[lane + i * 64];
+      for (int i = 0; i < PER; ++i)
+        if (lane + i * 64 < D) acc[i] = fmaf(wz, p[lane + i * 64], acc[i]);
+    }
   }
+  denom = wave_sum(denom);
   bf16_t* dst = a.out + (static_cast<long>(t.first_row + token) * a.q_heads + kvh * a.group + head_in_group) * D;
   const float inv = poisoned ? __uint_as_float(0x7fc00000u) : 1.f / denom;
 #pragma unroll

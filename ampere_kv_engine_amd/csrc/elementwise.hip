@@ -25,13 +25,64 @@ __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ 
 }
 
 // ---- residual add + RMSNorm: stream += delta (float32); out = T( T(stream * rsqrt(mean^2 + eps)) * w ) ----
+// One block per row.  A thread owns groups of 4 consecutive elements (16-byte accesses); a row of up to
+// 256 * 4 * kRowGroups elements stays in registers between the sum of squares and the scaling, longer rows are
+// read a second time.
+constexpr int kRowGroups = 4;
+
+template <typename T> __device__ __forceinline__ float4 load4(const T* p);
+template <> __device__ __forceinline__ float4 load4<float>(const float* p) { return *reinterpret_cast<const float4*>(p); }
+template <> __device__ __forceinline__ float4 load4<bf16_t>(const bf16_t* p) {
+  const uint2 v = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16),
+                     __uint_as_float(v.y & 0xffff0000u));
+}
+template <typename T> __device__ __forceinline__ void store4(T* p, float4 v);
+template <> __device__ __forceinline__ void store4<float>(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float4 v) {
+  uint2 packed;
+  packed.x = bf16_bits(v.x) | (static_cast<uint32_t>(bf16_bits(v.y)) << 16);
+  packed.y = bf16_bits(v.z) | (static_cast<uint32_t>(bf16_bits(v.w)) << 16);
+  *reinterpret_cast<uint2*>(p) = packed;
+}
+
 template <typename T>
-__global__ void add_rmsnorm_kernel(float* __restrict__ stream, const T* __restrict__ delta,
-                                   const float* __restrict__ weight, float eps, T* __restrict__ out, int hidden) {
+__global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ stream, const T* __restrict__ delta,
+                                                          const float* __restrict__ weight, float eps,
+                                                          T* __restrict__ out, int hidden) {
   __shared__ float scratch[16];
   const size_t base = static_cast<size_t>(blockIdx.x) * hidden;
   float* s = stream + base;
+  T* o = out + base;
   float acc = 0.f;
+  if ((hidden & 3) == 0 && hidden <= 256 * 4 * kRowGroups) {
+    float4 kept[kRowGroups];
+#pragma unroll
+    for (int j = 0; j < kRowGroups; ++j) {
+      const int i = (j * 256 + threadIdx.x) * 4;
+      if (i < hidden) {
+        float4 v = load4<float>(s + i);
+        if (delta != nullptr) {
+          const float4 d = load4<T>(delta + base + i);
+          v = make_float4(v.x + d.x, v.y + d.y, v.z + d.z, v.w + d.w);
+          store4<float>(s + i, v);
+        }
+        kept[j] = v;
+        acc += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+      }
+    }
+    const float scale = rsqrtf(block_sum(acc, scratch) / static_cast<float>(hidden) + eps);
+#pragma unroll
+    for (int j = 0; j < kRowGroups; ++j) {
+      const int i = (j * 256 + threadIdx.x) * 4;
+      if (i < hidden) {
+        const float4 v = kept[j], w = load4<float>(weight + i);
+        store4<T>(o + i, make_float4(rounded<T>(v.x * scale) * w.x, rounded<T>(v.y * scale) * w.y,
+                                     rounded<T>(v.z * scale) * w.z, rounded<T>(v.w * scale) * w.w));
+      }
+    }
+    return;
+  }
   if (delta != nullptr) {
     const T* d = delta + base;
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
@@ -47,7 +98,6 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ stream, const T* __restri
   }
   const float total = block_sum(acc, scratch);
   const float scale = rsqrtf(total / static_cast<float>(hidden) + eps);
-  T* o = out + base;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = from_float<T>(rounded<T>(s[i] * scale) * weight[i]);
 }
 

@@ -26,6 +26,14 @@ __device__ __forceinline__ floatx4 mfma16(uint4 a, uint4 b, floatx4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
+typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;
+
+// A 16-byte read of data that is used once: it does not displace what others re-read from the caches.
+__device__ __forceinline__ uint4 load_once(const uint4* p) {
+  const uintx4 v = __builtin_nontemporal_load(reinterpret_cast<const uintx4*>(p));
+  return make_uint4(v[0], v[1], v[2], v[3]);
+}
+
 template <typename TY> __device__ __forceinline__ void store4(TY* p, floatx4 v);
 template <> __device__ __forceinline__ void store4<float>(float* p, floatx4 v) {
   *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
@@ -52,14 +60,14 @@ __device__ __forceinline__ void store_tile(TY* y, floatx4 acc, int token, int fe
 }
 
 // ---- rows <= 16 * MT --------------------------------------------------------------------------------------------
-constexpr int kUnroll = 8;  // weight tiles in flight per wave
-
 template <int MT, typename TY>
 __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __restrict__ x, const uint4* __restrict__ wp,
                                                             TY* __restrict__ y, int rows, int outs, int k,
                                                             int k_tiles, int n_tiles, int k_split) {
+  constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);  // k-tiles per group; two groups are in flight
   extern __shared__ float red[];  // [wave][MT][4][64]
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+  const int lane = threadIdx.x & 63, waves = blockDim.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in every lane: keeps addresses scalar
   const int r = lane & 15, g = lane >> 4;
   const int row_tile = blockIdx.x * (waves / k_split) + wave / k_split;
   const int part = wave % k_split;
@@ -69,26 +77,51 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  if (row_tile < n_tiles) {
-    const uint4* wt = wp + static_cast<size_t>(row_tile) * k_tiles * 64 + lane;
+  if (row_tile < n_tiles && kt0 < kt1) {
+    // Addresses: a scalar base per wave plus a 32-bit lane offset, so that a load is one instruction.
+    const char* w_wave = reinterpret_cast<const char*>(wp) + static_cast<size_t>(row_tile) * k_tiles * 1024;
+    const uint32_t w_lane = lane * 16u;
+    const char* x_bytes = reinterpret_cast<const char*>(x);
+    uint32_t x_lane[MT];
+    bool x_row[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      x_row[mt] = mt * 16 + r < rows;
+      x_lane[mt] = static_cast<uint32_t>(mt * 16 + r) * static_cast<uint32_t>(k) * 2u + g * 16u;
+    }
+    const bool ragged = (k & 31) != 0;  // the last k-tile reaches beyond x's row
     const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
-    for (int kt = kt0; kt < kt1; kt += kUnroll) {
-      uint4 a[kUnroll];
+    // Two sets of operand registers: while the matrix cores work on one group of U k-tiles, the loads of the next
+    // group are already on their way.  Weights are read once and never again: their loads are marked nontemporal,
+    // which leaves the caches to the activations that every wave reads.
+    uint4 a0[U], a1[U], b0[MT][U], b1[MT][U];
+    auto fetch = [&](int kt, uint4 (&a)[U], uint4 (&b)[MT][U]) {
+      const char* w_at = w_wave + static_cast<size_t>(kt) * 1024;
+      const char* x_at = x_bytes + static_cast<size_t>(kt) * 64;
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) a[u] = (kt + u < kt1) ? wt[static_cast<size_t>(kt + u) * 64] : zero;
+      for (int u = 0; u < U; ++u)
+        a[u] = (kt + u < kt1) ? load_once(reinterpret_cast<const uint4*>(w_at + w_lane + u * 1024u)) : zero;
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const int token = mt * 16 + r;
-        uint4 b[kUnroll];
+      for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) {
-          const int at = (kt + u) * 32 + g * 8;
-          b[u] = (kt + u < kt1 && token < rows && at < k)
-                     ? *reinterpret_cast<const uint4*>(x + static_cast<size_t>(token) * k + at) : zero;
+        for (int u = 0; u < U; ++u) {
+          const bool inside = !ragged || (kt + u) * 32 + g * 8 < k;
+          b[mt][u] = (kt + u < kt1 && x_row[mt] && inside)
+                         ? *reinterpret_cast<const uint4*>(x_at + x_lane[mt] + u * 64u) : zero;
         }
+    };
+    auto multiply = [&](const uint4 (&a)[U], const uint4 (&b)[MT][U]) {
 #pragma unroll
-        for (int u = 0; u < kUnroll; ++u) acc[mt] = mfma16(a[u], b[u], acc[mt]);
-      }
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int u = 0; u < U; ++u) acc[mt] = mfma16(a[u], b[mt][u], acc[mt]);
+    };
+    fetch(kt0, a0, b0);
+    for (int kt = kt0; kt < kt1; kt += 2 * U) {
+      fetch(kt + U, a1, b1);      // beyond kt1 this fills zeros
+      multiply(a0, b0);
+      fetch(kt + 2 * U, a0, b0);
+      multiply(a1, b1);
     }
   }
   if (k_split > 1) {
