@@ -37,8 +37,10 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
 typedef __attribute__((ext_vector_type(2))) float floatx2;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;  // 16 bytes of operand: 8 bfloat16 (plain vector
+typedef __attribute__((ext_vector_type(2))) unsigned int uintx2;  // types: the compiler keeps them in registers)
 
-__device__ __forceinline__ floatx4 mfma16(uint4 a, uint4 b, floatx4 c) {
+__device__ __forceinline__ floatx4 mfma16(uintx4 a, uintx4 b, floatx4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
@@ -127,14 +129,14 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
   const Tile t = find_tile(a, blockIdx.x);
   if (!t.found) return;
   const int kvh = blockIdx.y / a.head_groups, hg = blockIdx.y % a.head_groups;
-  const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+  const uintx4 zero = uintx4{0u, 0u, 0u, 0u};
   const int page_size = 1 << a.page_shift, page_mask = page_size - 1;
 
   // this lane's columns: one per NQ tile
   bool col_valid[NQ];
   int col_pos[NQ], col_low[NQ];
   long col_at[NQ];  // element offset of the column's query / output row
-  uint4 qreg[NQ][KT];
+  uintx4 qreg[NQ][KT];
 #pragma unroll
   for (int nq = 0; nq < NQ; ++nq) {
     const int c = nq * 16 + r16;
@@ -146,7 +148,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
       const int dim = kt * 32 + g * 8;
-      qreg[nq][kt] = (col_valid[nq] && dim < D) ? *reinterpret_cast<const uint4*>(a.q + col_at[nq] + dim) : zero;
+      qreg[nq][kt] = (col_valid[nq] && dim < D) ? *reinterpret_cast<const uintx4*>(a.q + col_at[nq] + dim) : zero;
     }
   }
 
@@ -184,7 +186,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
 
   // Keys of the step at `base` into A operands.  CHECK: the step may reach outside [range_lo, range_hi]; rows outside
   // are zero and never looked up.
-  auto load_keys = [&](int base, uint4 (&dst)[2][KT], auto check) {
+  auto load_keys = [&](int base, uintx4 (&dst)[2][KT], auto check) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int key = base + key_in_step + j * 4;
@@ -201,13 +203,13 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) {
         const bool inside = (D % 32 == 0) || kt * 32 + g * 8 < D;
-        dst[j][kt] = (wanted && inside) ? *reinterpret_cast<const uint4*>(k_bytes + at + kt * 64u) : zero;
+        dst[j][kt] = (wanted && inside) ? *reinterpret_cast<const uintx4*>(k_bytes + at + kt * 64u) : zero;
       }
     }
   };
   // Values of the step at `base` into A operands: lane (dim row r16 of tile dt, keys base + 8g .. + 7).  CHECK: slots
   // of keys beyond the range are zeroed (they were never written and may hold anything, NaN included).
-  auto load_values = [&](int base, uint4 (&dst)[DT], auto check) {
+  auto load_values = [&](int base, uintx4 (&dst)[DT], auto check) {
     const int key = base + g * 8;
     if (!decltype(check)::value && page_size >= 8) {
       int page = table[key >> a.page_shift];
@@ -217,7 +219,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
       }
       const uint32_t at = static_cast<uint32_t>(page) * page_bytes + v_lane + static_cast<uint32_t>(key & page_mask) * 2u;
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) dst[dt] = *reinterpret_cast<const uint4*>(v_bytes + at + dt * v_tile);
+      for (int dt = 0; dt < DT; ++dt) dst[dt] = *reinterpret_cast<const uintx4*>(v_bytes + at + dt * v_tile);
       return;
     }
     const int live = min(8, range_hi - key + 1);
@@ -243,26 +245,26 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
     for (int w = 0; w < 4; ++w) keep[w] = live >= 2 * w + 2 ? 0xffffffffu : (live == 2 * w + 1 ? 0x0000ffffu : 0u);
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      uint4 v = zero;
+      uintx4 v = zero;
       if (page_size >= 8) {
-        if (have[0]) v = *reinterpret_cast<const uint4*>(v_bytes + at[0] + dt * v_tile);
+        if (have[0]) v = *reinterpret_cast<const uintx4*>(v_bytes + at[0] + dt * v_tile);
       } else {
         if (have[0]) {
-          const uint2 h = *reinterpret_cast<const uint2*>(v_bytes + at[0] + dt * v_tile);
+          const uintx2 h = *reinterpret_cast<const uintx2*>(v_bytes + at[0] + dt * v_tile);
           v.x = h.x;
           v.y = h.y;
         }
         if (have[1]) {
-          const uint2 h = *reinterpret_cast<const uint2*>(v_bytes + at[1] + dt * v_tile);
+          const uintx2 h = *reinterpret_cast<const uintx2*>(v_bytes + at[1] + dt * v_tile);
           v.z = h.x;
           v.w = h.y;
         }
       }
-      dst[dt] = make_uint4(v.x & keep[0], v.y & keep[1], v.z & keep[2], v.w & keep[3]);
+      dst[dt] = uintx4{v.x & keep[0], v.y & keep[1], v.z & keep[2], v.w & keep[3]};
     }
   };
 
-  uint4 kreg[2][KT], knext[PIPE ? 2 : 1][PIPE ? KT : 1], vreg[DT];
+  uintx4 kreg[2][KT], knext[PIPE ? 2 : 1][PIPE ? KT : 1], vreg[DT];
   const std::true_type checked{};
   const std::false_type unchecked{};
   auto inside = [&](int base) { return base >= range_lo && base + 31 <= range_hi; };
@@ -281,7 +283,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
         for (int nq = 0; nq < NQ; ++nq) s[nq][j] = mfma16(kreg[j][kt], qreg[nq][kt], s[nq][j]);
     }
     // ---- running maximum and sum per column (a column lives in the 4 lanes with the same r16) ---------------------
-    uint4 preg[NQ], plow[NQ];  // softmax weights as bfloat16 pairs: rounded value, and what the rounding lost
+    uintx4 preg[NQ], plow[NQ];  // softmax weights as bfloat16 pairs: rounded value, and what the rounding lost
     float correction[NQ];
     bool rescale = false;
 #pragma unroll
@@ -323,8 +325,8 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
         const floatx2 rest = {p[e][0] - __uint_as_float(high[e] << 16), p[e][1] - __uint_as_float(high[e] & 0xffff0000u)};
         low[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(rest, bf16x2));
       }
-      preg[nq] = make_uint4(high[0], high[1], high[2], high[3]);
-      plow[nq] = make_uint4(low[0], low[1], low[2], low[3]);
+      preg[nq] = uintx4{high[0], high[1], high[2], high[3]};
+      plow[nq] = uintx4{low[0], low[1], low[2], low[3]};
     }
     if (__any(rescale)) {  // the maxima rarely move after the first steps
 #pragma unroll
@@ -395,10 +397,10 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
       const float inv = poisoned ? nan : 1.f / l[nq];
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
-        uint2 packed;
+        uintx2 packed;
         packed.x = bf16_bits(o[nq][dt][0] * inv) | (static_cast<uint32_t>(bf16_bits(o[nq][dt][1] * inv)) << 16);
         packed.y = bf16_bits(o[nq][dt][2] * inv) | (static_cast<uint32_t>(bf16_bits(o[nq][dt][3] * inv)) << 16);
-        *reinterpret_cast<uint2*>(a.out + col_at[nq] + dt * 16 + g * 4) = packed;
+        *reinterpret_cast<uintx2*>(a.out + col_at[nq] + dt * 16 + g * 4) = packed;
       }
     }
   }

@@ -21,18 +21,15 @@ namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
+typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;  // 16 bytes of operand: 8 bfloat16 (a plain vector
+                                                                 // type: the compiler keeps it in registers)
 
-__device__ __forceinline__ floatx4 mfma16(uint4 a, uint4 b, floatx4 c) {
+__device__ __forceinline__ floatx4 mfma16(uintx4 a, uintx4 b, floatx4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
-typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;
-
 // A 16-byte read of data that is used once: it does not displace what others re-read from the caches.
-__device__ __forceinline__ uint4 load_once(const uint4* p) {
-  const uintx4 v = __builtin_nontemporal_load(reinterpret_cast<const uintx4*>(p));
-  return make_uint4(v[0], v[1], v[2], v[3]);
-}
+__device__ __forceinline__ uintx4 load_once(const uintx4* p) { return __builtin_nontemporal_load(p); }
 
 template <typename TY> __device__ __forceinline__ void store4(TY* p, floatx4 v);
 template <> __device__ __forceinline__ void store4<float>(float* p, floatx4 v) {
@@ -61,7 +58,7 @@ __device__ __forceinline__ void store_tile(TY* y, floatx4 acc, int token, int fe
 
 // ---- rows <= 16 * MT --------------------------------------------------------------------------------------------
 template <int MT, typename TY>
-__global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __restrict__ x, const uint4* __restrict__ wp,
+__global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __restrict__ x, const uintx4* __restrict__ wp,
                                                             TY* __restrict__ y, int rows, int outs, int k,
                                                             int k_tiles, int n_tiles, int k_split) {
   constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);  // k-tiles per group; two groups are in flight
@@ -90,27 +87,27 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
       x_lane[mt] = static_cast<uint32_t>(mt * 16 + r) * static_cast<uint32_t>(k) * 2u + g * 16u;
     }
     const bool ragged = (k & 31) != 0;  // the last k-tile reaches beyond x's row
-    const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+    const uintx4 zero = {0u, 0u, 0u, 0u};
     // Two sets of operand registers: while the matrix cores work on one group of U k-tiles, the loads of the next
     // group are already on their way.  Weights are read once and never again: their loads are marked nontemporal,
     // which leaves the caches to the activations that every wave reads.
-    uint4 a0[U], a1[U], b0[MT][U], b1[MT][U];
-    auto fetch = [&](int kt, uint4 (&a)[U], uint4 (&b)[MT][U]) {
+    uintx4 a0[U], a1[U], b0[MT][U], b1[MT][U];
+    auto fetch = [&](int kt, uintx4 (&a)[U], uintx4 (&b)[MT][U]) {
       const char* w_at = w_wave + static_cast<size_t>(kt) * 1024;
       const char* x_at = x_bytes + static_cast<size_t>(kt) * 64;
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        a[u] = (kt + u < kt1) ? load_once(reinterpret_cast<const uint4*>(w_at + w_lane + u * 1024u)) : zero;
+        a[u] = (kt + u < kt1) ? load_once(reinterpret_cast<const uintx4*>(w_at + w_lane + u * 1024u)) : zero;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int u = 0; u < U; ++u) {
           const bool inside = !ragged || (kt + u) * 32 + g * 8 < k;
           b[mt][u] = (kt + u < kt1 && x_row[mt] && inside)
-                         ? *reinterpret_cast<const uint4*>(x_at + x_lane[mt] + u * 64u) : zero;
+                         ? *reinterpret_cast<const uintx4*>(x_at + x_lane[mt] + u * 64u) : zero;
         }
     };
-    auto multiply = [&](const uint4 (&a)[U], const uint4 (&b)[MT][U]) {
+    auto multiply = [&](const uintx4 (&a)[U], const uintx4 (&b)[MT][U]) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -153,7 +150,7 @@ int launch_skinny(const void* x, const void* wp, void* y, int rows, int outs, in
   const int blocks = (n_tiles + tiles_per_block - 1) / tiles_per_block;
   const size_t lds = k_split > 1 ? static_cast<size_t>(waves) * MT * 4 * 64 * sizeof(float) : 0;
   linear_skinny_kernel<MT, TY><<<blocks, waves * 64, lds, stream>>>(
-      static_cast<const bf16_t*>(x), static_cast<const uint4*>(wp), static_cast<TY*>(y), rows, outs, k, k_tiles,
+      static_cast<const bf16_t*>(x), static_cast<const uintx4*>(wp), static_cast<TY*>(y), rows, outs, k, k_tiles,
       n_tiles, k_split);
   return AKV_LAUNCH_STATUS();
 }
@@ -171,92 +168,127 @@ int dispatch_skinny(const void* x, const void* wp, void* y, int rows, int outs, 
 }
 
 // ---- rows > 64 ----------------------------------------------------------------------------------------------------
-// Block: 256 threads = 2 x 2 waves; block tile 128 tokens x 128 features; wave tile 64 x 64 = 4 x 4 MFMA tiles.
-// Per stage of 64 k: activations [128 tokens][64 k] go through LDS laid out [k chunk of 8][token][8] so that a
-// wave's B-operand read (16 consecutive tokens of one chunk) is 256 consecutive bytes; weights come from the packed
-// layout directly into registers.
-constexpr int kWideM = 128, kWideN = 128, kWideK = 64;
+// Block: 256 threads = 2 x 2 waves; block tile 256 tokens x 128 features; wave tile 128 tokens x 64 features
+// = 8 x 4 MFMA tiles (128 accumulator registers).  Per stage of 64 k the block's activations [256 tokens][64 k] go
+// through LDS, double-buffered, laid out [k chunk of 8][token] with the token index XOR-swizzled by the chunk so
+// that both the staging writes (8 chunks of one token) and the operand reads (16 tokens of one chunk) are free of
+// bank conflicts.  Weights come from the packed layout straight into A operands, one k-tile ahead of their use.
+// Blocks are numbered so that the blocks sharing a band of 128 weight rows run on the same XCD (one L2 each: the
+// band is fetched from memory once), while XCDs work on different bands.
+constexpr int kWideM = 256, kWideN = 128, kWideK = 64, kXcds = 8;
 
 template <typename TY>
-__global__ __launch_bounds__(256) void linear_wide_kernel(const bf16_t* __restrict__ x, const uint4* __restrict__ wp,
+__global__ __launch_bounds__(256) void linear_wide_kernel(const bf16_t* __restrict__ x, const uintx4* __restrict__ wp,
                                                           TY* __restrict__ y, int rows, int outs, int k, int k_tiles,
-                                                          int n_tiles) {
-  __shared__ uint4 xs[2][kWideK / 8][kWideM];  // 2 stages x 8 chunks x 128 tokens x 16 B = 32 KB
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+                                                          int n_tiles, int n_blocks, int m_blocks) {
+  __shared__ uintx4 xs[2][kWideK / 8][kWideM];  // 2 stages x 8 chunks x 256 tokens x 16 B = 64 KB
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, g = lane >> 4;
+  // block -> (band of weight rows, block of tokens): consecutive blocks of one XCD share the band
+  const int xcd = blockIdx.x % kXcds, turn = blockIdx.x / kXcds;
+  const int n_block = (turn / m_blocks) * kXcds + xcd, m_block = turn % m_blocks;
+  if (n_block >= n_blocks) return;
   const int wave_m = wave & 1, wave_n = wave >> 1;
-  const int token0 = blockIdx.y * kWideM, tile0 = blockIdx.x * (kWideN / 16) + wave_n * 4;
-  const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+  const int token0 = m_block * kWideM, tile0 = n_block * (kWideN / 16) + wave_n * 4;
+  const uintx4 zero = {0u, 0u, 0u, 0u};
   const int stages = (k_tiles + 1) / 2;
 
-  floatx4 acc[4][4];  // [feature tile][token tile]
+  floatx4 acc[4][8];  // [feature tile][token tile]
 #pragma unroll
   for (int n = 0; n < 4; ++n)
 #pragma unroll
-    for (int m = 0; m < 4; ++m) acc[n][m] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int m = 0; m < 8; ++m) acc[n][m] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  // each thread moves 4 chunks of 16 B per stage: chunk c = e % 8 of token e / 8 (8 consecutive threads = 128 B of a row)
-  uint4 moving[4];
-  auto fetch = [&](int stage) {
+  // staging: a thread moves 8 chunks of 16 B per stage; chunk c = e % 8 of token e / 8, so that 8 consecutive threads
+  // read 128 consecutive bytes of one row of x
+  const char* x_bytes = reinterpret_cast<const char*>(x);
+  uint32_t x_at[8];
+  bool x_row[8];
 #pragma unroll
-    for (int p = 0; p < 4; ++p) {
+  for (int p = 0; p < 8; ++p) {
+    const int e = p * 256 + threadIdx.x, token = token0 + e / 8;
+    x_row[p] = token < rows;
+    x_at[p] = static_cast<uint32_t>(token) * static_cast<uint32_t>(k) * 2u + (e % 8) * 16u;
+  }
+  uintx4 moving[8];
+  auto fetch = [&](int stage) {
+    const char* at = x_bytes + static_cast<size_t>(stage) * (kWideK * 2);
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
       const int e = p * 256 + threadIdx.x;
-      const int token = token0 + e / 8, at = stage * kWideK + (e % 8) * 8;
-      moving[p] = (token < rows && at < k) ? *reinterpret_cast<const uint4*>(x + static_cast<size_t>(token) * k + at) : zero;
+      const bool inside = stage * kWideK + (e % 8) * 8 < k;
+      moving[p] = (x_row[p] && inside) ? *reinterpret_cast<const uintx4*>(at + x_at[p]) : zero;
     }
   };
   auto stash = [&](int buffer) {
 #pragma unroll
-    for (int p = 0; p < 4; ++p) {
-      const int e = p * 256 + threadIdx.x;
-      xs[buffer][e % 8][e / 8] = moving[p];
+    for (int p = 0; p < 8; ++p) {
+      const int e = p * 256 + threadIdx.x, c = e % 8, t = e / 8;
+      xs[buffer][c][t ^ (c << 1)] = moving[p];
     }
   };
-  uint4 a[2][4];  // weights of the stage's two k-tiles, 4 feature tiles
-  auto weights = [&](int stage) {
+  // weights: the wave's 4 row tiles of one k-tile
+  const char* w_bytes = reinterpret_cast<const char*>(wp);
+  uint32_t w_at[4];
+  bool w_row[4];
 #pragma unroll
-    for (int half = 0; half < 2; ++half)
+  for (int n = 0; n < 4; ++n) {
+    w_row[n] = tile0 + n < n_tiles;
+    w_at[n] = lane * 16u;
+  }
+  const size_t w_tile_row = static_cast<size_t>(k_tiles) * 1024;  // bytes of one row tile
+  auto weights = [&](int kt, uintx4 (&a)[4]) {
 #pragma unroll
-      for (int n = 0; n < 4; ++n) {
-        const int kt = stage * 2 + half, tile = tile0 + n;
-        a[half][n] = (kt < k_tiles && tile < n_tiles) ? wp[(static_cast<size_t>(tile) * k_tiles + kt) * 64 + lane] : zero;
-      }
+    for (int n = 0; n < 4; ++n) {
+      const char* at = w_bytes + (static_cast<size_t>(tile0 + n) * w_tile_row + static_cast<size_t>(kt) * 1024);
+      a[n] = (w_row[n] && kt < k_tiles) ? *reinterpret_cast<const uintx4*>(at + w_at[n]) : zero;
+    }
+  };
+  auto multiply = [&](int buffer, int half, const uintx4 (&a)[4]) {
+    uintx4 b[8];
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+      const int c = half * 4 + g, t = wave_m * 128 + m * 16 + r;
+      b[m] = xs[buffer][c][t ^ (c << 1)];
+    }
+#pragma unroll
+    for (int m = 0; m < 8; ++m)
+#pragma unroll
+      for (int n = 0; n < 4; ++n) acc[n][m] = mfma16(a[n], b[m], acc[n][m]);
   };
 
+  uintx4 a0[4], a1[4];
   fetch(0);
+  weights(0, a0);
   stash(0);
   __syncthreads();
   for (int stage = 0; stage < stages; ++stage) {
     const int buffer = stage & 1;
-    weights(stage);
-    if (stage + 1 < stages) fetch(stage + 1);
-#pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      uint4 b[4];
-#pragma unroll
-      for (int m = 0; m < 4; ++m) b[m] = xs[buffer][half * 4 + g][wave_m * 64 + m * 16 + r];
-#pragma unroll
-      for (int n = 0; n < 4; ++n)
-#pragma unroll
-        for (int m = 0; m < 4; ++m) acc[n][m] = mfma16(a[half][n], b[m], acc[n][m]);
-    }
+    if (stage + 1 < stages) fetch(stage + 1);   // next stage's activations travel while this stage computes
+    weights(stage * 2 + 1, a1);
+    multiply(buffer, 0, a0);
+    weights(stage * 2 + 2, a0);
+    multiply(buffer, 1, a1);
     if (stage + 1 < stages) stash(buffer ^ 1);
     __syncthreads();
   }
 #pragma unroll
   for (int n = 0; n < 4; ++n)
 #pragma unroll
-    for (int m = 0; m < 4; ++m)
-      store_tile<TY>(y, acc[n][m], token0 + wave_m * 64 + m * 16 + r, (tile0 + n) * 16 + g * 4, rows, outs);
+    for (int m = 0; m < 8; ++m)
+      store_tile<TY>(y, acc[n][m], token0 + wave_m * 128 + m * 16 + r, (tile0 + n) * 16 + g * 4, rows, outs);
 }
 
 template <typename TY>
 int launch_wide(const void* x, const void* wp, void* y, int rows, int outs, int k, int k_tiles, int n_tiles,
                 hipStream_t stream) {
-  dim3 grid((n_tiles * 16 + kWideN - 1) / kWideN, (rows + kWideM - 1) / kWideM);
-  if (grid.y > 65535) return -2;
-  linear_wide_kernel<TY><<<grid, 256, 0, stream>>>(static_cast<const bf16_t*>(x), static_cast<const uint4*>(wp),
-                                                    static_cast<TY*>(y), rows, outs, k, k_tiles, n_tiles);
+  const int n_blocks = (n_tiles * 16 + kWideN - 1) / kWideN, m_blocks = (rows + kWideM - 1) / kWideM;
+  const long blocks = static_cast<long>((n_blocks + kXcds - 1) / kXcds) * kXcds * m_blocks;
+  if (blocks > 0x7fffffffL || static_cast<long>(rows) * k * 2 >= (1L << 32)) return -2;
+  linear_wide_kernel<TY><<<static_cast<unsigned>(blocks), 256, 0, stream>>>(
+      static_cast<const bf16_t*>(x), static_cast<const uintx4*>(wp), static_cast<TY*>(y), rows, outs, k, k_tiles, n_tiles,
+      n_blocks, m_blocks);
   return AKV_LAUNCH_STATUS();
 }
 
