@@ -175,13 +175,16 @@ int dispatch_skinny(const void* x, const void* wp, void* y, int rows, int outs, 
 // bank conflicts.  Weights come from the packed layout straight into A operands, one k-tile ahead of their use.
 // Blocks are numbered so that the blocks sharing a band of 128 weight rows run on the same XCD (one L2 each: the
 // band is fetched from memory once), while XCDs work on different bands.
-constexpr int kWideM = 256, kWideN = 128, kWideK = 64, kXcds = 8;
+constexpr int kWideN = 128, kWideK = 64, kXcds = 8;
 
-template <typename TY>
-__global__ __launch_bounds__(256) void linear_wide_kernel(const bf16_t* __restrict__ x, const uintx4* __restrict__ wp,
+// MW: token tiles per wave (8: 256 tokens per block; 4: 128 tokens per block, for products with few weight rows,
+// which would otherwise leave compute units without a block).
+template <typename TY, int MW>
+__global__ __launch_bounds__(256, 2) void linear_wide_kernel(const bf16_t* __restrict__ x, const uintx4* __restrict__ wp,
                                                           TY* __restrict__ y, int rows, int outs, int k, int k_tiles,
                                                           int n_tiles, int n_blocks, int m_blocks) {
-  __shared__ uintx4 xs[2][kWideK / 8][kWideM];  // 2 stages x 8 chunks x 256 tokens x 16 B = 64 KB
+  constexpr int kWideM = 32 * MW;  // tokens per block
+  __shared__ uintx4 xs[2][kWideK / 8][kWideM];  // 2 stages x 8 chunks x tokens x 16 B (64 KB for 256 tokens)
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, g = lane >> 4;
@@ -194,28 +197,29 @@ __global__ __launch_bounds__(256) void linear_wide_kernel(const bf16_t* __restri
   const uintx4 zero = {0u, 0u, 0u, 0u};
   const int stages = (k_tiles + 1) / 2;
 
-  floatx4 acc[4][8];  // [feature tile][token tile]
+  floatx4 acc[4][MW];  // [feature tile][token tile]
 #pragma unroll
   for (int n = 0; n < 4; ++n)
 #pragma unroll
-    for (int m = 0; m < 8; ++m) acc[n][m] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int m = 0; m < MW; ++m) acc[n][m] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   // staging: a thread moves 8 chunks of 16 B per stage; chunk c = e % 8 of token e / 8, so that 8 consecutive threads
   // read 128 consecutive bytes of one row of x
   const char* x_bytes = reinterpret_cast<const char*>(x);
-  uint32_t x_at[8];
-  bool x_row[8];
+  constexpr int PX = MW;  // 16-byte chunks a thread stages: tokens * 8 / 256
+  uint32_t x_at[PX];
+  bool x_row[PX];
 #pragma unroll
-  for (int p = 0; p < 8; ++p) {
+  for (int p = 0; p < PX; ++p) {
     const int e = p * 256 + threadIdx.x, token = token0 + e / 8;
     x_row[p] = token < rows;
     x_at[p] = static_cast<uint32_t>(token) * static_cast<uint32_t>(k) * 2u + (e % 8) * 16u;
   }
-  uintx4 moving[8];
+  uintx4 moving[PX];
   auto fetch = [&](int stage) {
     const char* at = x_bytes + static_cast<size_t>(stage) * (kWideK * 2);
 #pragma unroll
-    for (int p = 0; p < 8; ++p) {
+    for (int p = 0; p < PX; ++p) {
       const int e = p * 256 + threadIdx.x;
       const bool inside = stage * kWideK + (e % 8) * 8 < k;
       moving[p] = (x_row[p] && inside) ? *reinterpret_cast<const uintx4*>(at + x_at[p]) : zero;
@@ -223,7 +227,7 @@ __global__ __launch_bounds__(256) void linear_wide_kernel(const bf16_t* __restri
   };
   auto stash = [&](int buffer) {
 #pragma unroll
-    for (int p = 0; p < 8; ++p) {
+    for (int p = 0; p < PX; ++p) {
       const int e = p * 256 + threadIdx.x, c = e % 8, t = e / 8;
       xs[buffer][c][t ^ (c << 1)] = moving[p];
     }
@@ -246,14 +250,14 @@ __global__ __launch_bounds__(256) void linear_wide_kernel(const bf16_t* __restri
     }
   };
   auto multiply = [&](int buffer, int half, const uintx4 (&a)[4]) {
-    uintx4 b[8];
+    uintx4 b[MW];
 #pragma unroll
-    for (int m = 0; m < 8; ++m) {
-      const int c = half * 4 + g, t = wave_m * 128 + m * 16 + r;
+    for (int m = 0; m < MW; ++m) {
+      const int c = half * 4 + g, t = wave_m * (16 * MW) + m * 16 + r;
       b[m] = xs[buffer][c][t ^ (c << 1)];
     }
 #pragma unroll
-    for (int m = 0; m < 8; ++m)
+    for (int m = 0; m < MW; ++m)
 #pragma unroll
       for (int n = 0; n < 4; ++n) acc[n][m] = mfma16(a[n], b[m], acc[n][m]);
   };
@@ -276,19 +280,28 @@ __global__ __launch_bounds__(256) void linear_wide_kernel(const bf16_t* __restri
 #pragma unroll
   for (int n = 0; n < 4; ++n)
 #pragma unroll
-    for (int m = 0; m < 8; ++m)
-      store_tile<TY>(y, acc[n][m], token0 + wave_m * 128 + m * 16 + r, (tile0 + n) * 16 + g * 4, rows, outs);
+    for (int m = 0; m < MW; ++m)
+      store_tile<TY>(y, acc[n][m], token0 + wave_m * (16 * MW) + m * 16 + r, (tile0 + n) * 16 + g * 4, rows, outs);
 }
 
 template <typename TY>
 int launch_wide(const void* x, const void* wp, void* y, int rows, int outs, int k, int k_tiles, int n_tiles,
                 hipStream_t stream) {
-  const int n_blocks = (n_tiles * 16 + kWideN - 1) / kWideN, m_blocks = (rows + kWideM - 1) / kWideM;
+  const int n_blocks = (n_tiles * 16 + kWideN - 1) / kWideN;
+  // 256 tokens per block when that still gives every compute unit its two blocks, else 128
+  const bool tall = static_cast<long>(n_blocks) * ((rows + 255) / 256) >= 512;
+  const int block_tokens = tall ? 256 : 128;
+  const int m_blocks = (rows + block_tokens - 1) / block_tokens;
   const long blocks = static_cast<long>((n_blocks + kXcds - 1) / kXcds) * kXcds * m_blocks;
   if (blocks > 0x7fffffffL || static_cast<long>(rows) * k * 2 >= (1L << 32)) return -2;
-  linear_wide_kernel<TY><<<static_cast<unsigned>(blocks), 256, 0, stream>>>(
-      static_cast<const bf16_t*>(x), static_cast<const uintx4*>(wp), static_cast<TY*>(y), rows, outs, k, k_tiles, n_tiles,
-      n_blocks, m_blocks);
+  if (tall)
+    linear_wide_kernel<TY, 8><<<static_cast<unsigned>(blocks), 256, 0, stream>>>(
+        static_cast<const bf16_t*>(x), static_cast<const uintx4*>(wp), static_cast<TY*>(y), rows, outs, k, k_tiles,
+        n_tiles, n_blocks, m_blocks);
+  else
+    linear_wide_kernel<TY, 4><<<static_cast<unsigned>(blocks), 256, 0, stream>>>(
+        static_cast<const bf16_t*>(x), static_cast<const uintx4*>(wp), static_cast<TY*>(y), rows, outs, k, k_tiles,
+        n_tiles, n_blocks, m_blocks);
   return AKV_LAUNCH_STATUS();
 }
 

@@ -72,7 +72,9 @@ class HipKernels:
             raise KernelError(f"the kernel library {path} could not be loaded: {error}") from error
         self.library_path = path
         self._attention_entry = {}      # head size -> entry point of that head size's attention library
-        self.decode_wave_target = 4096  # decode attention cuts the keys until about this many waves are at work
+        self.decode_wave_target = 2048  # decode attention cuts the keys until about this many waves are at work,
+        self.decode_min_segment = 128   # but into segments no shorter than this many keys
+        self.decode_max_splits = 32     # and no more than this many (the merge walks them one after the other)
         for name in ("akv_embed", "akv_add_rmsnorm", "akv_rmsnorm_rows", "akv_copy_rows", "akv_gather_rows",
                      "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
                      "akv_linear_tiled", "akv_linear_packed", "akv_attention_rows", "akv_sample"):
@@ -295,7 +297,9 @@ class HipKernels:
         if split:
             longest = max(ctx.host_seq_lens[seq_first:seq_first + seq_count])
             pairs = tiles * kv_heads * head_groups
-            num_splits = max(1, min((self.decode_wave_target + pairs - 1) // pairs, (longest + 127) // 128))
+            num_splits = max(1, min((self.decode_wave_target + pairs - 1) // pairs,
+                                    (longest + self.decode_min_segment - 1) // self.decode_min_segment,
+                                    self.decode_max_splits))
             seg_keys = ((longest + num_splits - 1) // num_splits + 31) // 32 * 32
             num_splits = (longest + seg_keys - 1) // seg_keys
             if num_splits > 1:
