@@ -43,6 +43,7 @@ def main() -> int:
                         help="fewer layers than the configuration has, where memory or time needs it")
     parser.add_argument("--points", default="1,64", help="further batch sizes to time (comma separated, '' for none)")
     parser.add_argument("--no-prefill", action="store_true")
+    parser.add_argument("--prefill-only", action="store_true", help="time the prefill alone (for kernel profiles)")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this engine has no multi-GPU path, run it with --gpus 1")
@@ -111,6 +112,11 @@ def main() -> int:
             engine.close(seq)
         return sorted(samples)[len(samples) // 2]
 
+    if args.prefill_only:
+        seconds = prefill()
+        print(json.dumps({"prefill_ms": round(seconds * 1000, 3), "tokens": PREFILL_TOKENS,
+                          "tok_per_s": round(PREFILL_TOKENS / seconds, 1), "layers": args.layers}))
+        return 0
     elapsed = decode(args.batch, args.steps, args.warmup)
     ms_per_step = elapsed / args.steps * 1000
     value = args.batch * args.steps / elapsed
