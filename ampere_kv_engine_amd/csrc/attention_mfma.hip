@@ -55,6 +55,7 @@ struct Args {
   const int* block_table;     // [requests, table_width]
   int table_width;
   int seq_first, seq_count;   // the launch covers requests seq_first .. seq_first + seq_count - 1
+  int tiles;                  // tiles over those requests
   int single_tokens;          // every request of the launch brings exactly one token: tile i is request seq_first + i
   int q_heads, kv_heads, group, heads_per_tile, head_groups, tokens_per_tile;
   int page_shift;             // page_size = 1 << page_shift, at least 4
@@ -126,8 +127,15 @@ __device__ __forceinline__ Tile find_tile(const Args& a, int slot) {
 template <int NQ, bool SPLIT, bool PIPE>
 __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
   const int lane = threadIdx.x, r16 = lane & 15, g = lane >> 4;
-  const Tile t = find_tile(a, blockIdx.x);
-  if (!t.found) return;
+  // Without SPLIT a block works on two tiles, one after the other: tile `tiles - 1 - x` and tile `x`.  Under the
+  // causal mask the late tiles of a prompt see many keys and the early ones few; a pair sees about the same number
+  // as every other pair, so the blocks finish together instead of waiting for the longest.
+  for (int pass = 0; pass < (SPLIT ? 1 : 2); ++pass) {
+  const int slot = SPLIT ? static_cast<int>(blockIdx.x)
+                         : (pass == 0 ? a.tiles - 1 - static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x));
+  if (!SPLIT && pass == 1 && slot >= a.tiles - 1 - slot) break;  // the middle tile was the first pass's
+  const Tile t = find_tile(a, slot);
+  if (!t.found) continue;
   const int kvh = blockIdx.y / a.head_groups, hg = blockIdx.y % a.head_groups;
   const uintx4 zero = uintx4{0u, 0u, 0u, 0u};
   const int page_size = 1 << a.page_shift, page_mask = page_size - 1;
@@ -270,7 +278,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
   auto inside = [&](int base) { return base >= range_lo && base + 31 <= range_hi; };
 
   // One step of 32 keys.  MASK: some column does not see the whole step (diagonal, window, segment edge).
-  auto step = [&](int base, auto mask) {
+  auto step = [&](int base, const uintx4 (&kreg)[2][KT], auto mask) {
     // ---- S^T = K . Q^T for two tiles of 16 keys --------------------------------------------------------------
     floatx4 s[NQ][2];
 #pragma unroll
@@ -341,39 +349,40 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
       for (int nq = 0; nq < NQ; ++nq) o[nq][dt] = mfma16(vreg[dt], plow[nq], mfma16(vreg[dt], preg[nq], o[nq][dt]));
   };
 
-  const int first_base = range_lo & ~31;
-  if (PIPE && first_base <= range_hi) {
-    if (inside(first_base)) load_keys(first_base, kreg, unchecked);
-    else load_keys(first_base, kreg, checked);
-  }
-  for (int base = first_base; base <= range_hi; base += 32) {
-    // memory first: this step's values (needed after the softmax) and the next step's keys (needed next turn)
+  // One turn: fetch this step's values and (PIPE) the next step's keys, then compute the step on `cur`.
+  auto turn = [&](int base, uintx4 (&cur)[2][KT], uintx4 (&next)[PIPE ? 2 : 1][PIPE ? KT : 1]) {
     const bool here = inside(base);
-    if (!PIPE) {
-      if (here) load_keys(base, kreg, unchecked);
-      else load_keys(base, kreg, checked);
+    if constexpr (!PIPE) {
+      if (here) load_keys(base, cur, unchecked);
+      else load_keys(base, cur, checked);
     }
+    // memory first: this step's values (needed after the softmax) and the next step's keys (needed next turn)
     if (here) load_values(base, vreg, unchecked);
     else load_values(base, vreg, checked);
-    const bool more = PIPE && base + 32 <= range_hi;
     if constexpr (PIPE) {
-      if (more) {
-        if (inside(base + 32)) load_keys(base + 32, knext, unchecked);
-        else load_keys(base + 32, knext, checked);
+      if (base + 32 <= range_hi) {
+        if (inside(base + 32)) load_keys(base + 32, next, unchecked);
+        else load_keys(base + 32, next, checked);
       }
     }
     // every valid column sees the whole step: below the diagonal, inside window and segment
     const bool whole = here && base + 31 <= t.first_pos && (a.window == 0 || base >= last_pos - a.window + 1);
-    if (whole) step(base, unchecked);
-    else step(base, checked);
-    if constexpr (PIPE) {
-      if (more) {
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-          for (int kt = 0; kt < KT; ++kt) kreg[j][kt] = knext[j][kt];
-      }
+    if (whole) step(base, cur, unchecked);
+    else step(base, cur, checked);
+  };
+  const int first_base = range_lo & ~31;
+  if constexpr (PIPE) {
+    if (first_base <= range_hi) {
+      if (inside(first_base)) load_keys(first_base, kreg, unchecked);
+      else load_keys(first_base, kreg, checked);
     }
+    for (int base = first_base; base <= range_hi; base += 64) {  // two turns: the key registers swap roles
+      turn(base, kreg, knext);
+      if (base + 32 > range_hi) break;
+      turn(base + 32, knext, kreg);
+    }
+  } else {
+    for (int base = first_base; base <= range_hi; base += 32) turn(base, kreg, knext);
   }
 
   // ---- results: lane holds, per column, dims dt * 16 + 4g .. + 3 ------------------------------------------------------
@@ -384,7 +393,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
     l[nq] += __shfl_xor(l[nq], 16, 64);
     l[nq] += __shfl_xor(l[nq], 32, 64);
     if (SPLIT) {
-      if (!col_valid[nq]) continue;  // the merge never reads the columns that are no (token, head) of the tile
+      if (!col_valid[nq]) continue;  // (next column) the merge never reads columns that are no (token, head) pair
       const int c = nq * 16 + r16;
       float* dst = a.partial + ((((static_cast<long>(blockIdx.x) * gridDim.y + blockIdx.y) * a.num_splits + blockIdx.z) * (16 * NQ)) + c) * PSTRIDE;
 #pragma unroll
@@ -404,6 +413,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
       }
     }
   }
+  }  // pass
 }
 
 // Merge of the segments' partial results: out = sum_z 2^(m_z - M) O_z / sum_z 2^(m_z - M) l_z, M = max_z m_z
@@ -443,13 +453,20 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(const Args a) {
       denom += w * src[z * split_stride + D + 1];
     }
     const int count = min(64, a.num_splits - z0);
-#pragma unroll 4
-    for (int zz = 0; zz < count; ++zz) {  // ascending segments: the order of the sum is fixed
-      const float wz = __shfl(w, zz, 64);
-      const float* p = src + (z0 + zz) * split_stride;
+    for (int zz0 = 0; zz0 < count; zz0 += 8) {  // ascending segments: the order of the sum is fixed
+      float v[8][PER];                            // eight segments' loads go out together
 #pragma unroll
-      for (int i = 0; i < PER; ++i)
-        if (lane + i * 64 < D) acc[i] = fmaf(wz, p[lane + i * 64], acc[i]);
+      for (int j = 0; j < 8; ++j) {
+        const float* p = src + (z0 + min(zz0 + j, count - 1)) * split_stride;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) v[j][i] = lane + i * 64 < D ? p[lane + i * 64] : 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float wz = zz0 + j < count ? __shfl(w, zz0 + j, 64) : 0.f;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) acc[i] = fmaf(wz, v[j][i], acc[i]);
+      }
     }
   }
   denom = wave_sum(denom);
@@ -463,12 +480,13 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(const Args a) {
 template <int NQ>
 int launch(const Args& a, int tiles, hipStream_t stream) {
   dim3 grid(tiles, a.kv_heads * a.head_groups, a.num_splits);
+  if (a.num_splits == 1) grid.x = (tiles + 1) / 2;  // a block takes a late tile and an early one
   if (a.num_splits > 1) {
-    attention_mfma_kernel<NQ, true, (NQ < 4)><<<grid, 64, 0, stream>>>(a);
+    attention_mfma_kernel<NQ, true, true><<<grid, 64, 0, stream>>>(a);
     grid.z = a.heads_per_tile * a.tokens_per_tile;  // the columns that can be (token, head) pairs
     attention_merge_kernel<NQ><<<grid, 64, 0, stream>>>(a);
   } else {
-    attention_mfma_kernel<NQ, false, (NQ < 4)><<<grid, 64, 0, stream>>>(a);
+    attention_mfma_kernel<NQ, false, true><<<grid, 64, 0, stream>>>(a);
   }
   return AKV_LAUNCH_STATUS();
 }
@@ -478,7 +496,7 @@ int launch(const Args& a, int tiles, hipStream_t stream) {
 #define AKV_CONCAT2(a, b) a##b
 #define AKV_CONCAT(a, b) AKV_CONCAT2(a, b)
 
-// Attention of requests seq_first .. seq_first + seq_count - 1 of the step.  `nq` (1, 2 or 4) sets the tile to
+// Attention of requests seq_first .. seq_first + seq_count - 1 of the step.  `nq` (1 or 2) sets the tile to
 // 16 * nq query columns; `tiles` is the number of tiles over those requests (sum of ceil(tokens / tokens_per_tile));
 // with num_splits > 1 `partial` must hold tiles * kv_heads * head_groups * num_splits * 16 * nq * (D + 4) floats.
 // page_size must be a power of two, at least 4.  `single_tokens` says that every request brings exactly one token.
@@ -506,6 +524,7 @@ extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
   a.table_width = table_width;
   a.seq_first = seq_first;
   a.seq_count = seq_count;
+  a.tiles = tiles;
   a.q_heads = q_heads;
   a.kv_heads = kv_heads;
   a.group = q_heads / kv_heads;
@@ -522,7 +541,6 @@ extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
   switch (nq) {
     case 1: return launch<1>(a, tiles, stream);
     case 2: return launch<2>(a, tiles, stream);
-    case 4: return launch<4>(a, tiles, stream);
     default: return -2;
   }
 }

@@ -57,26 +57,32 @@ __device__ __forceinline__ void store_tile(TY* y, floatx4 acc, int token, int fe
 }
 
 // ---- rows <= 16 * MT --------------------------------------------------------------------------------------------
-template <int MT, typename TY>
+// A wave owns RT consecutive row tiles and a part of k.  With more than 16 rows of x the activation operands weigh
+// more than the weights (MT operands per weight tile); giving a wave RT row tiles lets each of them serve RT weight
+// tiles, so the traffic from the caches stays near the traffic from memory.
+template <int MT, int RT, typename TY>
 __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __restrict__ x, const uintx4* __restrict__ wp,
                                                             TY* __restrict__ y, int rows, int outs, int k,
                                                             int k_tiles, int n_tiles, int k_split) {
-  constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);  // k-tiles per group; two groups are in flight
-  extern __shared__ float red[];  // [wave][MT][4][64]
+  constexpr int U = 8 / RT;  // k-tiles per group: 8 weight tiles (8 KB) per group and wave; two groups are in flight
+  extern __shared__ float red[];  // [group of waves with the same row tiles][RT][MT][4][64]
   const int lane = threadIdx.x & 63, waves = blockDim.x >> 6;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in every lane: keeps addresses scalar
   const int r = lane & 15, g = lane >> 4;
-  const int row_tile = blockIdx.x * (waves / k_split) + wave / k_split;
+  const int row_tile = (blockIdx.x * (waves / k_split) + wave / k_split) * RT;
   const int part = wave % k_split;
   const int per_part = (k_tiles + k_split - 1) / k_split;
   const int kt0 = part * per_part, kt1 = min(k_tiles, kt0 + per_part);
-  floatx4 acc[MT];
+  floatx4 acc[RT][MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) acc[mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   if (row_tile < n_tiles && kt0 < kt1) {
     // Addresses: a scalar base per wave plus a 32-bit lane offset, so that a load is one instruction.
-    const char* w_wave = reinterpret_cast<const char*>(wp) + static_cast<size_t>(row_tile) * k_tiles * 1024;
+    const size_t w_tile_row = static_cast<size_t>(k_tiles) * 1024;  // bytes of one row tile
+    const char* w_wave = reinterpret_cast<const char*>(wp) + static_cast<size_t>(row_tile) * w_tile_row;
     const uint32_t w_lane = lane * 16u;
     const char* x_bytes = reinterpret_cast<const char*>(x);
     uint32_t x_lane[MT];
@@ -91,13 +97,16 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
     // Two sets of operand registers: while the matrix cores work on one group of U k-tiles, the loads of the next
     // group are already on their way.  Weights are read once and never again: their loads are marked nontemporal,
     // which leaves the caches to the activations that every wave reads.
-    uintx4 a0[U], a1[U], b0[MT][U], b1[MT][U];
-    auto fetch = [&](int kt, uintx4 (&a)[U], uintx4 (&b)[MT][U]) {
+    uintx4 a0[RT][U], a1[RT][U], b0[MT][U], b1[MT][U];
+    auto fetch = [&](int kt, uintx4 (&a)[RT][U], uintx4 (&b)[MT][U]) {
       const char* w_at = w_wave + static_cast<size_t>(kt) * 1024;
       const char* x_at = x_bytes + static_cast<size_t>(kt) * 64;
 #pragma unroll
-      for (int u = 0; u < U; ++u)
-        a[u] = (kt + u < kt1) ? load_once(reinterpret_cast<const uintx4*>(w_at + w_lane + u * 1024u)) : zero;
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          a[rt][u] = (kt + u < kt1 && row_tile + rt < n_tiles)
+                         ? load_once(reinterpret_cast<const uintx4*>(w_at + rt * w_tile_row + w_lane + u * 1024u)) : zero;
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -107,11 +116,13 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
                          ? *reinterpret_cast<const uintx4*>(x_at + x_lane[mt] + u * 64u) : zero;
         }
     };
-    auto multiply = [&](const uintx4 (&a)[U], const uintx4 (&b)[MT][U]) {
+    auto multiply = [&](const uintx4 (&a)[RT][U], const uintx4 (&b)[MT][U]) {
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
+      for (int u = 0; u < U; ++u)
 #pragma unroll
-        for (int u = 0; u < U; ++u) acc[mt] = mfma16(a[u], b[mt][u], acc[mt]);
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = mfma16(a[rt][u], b[mt][u], acc[rt][mt]);
     };
     fetch(kt0, a0, b0);
     for (int kt = kt0; kt < kt1; kt += 2 * U) {
@@ -122,34 +133,50 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
     }
   }
   if (k_split > 1) {
+    // The parts of k are added in LDS one after the other - part 0, then + part 1, ... - so the order of the sum is
+    // fixed; the buffer holds one set of accumulators per group of waves that share their row tiles.
+    float* mine = red + static_cast<size_t>(wave / k_split) * (RT * MT * 4 * 64);
+    for (int turn = 0; turn < k_split; ++turn) {
+      if (part == turn) {
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+        for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) red[((wave * MT + mt) * 4 + i) * 64 + lane] = acc[mt][i];
-    __syncthreads();
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              float* slot = mine + ((rt * MT + mt) * 4 + i) * 64 + lane;
+              *slot = turn == 0 ? acc[rt][mt][i] : *slot + acc[rt][mt][i];
+            }
+      }
+      __syncthreads();
+    }
     if (part != 0) return;
-    for (int other = 1; other < k_split; ++other)  // fixed order: part 0 + part 1 + ...
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[mt][i] += red[(((wave + other) * MT + mt) * 4 + i) * 64 + lane];
+        for (int i = 0; i < 4; ++i) acc[rt][mt][i] = mine[((rt * MT + mt) * 4 + i) * 64 + lane];
   }
-  if (row_tile >= n_tiles) return;
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) store_tile<TY>(y, acc[mt], mt * 16 + r, row_tile * 16 + g * 4, rows, outs);
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      if (row_tile + rt < n_tiles) store_tile<TY>(y, acc[rt][mt], mt * 16 + r, (row_tile + rt) * 16 + g * 4, rows, outs);
 }
 
-template <int MT, typename TY>
+template <int MT, int RT, typename TY>
 int launch_skinny(const void* x, const void* wp, void* y, int rows, int outs, int k, int k_tiles, int n_tiles,
                   hipStream_t stream) {
   // enough waves to keep every CU's memory pipe full: split k over the waves of a block when there are few row tiles
+  const int wave_rows = (n_tiles + RT - 1) / RT;
   int k_split = 1;
-  while (k_split < 8 && n_tiles * k_split < 2048 && k_tiles / (k_split * 2) >= 4) k_split *= 2;
+  while (k_split < 8 && wave_rows * k_split < 2048 && k_tiles / (k_split * 2) >= 4) k_split *= 2;
   const int waves = k_split == 8 ? 8 : 4;
-  const int tiles_per_block = waves / k_split;
-  const int blocks = (n_tiles + tiles_per_block - 1) / tiles_per_block;
-  const size_t lds = k_split > 1 ? static_cast<size_t>(waves) * MT * 4 * 64 * sizeof(float) : 0;
-  linear_skinny_kernel<MT, TY><<<blocks, waves * 64, lds, stream>>>(
+  const int rows_per_block = waves / k_split;
+  const int blocks = (wave_rows + rows_per_block - 1) / rows_per_block;
+  const size_t lds = k_split > 1 ? static_cast<size_t>(rows_per_block) * RT * MT * 4 * 64 * sizeof(float) : 0;
+  linear_skinny_kernel<MT, RT, TY><<<blocks, waves * 64, lds, stream>>>(
       static_cast<const bf16_t*>(x), static_cast<const uintx4*>(wp), static_cast<TY*>(y), rows, outs, k, k_tiles,
       n_tiles, k_split);
   return AKV_LAUNCH_STATUS();
@@ -159,10 +186,15 @@ template <typename TY>
 int dispatch_skinny(const void* x, const void* wp, void* y, int rows, int outs, int k, int k_tiles, int n_tiles,
                     hipStream_t stream) {
   switch ((rows + 15) / 16) {
-    case 1: return launch_skinny<1, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
-    case 2: return launch_skinny<2, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
-    case 3: return launch_skinny<3, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
-    case 4: return launch_skinny<4, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+    case 1: return launch_skinny<1, 1, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+    case 2: return launch_skinny<2, 2, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+    // four row tiles per wave where that still leaves a thousand waves, two otherwise
+    case 3:
+      return n_tiles >= 512 ? launch_skinny<3, 4, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream)
+                            : launch_skinny<3, 2, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+    case 4:
+      return n_tiles >= 512 ? launch_skinny<4, 4, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream)
+                            : launch_skinny<4, 2, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
     default: return -2;
   }
 }
