@@ -68,11 +68,6 @@ class BlockTable:
     def num_held(self) -> int:
         return len(self._pages) - self._first_live
 
-    def pages_missing_for(self, num_tokens: int) -> int:
-        """Pages `append_tokens(num_tokens)` would take from the pool, counting those it gives back first."""
-        required = (self._length + num_tokens + self.page_size - 1) // self.page_size
-        return max(0, required - len(self._pages)) - self._passed_pages(self._length)
-
     def _passed_pages(self, next_position: int) -> int:
         """Live pages that lie wholly before the oldest key a query at `next_position` may read."""
         if self.window is None:

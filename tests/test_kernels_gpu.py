@@ -439,3 +439,31 @@ def test_sizes_are_refused_not_miscomputed(hip):
         hip.linear(torch.zeros(2, 3), torch.zeros(4, 3, device="cuda"), torch.zeros(2, 4, device="cuda"))
     with pytest.raises(KernelError):
         hip.linear(torch.zeros(2, 3, device="cuda"), torch.zeros(4, 5, device="cuda"), torch.zeros(2, 4, device="cuda"))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("history", [40, 100])
+def test_attention_window_edge(hip, ref, dtype, history):
+    """One key just inside the window and one just outside it both match the query far better than the rest: the
+    output must be the inside key's value, and must change when the window moves by one."""
+    window, dim, page = 17, 32, 8
+    portions = [(history, 1)]
+    pos = history                                        # the query's position; it sees keys pos - window + 1 .. pos
+    inside, outside = pos - window + 1, pos - window
+    for w, winner in ((window, inside), (window + 1, outside)):
+        q, k_pages, v_pages, ctx, meta, keys, values = _attention_case(dtype, 2, 1, dim, page, portions, None, 41)
+        table = meta.block_table[0]
+        direction = torch.randn(dim, generator=torch.Generator().manual_seed(5))
+        direction = direction / direction.norm() * 6.0
+        for key, gain in ((inside, 1.0), (outside, 1.5)):   # the outside key wins whenever it is seen
+            k_pages[int(table[key // page]), 0, key % page] = (direction * gain).to(dtype)
+        q[0] = (direction.repeat(2) * 4.0).to(dtype)
+        ctx.num_decode_seqs = 1
+        want = torch.empty_like(q)
+        ref.attention(q, k_pages, v_pages, ctx, meta, 2, 1, dim, dim ** -0.5, w, want)
+        cctx, cmeta = _to_cuda(ctx, meta)
+        got = torch.empty_like(q, device="cuda")
+        hip.attention(q.cuda(), k_pages.cuda(), v_pages.cuda(), cctx, cmeta, 2, 1, dim, dim ** -0.5, w, got)
+        torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(dtype))
+        seen_value = v_pages[int(table[winner // page]), 0, :, winner % page].float()
+        torch.testing.assert_close(got.cpu().float()[0, :dim], seen_value, rtol=0.05, atol=0.05)
