@@ -144,9 +144,20 @@ __global__ void gather_rows_kernel(const float* __restrict__ stream, const T* __
 }
 
 // ---- SwiGLU: out[n, i] = silu(gate_up[n, i]) * gate_up[n, inter + i] ----------------------------------------
+// A thread handles 4 consecutive outputs (16-byte accesses for float32, 8-byte for bfloat16) when `inter` allows.
 template <typename T>
 __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, long tokens, int inter) {
   const long index = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if ((inter & 3) == 0) {
+    const int quads = inter / 4;
+    if (index >= tokens * quads) return;
+    const long n = index / quads;
+    const int i = static_cast<int>(index % quads) * 4;
+    const float4 g = load4<T>(gate_up + n * 2 * inter + i), u = load4<T>(gate_up + n * 2 * inter + inter + i);
+    store4<T>(out + n * inter + i, make_float4(g.x / (1.f + expf(-g.x)) * u.x, g.y / (1.f + expf(-g.y)) * u.y,
+                                               g.z / (1.f + expf(-g.z)) * u.z, g.w / (1.f + expf(-g.w)) * u.w));
+    return;
+  }
   if (index >= tokens * inter) return;
   const long n = index / inter;
   const int i = static_cast<int>(index % inter);
@@ -215,81 +226,101 @@ __global__ void kv_write_kernel(const T* __restrict__ k, long k_stride, const T*
 }
 
 // ---- fused: per-head RMSNorm of q and k, rotation of q and k, q out, k and v into the token's cache slot -------
-// One wave per (token, head) over the q_heads + 2 * kv_heads heads of a qkv row.  Any of the three steps can be
-// switched off: q_weight/k_weight null (no norm), table null (no rotation), slot_map null (no cache write).
+// One wave per (token, group of `heads_per_wave` heads) of the q_heads + 2 * kv_heads heads of a qkv row (many
+// heads per wave when there are many tokens, one when there are few and latency counts).  A lane owns
+// the rotation pairs (j, j + dim/2) for j = lane, lane + 64, ...: both members of a pair sit in its registers, so
+// the rotation needs no exchange, and the token's position, cache slot and the pair's cos/sin are fetched once for
+// all the heads of the group.  Any step can be switched off: q_weight/k_weight null (no norm), table null (no
+// rotation), slot_map null (no cache write).
+constexpr int kMaxPairsPerLane = 2;  // head sizes up to 256
+
 template <typename T>
-__global__ void qk_norm_rope_write_kernel(const T* __restrict__ qkv, const float* __restrict__ q_weight,
-                                          const float* __restrict__ k_weight, float eps,
-                                          const float* __restrict__ table, int table_positions,
-                                          const int* __restrict__ positions, const int* __restrict__ slot_map,
-                                          T* __restrict__ k_pages, T* __restrict__ v_pages, T* __restrict__ q_out,
-                                          long tokens, int q_heads, int kv_heads, int dim, int page_size,
-                                          long num_slots) {
-  extern __shared__ float lds[];
+__global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
+    const T* __restrict__ qkv, const float* __restrict__ q_weight, const float* __restrict__ k_weight, float eps,
+    const float* __restrict__ table, int table_positions, const int* __restrict__ positions,
+    const int* __restrict__ slot_map, T* __restrict__ k_pages, T* __restrict__ v_pages, T* __restrict__ q_out,
+    long tokens, int q_heads, int kv_heads, int dim, int page_size, long num_slots, int heads_per_wave) {
   const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
-  const int heads = q_heads + 2 * kv_heads;
-  const long row = static_cast<long>(blockIdx.x) * waves + wave;
-  if (row >= tokens * heads) return;
-  const long n = row / heads;
-  const int h = static_cast<int>(row % heads);
-  const T* src = qkv + row * dim;  // a qkv row is heads * dim wide, so (n, h) starts at row * dim
-  float* mine = lds + wave * dim;
-
-  T* dst;  // where this head's result goes
-  if (h < q_heads) {
-    dst = q_out + (n * q_heads + h) * dim;
-  } else {
-    if (slot_map == nullptr) return;
-    const long slot = slot_map[n];
-    if (slot < 0 || slot >= num_slots) return;
-    const int kvh = (h - q_heads) % kv_heads;
-    const long page = slot / page_size, offset = slot % page_size;
-    if (h >= q_heads + kv_heads) {  // value: copied as it is, into the [dim, page_size] layout
-      const long at = (page * kv_heads + kvh) * dim * page_size + offset;
-      for (int i = lane; i < dim; i += kWave) v_pages[at + static_cast<long>(i) * page_size] = src[i];
-      return;
-    }
-    dst = k_pages + ((page * kv_heads + kvh) * page_size + offset) * dim;
-  }
-
-  const float* weight = h < q_heads ? q_weight : k_weight;
-  float scale = 1.f;
-  if (weight != nullptr) {
-    float acc = 0.f;
-    for (int i = lane; i < dim; i += kWave) {
-      const float v = to_float(src[i]);
-      acc += v * v;
-    }
-    scale = rsqrtf(wave_sum(acc) / static_cast<float>(dim) + eps);
-  }
-  if (table == nullptr) {
-    for (int i = lane; i < dim; i += kWave) {
-      const float v = to_float(src[i]);
-      dst[i] = weight != nullptr ? from_float<T>(rounded<T>(v * scale) * weight[i]) : src[i];
-    }
-    return;
-  }
-  for (int i = lane; i < dim; i += kWave) {
-    const float v = to_float(src[i]);
-    mine[i] = weight != nullptr ? rounded<T>(rounded<T>(v * scale) * weight[i]) : v;
-  }
-  // the wave's own writes to its LDS row must be visible to its other lanes before the pairs are read
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const int heads = q_heads + 2 * kv_heads, groups = (heads + heads_per_wave - 1) / heads_per_wave;
+  const long item = static_cast<long>(blockIdx.x) * waves + wave;
+  if (item >= tokens * groups) return;
+  const long n = item / groups;
+  const int first_head = static_cast<int>(item % groups) * heads_per_wave;
   const int half = dim / 2;
-  const int pos = positions[n];
-  const bool bad = pos < 0 || pos >= table_positions;
-  for (int j = lane; j < half; j += kWave) {
-    if (bad) {
-      dst[j] = from_float<T>(__uint_as_float(0x7fc00000u));
-      dst[j + half] = from_float<T>(__uint_as_float(0x7fc00000u));
+  const float nan = __uint_as_float(0x7fc00000u);
+
+  // per token: the pair's cos/sin, the cache slot
+  float cs[kMaxPairsPerLane], sn[kMaxPairsPerLane];
+  float wq_lo[kMaxPairsPerLane], wq_hi[kMaxPairsPerLane], wk_lo[kMaxPairsPerLane], wk_hi[kMaxPairsPerLane];
+#pragma unroll
+  for (int p = 0; p < kMaxPairsPerLane; ++p) {
+    const int j = lane + p * kWave;
+    cs[p] = 1.f;
+    sn[p] = 0.f;
+    wq_lo[p] = wq_hi[p] = wk_lo[p] = wk_hi[p] = 1.f;
+    if (j < half) {
+      if (table != nullptr) {
+        const int pos = positions[n];
+        if (pos < 0 || pos >= table_positions) {
+          cs[p] = sn[p] = nan;
+        } else {
+          cs[p] = table[(static_cast<long>(pos) * half + j) * 2];
+          sn[p] = table[(static_cast<long>(pos) * half + j) * 2 + 1];
+        }
+      }
+      if (q_weight != nullptr) {
+        wq_lo[p] = q_weight[j];
+        wq_hi[p] = q_weight[j + half];
+        wk_lo[p] = k_weight[j];
+        wk_hi[p] = k_weight[j + half];
+      }
+    }
+  }
+  long slot = -1;
+  if (slot_map != nullptr) {
+    slot = slot_map[n];
+    if (slot < 0 || slot >= num_slots) slot = -1;  // host checks the map; never write outside the pool
+  }
+  const long page = slot >= 0 ? slot / page_size : 0, offset = slot >= 0 ? slot % page_size : 0;
+
+  for (int h = first_head; h < min(first_head + heads_per_wave, heads); ++h) {
+    const T* src = qkv + (n * heads + h) * dim;
+    if (h >= q_heads + kv_heads) {  // value: copied as it is, into the [dim, page_size] layout
+      if (slot < 0) continue;
+      const long at = (page * kv_heads + (h - q_heads - kv_heads)) * dim * page_size + offset;
+      for (int i = lane; i < dim; i += kWave) v_pages[at + static_cast<long>(i) * page_size] = src[i];
       continue;
     }
-    const float c = table[(static_cast<long>(pos) * half + j) * 2], s = table[(static_cast<long>(pos) * half + j) * 2 + 1];
-    const float lo = mine[j], hi = mine[j + half];
-    dst[j] = from_float<T>(lo * c - hi * s);
-    dst[j + half] = from_float<T>(hi * c + lo * s);
+    const bool is_q = h < q_heads;
+    if (!is_q && slot < 0) continue;
+    T* dst = is_q ? q_out + (n * q_heads + h) * dim
+                  : k_pages + ((page * kv_heads + (h - q_heads)) * page_size + offset) * dim;
+    float lo[kMaxPairsPerLane], hi[kMaxPairsPerLane];
+    float acc = 0.f;
+#pragma unroll
+    for (int p = 0; p < kMaxPairsPerLane; ++p) {
+      const int j = lane + p * kWave;
+      lo[p] = hi[p] = 0.f;
+      if (j < half) {
+        lo[p] = to_float(src[j]);
+        hi[p] = to_float(src[j + half]);
+        acc += lo[p] * lo[p] + hi[p] * hi[p];
+      }
+    }
+    const bool normed = q_weight != nullptr;
+    const float scale = normed ? rsqrtf(wave_sum(acc) / static_cast<float>(dim) + eps) : 1.f;
+#pragma unroll
+    for (int p = 0; p < kMaxPairsPerLane; ++p) {
+      const int j = lane + p * kWave;
+      if (j >= half) continue;
+      float a = lo[p], b = hi[p];
+      if (normed) {  // normalise, round to the activation type, times the weight, round again
+        a = rounded<T>(rounded<T>(a * scale) * (is_q ? wq_lo[p] : wk_lo[p]));
+        b = rounded<T>(rounded<T>(b * scale) * (is_q ? wq_hi[p] : wk_hi[p]));
+      }
+      dst[j] = from_float<T>(a * cs[p] - b * sn[p]);
+      dst[j + half] = from_float<T>(b * cs[p] + a * sn[p]);
+    }
   }
 }
 
@@ -348,7 +379,7 @@ int akv_gather_rows(const float* stream_buf, const void* pending, int dtype, con
 int akv_swiglu(const void* gate_up, void* out, int dtype, long tokens, int inter, hipStream_t stream) {
   if (tokens <= 0) return 0;
   AKV_DISPATCH(dtype, T,
-               swiglu_kernel<T><<<blocks_for(tokens * inter, 256), 256, 0, stream>>>(
+               swiglu_kernel<T><<<blocks_for((inter & 3) == 0 ? tokens * (inter / 4) : tokens * inter, 256), 256, 0, stream>>>(
                    static_cast<const T*>(gate_up), static_cast<T*>(out), tokens, inter));
   return AKV_LAUNCH_STATUS();
 }
@@ -385,13 +416,14 @@ int akv_qk_norm_rope_write(const void* qkv, const float* q_weight, const float* 
                            void* k_pages, void* v_pages, void* q_out, int dtype, long tokens, int q_heads,
                            int kv_heads, int dim, int page_size, long num_pages, hipStream_t stream) {
   if (tokens <= 0) return 0;
-  const long rows = tokens * (q_heads + 2 * kv_heads);
-  const size_t lds = 4 * static_cast<size_t>(dim) * sizeof(float);
+  if (dim > 2 * kMaxPairsPerLane * kWave || (dim & 1) != 0) return -2;
+  const int heads_per_wave = tokens >= 512 ? 8 : (tokens >= 64 ? 2 : 1);
+  const long items = tokens * ((q_heads + 2 * kv_heads + heads_per_wave - 1) / heads_per_wave);
   AKV_DISPATCH(dtype, T,
-               qk_norm_rope_write_kernel<T><<<blocks_for(rows, 4), 256, lds, stream>>>(
+               qk_norm_rope_write_kernel<T><<<blocks_for(items, 4), 256, 0, stream>>>(
                    static_cast<const T*>(qkv), q_weight, k_weight, eps, table, table_positions, positions, slot_map,
                    static_cast<T*>(k_pages), static_cast<T*>(v_pages), static_cast<T*>(q_out), tokens, q_heads,
-                   kv_heads, dim, page_size, num_pages * page_size));
+                   kv_heads, dim, page_size, num_pages * page_size, heads_per_wave));
   return AKV_LAUNCH_STATUS();
 }
 

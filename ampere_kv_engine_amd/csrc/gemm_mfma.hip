@@ -247,8 +247,7 @@ __global__ __launch_bounds__(256, 2) void linear_wide_kernel(const bf16_t* __res
     x_row[p] = token < rows;
     x_at[p] = static_cast<uint32_t>(token) * static_cast<uint32_t>(k) * 2u + (e % 8) * 16u;
   }
-  uintx4 moving[PX];
-  auto fetch = [&](int stage) {
+  auto fetch = [&](int stage, uintx4 (&moving)[PX]) {
     const char* at = x_bytes + static_cast<size_t>(stage) * (kWideK * 2);
 #pragma unroll
     for (int p = 0; p < PX; ++p) {
@@ -257,7 +256,7 @@ __global__ __launch_bounds__(256, 2) void linear_wide_kernel(const bf16_t* __res
       moving[p] = (x_row[p] && inside) ? *reinterpret_cast<const uintx4*>(at + x_at[p]) : zero;
     }
   };
-  auto stash = [&](int buffer) {
+  auto stash = [&](int buffer, const uintx4 (&moving)[PX]) {
 #pragma unroll
     for (int p = 0; p < PX; ++p) {
       const int e = p * 256 + threadIdx.x, c = e % 8, t = e / 8;
@@ -294,20 +293,51 @@ __global__ __launch_bounds__(256, 2) void linear_wide_kernel(const bf16_t* __res
       for (int n = 0; n < 4; ++n) acc[n][m] = mfma16(a[n], b[m], acc[n][m]);
   };
 
-  uintx4 a0[4], a1[4];
-  fetch(0);
-  weights(0, a0);
-  stash(0);
-  __syncthreads();
-  for (int stage = 0; stage < stages; ++stage) {
-    const int buffer = stage & 1;
-    if (stage + 1 < stages) fetch(stage + 1);   // next stage's activations travel while this stage computes
-    weights(stage * 2 + 1, a1);
-    multiply(buffer, 0, a0);
-    weights(stage * 2 + 2, a0);
-    multiply(buffer, 1, a1);
-    if (stage + 1 < stages) stash(buffer ^ 1);
+  if constexpr (MW <= 4) {
+    // Registers allow two sets of everything: the weights of a whole stage (two k-tiles) are fetched one stage ahead,
+    // the activations two stages ahead (they wait in registers for one stage, then go to the LDS buffer that the
+    // stage before has just finished reading).
+    uintx4 a0[2][4], a1[2][4], m0[PX], m1[PX];
+    auto run_stage = [&](int stage, const uintx4 (&cur)[2][4], uintx4 (&next)[2][4], uintx4 (&arriving)[PX],
+                         const uintx4 (&arrived)[PX]) {
+      const int buffer = stage & 1;
+      if (stage + 2 < stages) fetch(stage + 2, arriving);
+      if (stage + 1 < stages) {
+        weights(stage * 2 + 2, next[0]);
+        weights(stage * 2 + 3, next[1]);
+      }
+      multiply(buffer, 0, cur[0]);
+      multiply(buffer, 1, cur[1]);
+      if (stage + 1 < stages) stash(buffer ^ 1, arrived);
+      __syncthreads();
+    };
+    fetch(0, m0);
+    stash(0, m0);
+    if (stages > 1) fetch(1, m1);
+    weights(0, a0[0]);
+    weights(1, a0[1]);
     __syncthreads();
+    for (int stage = 0; stage < stages; stage += 2) {
+      run_stage(stage, a0, a1, m0, m1);
+      if (stage + 1 < stages) run_stage(stage + 1, a1, a0, m1, m0);
+    }
+  } else {
+    // weights are fetched one k-tile ahead, activations one stage ahead
+    uintx4 a0[4], a1[4], moving[PX];
+    fetch(0, moving);
+    stash(0, moving);
+    weights(0, a0);
+    __syncthreads();
+    for (int stage = 0; stage < stages; ++stage) {
+      const int buffer = stage & 1;
+      if (stage + 1 < stages) fetch(stage + 1, moving);
+      weights(stage * 2 + 1, a1);
+      multiply(buffer, 0, a0);
+      weights(stage * 2 + 2, a0);
+      multiply(buffer, 1, a1);
+      if (stage + 1 < stages) stash(buffer ^ 1, moving);
+      __syncthreads();
+    }
   }
 #pragma unroll
   for (int n = 0; n < 4; ++n)
