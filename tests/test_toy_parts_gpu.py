@@ -169,3 +169,146 @@ def test_the_state_carries_across_portions_and_between_mixed_requests(tmp_path):
     engine.close(a), engine.close(b)
     torch.testing.assert_close(torch.cat(parts_a), whole_a, rtol=1e-4, atol=1e-5)
     torch.testing.assert_close(torch.cat(parts_b), whole_b, rtol=1e-4, atol=1e-5)
+
+
+# ---- a feed-forward with routing and another position encoding, also defined here only -----------------------------
+
+class RoutedFeedForward(Part):
+    """Top-1 of `experts` small SwiGLU experts per token: router logits in float32, the chosen expert's output times
+    its softmax weight.  Token-wise, so nothing about cache or batch touches it."""
+    graph_safe = False
+
+    def __init__(self, spec, runtime):
+        self.rt, self.hidden, self.inter, self.experts = runtime, int(spec["hidden_size"]), int(spec["intermediate_size"]), int(spec["experts"])
+        self.router = self.gate_up = self.down = None
+
+    def tensors(self, prefix):
+        specs = [TensorSpec(prefix + "moe.router.weight", (self.experts, self.hidden))]
+        for e in range(self.experts):
+            specs += [TensorSpec(f"{prefix}moe.experts.{e}.gate_up.weight", (2 * self.inter, self.hidden)),
+                      TensorSpec(f"{prefix}moe.experts.{e}.down.weight", (self.hidden, self.inter))]
+        return specs
+
+    def load(self, fetch, prefix):
+        specs = self.tensors(prefix)
+        self.router = fetch(specs[0]).float()
+        self.gate_up = [self.rt.kernels.prepare_linear(fetch(s)) for s in specs[1::2]]
+        self.down = [self.rt.kernels.prepare_linear(fetch(s)) for s in specs[2::2]]
+
+    def forward(self, x, ctx):
+        k = self.rt.kernels
+        logits = x.float() @ self.router.T                        # router logits in float32
+        weight, choice = logits.softmax(-1).max(-1)
+        out = ctx.arena.take(tuple(x.shape), self.rt.dtype)
+        out.zero_()
+        for e in range(self.experts):
+            rows = (choice == e).nonzero().flatten()
+            if rows.numel() == 0:
+                continue
+            xe = x[rows].contiguous()
+            gate_up = torch.empty((rows.numel(), 2 * self.inter), dtype=self.rt.dtype, device=x.device)
+            k.linear(xe, self.gate_up[e], gate_up)                # the framework's own products and activation
+            act = torch.empty((rows.numel(), self.inter), dtype=self.rt.dtype, device=x.device)
+            k.swiglu(gate_up, act)
+            ye = torch.empty((rows.numel(), self.hidden), dtype=self.rt.dtype, device=x.device)
+            k.linear(act, self.down[e], ye)
+            out[rows] = (ye.float() * weight[rows, None]).to(self.rt.dtype)
+        return out
+
+
+class AdjacentPairRotary(Part):
+    """Another rotary encoding: pairs (2j, 2j + 1) instead of (j, j + d/2), angles position * theta^(-2j/d)."""
+
+    def __init__(self, spec, runtime):
+        self.head_dim, self.theta = int(spec["head_dim"]), float(spec["theta"])
+        self.inv_freq = 1.0 / (self.theta ** (torch.arange(0, self.head_dim, 2, dtype=torch.float32) / self.head_dim))
+        self.table = None
+
+    def apply(self, x, positions):
+        angles = positions.float()[:, None].to(x.device) * self.inv_freq.to(x.device)[None, :]
+        cos, sin = angles.cos()[:, None, :], angles.sin()[:, None, :]
+        even, odd = x[..., 0::2].float(), x[..., 1::2].float()
+        rotated = torch.stack((even * cos - odd * sin, odd * cos + even * sin), dim=-1).flatten(-2)
+        x.copy_(rotated.to(x.dtype))
+        return x
+
+
+@dataclass(frozen=True)
+class RoutedConfig(ToyConfig):
+    architecture = "ToyRoutedForCausalLM"
+
+    def to_model_spec(self):
+        h = self.hidden_size
+        norm = part("rmsnorm", size=h, eps=self.eps)
+        block = part("prenorm", hidden_size=h, norm=norm)
+        attention = part("attention", hidden_size=h, q_heads=2, kv_heads=2, head_dim=16, window=None, qk_norm=None,
+                         position=part("adjacent_pair_rotary", head_dim=16, theta=1e4), scale=0.25, name="self_attn")
+        dense = part("swiglu", hidden_size=h, intermediate_size=40, name="mlp")
+        routed = part("routed", hidden_size=h, intermediate_size=24, experts=3)
+        layers = (LayerSpec(block, attention, routed, "model.layers.0."), LayerSpec(block, attention, dense, "model.layers.1."))
+        return ModelSpec(self.architecture, self.vocab_size, h,
+                         part("embedding", vocab_size=self.vocab_size, hidden_size=h, name="model.embed_tokens.weight"),
+                         layers, (RunEntry(0, 0), RunEntry(1, 1)),
+                         part("rmsnorm", size=h, eps=self.eps, name="model.norm.weight"),
+                         part("linear_head", vocab_size=self.vocab_size, hidden_size=h, name="lm_head.weight", tied_to=None))
+
+
+def plain_routed_logits(folder, config, ids):
+    from safetensors.torch import load_file
+    w = {k: v.float() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    h = w["model.embed_tokens.weight"][torch.tensor(ids)]
+    n = len(ids)
+    inv_freq = 1.0 / (1e4 ** (torch.arange(0, 16, 2, dtype=torch.float32) / 16))
+
+    def rotate(x):
+        angles = torch.arange(n).float()[:, None] * inv_freq[None, :]
+        cos, sin = angles.cos()[:, None, :], angles.sin()[:, None, :]
+        even, odd = x[..., 0::2], x[..., 1::2]
+        return torch.stack((even * cos - odd * sin, odd * cos + even * sin), dim=-1).flatten(-2)
+
+    for layer in range(2):
+        p = f"model.layers.{layer}."
+        x = P.rms_norm(h, w[p + "input_layernorm.weight"], config.eps)
+        q = rotate((x @ w[p + "self_attn.q_proj.weight"].T).reshape(n, 2, 16))
+        k = rotate((x @ w[p + "self_attn.k_proj.weight"].T).reshape(n, 2, 16))
+        v = (x @ w[p + "self_attn.v_proj.weight"].T).reshape(n, 2, 16)
+        h = h + P.causal_attention(q, k, v).reshape(n, 32) @ w[p + "self_attn.o_proj.weight"].T
+        x = P.rms_norm(h, w[p + "post_attention_layernorm.weight"], config.eps)
+        if layer == 0:
+            probs = (x @ w[p + "moe.router.weight"].T).softmax(-1)
+            weight, choice = probs.max(-1)
+            y = torch.zeros_like(x)
+            for t in range(n):
+                e = int(choice[t])
+                gu = x[t] @ w[f"{p}moe.experts.{e}.gate_up.weight"].T
+                g, u = gu[:24], gu[24:]
+                y[t] = ((g * torch.sigmoid(g) * u) @ w[f"{p}moe.experts.{e}.down.weight"].T) * weight[t]
+            h = h + y
+        else:
+            h = h + P.swiglu_feed_forward(x, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    return P.rms_norm(h, w["model.norm.weight"], config.eps) @ w["lm_head.weight"].T
+
+
+def test_a_routed_feed_forward_and_another_position_encoding(tmp_path):
+    """Different feed-forwards in different layers (routed experts, dense), attention without q/k norm and with a
+    position encoding the fused kernel does not know: registered and stepped, whole and in portions."""
+    register_part("feed_forward", "routed", RoutedFeedForward, replace=True)
+    register_part("position", "adjacent_pair_rotary", AdjacentPairRotary, replace=True)
+    register_architecture(RoutedConfig.architecture, RoutedConfig, replace=True)
+    config = RoutedConfig(vocab_size=97, hidden_size=32, decay=0.0, eps=1e-5)
+    folder = write_random_model(str(tmp_path / "routed"), config, seed=11)
+    engine = Engine.from_folder(folder, EngineConfig(dtype="float32", page_size=8, num_pages=16, max_seqs=2,
+                                                     max_batched_tokens=64, max_seq_len=64, device="cuda:0"))
+    assert not engine._recordable and not engine.model.blocks[0].mixer.fused
+    assert [type(b.feed_forward).__name__ for b in engine.model.blocks] == ["RoutedFeedForward", "SwiGLU"]
+    ids = random_ids(97, 21, seed=12)
+    want = plain_routed_logits(folder, config, ids)
+    seq = engine.open("whole")
+    got = engine.step([StepEntry(seq, ids, list(range(21)))]).cpu()
+    engine.close(seq)
+    torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-5)
+    seq, parts = engine.open("cut"), []
+    for lo, hi in ((0, 9), (9, 11), (11, 12), (12, 21)):
+        parts.append(engine.step([StepEntry(seq, ids[lo:hi], list(range(hi - lo)))]).cpu())
+    engine.close(seq)
+    torch.testing.assert_close(torch.cat(parts), want, rtol=1e-4, atol=1e-5)
