@@ -11,6 +11,10 @@
 //   linear_wide    rows  > 64 (prefill): 128 x 128 output tiles per block, activations staged through LDS,
 //                  weights straight from the packed layout into the A operand.
 // In both, a row of x meets the weights in the same k order whatever else is in the batch.
+//
+// GATED variants compute a gated feed-forward's first half in one pass: the packed matrix alternates a tile of 16 gate
+// rows with the tile of the 16 up rows of the same features, a wave always owns such pairs, and what it stores is
+// silu(gate) * up, taken from the float32 accumulators - the stacked product never goes to memory.
 
 #include "common.h"
 #include "api.h"
@@ -56,11 +60,18 @@ __device__ __forceinline__ void store_tile(TY* y, floatx4 acc, int token, int fe
   }
 }
 
+__device__ __forceinline__ floatx4 silu_times(floatx4 gate, floatx4 up) {
+  floatx4 v;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v[i] = gate[i] / (1.f + expf(-gate[i])) * up[i];
+  return v;
+}
+
 // ---- rows <= 16 * MT --------------------------------------------------------------------------------------------
 // A wave owns RT consecutive row tiles and a part of k.  With more than 16 rows of x the activation operands weigh
 // more than the weights (MT operands per weight tile); giving a wave RT row tiles lets each of them serve RT weight
 // tiles, so the traffic from the caches stays near the traffic from memory.
-template <int MT, int RT, typename TY>
+template <int MT, int RT, typename TY, bool GATED>
 __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __restrict__ x, const uintx4* __restrict__ wp,
                                                             TY* __restrict__ y, int rows, int outs, int k,
                                                             int k_tiles, int n_tiles, int k_split) {
@@ -158,14 +169,25 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[rt][mt][i] = mine[((rt * MT + mt) * 4 + i) * 64 + lane];
   }
+  if constexpr (GATED) {
+    static_assert(RT % 2 == 0, "a wave must own gate and up tiles in pairs");
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
+    for (int rt = 0; rt < RT; rt += 2)
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-      if (row_tile + rt < n_tiles) store_tile<TY>(y, acc[rt][mt], mt * 16 + r, (row_tile + rt) * 16 + g * 4, rows, outs);
+      for (int mt = 0; mt < MT; ++mt)
+        if (row_tile + rt < n_tiles)
+          store_tile<TY>(y, silu_times(acc[rt][mt], acc[rt + 1][mt]), mt * 16 + r, ((row_tile + rt) >> 1) * 16 + g * 4,
+                         rows, outs);
+  } else {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        if (row_tile + rt < n_tiles) store_tile<TY>(y, acc[rt][mt], mt * 16 + r, (row_tile + rt) * 16 + g * 4, rows, outs);
+  }
 }
 
-template <int MT, int RT, typename TY>
+template <int MT, int RT, typename TY, bool GATED>
 int launch_skinny(const void* x, const void* wp, void* y, int rows, int outs, int k, int k_tiles, int n_tiles,
                   hipStream_t stream) {
   // enough waves to keep every CU's memory pipe full: split k over the waves of a block when there are few row tiles
@@ -176,25 +198,25 @@ int launch_skinny(const void* x, const void* wp, void* y, int rows, int outs, in
   const int rows_per_block = waves / k_split;
   const int blocks = (wave_rows + rows_per_block - 1) / rows_per_block;
   const size_t lds = k_split > 1 ? static_cast<size_t>(rows_per_block) * RT * MT * 4 * 64 * sizeof(float) : 0;
-  linear_skinny_kernel<MT, RT, TY><<<blocks, waves * 64, lds, stream>>>(
+  linear_skinny_kernel<MT, RT, TY, GATED><<<blocks, waves * 64, lds, stream>>>(
       static_cast<const bf16_t*>(x), static_cast<const uintx4*>(wp), static_cast<TY*>(y), rows, outs, k, k_tiles,
       n_tiles, k_split);
   return AKV_LAUNCH_STATUS();
 }
 
-template <typename TY>
+template <typename TY, bool GATED>
 int dispatch_skinny(const void* x, const void* wp, void* y, int rows, int outs, int k, int k_tiles, int n_tiles,
                     hipStream_t stream) {
   switch ((rows + 15) / 16) {
-    case 1: return launch_skinny<1, 1, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
-    case 2: return launch_skinny<2, 2, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+    case 1: return launch_skinny<1, GATED ? 2 : 1, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+    case 2: return launch_skinny<2, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
     // four row tiles per wave where that still leaves a thousand waves, two otherwise
     case 3:
-      return n_tiles >= 512 ? launch_skinny<3, 4, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream)
-                            : launch_skinny<3, 2, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+      return n_tiles >= 512 ? launch_skinny<3, 4, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream)
+                            : launch_skinny<3, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
     case 4:
-      return n_tiles >= 512 ? launch_skinny<4, 4, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream)
-                            : launch_skinny<4, 2, TY>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+      return n_tiles >= 512 ? launch_skinny<4, 4, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream)
+                            : launch_skinny<4, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
     default: return -2;
   }
 }
@@ -211,7 +233,7 @@ constexpr int kWideN = 128, kWideK = 64, kXcds = 8;
 
 // MW: token tiles per wave (8: 256 tokens per block; 4: 128 tokens per block, for products with few weight rows,
 // which would otherwise leave compute units without a block).
-template <typename TY, int MW>
+template <typename TY, int MW, bool GATED>
 __global__ __launch_bounds__(256, 2) void linear_wide_kernel(const bf16_t* __restrict__ x, const uintx4* __restrict__ wp,
                                                           TY* __restrict__ y, int rows, int outs, int k, int k_tiles,
                                                           int n_tiles, int n_blocks, int m_blocks) {
@@ -339,14 +361,23 @@ __global__ __launch_bounds__(256, 2) void linear_wide_kernel(const bf16_t* __res
       __syncthreads();
     }
   }
+  if constexpr (GATED) {
 #pragma unroll
-  for (int n = 0; n < 4; ++n)
+    for (int n = 0; n < 4; n += 2)
 #pragma unroll
-    for (int m = 0; m < MW; ++m)
-      store_tile<TY>(y, acc[n][m], token0 + wave_m * (16 * MW) + m * 16 + r, (tile0 + n) * 16 + g * 4, rows, outs);
+      for (int m = 0; m < MW; ++m)
+        store_tile<TY>(y, silu_times(acc[n][m], acc[n + 1][m]), token0 + wave_m * (16 * MW) + m * 16 + r,
+                       ((tile0 + n) >> 1) * 16 + g * 4, rows, outs);
+  } else {
+#pragma unroll
+    for (int n = 0; n < 4; ++n)
+#pragma unroll
+      for (int m = 0; m < MW; ++m)
+        store_tile<TY>(y, acc[n][m], token0 + wave_m * (16 * MW) + m * 16 + r, (tile0 + n) * 16 + g * 4, rows, outs);
+  }
 }
 
-template <typename TY>
+template <typename TY, bool GATED>
 int launch_wide(const void* x, const void* wp, void* y, int rows, int outs, int k, int k_tiles, int n_tiles,
                 hipStream_t stream) {
   const int n_blocks = (n_tiles * 16 + kWideN - 1) / kWideN;
@@ -357,16 +388,31 @@ int launch_wide(const void* x, const void* wp, void* y, int rows, int outs, int 
   const long blocks = static_cast<long>((n_blocks + kXcds - 1) / kXcds) * kXcds * m_blocks;
   if (blocks > 0x7fffffffL || static_cast<long>(rows) * k * 2 >= (1L << 32)) return -2;
   if (tall)
-    linear_wide_kernel<TY, 8><<<static_cast<unsigned>(blocks), 256, 0, stream>>>(
+    linear_wide_kernel<TY, 8, GATED><<<static_cast<unsigned>(blocks), 256, 0, stream>>>(
         static_cast<const bf16_t*>(x), static_cast<const uintx4*>(wp), static_cast<TY*>(y), rows, outs, k, k_tiles,
         n_tiles, n_blocks, m_blocks);
   else
-    linear_wide_kernel<TY, 4><<<static_cast<unsigned>(blocks), 256, 0, stream>>>(
+    linear_wide_kernel<TY, 4, GATED><<<static_cast<unsigned>(blocks), 256, 0, stream>>>(
         static_cast<const bf16_t*>(x), static_cast<const uintx4*>(wp), static_cast<TY*>(y), rows, outs, k, k_tiles,
         n_tiles, n_blocks, m_blocks);
   return AKV_LAUNCH_STATUS();
 }
 
+}  // namespace
+
+namespace {
+template <bool GATED>
+int linear_packed(const void* x, const void* wp, void* y, int y_dtype, int rows, int outs, int k, int n_tiles,
+                  int k_tiles, hipStream_t stream) {
+  if (rows <= 64) {
+    if (y_dtype == kF32) return dispatch_skinny<float, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+    if (y_dtype == kBF16) return dispatch_skinny<bf16_t, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+    return -1;
+  }
+  if (y_dtype == kF32) return launch_wide<float, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+  if (y_dtype == kBF16) return launch_wide<bf16_t, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+  return -1;
+}
 }  // namespace
 
 // x [rows, k] bfloat16 row-major; wp the packed weight of `n_tiles` x `k_tiles` tiles; y [rows, outs] bfloat16 or
@@ -375,12 +421,14 @@ extern "C" int akv_linear_packed(const void* x, const void* wp, void* y, int y_d
                                  int n_tiles, int k_tiles, hipStream_t stream) {
   if (rows <= 0 || outs <= 0) return 0;
   if ((k & 7) != 0 || n_tiles * 16 < outs || k_tiles * 32 < k) return -2;
-  if (rows <= 64) {
-    if (y_dtype == kF32) return dispatch_skinny<float>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
-    if (y_dtype == kBF16) return dispatch_skinny<bf16_t>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
-    return -1;
-  }
-  if (y_dtype == kF32) return launch_wide<float>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
-  if (y_dtype == kBF16) return launch_wide<bf16_t>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
-  return -1;
+  return linear_packed<false>(x, wp, y, y_dtype, rows, outs, k, n_tiles, k_tiles, stream);
+}
+
+// The gated pair in one pass: wp holds 2 * inter / 16 row tiles, gate tile t at 2t and up tile t at 2t + 1;
+// y [rows, inter] = silu(x Wgate^T) * (x Wup^T).  inter must be a multiple of 16.
+extern "C" int akv_linear_packed_swiglu(const void* x, const void* wp, void* y, int y_dtype, int rows, int inter,
+                                        int k, int n_tiles, int k_tiles, hipStream_t stream) {
+  if (rows <= 0 || inter <= 0) return 0;
+  if ((k & 7) != 0 || (inter & 15) != 0 || n_tiles * 8 != inter || k_tiles * 32 < k) return -2;
+  return linear_packed<true>(x, wp, y, y_dtype, rows, inter, k, n_tiles, k_tiles, stream);
 }

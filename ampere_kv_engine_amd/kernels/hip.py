@@ -43,6 +43,21 @@ class PackedWeight:
         return full.reshape(self.n_tiles * 16, self.k_tiles * 32)[:self.outs, :self.k].contiguous()
 
 
+class GatedWeight:
+    """Gate and up matrices [inter, k] of a gated feed-forward as ONE packed matrix whose row tiles alternate:
+    tile 2t holds gate rows 16t .. 16t + 15, tile 2t + 1 the up rows of the same features."""
+
+    def __init__(self, gate: torch.Tensor, up: torch.Tensor):
+        inter, k = gate.shape
+        self.inter, self.k = inter, k
+        paired = torch.stack((gate.view(inter // 16, 16, k), up.view(inter // 16, 16, k)), dim=1).reshape(2 * inter, k)
+        self.packed = PackedWeight(paired)
+
+    def unpack(self) -> tuple[torch.Tensor, torch.Tensor]:
+        paired = self.packed.unpack().view(self.inter // 16, 2, 16, self.k)
+        return paired[:, 0].reshape(self.inter, self.k), paired[:, 1].reshape(self.inter, self.k)
+
+
 def _code(t: torch.Tensor) -> int:
     try:
         return _DTYPE_CODE[t.dtype]
@@ -77,7 +92,7 @@ class HipKernels:
         self.decode_max_splits = 32     # and no more than this many (the merge walks them one after the other)
         for name in ("akv_embed", "akv_add_rmsnorm", "akv_rmsnorm_rows", "akv_copy_rows", "akv_gather_rows",
                      "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
-                     "akv_linear_tiled", "akv_linear_packed", "akv_attention_rows", "akv_sample"):
+                     "akv_linear_tiled", "akv_linear_packed", "akv_linear_packed_swiglu", "akv_attention_rows", "akv_sample"):
             getattr(self.lib, name).restype = ctypes.c_int
 
     # ---- helpers -----------------------------------------------------------------------------------------
@@ -199,6 +214,25 @@ class HipKernels:
         self._dense(out, "out", None, (rows, outs))
         self._check(self.lib.akv_linear_tiled(_ptr(x), _code(x), _ptr(weight), _code(weight), _ptr(out), _code(out),
                                               rows, outs, k, self._stream()), "linear")
+
+    def prepare_gated_linear(self, gate: torch.Tensor, up: torch.Tensor):
+        """The packing for `gated_linear`, or None where the two matrices have to stay a stacked product followed by
+        `swiglu` (float32 weights, sizes the packed kernels do not take)."""
+        if (gate.dtype == torch.bfloat16 and up.dtype == torch.bfloat16 and gate.shape == up.shape
+                and gate.shape[1] % 8 == 0 and gate.shape[0] % 16 == 0):
+            return GatedWeight(gate, up)
+        return None
+
+    def gated_linear(self, x, weight: GatedWeight, out):
+        """out [rows, inter] = silu(x Wgate^T) * (x Wup^T), from float32 accumulators, in one kernel."""
+        rows = x.shape[0]
+        packed = weight.packed
+        self._dense(x, "x", torch.bfloat16, (rows, weight.k))
+        self._dense(out, "out", None, (rows, weight.inter))
+        self._dense(packed.data, "packed weight", torch.bfloat16)
+        self._check(self.lib.akv_linear_packed_swiglu(_ptr(x), _ptr(packed.data), _ptr(out), _code(out), rows,
+                                                      weight.inter, weight.k, packed.n_tiles, packed.k_tiles,
+                                                      self._stream()), "gated_linear")
 
     def swiglu(self, gate_up, out):
         tokens, inter = out.shape

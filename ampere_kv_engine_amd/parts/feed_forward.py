@@ -1,7 +1,11 @@
 """Feed-forwards.  `swiglu` is the dense gated one of the reference (ampere_kv/runner.py:172-177):
-down( silu(x Wg^T) * (x Wu^T) ), silu on the gate only; gate and up are one stacked product."""
+down( silu(x Wg^T) * (x Wu^T) ), silu on the gate only.  Gate and up are one product: where the kernel set can, it
+also applies the activation before anything is stored (`gated_linear`); otherwise the stacked product is followed
+by the `swiglu` kernel."""
 
 from __future__ import annotations
+
+import torch
 
 from .base import Part, register_part
 from .linear import Linear
@@ -17,6 +21,7 @@ class SwiGLU(Part):
         self.name = spec.get("name", "mlp")
         self.gate_up = Linear(runtime, self.hidden, [self.inter, self.inter], ["gate_proj.weight", "up_proj.weight"])
         self.down = Linear(runtime, self.inter, [self.hidden], ["down_proj.weight"])
+        self.gated = None           # the kernel set's packing of gate and up for the one-pass product, if it has one
 
     def _prefix(self, prefix):
         return f"{prefix}{self.name}."
@@ -25,19 +30,28 @@ class SwiGLU(Part):
         return self.gate_up.tensors(self._prefix(prefix)) + self.down.tensors(self._prefix(prefix))
 
     def load(self, fetch, prefix):
-        self.gate_up.load(fetch, self._prefix(prefix))
+        gate, up = (fetch(spec) for spec in self.gate_up.tensors(self._prefix(prefix)))
+        self.gated = self.rt.kernels.prepare_gated_linear(gate.contiguous(), up.contiguous())
+        if self.gated is None:
+            self.gate_up.adopt(torch.cat((gate, up), dim=0).contiguous())
+        else:
+            self._gated_bytes = gate.numel() * gate.element_size() + up.numel() * up.element_size()
         self.down.load(fetch, self._prefix(prefix))
 
     def weight_bytes(self):
-        return self.gate_up.weight_bytes() + self.down.weight_bytes()
+        first = self._gated_bytes if self.gated is not None else self.gate_up.weight_bytes()
+        return first + self.down.weight_bytes()
 
     def forward(self, x, ctx):
         """x [tokens, hidden] -> [tokens, hidden], both in the activation dtype."""
         tokens = x.shape[0]
-        gate_up = ctx.arena.take((tokens, 2 * self.inter), self.rt.dtype)
-        self.gate_up.forward(x, gate_up)
         act = ctx.arena.take((tokens, self.inter), self.rt.dtype)
-        self.rt.kernels.swiglu(gate_up, act)
+        if self.gated is not None:
+            self.rt.kernels.gated_linear(x, self.gated, act)
+        else:
+            gate_up = ctx.arena.take((tokens, 2 * self.inter), self.rt.dtype)
+            self.gate_up.forward(x, gate_up)
+            self.rt.kernels.swiglu(gate_up, act)
         out = ctx.arena.take((tokens, self.hidden), self.rt.dtype)
         return self.down.forward(act, out)
 

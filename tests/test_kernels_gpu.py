@@ -151,6 +151,43 @@ def test_linear_packed_rows_do_not_depend_on_the_batch(hip):
             assert torch.equal(part, whole[first:first + n])
 
 
+@pytest.mark.parametrize("y_dtype", DTYPES)
+@pytest.mark.parametrize("rows", [1, 7, 16, 17, 40, 64, 65, 128, 300])
+@pytest.mark.parametrize("inter,k", [(16, 96), (48, 4096), (208, 200), (4112, 256), (1040, 1000)])
+def test_gated_linear(hip, ref, y_dtype, rows, inter, k):
+    """silu(x Wg^T) * (x Wu^T) in one pass over gate and up tiles that alternate in the packing: numbers of tiles
+    that fill no wave's or block's share, few rows and many."""
+    from ampere_kv_engine_amd.kernels.hip import GatedWeight
+    x = rand(rows, k, dtype=torch.bfloat16, seed=35)
+    gate = rand(inter, k, dtype=torch.bfloat16, seed=36, scale=0.08)
+    up = rand(inter, k, dtype=torch.bfloat16, seed=37, scale=0.05)
+    weight = hip.prepare_gated_linear(gate.cuda(), up.cuda())
+    assert isinstance(weight, GatedWeight)
+    back = weight.unpack()
+    assert torch.equal(back[0].cpu(), gate) and torch.equal(back[1].cpu(), up)
+    want = torch.empty(rows, inter, dtype=y_dtype)
+    ref.gated_linear(x, (gate, up), want)
+    got = torch.full((rows, inter), float("nan"), dtype=y_dtype, device="cuda")
+    hip.gated_linear(x.cuda(), weight, got)
+    t = dict(rtol=2e-4, atol=2e-5 * k ** 0.5) if y_dtype == torch.float32 else tol(torch.bfloat16)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **t)
+
+
+def test_gated_linear_rows_do_not_depend_on_the_batch_and_other_sizes_stay_stacked(hip):
+    x = rand(200, 512, dtype=torch.bfloat16, seed=38).cuda()
+    weight = hip.prepare_gated_linear(rand(304, 512, dtype=torch.bfloat16, seed=39).cuda(),
+                                      rand(304, 512, dtype=torch.bfloat16, seed=40).cuda())
+    for count in (40, 200):
+        whole = torch.empty(count, 304, device="cuda")
+        hip.gated_linear(x[:count].contiguous(), weight, whole)
+        for first, n in ((0, 1), (17, 3), (39, 1)) if count == 40 else ((0, 70), (100, 100)):
+            part = torch.empty(n, 304, device="cuda")
+            hip.gated_linear(x[first:first + n].contiguous(), weight, part)
+            assert torch.equal(part, whole[first:first + n])
+    assert hip.prepare_gated_linear(torch.zeros(40, 64, dtype=torch.bfloat16), torch.zeros(40, 64, dtype=torch.bfloat16)) is None
+    assert hip.prepare_gated_linear(torch.zeros(48, 64), torch.zeros(48, 64)) is None
+
+
 def test_linear_keeps_other_weights_row_major(hip):
     assert isinstance(hip.prepare_linear(torch.zeros(4, 12, dtype=torch.bfloat16, device="cuda")), torch.Tensor)   # k % 8
     assert isinstance(hip.prepare_linear(torch.zeros(4, 16, device="cuda")), torch.Tensor)                         # float32

@@ -58,6 +58,13 @@ class TorchKernels:
     def linear(self, x, weight, out):
         out.copy_((x.float() @ weight.float().T).to(out.dtype))
 
+    def prepare_gated_linear(self, gate, up):
+        return (gate, up)
+
+    def gated_linear(self, x, weight, out):
+        g, u = x.float() @ weight[0].float().T, x.float() @ weight[1].float().T
+        out.copy_((g * torch.sigmoid(g) * u).to(out.dtype))
+
     def swiglu(self, gate_up, out):
         inter = out.shape[-1]
         g, u = gate_up[:, :inter].float(), gate_up[:, inter:].float()
