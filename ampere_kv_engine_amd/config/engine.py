@@ -21,6 +21,9 @@ class EngineConfig:
     max_seq_len: int = 8192          # longest sequence a request may reach (block-table width, rotary table)
     device: str = "cuda:0"
     decode_graphs: bool = True       # replay a recorded HIP graph for steps in which every request brings one token
+    # bfloat16 products of more rows than this go to the BLAS library, which reads the matrices row-major: they are
+    # then kept twice (row-major and packed for the engine's own kernels).  None: one copy, own kernels only.
+    library_products_above: int | None = 16
 
     def __post_init__(self):
         if self.dtype not in DTYPES:
@@ -29,6 +32,9 @@ class EngineConfig:
             value = getattr(self, name)
             if not isinstance(value, int) or value <= 0:
                 raise ValueError(f"{name} must be a positive integer, got {value!r}")
+        above = self.library_products_above
+        if above is not None and (not isinstance(above, int) or above < 0):
+            raise ValueError(f"library_products_above must be None or a non-negative integer, got {above!r}")
 
     @property
     def max_pages_per_seq(self) -> int:

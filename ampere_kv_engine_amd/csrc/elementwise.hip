@@ -71,12 +71,18 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ st
         acc += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
       }
     }
+    float4 gain[kRowGroups];  // asked for before the sum, so that they arrive while it is formed
+#pragma unroll
+    for (int j = 0; j < kRowGroups; ++j) {
+      const int i = (j * 256 + threadIdx.x) * 4;
+      if (i < hidden) gain[j] = load4<float>(weight + i);
+    }
     const float scale = rsqrtf(block_sum(acc, scratch) / static_cast<float>(hidden) + eps);
 #pragma unroll
     for (int j = 0; j < kRowGroups; ++j) {
       const int i = (j * 256 + threadIdx.x) * 4;
       if (i < hidden) {
-        const float4 v = kept[j], w = load4<float>(weight + i);
+        const float4 v = kept[j], w = gain[j];
         store4<T>(o + i, make_float4(rounded<T>(v.x * scale) * w.x, rounded<T>(v.y * scale) * w.y,
                                      rounded<T>(v.z * scale) * w.z, rounded<T>(v.w * scale) * w.w));
       }

@@ -71,12 +71,15 @@ __device__ __forceinline__ floatx4 silu_times(floatx4 gate, floatx4 up) {
 // A wave owns RT consecutive row tiles and a part of k.  With more than 16 rows of x the activation operands weigh
 // more than the weights (MT operands per weight tile); giving a wave RT row tiles lets each of them serve RT weight
 // tiles, so the traffic from the caches stays near the traffic from memory.
+// whether every wave of a block gets LDS for its own accumulators in the sum over the parts of k (8 waves, <= 64 KB)
+template <int MT, int RT> constexpr bool kSkinnyOwnSets = RT * MT <= 8;
+
 template <int MT, int RT, typename TY, bool GATED>
 __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __restrict__ x, const uintx4* __restrict__ wp,
                                                             TY* __restrict__ y, int rows, int outs, int k,
                                                             int k_tiles, int n_tiles, int k_split) {
   constexpr int U = 8 / RT;  // k-tiles per group: 8 weight tiles (8 KB) per group and wave; two groups are in flight
-  extern __shared__ float red[];  // [group of waves with the same row tiles][RT][MT][4][64]
+  extern __shared__ float red[];  // [wave, or group of waves with the same row tiles][RT][MT][4][64]
   const int lane = threadIdx.x & 63, waves = blockDim.x >> 6;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in every lane: keeps addresses scalar
   const int r = lane & 15, g = lane >> 4;
@@ -144,30 +147,55 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
     }
   }
   if (k_split > 1) {
-    // The parts of k are added in LDS one after the other - part 0, then + part 1, ... - so the order of the sum is
-    // fixed; the buffer holds one set of accumulators per group of waves that share their row tiles.
-    float* mine = red + static_cast<size_t>(wave / k_split) * (RT * MT * 4 * 64);
-    for (int turn = 0; turn < k_split; ++turn) {
-      if (part == turn) {
+    // The parts of k are summed through LDS in a fixed order: part 0 + part 1 + part 2 ...  Where a set of
+    // accumulators per wave fits, every wave writes its own and the wave of part 0 adds them up after one barrier;
+    // otherwise one set per group of waves that share their row tiles is passed from part to part.
+    constexpr int kSet = RT * MT * 4 * 64;  // floats of one wave's accumulators
+    if constexpr (kSkinnyOwnSets<MT, RT>) {
+      float* mine = red + static_cast<size_t>(wave) * kSet;
+      if (part != 0) {
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              float* slot = mine + ((rt * MT + mt) * 4 + i) * 64 + lane;
-              *slot = turn == 0 ? acc[rt][mt][i] : *slot + acc[rt][mt][i];
-            }
+            for (int i = 0; i < 4; ++i) mine[((rt * MT + mt) * 4 + i) * 64 + lane] = acc[rt][mt][i];
       }
       __syncthreads();
+      if (part != 0) return;
+      for (int other = 1; other < k_split; ++other) {
+        const float* theirs = mine + static_cast<size_t>(other) * kSet;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[rt][mt][i] += theirs[((rt * MT + mt) * 4 + i) * 64 + lane];
+      }
+    } else {
+      float* mine = red + static_cast<size_t>(wave / k_split) * kSet;
+      for (int turn = 0; turn < k_split; ++turn) {
+        if (part == turn) {
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                float* slot = mine + ((rt * MT + mt) * 4 + i) * 64 + lane;
+                *slot = turn == 0 ? acc[rt][mt][i] : *slot + acc[rt][mt][i];
+              }
+        }
+        __syncthreads();
+      }
+      if (part != 0) return;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[rt][mt][i] = mine[((rt * MT + mt) * 4 + i) * 64 + lane];
     }
-    if (part != 0) return;
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[rt][mt][i] = mine[((rt * MT + mt) * 4 + i) * 64 + lane];
   }
   if constexpr (GATED) {
     static_assert(RT % 2 == 0, "a wave must own gate and up tiles in pairs");
@@ -197,7 +225,8 @@ int launch_skinny(const void* x, const void* wp, void* y, int rows, int outs, in
   const int waves = k_split == 8 ? 8 : 4;
   const int rows_per_block = waves / k_split;
   const int blocks = (wave_rows + rows_per_block - 1) / rows_per_block;
-  const size_t lds = k_split > 1 ? static_cast<size_t>(rows_per_block) * RT * MT * 4 * 64 * sizeof(float) : 0;
+  const size_t sets = kSkinnyOwnSets<MT, RT> ? waves : rows_per_block;
+  const size_t lds = k_split > 1 ? sets * RT * MT * 4 * 64 * sizeof(float) : 0;
   linear_skinny_kernel<MT, RT, TY, GATED><<<blocks, waves * 64, lds, stream>>>(
       static_cast<const bf16_t*>(x), static_cast<const uintx4*>(wp), static_cast<TY*>(y), rows, outs, k, k_tiles,
       n_tiles, k_split);

@@ -34,7 +34,7 @@ class Engine:
         self.dtype = _TORCH_DTYPE[engine_config.dtype]
         if kernels is None:
             from ..kernels.hip import HipKernels
-            kernels = HipKernels(self.device)
+            kernels = HipKernels(self.device, library_products_above=engine_config.library_products_above)
         self.kernels = kernels
         self.runtime = Runtime(kernels=kernels, dtype=self.dtype, device=self.device,
                                max_seq_len=engine_config.max_seq_len, page_size=engine_config.page_size)

@@ -25,9 +25,10 @@ class PackedWeight:
     """A bfloat16 matrix [outs, k] re-laid for the matrix cores: tiles of 16 rows x 32 k, 1 KB each, stored
     [row tile][k tile][lane][8] with lane = (k chunk of 8) * 16 + row; rows and k beyond the matrix are zero."""
 
-    def __init__(self, matrix: torch.Tensor):
+    def __init__(self, matrix: torch.Tensor, keep_row_major: bool = False):
         outs, k = matrix.shape
         self.outs, self.k = outs, k
+        self.row_major = matrix if keep_row_major else None   # what a library product reads
         self.n_tiles, self.k_tiles = (outs + 15) // 16, (k + 31) // 32
         padded = matrix
         if outs % 16 or k % 32:
@@ -47,9 +48,11 @@ class GatedWeight:
     """Gate and up matrices [inter, k] of a gated feed-forward as ONE packed matrix whose row tiles alternate:
     tile 2t holds gate rows 16t .. 16t + 15, tile 2t + 1 the up rows of the same features."""
 
-    def __init__(self, gate: torch.Tensor, up: torch.Tensor):
+    def __init__(self, gate: torch.Tensor, up: torch.Tensor, keep_row_major: bool = False):
         inter, k = gate.shape
         self.inter, self.k = inter, k
+        # what a library product reads: gate rows, then up rows
+        self.stacked = torch.cat((gate, up), dim=0).contiguous() if keep_row_major else None
         paired = torch.stack((gate.view(inter // 16, 16, k), up.view(inter // 16, 16, k)), dim=1).reshape(2 * inter, k)
         self.packed = PackedWeight(paired)
 
@@ -72,7 +75,11 @@ def _ptr(t: torch.Tensor | None):
 class HipKernels:
     name = "hip-gfx950"
 
-    def __init__(self, device: torch.device | str = "cuda:0"):
+    def __init__(self, device: torch.device | str = "cuda:0", library_products_above: int | None = 16):
+        """`library_products_above`: bfloat16 products of more rows than this go to the BLAS library (torch.mm),
+        which then needs the matrices row-major beside their packing; None keeps the packing alone and every
+        product in this library's own kernels."""
+        self.library_products_above = library_products_above
         self.device = torch.device(device)
         if self.device.type == "cuda" and self.device.index is None:
             self.device = torch.device("cuda", 0)
@@ -195,14 +202,21 @@ class HipKernels:
         """bfloat16 matrices whose k is a multiple of 8 are packed for the MFMA kernels; others stay row-major and
         go through the plain tiled kernel."""
         if matrix.dtype == torch.bfloat16 and matrix.shape[1] % 8 == 0:
-            return PackedWeight(matrix)
+            return PackedWeight(matrix, keep_row_major=self.library_products_above is not None)
         return matrix
+
+    def _library_product(self, rows: int, row_major, out) -> bool:
+        return (row_major is not None and self.library_products_above is not None
+                and rows > self.library_products_above and out.dtype == torch.bfloat16)
 
     def linear(self, x, weight, out):
         if isinstance(weight, PackedWeight):
             rows, k = x.shape
             self._dense(x, "x", torch.bfloat16, (rows, weight.k))
             self._dense(out, "out", None, (rows, weight.outs))
+            if self._library_product(rows, weight.row_major, out):
+                torch.mm(x, weight.row_major.t(), out=out)
+                return
             self._dense(weight.data, "packed weight", torch.bfloat16)
             self._check(self.lib.akv_linear_packed(_ptr(x), _ptr(weight.data), _ptr(out), _code(out), rows, weight.outs,
                                                    weight.k, weight.n_tiles, weight.k_tiles, self._stream()), "linear")
@@ -220,15 +234,30 @@ class HipKernels:
         `swiglu` (float32 weights, sizes the packed kernels do not take)."""
         if (gate.dtype == torch.bfloat16 and up.dtype == torch.bfloat16 and gate.shape == up.shape
                 and gate.shape[1] % 8 == 0 and gate.shape[0] % 16 == 0):
-            return GatedWeight(gate, up)
+            return GatedWeight(gate, up, keep_row_major=self.library_products_above is not None)
         return None
 
-    def gated_linear(self, x, weight: GatedWeight, out):
-        """out [rows, inter] = silu(x Wgate^T) * (x Wup^T), from float32 accumulators, in one kernel."""
+    def gated_scratch(self, weight: GatedWeight, rows: int, dtype: torch.dtype):
+        """Shape of the buffer `gated_linear` wants for this many rows (the stacked product of the library path),
+        or None."""
+        probe = torch.empty((), dtype=dtype)
+        return (rows, 2 * weight.inter) if self._library_product(rows, weight.stacked, probe) else None
+
+    def gated_linear(self, x, weight: GatedWeight, out, scratch=None):
+        """out [rows, inter] = silu(x Wgate^T) * (x Wup^T): one kernel, from float32 accumulators; with many rows the
+        library's stacked product into `scratch`, then the activation kernel."""
         rows = x.shape[0]
         packed = weight.packed
         self._dense(x, "x", torch.bfloat16, (rows, weight.k))
         self._dense(out, "out", None, (rows, weight.inter))
+        if self._library_product(rows, weight.stacked, out):
+            if scratch is None:
+                raise KernelError(f"gated_linear of {rows} rows takes the library path and needs the scratch buffer "
+                                  "that gated_scratch() describes")
+            self._dense(scratch, "scratch", torch.bfloat16, (rows, 2 * weight.inter))
+            torch.mm(x, weight.stacked.t(), out=scratch)
+            self.swiglu(scratch, out)
+            return
         self._dense(packed.data, "packed weight", torch.bfloat16)
         self._check(self.lib.akv_linear_packed_swiglu(_ptr(x), _ptr(packed.data), _ptr(out), _code(out), rows,
                                                       weight.inter, weight.k, packed.n_tiles, packed.k_tiles,

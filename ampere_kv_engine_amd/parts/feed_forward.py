@@ -47,7 +47,9 @@ class SwiGLU(Part):
         tokens = x.shape[0]
         act = ctx.arena.take((tokens, self.inter), self.rt.dtype)
         if self.gated is not None:
-            self.rt.kernels.gated_linear(x, self.gated, act)
+            shape = self.rt.kernels.gated_scratch(self.gated, tokens, self.rt.dtype)
+            scratch = ctx.arena.take(shape, self.rt.dtype) if shape is not None else None
+            self.rt.kernels.gated_linear(x, self.gated, act, scratch)
         else:
             gate_up = ctx.arena.take((tokens, 2 * self.inter), self.rt.dtype)
             self.gate_up.forward(x, gate_up)

@@ -61,3 +61,31 @@ def test_trace_run_program(case, dtype, tmp_path):
             row += count
             fed[item["id"]] += count
         assert row == data.shape[0]
+
+
+def test_recorded_decode_steps_of_many_requests(case):
+    """More than 16 requests decode together: the products of such a step come from the BLAS library, also inside the
+    recorded graph.  Every replay is checked against the plain implementation, with eager work between replays."""
+    from conftest import random_ids
+    from ampere_kv_engine_amd.config import EngineConfig
+    from ampere_kv_engine_amd.engine import Engine, StepEntry
+    from plain.qwen3_plain import PlainQwen3
+    live, decoded, page = 24, 10, case["page_size"]
+    engine = Engine.from_folder(case["folder"], EngineConfig(dtype="bfloat16", page_size=page, num_pages=live * (48 // page + 1),
+                                                             max_seqs=live, max_batched_tokens=1024, max_seq_len=64))
+    assert engine.kernels.library_products_above == 16 and engine._recordable
+    plain = PlainQwen3(case["folder"])
+    ids = [random_ids(case["raw"]["vocab_size"], 14 + i % 7 + decoded, seed=300 + i) for i in range(live)]
+    want = [plain.logits(tokens) for tokens in ids]
+    seqs = [engine.open(f"r{i}") for i in range(live)]
+    engine.step([StepEntry(seq, tokens[:-decoded], []) for seq, tokens in zip(seqs, ids)])
+    for step in range(decoded):
+        entries = [StepEntry(seq, [tokens[len(tokens) - decoded + step]], [0]) for seq, tokens in zip(seqs, ids)]
+        got = engine.step(entries).cpu()
+        for i, tokens in enumerate(ids):
+            expected = want[i][len(tokens) - decoded + step]
+            torch.testing.assert_close(got[i], expected, **tolerance("bfloat16", want[i]), msg=lambda m: f"step {step} request {i}: {m}")
+        torch.cuda.synchronize()
+    assert sum(graph is not None for graph, _ in engine._graphs.values()) == 1
+    for seq in seqs:
+        engine.close(seq)

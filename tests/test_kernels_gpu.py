@@ -17,8 +17,21 @@ DTYPES = [torch.float32, torch.bfloat16]
 
 @pytest.fixture(scope="module")
 def hip():
+    """The kernel set as the engine builds it: the BLAS library takes bfloat16 products of more than 16 rows."""
     from ampere_kv_engine_amd.kernels.hip import HipKernels
     return HipKernels("cuda:0")
+
+
+@pytest.fixture(scope="module")
+def hip_own():
+    """Every product in the engine's own kernels, whatever the number of rows."""
+    from ampere_kv_engine_amd.kernels.hip import HipKernels
+    return HipKernels("cuda:0", library_products_above=None)
+
+
+@pytest.fixture(params=["own", "library"])
+def hip_either(request, hip, hip_own):
+    return hip if request.param == "library" else hip_own
 
 
 @pytest.fixture(scope="module")
@@ -122,7 +135,8 @@ def test_linear(hip, ref, x_dtype, w_dtype, y_dtype, rows, outs, k):
 @pytest.mark.parametrize("y_dtype", DTYPES)
 @pytest.mark.parametrize("rows", [1, 5, 16, 17, 33, 64, 65, 130, 300])
 @pytest.mark.parametrize("outs,k", [(379, 96), (64, 4096), (200, 200), (8192, 256), (1040, 1000)])
-def test_linear_packed(hip, ref, y_dtype, rows, outs, k):
+def test_linear_packed(hip_either, ref, y_dtype, rows, outs, k):
+    hip = hip_either
     """bfloat16 weights packed for the matrix cores: few rows (k split over waves), many rows (LDS-staged tiles),
     sizes that are no multiple of the 16 x 32 tile."""
     from ampere_kv_engine_amd.kernels.hip import PackedWeight
@@ -138,7 +152,8 @@ def test_linear_packed(hip, ref, y_dtype, rows, outs, k):
     torch.testing.assert_close(got.cpu().float(), want.float(), **t)
 
 
-def test_linear_packed_rows_do_not_depend_on_the_batch(hip):
+def test_linear_packed_rows_do_not_depend_on_the_batch(hip_own):
+    hip = hip_own
     """A row's result is bit-identical alone and among up to 64 rows (one kernel), and among more (the other)."""
     x = rand(200, 512, dtype=torch.bfloat16, seed=33).cuda()
     packed = hip.prepare_linear(rand(300, 512, dtype=torch.bfloat16, seed=34).cuda())
@@ -154,7 +169,8 @@ def test_linear_packed_rows_do_not_depend_on_the_batch(hip):
 @pytest.mark.parametrize("y_dtype", DTYPES)
 @pytest.mark.parametrize("rows", [1, 7, 16, 17, 40, 64, 65, 128, 300])
 @pytest.mark.parametrize("inter,k", [(16, 96), (48, 4096), (208, 200), (4112, 256), (1040, 1000)])
-def test_gated_linear(hip, ref, y_dtype, rows, inter, k):
+def test_gated_linear(hip_either, ref, y_dtype, rows, inter, k):
+    hip = hip_either
     """silu(x Wg^T) * (x Wu^T) in one pass over gate and up tiles that alternate in the packing: numbers of tiles
     that fill no wave's or block's share, few rows and many."""
     from ampere_kv_engine_amd.kernels.hip import GatedWeight
@@ -168,12 +184,15 @@ def test_gated_linear(hip, ref, y_dtype, rows, inter, k):
     want = torch.empty(rows, inter, dtype=y_dtype)
     ref.gated_linear(x, (gate, up), want)
     got = torch.full((rows, inter), float("nan"), dtype=y_dtype, device="cuda")
-    hip.gated_linear(x.cuda(), weight, got)
+    shape = hip.gated_scratch(weight, rows, y_dtype)
+    assert (shape is not None) == (hip.library_products_above is not None and rows > 16 and y_dtype == torch.bfloat16)
+    hip.gated_linear(x.cuda(), weight, got, torch.empty(shape, dtype=y_dtype, device="cuda") if shape else None)
     t = dict(rtol=2e-4, atol=2e-5 * k ** 0.5) if y_dtype == torch.float32 else tol(torch.bfloat16)
     torch.testing.assert_close(got.cpu().float(), want.float(), **t)
 
 
-def test_gated_linear_rows_do_not_depend_on_the_batch_and_other_sizes_stay_stacked(hip):
+def test_gated_linear_rows_do_not_depend_on_the_batch_and_other_sizes_stay_stacked(hip_own):
+    hip = hip_own
     x = rand(200, 512, dtype=torch.bfloat16, seed=38).cuda()
     weight = hip.prepare_gated_linear(rand(304, 512, dtype=torch.bfloat16, seed=39).cuda(),
                                       rand(304, 512, dtype=torch.bfloat16, seed=40).cuda())

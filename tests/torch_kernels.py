@@ -61,7 +61,10 @@ class TorchKernels:
     def prepare_gated_linear(self, gate, up):
         return (gate, up)
 
-    def gated_linear(self, x, weight, out):
+    def gated_scratch(self, weight, rows, dtype):
+        return None
+
+    def gated_linear(self, x, weight, out, scratch=None):
         g, u = x.float() @ weight[0].float().T, x.float() @ weight[1].float().T
         out.copy_((g * torch.sigmoid(g) * u).to(out.dtype))
 
