@@ -63,6 +63,7 @@ struct Args {
   float scale_log2;           // softmax scale * log2(e)
   int window;                 // 0: none
   int seg_keys, num_splits;
+  int units;                  // compute units of the device (block order of the shared kernel)
 };
 
 // Which request and which of its tiles this block works on.
@@ -73,7 +74,7 @@ struct Tile {
 
 // Tiles are numbered request by request.  The wave looks at 64 requests at a time: every lane counts the tiles of
 // one request, a prefix sum over the lanes places them, and the lane whose span holds `slot` owns the answer.
-__device__ __forceinline__ Tile find_tile(const Args& a, int slot) {
+__device__ __forceinline__ Tile find_tile(const Args& a, int slot, int per_tile) {
   Tile t{};
   t.found = false;
   const int lane = threadIdx.x & 63, end = a.seq_first + a.seq_count;
@@ -94,7 +95,7 @@ __device__ __forceinline__ Tile find_tile(const Args& a, int slot) {
       begin = a.q_start[r];
       count = a.q_start[r + 1] - begin;
     }
-    const int tiles = (count + a.tokens_per_tile - 1) / a.tokens_per_tile;
+    const int tiles = (count + per_tile - 1) / per_tile;
     int upto = tiles;  // inclusive prefix sum over the wave
 #pragma unroll
     for (int step = 1; step < 64; step <<= 1) {
@@ -108,9 +109,9 @@ __device__ __forceinline__ Tile find_tile(const Args& a, int slot) {
       const int local = slot - (before + __shfl(upto - tiles, owner, 64));
       const int o_begin = __shfl(begin, owner, 64), o_count = __shfl(count, owner, 64);
       t.request = r0 + owner;
-      t.first_row = o_begin + local * a.tokens_per_tile;
-      t.tokens = min(a.tokens_per_tile, o_count - local * a.tokens_per_tile);
-      t.first_pos = a.seq_lens[t.request] - o_count + local * a.tokens_per_tile;
+      t.first_row = o_begin + local * per_tile;
+      t.tokens = min(per_tile, o_count - local * per_tile);
+      t.first_pos = a.seq_lens[t.request] - o_count + local * per_tile;
       t.found = true;
       return t;
     }
@@ -134,7 +135,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
   const int slot = SPLIT ? static_cast<int>(blockIdx.x)
                          : (pass == 0 ? a.tiles - 1 - static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x));
   if (!SPLIT && pass == 1 && slot >= a.tiles - 1 - slot) break;  // the middle tile was the first pass's
-  const Tile t = find_tile(a, slot);
+  const Tile t = find_tile(a, slot, a.tokens_per_tile);
   if (!t.found) continue;
   const int kvh = blockIdx.y / a.head_groups, hg = blockIdx.y % a.head_groups;
   const uintx4 zero = uintx4{0u, 0u, 0u, 0u};
@@ -416,12 +417,335 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
   }  // pass
 }
 
+// ---- prompt portions: four waves share every key and value through LDS ------------------------------------------------
+// A block of 4 waves works on 4 consecutive tiles of one request and one kv head (4 * 16 * NQ columns).  The keys and
+// values of a step of 32 keys are fetched from the pages ONCE per block - every thread moves a few 16-byte pieces into
+// LDS, double-buffered, one barrier per step - and each wave reads its MFMA A operands from there.  Against one wave
+// per tile this takes three quarters of the traffic off the vector memory pipe and the address arithmetic off the
+// waves, and leaves registers for two blocks per compute unit.  In LDS a key row is padded by 16 bytes and stored at the
+// MFMA row it feeds (tile j, row rho), a value row (one dim, 32 keys) is padded by 16 bytes: operand reads of the 16
+// lanes of a group then fall into different banks.  Pages must hold at least 8 tokens (an aligned run of 8 keys of a
+// value row is one 16-byte piece).
+constexpr int kSharedWaves = 4;
+constexpr int KROW = D + 8;   // bfloat16 per key row in LDS
+constexpr int VROW = 32 + 8;  // bfloat16 per value row in LDS
+constexpr float kLazy = 8.f;  // the exponentials' reference point trails the maximum by at most 2^kLazy
+
+template <int NQ>
+__global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) void attention_shared_kernel(const Args a) {
+  __shared__ __align__(16) bf16_t k_lds[2][32 * KROW];
+  __shared__ __align__(16) bf16_t v_lds[2][D * VROW];
+  __shared__ int bad_page;
+  const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // Late tiles of a prompt see the most keys.  Blocks are ranked longest first, and the ranks are dealt out to the
+  // compute units like cards in a snake: the first `units` blocks take the longest, the next `units` blocks the
+  // following ranks in ascending order, so that the two blocks that share a unit add up to about the same work.
+  const int heads = a.kv_heads * a.head_groups, round = 2 * a.units;
+  const int turn = static_cast<int>(blockIdx.x) / round, within = static_cast<int>(blockIdx.x) % round;
+  const int total = a.tiles * heads, in_round = min(round, total - turn * round);
+  // a short last round has in_round < round blocks: its second part, if any, mirrors onto the ranks that exist
+  const int rank = turn * round + (within < a.units ? within : in_round - 1 - (within - a.units));
+  Tile t = find_tile(a, a.tiles - 1 - rank / heads, kSharedWaves * a.tokens_per_tile);
+  if (!t.found) return;  // the same in every wave of the block
+  t.request = __builtin_amdgcn_readfirstlane(t.request);  // the same in every lane: addresses built on it stay scalar
+  t.first_row = __builtin_amdgcn_readfirstlane(t.first_row);
+  t.tokens = __builtin_amdgcn_readfirstlane(t.tokens);
+  t.first_pos = __builtin_amdgcn_readfirstlane(t.first_pos);
+  const int kvh = (rank % heads) / a.head_groups, hg = (rank % heads) % a.head_groups;
+  const uintx4 zero = uintx4{0u, 0u, 0u, 0u};
+  const int page_mask = (1 << a.page_shift) - 1;
+  if (tid == 0) bad_page = 0;
+
+  // this wave's tile inside the block's, and this lane's columns
+  const int wave_token0 = wave * a.tokens_per_tile;
+  const bool wave_active = wave_token0 < t.tokens;
+  const int wave_first_pos = t.first_pos + wave_token0;
+  const int wave_last_pos = t.first_pos + min(t.tokens, wave_token0 + a.tokens_per_tile) - 1;
+  bool col_valid[NQ];
+  int col_pos[NQ], col_low[NQ];
+  long col_at[NQ];
+  uintx4 qreg[NQ][KT];
+#pragma unroll
+  for (int nq = 0; nq < NQ; ++nq) {
+    const int c = nq * 16 + r16;
+    const int token = wave_token0 + c / a.heads_per_tile, head_in_group = hg * a.heads_per_tile + c % a.heads_per_tile;
+    col_valid[nq] = token < t.tokens && c / a.heads_per_tile < a.tokens_per_tile && head_in_group < a.group;
+    col_pos[nq] = t.first_pos + token;
+    col_low[nq] = a.window > 0 ? max(0, col_pos[nq] - a.window + 1) : 0;
+    col_at[nq] = (static_cast<long>(t.first_row + token) * a.q_heads + kvh * a.group + head_in_group) * D;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+      const int dim = kt * 32 + g * 8;
+      qreg[nq][kt] = (col_valid[nq] && dim < D) ? *reinterpret_cast<const uintx4*>(a.q + col_at[nq] + dim) : zero;
+    }
+  }
+  // keys the block looks at
+  const int last_pos = t.first_pos + t.tokens - 1;
+  const int range_lo = a.window > 0 ? max(0, t.first_pos - a.window + 1) : 0;
+  const int range_hi = last_pos;
+
+  // The sum of a column's weights is accumulated by the matrix cores from the weights as they enter the weighted
+  // sum: numerator and denominator carry the same rounding, and no lane has to add its keys up.
+  const uintx4 ones = uintx4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+  float m[NQ];
+  floatx4 l[NQ], o[NQ][DT];
+#pragma unroll
+  for (int nq = 0; nq < NQ; ++nq) {
+    m[nq] = -INFINITY;
+    l[nq] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[nq][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  // ---- the block's loads: pieces of 16 bytes, piece p * 256 + tid ------------------------------------------------------
+  const int* table = a.block_table + static_cast<long>(t.request) * a.table_width;
+  const char* k_bytes = reinterpret_cast<const char*>(a.k_pages);
+  const char* v_bytes = reinterpret_cast<const char*>(a.v_pages);
+  const uint32_t page_bytes = static_cast<uint32_t>(a.kv_heads) * D * 2u << a.page_shift;
+  const uint32_t head_bytes = static_cast<uint32_t>(kvh) * D * 2u << a.page_shift;
+  constexpr int kKeyPieces = 32 * (D / 8), kValuePieces = D * 4;
+  constexpr int PK = (kKeyPieces + 255) / 256, PV = (kValuePieces + 255) / 256;
+  const int run_shift = min(2, a.page_shift - 3);  // aligned runs of 8 keys of this step in one page row: 1, 2 or 4
+  const std::true_type checked{};
+  const std::false_type unchecked{};
+  bool bad = false;
+  // What a thread moves does not change from step to step: which key of the step and which 16 bytes of its row
+  // (keys), which dim and which run of 8 keys (values), which of the step's pages that is, and where the piece goes
+  // in LDS.  What changes - the step's 1, 2 or 4 page ids - is the same for every thread: it is read and checked with
+  // scalar instructions, one step before the loads that need it are issued, so no load waits for the table entry
+  // that addresses it and no lane spends arithmetic on it.
+  const int step_pages = max(1, 32 >> a.page_shift), span = min(32, 1 << a.page_shift);
+  int k_sel[PK], v_sel[PV];             // which of the step's pages holds the piece
+  uint32_t k_from[PK], v_from[PV];      // byte offset inside the page, without what the step's first key adds
+  uint32_t k_to[PK], v_to[PV];          // element offset in the LDS buffer
+  bool k_mine[PK], v_mine[PV];
+#pragma unroll
+  for (int p = 0; p < PK; ++p) {
+    const int c = p * 256 + tid, key = c / (D / 8);
+    k_mine[p] = c < kKeyPieces;
+    k_sel[p] = step_pages == 1 ? 0 : key >> a.page_shift;
+    k_from[p] = head_bytes + (c % (D / 8)) * 16u + static_cast<uint32_t>(key & page_mask) * (D * 2u);
+    k_to[p] = (((key >> 2) & 1) * 16 + (key >> 3) * 4 + (key & 3)) * KROW + (c % (D / 8)) * 8;  // tile j, row rho
+  }
+#pragma unroll
+  for (int p = 0; p < PV; ++p) {
+    const int c = p * 256 + tid;
+    const int run = (c / D) >> run_shift, within = c - ((run * D) << run_shift);
+    const int dim = within >> run_shift, piece = (run << run_shift) + (within & ((1 << run_shift) - 1));
+    v_mine[p] = c < kValuePieces;
+    v_sel[p] = step_pages == 1 ? 0 : (piece * 8) >> a.page_shift;
+    v_from[p] = head_bytes + (static_cast<uint32_t>(dim) << (a.page_shift + 1)) + static_cast<uint32_t>((piece * 8) & page_mask) * 2u;
+    v_to[p] = dim * VROW + piece * 8;
+  }
+  // key of a piece relative to the step's first: only steps at the edge of the range ask, so it is not kept
+  auto k_key = [&](int p) { return (p * 256 + tid) / (D / 8); };
+  auto v_key = [&](int p) {
+    const int c = p * 256 + tid, run = (c / D) >> run_shift, within = c - ((run * D) << run_shift);
+    return ((run << run_shift) + (within & ((1 << run_shift) - 1))) * 8;
+  };
+  // The page ids of the step at `base`.  CHECK: the step may reach outside [range_lo, range_hi]; pages wholly
+  // outside are not looked up (their entries may lie beyond the table).
+  auto page_wanted = [&](int base, int i) {
+    const int first = base + (i << a.page_shift);
+    return first <= range_hi && first + span - 1 >= range_lo;
+  };
+  auto lookup = [&](int base, int (&pages)[4], auto check) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      pages[i] = 0;
+      if (i < step_pages && (!decltype(check)::value || page_wanted(base, i))) pages[i] = table[(base >> a.page_shift) + i];
+    }
+  };
+  auto fetch = [&](int base, const int (&pages)[4], uintx4 (&kst)[PK], uintx4 (&vst)[PV], auto check) {
+    uint32_t at[4];  // byte offset of each of the step's pages
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int page = pages[i];
+      if (i < step_pages && (!decltype(check)::value || page_wanted(base, i)) && (page < 0 || page >= a.num_pages)) {
+        bad = true;
+        page = 0;
+      }
+      at[i] = static_cast<uint32_t>(page) * page_bytes;
+    }
+    auto of = [&](int sel) { return sel == 0 ? at[0] : (sel == 1 ? at[1] : (sel == 2 ? at[2] : at[3])); };
+    const uint32_t in_page = static_cast<uint32_t>(base & page_mask);  // pages of more than 32 tokens: where the step begins
+#pragma unroll
+    for (int p = 0; p < PK; ++p) {
+      bool wanted = k_mine[p];
+      if (decltype(check)::value) {
+        const int key = base + k_key(p);
+        wanted = wanted && key >= range_lo && key <= range_hi;
+      }
+      kst[p] = zero;
+      if (wanted) kst[p] = *reinterpret_cast<const uintx4*>(k_bytes + of(k_sel[p]) + in_page * (D * 2u) + k_from[p]);
+    }
+#pragma unroll
+    for (int p = 0; p < PV; ++p) {
+      int live = 8;
+      bool wanted = v_mine[p];
+      if (decltype(check)::value) {
+        const int key = base + v_key(p);
+        live = min(8, range_hi - key + 1);
+        wanted = wanted && live > 0 && key + 7 >= range_lo;
+      }
+      uintx4 v = zero;
+      if (wanted) {
+        v = *reinterpret_cast<const uintx4*>(v_bytes + of(v_sel[p]) + in_page * 2u + v_from[p]);
+        if (decltype(check)::value && live < 8) {  // slots beyond the last key were never written: anything, NaN included
+          uint32_t keep[4];
+#pragma unroll
+          for (int w = 0; w < 4; ++w) keep[w] = live >= 2 * w + 2 ? 0xffffffffu : (live == 2 * w + 1 ? 0x0000ffffu : 0u);
+          v = uintx4{v.x & keep[0], v.y & keep[1], v.z & keep[2], v.w & keep[3]};
+        }
+      }
+      vst[p] = v;
+    }
+  };
+  auto stash = [&](int buffer, const uintx4 (&kst)[PK], const uintx4 (&vst)[PV]) {
+#pragma unroll
+    for (int p = 0; p < PK; ++p)
+      if (k_mine[p]) *reinterpret_cast<uintx4*>(&k_lds[buffer][k_to[p]]) = kst[p];
+#pragma unroll
+    for (int p = 0; p < PV; ++p)
+      if (v_mine[p]) *reinterpret_cast<uintx4*>(&v_lds[buffer][v_to[p]]) = vst[p];
+  };
+
+  // One step of 32 keys from LDS.  MASK: some column does not see the whole step.
+  auto step = [&](int base, int buffer, auto mask) {
+    floatx4 s[NQ][2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+      for (int nq = 0; nq < NQ; ++nq) s[nq][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) {
+        const bool inside = (D % 32 == 0) || kt * 32 + g * 8 < D;
+        const uintx4 keys = inside ? *reinterpret_cast<const uintx4*>(&k_lds[buffer][(j * 16 + r16) * KROW + kt * 32 + g * 8])
+                                   : zero;
+#pragma unroll
+        for (int nq = 0; nq < NQ; ++nq) s[nq][j] = mfma16(keys, qreg[nq][kt], s[nq][j]);
+      }
+    }
+    uintx4 preg[NQ], plow[NQ];
+    float correction[NQ];
+    bool rescale = false;
+#pragma unroll
+    for (int nq = 0; nq < NQ; ++nq) {
+      if (decltype(mask)::value) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int key = base + g * 8 + j * 4 + i;
+            const bool seen = col_valid[nq] && key <= col_pos[nq] && key >= col_low[nq];
+            if (!seen) s[nq][j][i] = -INFINITY;
+          }
+      }
+      float top = fmaxf(fmaxf(fmaxf(s[nq][0][0], s[nq][0][1]), fmaxf(s[nq][0][2], s[nq][0][3])),
+                        fmaxf(fmaxf(s[nq][1][0], s[nq][1][1]), fmaxf(s[nq][1][2], s[nq][1][3])));
+      top = fmaxf(top, __shfl_xor(top, 16, 64));
+      top = fmaxf(top, __shfl_xor(top, 32, 64));
+      // The reference point of the exponentials follows the maximum lazily: it moves only when the maximum has grown
+      // by more than 2^kLazy, so weights stay below 2^kLazy (harmless in float32 sums, and bfloat16 keeps its relative
+      // precision) and the accumulators are rescaled a few times per row instead of at every step.
+      const float scaled = top * a.scale_log2;                 // the scale is positive: max commutes with it
+      const bool moved = scaled > m[nq] + kLazy;               // also the first keys seen: m is -inf
+      const float m_new = moved ? scaled : m[nq];
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;   // nothing seen yet: every weight is 0, no NaN
+      correction[nq] = moved ? __builtin_amdgcn_exp2f(m[nq] - m_safe) : 1.f;
+      rescale = rescale || moved;
+      m[nq] = m_new;
+      // A weight enters the second product as two bfloat16 numbers (p = high + low, 16 bits of mantissa together),
+      // so that the weighted sum does not carry the 2^-9 relative error of a single bfloat16.
+      uint32_t high[4], low[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        floatx2 p;
+        p[0] = __builtin_amdgcn_exp2f(fmaf(s[nq][e >> 1][(e & 1) * 2], a.scale_log2, -m_safe));
+        p[1] = __builtin_amdgcn_exp2f(fmaf(s[nq][e >> 1][(e & 1) * 2 + 1], a.scale_log2, -m_safe));
+        high[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(p, bf16x2));
+        const floatx2 rest = {p[0] - __uint_as_float(high[e] << 16), p[1] - __uint_as_float(high[e] & 0xffff0000u)};
+        low[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(rest, bf16x2));
+      }
+      preg[nq] = uintx4{high[0], high[1], high[2], high[3]};
+      plow[nq] = uintx4{low[0], low[1], low[2], low[3]};
+    }
+    if (__any(rescale)) {
+#pragma unroll
+      for (int nq = 0; nq < NQ; ++nq) {
+        l[nq] *= correction[nq];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o[nq][dt] *= correction[nq];
+      }
+    }
+    // O^T += V^T . P^T, and the weights' sums from the same two-part weights: a row of ones beside the value rows
+#pragma unroll
+    for (int nq = 0; nq < NQ; ++nq) l[nq] = mfma16(ones, plow[nq], mfma16(ones, preg[nq], l[nq]));
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const uintx4 values = *reinterpret_cast<const uintx4*>(&v_lds[buffer][(dt * 16 + r16) * VROW + g * 8]);
+#pragma unroll
+      for (int nq = 0; nq < NQ; ++nq) o[nq][dt] = mfma16(values, plow[nq], mfma16(values, preg[nq], o[nq][dt]));
+    }
+  };
+
+  uintx4 kst[PK], vst[PV];
+  int pages[4];
+  const int first_base = range_lo & ~31;
+  auto inside = [&](int base) { return base >= range_lo && base + 31 <= range_hi; };
+  auto lookup_step = [&](int base) {
+    if (inside(base)) lookup(base, pages, unchecked);
+    else lookup(base, pages, checked);
+  };
+  auto fetch_step = [&](int base) {
+    if (inside(base)) fetch(base, pages, kst, vst, unchecked);
+    else fetch(base, pages, kst, vst, checked);
+  };
+  lookup_step(first_base);
+  fetch_step(first_base);
+  if (first_base + 32 <= range_hi) lookup_step(first_base + 32);
+  stash(0, kst, vst);
+  __syncthreads();
+  int buffer = 0;
+  for (int base = first_base; base <= range_hi; base += 32, buffer ^= 1) {
+    const bool more = base + 32 <= range_hi;
+    if (more) fetch_step(base + 32);
+    if (base + 64 <= range_hi) lookup_step(base + 64);
+    // the wave's tokens see some key of this step
+    if (wave_active && base <= wave_last_pos && (a.window == 0 || base + 31 >= wave_first_pos - a.window + 1)) {
+      const bool whole = base >= range_lo && base + 31 <= wave_first_pos &&
+                         (a.window == 0 || base >= wave_last_pos - a.window + 1);
+      if (whole) step(base, buffer, unchecked);
+      else step(base, buffer, checked);
+    }
+    if (more) stash(buffer ^ 1, kst, vst);
+    __syncthreads();
+  }
+  if (bad) bad_page = 1;
+  __syncthreads();
+  const bool poisoned = bad_page != 0;
+  const float nan = __uint_as_float(0x7fc00000u);
+#pragma unroll
+  for (int nq = 0; nq < NQ; ++nq) {
+    if (!col_valid[nq]) continue;
+    const float inv = poisoned ? nan : 1.f / l[nq][0];  // every row of the ones tile holds the column's sum
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      uintx2 packed;
+      packed.x = bf16_bits(o[nq][dt][0] * inv) | (static_cast<uint32_t>(bf16_bits(o[nq][dt][1] * inv)) << 16);
+      packed.y = bf16_bits(o[nq][dt][2] * inv) | (static_cast<uint32_t>(bf16_bits(o[nq][dt][3] * inv)) << 16);
+      *reinterpret_cast<uintx2*>(a.out + col_at[nq] + dt * 16 + g * 4) = packed;
+    }
+  }
+}
+
 // Merge of the segments' partial results: out = sum_z 2^(m_z - M) O_z / sum_z 2^(m_z - M) l_z, M = max_z m_z
 // (csrc/paged_decode.cu:528-544 of the reference has the same rule in base e).  One wave per (tile, head group,
 // column); a lane owns dims lane, lane + 64, ...; the segments are summed in ascending order.
 template <int NQ>
 __global__ __launch_bounds__(64) void attention_merge_kernel(const Args a) {
-  const Tile t = find_tile(a, blockIdx.x);
+  const Tile t = find_tile(a, blockIdx.x, a.tokens_per_tile);
   if (!t.found) return;
   const int kvh = blockIdx.y / a.head_groups, hg = blockIdx.y % a.head_groups;
   const int c = blockIdx.z, lane = threadIdx.x;
@@ -478,8 +802,15 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(const Args a) {
 }
 
 template <int NQ>
-int launch(const Args& a, int tiles, hipStream_t stream) {
+int launch(const Args& a, int tiles, bool shared, hipStream_t stream) {
   dim3 grid(tiles, a.kv_heads * a.head_groups, a.num_splits);
+  if (shared) {
+    if constexpr (NQ == 1) {  // one tile of 16 columns per wave: three blocks fit a compute unit
+      attention_shared_kernel<1><<<dim3(tiles * a.kv_heads * a.head_groups), 64 * kSharedWaves, 0, stream>>>(a);
+      return AKV_LAUNCH_STATUS();
+    }
+    return -2;
+  }
   if (a.num_splits == 1) grid.x = (tiles + 1) / 2;  // a block takes a late tile and an early one
   if (a.num_splits > 1) {
     attention_mfma_kernel<NQ, true, true><<<grid, 64, 0, stream>>>(a);
@@ -500,17 +831,19 @@ int launch(const Args& a, int tiles, hipStream_t stream) {
 // 16 * nq query columns; `tiles` is the number of tiles over those requests (sum of ceil(tokens / tokens_per_tile));
 // with num_splits > 1 `partial` must hold tiles * kv_heads * head_groups * num_splits * 16 * nq * (D + 4) floats.
 // page_size must be a power of two, at least 4.  `single_tokens` says that every request brings exactly one token.
+// `shared`: blocks of four waves that share keys and values through LDS; `tiles` then counts tiles of
+// 4 * tokens_per_tile tokens, nq and num_splits must be 1 and pages hold at least 8 tokens.
 extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
     const void* q, const void* k_pages, const void* v_pages, void* out, float* partial, const int* q_start,
     const int* seq_lens, const int* block_table, int table_width, int seq_first, int seq_count, int tiles, int nq,
     int q_heads, int kv_heads, int heads_per_tile, int head_groups, int tokens_per_tile, int page_size, long num_pages,
-    float scale, int window, int seg_keys, int num_splits, int single_tokens, hipStream_t stream) {
+    float scale, int window, int seg_keys, int num_splits, int single_tokens, int shared, hipStream_t stream) {
   if (tiles <= 0 || seq_count <= 0) return 0;
   int page_shift = 0;
   while ((1 << page_shift) < page_size) ++page_shift;
   if (page_size < 4 || (1 << page_shift) != page_size || q_heads % kv_heads != 0 ||
       heads_per_tile * tokens_per_tile > 16 * nq || kv_heads * head_groups > 65535 || num_splits > 65535 ||
-      num_splits < 1 || (single_tokens && tiles != seq_count))
+      num_splits < 1 || (single_tokens && tiles != seq_count) || (shared && (page_size < 8 || num_splits != 1 || nq != 1)))
     return -2;
   Args a;
   a.q = static_cast<const bf16_t*>(q);
@@ -538,9 +871,22 @@ extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
   a.window = window;
   a.seg_keys = seg_keys;
   a.num_splits = num_splits;
+  a.units = 1;
+  if (shared) {
+    static int units_of[64] = {0};  // compute units per device, asked once
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return -3;
+    if (units_of[device] == 0) {
+      int count = 0;
+      if (hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count <= 0) return -3;
+      units_of[device] = count;
+    }
+    a.units = units_of[device];
+    if (static_cast<long>(tiles) * kv_heads * head_groups > 0x7fffffffL) return -2;
+  }
   switch (nq) {
-    case 1: return launch<1>(a, tiles, stream);
-    case 2: return launch<2>(a, tiles, stream);
+    case 1: return launch<1>(a, tiles, shared != 0, stream);
+    case 2: return launch<2>(a, tiles, shared != 0, stream);
     default: return -2;
   }
 }

@@ -97,6 +97,7 @@ class HipKernels:
         self.decode_wave_target = 2048  # decode attention cuts the keys until about this many waves are at work,
         self.decode_min_segment = 128   # but into segments no shorter than this many keys
         self.decode_max_splits = 32     # and no more than this many (the merge walks them one after the other)
+        self.share_prompt_tiles = True  # prompt portions: blocks of four waves share keys and values through LDS
         for name in ("akv_embed", "akv_add_rmsnorm", "akv_rmsnorm_rows", "akv_copy_rows", "akv_gather_rows",
                      "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
                      "akv_linear_tiled", "akv_linear_packed", "akv_linear_packed_swiglu", "akv_attention_rows", "akv_sample"):
@@ -345,16 +346,18 @@ class HipKernels:
         return self._attention_entry[head_dim]
 
     def _attention_mfma(self, q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out,
-                        page_size, num_pages, seq_first, seq_count, nq, split):
+                        page_size, num_pages, seq_first, seq_count, nq, split, shared=False):
         """Requests seq_first .. seq_first + seq_count - 1 of the step on the MFMA kernel, in tiles of 16 * nq
         (token, head-of-group) columns; `split` says that each of them brings one token (decode) and cuts the keys
-        over several waves."""
+        over several waves; `shared` (prompt portions, pages of 8 tokens and more) lets blocks of four waves, four
+        tiles, fetch every key and value once into LDS."""
         group = q_heads // kv_heads
         heads_per_tile = min(group, 16 * nq)
         head_groups = (group + heads_per_tile - 1) // heads_per_tile
         tokens_per_tile = (16 * nq) // heads_per_tile
         starts = ctx.host_q_start
-        tiles = sum((starts[r + 1] - starts[r] + tokens_per_tile - 1) // tokens_per_tile
+        per_tile = tokens_per_tile * (4 if shared else 1)
+        tiles = sum((starts[r + 1] - starts[r] + per_tile - 1) // per_tile
                     for r in range(seq_first, seq_first + seq_count))
         num_splits, seg_keys, partial = 1, 0, None
         if split:
@@ -374,7 +377,8 @@ class HipKernels:
             _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial), _ptr(ctx.q_start), _ptr(ctx.seq_lens),
             _ptr(meta.block_table), meta.width, seq_first, seq_count, tiles, nq, q_heads, kv_heads, heads_per_tile,
             head_groups, tokens_per_tile, page_size, ctypes.c_long(num_pages), ctypes.c_float(scale),
-            int(window) if window is not None else 0, seg_keys, num_splits, 1 if split else 0, self._stream()),
+            int(window) if window is not None else 0, seg_keys, num_splits, 1 if split else 0, 1 if shared else 0,
+            self._stream()),
             "attention")
 
     def attention(self, q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out):
@@ -397,7 +401,9 @@ class HipKernels:
             if decodes:      # single tokens against long histories: one small tile each, keys split over waves
                 self._attention_mfma(*common, 0, decodes, 1, True)
             if ctx.num_seqs > decodes:
-                self._attention_mfma(*common, decodes, ctx.num_seqs - decodes, 2 if head_dim <= 128 else 1, False)
+                shared = page_size >= 8 and self.share_prompt_tiles
+                nq = 1 if shared or head_dim > 128 else 2
+                self._attention_mfma(*common, decodes, ctx.num_seqs - decodes, nq, False, shared=shared)
             return
         self._dense(ctx.seq_of_token, "seq_of_token", torch.int32, (tokens,))
         self._dense(ctx.positions, "positions", torch.int32, (tokens,))
