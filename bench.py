@@ -9,7 +9,8 @@ not change the time a step takes).  One JSON line is printed:
   value     decoded tokens per second at the default batch
   prefill   one request's 2,048-token prompt fed whole: tokens/s, ms, and flops / time / bf16 MFMA peak
   roofline  bytes a decode step has to read (every weight once + the live requests' cache) / its time / HBM peak
-  points    decoded tokens per second at batch 1 and 64
+  points    decoded tokens per second at batch 1 and 64; prefill tokens per second with every product in the engine's
+            own kernels (by default bfloat16 products of more than 16 rows go to the BLAS library)
 Peaks are MI355X's published ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s.
 """
 
@@ -134,7 +135,8 @@ def main() -> int:
                    "kv_heads": config.num_key_value_heads, "head_dim": config.head_dim,
                    "intermediate": config.intermediate_size, "vocab": config.vocab_size, "page_size": PAGE_SIZE,
                    "prefill_tokens": PREFILL_TOKENS, "rope_theta": config.rope_theta, "rms_norm_eps": config.rms_norm_eps,
-                   "tied_embeddings": config.tie_word_embeddings},
+                   "tied_embeddings": config.tie_word_embeddings,
+                   "library_products_above_rows": engine.config.library_products_above},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
     }
@@ -153,6 +155,10 @@ def main() -> int:
         flops += 2 * config.vocab_size * config.hidden_size                     # the head on the one wanted row
         record["prefill"] = {"value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS,
                              "ms": round(seconds * 1000, 3), "frac": round(flops / seconds / BF16_PEAK_FLOPS, 4)}
+        if points and engine.kernels.library_products_above is not None:
+            kept, engine.kernels.library_products_above = engine.kernels.library_products_above, None
+            record["points"]["prefill_own_products"] = round(PREFILL_TOKENS / prefill(), 1)
+            engine.kernels.library_products_above = kept
     print(json.dumps(record))
     return 0
 
