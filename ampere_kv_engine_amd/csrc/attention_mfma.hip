@@ -183,8 +183,8 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
   const int* table = a.block_table + static_cast<long>(t.request) * a.table_width;
   const int key_in_step = (r16 >> 2) * 8 + (r16 & 3);  // + j * 4: this lane's key row of tile j
 
-  // Addresses are 32-bit byte offsets from the page tensors (the host refuses tensors of 4 GB and more), so that a
-  // load is one instruction on a scalar base and a lane offset instead of 64-bit arithmetic per lane.
+  // A page's byte offset is 64-bit (pools of many gigabytes); what is added inside a page fits 32 bits and is
+  // prepared once per lane.
   const char* k_bytes = reinterpret_cast<const char*>(a.k_pages);
   const char* v_bytes = reinterpret_cast<const char*>(a.v_pages);
   const uint32_t page_bytes = static_cast<uint32_t>(a.kv_heads) * D * 2u << a.page_shift;  // one page, all kv heads
@@ -208,7 +208,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
           page = 0;
         }
       }
-      const uint32_t at = static_cast<uint32_t>(page) * page_bytes + k_lane + static_cast<uint32_t>(key & page_mask) * (D * 2u);
+      const size_t at = static_cast<size_t>(page) * page_bytes + (k_lane + static_cast<uint32_t>(key & page_mask) * (D * 2u));
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) {
         const bool inside = (D % 32 == 0) || kt * 32 + g * 8 < D;
@@ -226,14 +226,14 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
         poisoned = true;
         page = 0;
       }
-      const uint32_t at = static_cast<uint32_t>(page) * page_bytes + v_lane + static_cast<uint32_t>(key & page_mask) * 2u;
+      const size_t at = static_cast<size_t>(page) * page_bytes + (v_lane + static_cast<uint32_t>(key & page_mask) * 2u);
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) dst[dt] = *reinterpret_cast<const uintx4*>(v_bytes + at + dt * v_tile);
       return;
     }
     const int live = min(8, range_hi - key + 1);
     bool have[2] = {false, false};
-    uint32_t at[2] = {0u, 0u};
+    size_t at[2] = {0u, 0u};
     if (live > 0 && key + 7 >= range_lo) {
       // pages of 8 and more hold the 8 keys together; pages of 4 hold them in two pages
 #pragma unroll
@@ -245,7 +245,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
         if (page < 0 || page >= a.num_pages) poisoned = true;
         else {
           have[half] = true;
-          at[half] = static_cast<uint32_t>(page) * page_bytes + v_lane + static_cast<uint32_t>(first & page_mask) * 2u;
+          at[half] = static_cast<size_t>(page) * page_bytes + (v_lane + static_cast<uint32_t>(first & page_mask) * 2u);
         }
       }
     }
@@ -558,7 +558,7 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
     }
   };
   auto fetch = [&](int base, const int (&pages)[4], uintx4 (&kst)[PK], uintx4 (&vst)[PV], auto check) {
-    uint32_t at[4];  // byte offset of each of the step's pages
+    size_t at[4];  // byte offset of each of the step's pages
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       int page = pages[i];
@@ -566,7 +566,7 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
         bad = true;
         page = 0;
       }
-      at[i] = static_cast<uint32_t>(page) * page_bytes;
+      at[i] = static_cast<size_t>(page) * page_bytes;
     }
     auto of = [&](int sel) { return sel == 0 ? at[0] : (sel == 1 ? at[1] : (sel == 2 ? at[2] : at[3])); };
     const uint32_t in_page = static_cast<uint32_t>(base & page_mask);  // pages of more than 32 tokens: where the step begins

@@ -389,8 +389,7 @@ class HipKernels:
         self._dense(meta.block_table, "block_table", torch.int32, (ctx.num_seqs, meta.width))
         if ctx.max_seq_len > meta.width * page_size:
             raise KernelError(f"a request of {ctx.max_seq_len} tokens does not fit a block table of {meta.width} pages")
-        small = k_pages.numel() * k_pages.element_size() < 2 ** 32       # the kernel addresses pages with 32 bits
-        if q.dtype == torch.bfloat16 and page_size >= 4 and page_size & (page_size - 1) == 0 and small:
+        if q.dtype == torch.bfloat16 and page_size >= 4 and page_size & (page_size - 1) == 0:
             self._dense(ctx.q_start, "q_start", torch.int32, (ctx.num_seqs + 1,))
             self._dense(ctx.seq_lens, "seq_lens", torch.int32, (ctx.num_seqs,))
             if ctx.host_q_start[ctx.num_seqs] != tokens or len(ctx.host_seq_lens) != ctx.num_seqs:

@@ -438,6 +438,29 @@ def test_attention_decodes_beside_portions(hip, ref):
     torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(torch.bfloat16))
 
 
+def test_attention_over_a_pool_of_more_than_4_gb(hip, ref):
+    """The request's pages lie at the end of a pool whose key tensor alone has 4.6 GB: page offsets need 64 bits.
+    One single token (split-key kernel) and one prompt portion (shared-tile kernel)."""
+    q_heads, kv_heads, dim, page_size = 8, 8, 128, 16
+    portions = [(300, 1), (0, 150)]
+    q, k_pages, v_pages, ctx, meta, _, _ = _attention_case(torch.bfloat16, q_heads, kv_heads, dim, page_size, portions, None, 29)
+    ctx.num_decode_seqs = 1
+    want = torch.empty_like(q)
+    ref.attention(q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, dim, dim ** -0.5, None, want)
+    pool = 140_000                                     # x 32 KB per page and tensor
+    shift = pool - k_pages.shape[0]
+    k_big = torch.empty((pool, kv_heads, page_size, dim), dtype=torch.bfloat16, device="cuda")
+    v_big = torch.empty((pool, kv_heads, dim, page_size), dtype=torch.bfloat16, device="cuda")
+    assert k_big.numel() * 2 > 2 ** 32
+    k_big[shift:] = k_pages.cuda()
+    v_big[shift:] = v_pages.cuda()
+    cctx, cmeta = _to_cuda(ctx, meta)
+    cmeta.block_table = torch.where(cmeta.block_table >= 0, cmeta.block_table + shift, cmeta.block_table)
+    got = torch.full_like(q, float("nan"), device="cuda")
+    hip.attention(q.cuda(), k_big, v_big, cctx, cmeta, q_heads, kv_heads, dim, dim ** -0.5, None, got)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(torch.bfloat16))
+
+
 def test_attention_poisons_a_foreign_page(hip):
     """A table entry inside a request's length that is no page of the pool gives NaN, not a read outside the pool."""
     portions = [(40, 1), (40, 5)]
