@@ -44,14 +44,27 @@ __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ 
   const uint32_t draw = t > 0.f ? draws[row] : 0u;
   float value = -INFINITY;
   int index = vocab;  // "none yet"; any real index is lower
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-    float score = x[i];
-    if (t > 0.f) {
-      const uint32_t bits = philox_first(static_cast<uint32_t>(i), draw, k0, k1);
-      const float u = (static_cast<float>(bits >> 8) + 0.5f) * 0x1p-24f;
-      score = score / t - logf(-logf(u));
+  // eight loads of a thread are on their way before the first is looked at; ids still ascend per thread, so the
+  // first maximum stays
+  constexpr int kAhead = 8;
+  for (int i0 = threadIdx.x; i0 < vocab; i0 += kAhead * blockDim.x) {
+    float fetched[kAhead];
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      const int i = i0 + u * blockDim.x;
+      fetched[u] = i < vocab ? x[i] : -INFINITY;
     }
-    if (score > value) { value = score; index = i; }  // ascending i per thread: the first maximum stays
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      const int i = i0 + u * blockDim.x;
+      float score = fetched[u];
+      if (t > 0.f && i < vocab) {
+        const uint32_t bits = philox_first(static_cast<uint32_t>(i), draw, k0, k1);
+        const float u01 = (static_cast<float>(bits >> 8) + 0.5f) * 0x1p-24f;
+        score = score / t - logf(-logf(u01));
+      }
+      if (i < vocab && score > value) { value = score; index = i; }
+    }
   }
   for (int offset = kWave / 2; offset > 0; offset >>= 1) {
     const float other_value = __shfl_xor(value, offset, kWave);
