@@ -349,6 +349,16 @@ __global__ __launch_bounds__(256, 2) void linear_wide_kernel(const bf16_t* __res
     for (int m = 0; m < MW; ++m)
 #pragma unroll
       for (int n = 0; n < 4; ++n) acc[n][m] = mfma16(a[n], b[m], acc[n][m]);
+    // Order for the instruction scheduler: two operand reads from LDS go out first, then every group of 4 matrix
+    // instructions is followed by the read of the operand two groups ahead, so that the matrix pipe does not wait for
+    // LDS (left alone, the scheduler puts every read right before its use).
+    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+#pragma unroll
+    for (int m = 0; m < MW - 2; ++m) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
   };
 
   if constexpr (MW <= 4) {
