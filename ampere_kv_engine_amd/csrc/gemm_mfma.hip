@@ -115,20 +115,40 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
     auto fetch = [&](int kt, uintx4 (&a)[RT][U], uintx4 (&b)[MT][U]) {
       const char* w_at = w_wave + static_cast<size_t>(kt) * 1024;
       const char* x_at = x_bytes + static_cast<size_t>(kt) * 64;
+      if (kt + U <= kt1 && row_tile + RT <= n_tiles) {  // the whole group exists: no test per load
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt)
+        for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-        for (int u = 0; u < U; ++u)
-          a[rt][u] = (kt + u < kt1 && row_tile + rt < n_tiles)
-                         ? load_once(reinterpret_cast<const uintx4*>(w_at + rt * w_tile_row + w_lane + u * 1024u)) : zero;
+          for (int u = 0; u < U; ++u)
+            a[rt][u] = load_once(reinterpret_cast<const uintx4*>(w_at + rt * w_tile_row + w_lane + u * 1024u));
+      } else {
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
+        for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const bool inside = !ragged || (kt + u) * 32 + g * 8 < k;
-          b[mt][u] = (kt + u < kt1 && x_row[mt] && inside)
-                         ? *reinterpret_cast<const uintx4*>(x_at + x_lane[mt] + u * 64u) : zero;
+          for (int u = 0; u < U; ++u)
+            a[rt][u] = (kt + u < kt1 && row_tile + rt < n_tiles)
+                           ? load_once(reinterpret_cast<const uintx4*>(w_at + rt * w_tile_row + w_lane + u * 1024u)) : zero;
+      }
+      if (kt + U <= kt1 && !ragged) {  // one test per row tile of x instead of one per load
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+          for (int u = 0; u < U; ++u) b[mt][u] = zero;
+          if (x_row[mt]) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) b[mt][u] = *reinterpret_cast<const uintx4*>(x_at + x_lane[mt] + u * 64u);
+          }
         }
+      } else {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int u = 0; u < U; ++u) {
+            const bool inside = !ragged || (kt + u) * 32 + g * 8 < k;
+            b[mt][u] = (kt + u < kt1 && x_row[mt] && inside)
+                           ? *reinterpret_cast<const uintx4*>(x_at + x_lane[mt] + u * 64u) : zero;
+          }
+      }
     };
     auto multiply = [&](const uintx4 (&a)[RT][U], const uintx4 (&b)[MT][U]) {
 #pragma unroll
