@@ -12,6 +12,11 @@ not change the time a step takes).  One JSON line is printed:
   points    decoded tokens per second at batch 1 and 64; prefill tokens per second with every product in the engine's
             own kernels (by default bfloat16 products of more than 16 rows go to the BLAS library)
 Peaks are MI355X's published ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s.
+
+Two further workloads run through the scheduler and print a line of their own (`--workload`):
+  serving-14b   Qwen3-14B layer sizes: 32 requests, prompt lengths uniform in [128, 4096], 256 tokens each,
+                prompts fed in portions of at most 2,048 tokens beside the decoding requests
+  batch-32b     Qwen3-32B layer sizes: 16 requests with 8,192-token prompts, 128 greedy tokens each
 """
 
 from __future__ import annotations
@@ -29,8 +34,58 @@ sys.path.insert(0, ROOT)
 QWEN3_8B = dict(architectures=["Qwen3ForCausalLM"], num_hidden_layers=36, hidden_size=4096, num_attention_heads=32,
                 num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=151936, rope_theta=1000000.0,
                 rms_norm_eps=1e-6, tie_word_embeddings=False, hidden_act="silu")
+# BASELINE.json configs[3] and configs[4]: the layer sizes of the two larger dense models
+QWEN3_14B = dict(QWEN3_8B, num_hidden_layers=40, hidden_size=5120, num_attention_heads=40, intermediate_size=17408)
+QWEN3_32B = dict(QWEN3_8B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, intermediate_size=25600)
 PAGE_SIZE, CONTEXT, PREFILL_TOKENS = 16, 8192, 2048
 HBM_PEAK_GBS, BF16_PEAK_FLOPS = 8000.0, 2.5e15
+
+
+def scheduler_workload(name: str, layers: int | None) -> int:
+    """A fixed set of requests through the scheduler, from submission to the last token; one JSON line."""
+    import torch
+    from ampere_kv_engine_amd.config import EngineConfig, Qwen3Config
+    from ampere_kv_engine_amd.engine import Engine
+    from ampere_kv_engine_amd.engine.scheduler import Scheduler
+
+    generator = torch.Generator().manual_seed(0)
+    if name == "serving-14b":
+        raw, new_tokens = QWEN3_14B, 256
+        prompts = torch.randint(128, 4097, (32,), generator=generator).tolist()
+    else:
+        raw, new_tokens = QWEN3_32B, 128
+        prompts = [8192] * 16
+    raw = dict(raw, num_hidden_layers=layers or raw["num_hidden_layers"])
+    config = Qwen3Config.from_dict(raw)
+    longest = max(prompts) + new_tokens
+    pages = sum((p + new_tokens + 2 * PAGE_SIZE) // PAGE_SIZE for p in prompts) + 8
+    engine = Engine.from_random(config, seed=0, engine_config=EngineConfig(
+        dtype="bfloat16", page_size=PAGE_SIZE, num_pages=pages, max_seqs=len(prompts),
+        max_batched_tokens=PREFILL_TOKENS + len(prompts), max_seq_len=longest + PAGE_SIZE, device="cuda:0"))
+    samples = []
+    for run in range(3):                                    # the first run warms up (graphs are recorded in it)
+        scheduler = Scheduler(engine, prefill_chunk_size=PREFILL_TOKENS)
+        ids = [torch.randint(0, config.vocab_size, (p,), generator=generator).tolist() for p in prompts]
+        torch.cuda.synchronize(engine.device)
+        started = time.perf_counter()
+        requests = [scheduler.submit(f"{run}_{i}", tokens, max_new_tokens=new_tokens, ignore_eos=True)
+                    for i, tokens in enumerate(ids)]
+        scheduler.run_until_idle()
+        torch.cuda.synchronize(engine.device)
+        if run:
+            samples.append(time.perf_counter() - started)
+        assert all(len(r.output_ids) == new_tokens for r in requests)
+        assert engine.cache.num_free_pages == [pages]
+    seconds = sorted(samples)[len(samples) // 2]
+    print(json.dumps({
+        "workload": name, "seconds": round(seconds, 3), "samples": [round(x, 3) for x in samples],
+        "output_tok_per_s": round(len(prompts) * new_tokens / seconds, 1),
+        "all_tok_per_s": round((sum(prompts) + len(prompts) * new_tokens) / seconds, 1),
+        "requests": len(prompts), "prompt_tokens": sum(prompts), "new_tokens_each": new_tokens,
+        "rounds": scheduler.rounds, "layers": raw["num_hidden_layers"], "hidden": config.hidden_size,
+        "q_heads": config.num_attention_heads, "intermediate": config.intermediate_size, "dtype": "bf16",
+        "data": "synthetic: random-init weights, uniform random token ids"}))
+    return 0
 
 
 def main() -> int:
@@ -45,10 +100,15 @@ def main() -> int:
     parser.add_argument("--points", default="1,64", help="further batch sizes to time (comma separated, '' for none)")
     parser.add_argument("--no-prefill", action="store_true")
     parser.add_argument("--prefill-only", action="store_true", help="time the prefill alone (for kernel profiles)")
+    parser.add_argument("--workload", choices=["decode", "serving-14b", "batch-32b"], default="decode",
+                        help="decode: the headline measurement; the others run a set of requests through the scheduler")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this engine has no multi-GPU path, run it with --gpus 1")
         return 2
+
+    if args.workload != "decode":
+        return scheduler_workload(args.workload, args.layers if args.layers != QWEN3_8B["num_hidden_layers"] else None)
 
     import torch
     from ampere_kv_engine_amd.config import EngineConfig, Qwen3Config
