@@ -26,9 +26,8 @@ __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ 
 
 // ---- residual add + RMSNorm: stream += delta (float32); out = T( T(stream * rsqrt(mean^2 + eps)) * w ) ----
 // One block per row.  A thread owns groups of 4 consecutive elements (16-byte accesses); a row of up to
-// 256 * 4 * kRowGroups elements stays in registers between the sum of squares and the scaling, longer rows are
-// read a second time.
-constexpr int kRowGroups = 4;
+// 256 * 4 * GROUPS elements (GROUPS = 4, 8 or 16: rows up to 16,384 wide) stays in registers between the sum of
+// squares and the scaling, longer rows are read a second time.
 
 template <typename T> __device__ __forceinline__ float4 load4(const T* p);
 template <> __device__ __forceinline__ float4 load4<float>(const float* p) { return *reinterpret_cast<const float4*>(p); }
@@ -46,7 +45,7 @@ template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float4 v) 
   *reinterpret_cast<uint2*>(p) = packed;
 }
 
-template <typename T>
+template <typename T, int GROUPS>
 __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ stream, const T* __restrict__ delta,
                                                           const float* __restrict__ weight, float eps,
                                                           T* __restrict__ out, int hidden) {
@@ -55,10 +54,10 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ st
   float* s = stream + base;
   T* o = out + base;
   float acc = 0.f;
-  if ((hidden & 3) == 0 && hidden <= 256 * 4 * kRowGroups) {
-    float4 kept[kRowGroups];
+  if ((hidden & 3) == 0 && hidden <= 256 * 4 * GROUPS) {
+    float4 kept[GROUPS];
 #pragma unroll
-    for (int j = 0; j < kRowGroups; ++j) {
+    for (int j = 0; j < GROUPS; ++j) {
       const int i = (j * 256 + threadIdx.x) * 4;
       if (i < hidden) {
         float4 v = load4<float>(s + i);
@@ -71,15 +70,15 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ st
         acc += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
       }
     }
-    float4 gain[kRowGroups];  // asked for before the sum, so that they arrive while it is formed
+    float4 gain[GROUPS];  // asked for before the sum, so that they arrive while it is formed
 #pragma unroll
-    for (int j = 0; j < kRowGroups; ++j) {
+    for (int j = 0; j < GROUPS; ++j) {
       const int i = (j * 256 + threadIdx.x) * 4;
       if (i < hidden) gain[j] = load4<float>(weight + i);
     }
     const float scale = rsqrtf(block_sum(acc, scratch) / static_cast<float>(hidden) + eps);
 #pragma unroll
-    for (int j = 0; j < kRowGroups; ++j) {
+    for (int j = 0; j < GROUPS; ++j) {
       const int i = (j * 256 + threadIdx.x) * 4;
       if (i < hidden) {
         const float4 v = kept[j], w = gain[j];
@@ -347,9 +346,16 @@ int akv_embed(const int* ids, const void* table, int table_dtype, float* out, in
 int akv_add_rmsnorm(float* stream_buf, const void* delta, const float* weight, float eps, void* out, int dtype,
                     int tokens, int hidden, hipStream_t stream) {
   if (tokens <= 0) return 0;
-  AKV_DISPATCH(dtype, T,
-               add_rmsnorm_kernel<T><<<tokens, 256, 0, stream>>>(stream_buf, static_cast<const T*>(delta), weight, eps,
-                                                                 static_cast<T*>(out), hidden));
+  if (hidden <= 4096) {
+    AKV_DISPATCH(dtype, T, (add_rmsnorm_kernel<T, 4><<<tokens, 256, 0, stream>>>(
+                               stream_buf, static_cast<const T*>(delta), weight, eps, static_cast<T*>(out), hidden)));
+  } else if (hidden <= 8192) {
+    AKV_DISPATCH(dtype, T, (add_rmsnorm_kernel<T, 8><<<tokens, 256, 0, stream>>>(
+                               stream_buf, static_cast<const T*>(delta), weight, eps, static_cast<T*>(out), hidden)));
+  } else {
+    AKV_DISPATCH(dtype, T, (add_rmsnorm_kernel<T, 16><<<tokens, 256, 0, stream>>>(
+                               stream_buf, static_cast<const T*>(delta), weight, eps, static_cast<T*>(out), hidden)));
+  }
   return AKV_LAUNCH_STATUS();
 }
 

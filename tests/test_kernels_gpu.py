@@ -67,7 +67,7 @@ def test_embed(hip, ref, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("hidden", [96, 1000, 4096])
+@pytest.mark.parametrize("hidden", [96, 1000, 4096, 5120, 8192, 10240, 16388, 18000])
 def test_add_rmsnorm(hip, ref, dtype, hidden):
     stream = rand(7, hidden, seed=2, scale=3.0)
     delta = rand(7, hidden, dtype=dtype, seed=3)
