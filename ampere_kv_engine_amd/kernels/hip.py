@@ -74,12 +74,18 @@ def _ptr(t: torch.Tensor | None):
 
 class HipKernels:
     name = "hip-gfx950"
+    OWN_SKINNY_ROWS = 64            # the most rows the engine's own decode product takes
 
-    def __init__(self, device: torch.device | str = "cuda:0", library_products_above: int | None = 16):
-        """`library_products_above`: bfloat16 products of more rows than this go to the BLAS library (torch.mm),
+    def __init__(self, device: torch.device | str = "cuda:0", library_products_above: int | None = 16,
+                 tune_products: bool = True):
+        """`library_products_above`: bfloat16 products of more rows than this may go to the BLAS library (torch.mm),
         which then needs the matrices row-major beside their packing; None keeps the packing alone and every
-        product in this library's own kernels."""
+        product in this library's own kernels.  `tune_products`: up to 64 rows the faster of the two is found out
+        once per matrix shape; False sends every product above the limit to the library."""
         self.library_products_above = library_products_above
+        self.tune_products = tune_products     # 17..64 rows: own kernel or library, whichever is faster for the shape
+        self._tuned = {}                       # (kind, outs, k, row tiles) -> "own" | "library"
+        self._spacer = None                    # the buffer whose fill precedes every timed run
         self.device = torch.device(device)
         if self.device.type == "cuda" and self.device.index is None:
             self.device = torch.device("cuda", 0)
@@ -210,17 +216,55 @@ class HipKernels:
         return (row_major is not None and self.library_products_above is not None
                 and rows > self.library_products_above and out.dtype == torch.bfloat16)
 
+    def _own_or_library(self, key: tuple, rows: int, own, library) -> None:
+        """A product that may go to the library.  More than 64 rows: it does.  Up to 64 rows (the range of the skinny
+        kernel, where neither side wins for every shape): whichever of the two is faster for a matrix of this shape
+        and this many tiles of 16 rows, found out at the first such call (never while a graph is recorded) and
+        remembered.  Each is timed twice on the device; before every timed run reads of 256 MB empty the caches, as
+        the other layers' weights do in a real step, and keep the device busy while the host queues the run, so that
+        the host's launch time is not part of what is measured."""
+        if rows > self.OWN_SKINNY_ROWS or not self.tune_products:
+            library()
+            return
+        key = (*key, (rows + 15) // 16)
+        choice = self._tuned.get(key)
+        if choice is None:
+            if torch.cuda.is_current_stream_capturing():
+                library()
+                return
+            if self._spacer is None:
+                self._spacer = torch.zeros(64 << 20, dtype=torch.float32, device=self.device)
+            timed = {"own": [], "library": []}
+            for _ in range(2):
+                for name, run in (("own", own), ("library", library)):
+                    for _ in range(4):      # ~0.25 ms of device work: more than the host needs to queue what follows
+                        self._spacer.sum()  # (reads: nothing is left to be written back while the run is timed)
+                    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    start.record()
+                    run()
+                    end.record()
+                    timed[name].append((start, end))
+            torch.cuda.synchronize(self.device)
+            best = {name: min(a.elapsed_time(b) for a, b in pairs) for name, pairs in timed.items()}
+            choice = self._tuned[key] = "own" if best["own"] <= best["library"] else "library"
+        (own if choice == "own" else library)()
+
     def linear(self, x, weight, out):
         if isinstance(weight, PackedWeight):
             rows, k = x.shape
             self._dense(x, "x", torch.bfloat16, (rows, weight.k))
             self._dense(out, "out", None, (rows, weight.outs))
-            if self._library_product(rows, weight.row_major, out):
-                torch.mm(x, weight.row_major.t(), out=out)
-                return
             self._dense(weight.data, "packed weight", torch.bfloat16)
-            self._check(self.lib.akv_linear_packed(_ptr(x), _ptr(weight.data), _ptr(out), _code(out), rows, weight.outs,
-                                                   weight.k, weight.n_tiles, weight.k_tiles, self._stream()), "linear")
+
+            def own():
+                self._check(self.lib.akv_linear_packed(_ptr(x), _ptr(weight.data), _ptr(out), _code(out), rows,
+                                                       weight.outs, weight.k, weight.n_tiles, weight.k_tiles,
+                                                       self._stream()), "linear")
+            if self._library_product(rows, weight.row_major, out):
+                self._own_or_library(("linear", weight.outs, weight.k), rows, own,
+                                     lambda: torch.mm(x, weight.row_major.t(), out=out))
+            else:
+                own()
             return
         rows, k = x.shape
         outs = weight.shape[0]
@@ -251,15 +295,23 @@ class HipKernels:
         packed = weight.packed
         self._dense(x, "x", torch.bfloat16, (rows, weight.k))
         self._dense(out, "out", None, (rows, weight.inter))
+        self._dense(packed.data, "packed weight", torch.bfloat16)
         if self._library_product(rows, weight.stacked, out):
             if scratch is None:
-                raise KernelError(f"gated_linear of {rows} rows takes the library path and needs the scratch buffer "
-                                  "that gated_scratch() describes")
+                raise KernelError(f"gated_linear of {rows} rows may take the library path and needs the scratch "
+                                  "buffer that gated_scratch() describes")
             self._dense(scratch, "scratch", torch.bfloat16, (rows, 2 * weight.inter))
-            torch.mm(x, weight.stacked.t(), out=scratch)
-            self.swiglu(scratch, out)
+
+            def own():
+                self._check(self.lib.akv_linear_packed_swiglu(_ptr(x), _ptr(packed.data), _ptr(out), _code(out), rows,
+                                                              weight.inter, weight.k, packed.n_tiles, packed.k_tiles,
+                                                              self._stream()), "gated_linear")
+
+            def library():
+                torch.mm(x, weight.stacked.t(), out=scratch)
+                self.swiglu(scratch, out)
+            self._own_or_library(("gated", weight.inter, weight.k), rows, own, library)
             return
-        self._dense(packed.data, "packed weight", torch.bfloat16)
         self._check(self.lib.akv_linear_packed_swiglu(_ptr(x), _ptr(packed.data), _ptr(out), _code(out), rows,
                                                       weight.inter, weight.k, packed.n_tiles, packed.k_tiles,
                                                       self._stream()), "gated_linear")

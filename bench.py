@@ -41,7 +41,7 @@ PAGE_SIZE, CONTEXT, PREFILL_TOKENS = 16, 8192, 2048
 HBM_PEAK_GBS, BF16_PEAK_FLOPS = 8000.0, 2.5e15
 
 
-def scheduler_workload(name: str, layers: int | None) -> int:
+def scheduler_workload(name: str, layers: int | None, library_above: int | None) -> int:
     """A fixed set of requests through the scheduler, from submission to the last token; one JSON line."""
     import torch
     from ampere_kv_engine_amd.config import EngineConfig, Qwen3Config
@@ -61,7 +61,8 @@ def scheduler_workload(name: str, layers: int | None) -> int:
     pages = sum((p + new_tokens + 2 * PAGE_SIZE) // PAGE_SIZE for p in prompts) + 8
     engine = Engine.from_random(config, seed=0, engine_config=EngineConfig(
         dtype="bfloat16", page_size=PAGE_SIZE, num_pages=pages, max_seqs=len(prompts),
-        max_batched_tokens=PREFILL_TOKENS + len(prompts), max_seq_len=longest + PAGE_SIZE, device="cuda:0"))
+        max_batched_tokens=PREFILL_TOKENS + len(prompts), max_seq_len=longest + PAGE_SIZE, device="cuda:0",
+        library_products_above=library_above))
     samples = []
     for run in range(3):                                    # the first run warms up (graphs are recorded in it)
         scheduler = Scheduler(engine, prefill_chunk_size=PREFILL_TOKENS)
@@ -84,7 +85,7 @@ def scheduler_workload(name: str, layers: int | None) -> int:
         "requests": len(prompts), "prompt_tokens": sum(prompts), "new_tokens_each": new_tokens,
         "rounds": scheduler.rounds, "layers": raw["num_hidden_layers"], "hidden": config.hidden_size,
         "q_heads": config.num_attention_heads, "intermediate": config.intermediate_size, "dtype": "bf16",
-        "data": "synthetic: random-init weights, uniform random token ids"}))
+        "library_products_above_rows": library_above, "data": "synthetic: random-init weights, uniform random token ids"}))
     return 0
 
 
@@ -102,13 +103,17 @@ def main() -> int:
     parser.add_argument("--prefill-only", action="store_true", help="time the prefill alone (for kernel profiles)")
     parser.add_argument("--workload", choices=["decode", "serving-14b", "batch-32b"], default="decode",
                         help="decode: the headline measurement; the others run a set of requests through the scheduler")
+    parser.add_argument("--library-above", type=int, default=16,
+                        help="bfloat16 products of more rows than this go to the BLAS library; -1: none does")
     args = parser.parse_args()
+    library_above = None if args.library_above < 0 else args.library_above
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this engine has no multi-GPU path, run it with --gpus 1")
         return 2
 
     if args.workload != "decode":
-        return scheduler_workload(args.workload, args.layers if args.layers != QWEN3_8B["num_hidden_layers"] else None)
+        return scheduler_workload(args.workload, args.layers if args.layers != QWEN3_8B["num_hidden_layers"] else None,
+                                  library_above)
 
     import torch
     from ampere_kv_engine_amd.config import EngineConfig, Qwen3Config
@@ -123,7 +128,7 @@ def main() -> int:
     pages = max_batch * ((tokens_per_request + PAGE_SIZE - 1) // PAGE_SIZE) + PREFILL_TOKENS // PAGE_SIZE + 2
     engine_config = EngineConfig(dtype="bfloat16", page_size=PAGE_SIZE, num_pages=pages, max_seqs=max_batch,
                                  max_batched_tokens=PREFILL_TOKENS, max_seq_len=tokens_per_request + PAGE_SIZE,
-                                 device="cuda:0")
+                                 device="cuda:0", library_products_above=library_above)
     engine = Engine.from_random(config, seed=0, engine_config=engine_config)
     for group in engine.cache.groups:       # any finite keys and values: their content does not change the timing
         group.pages.normal_(0.0, 0.5)

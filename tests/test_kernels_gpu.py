@@ -29,9 +29,16 @@ def hip_own():
     return HipKernels("cuda:0", library_products_above=None)
 
 
-@pytest.fixture(params=["own", "library"])
-def hip_either(request, hip, hip_own):
-    return hip if request.param == "library" else hip_own
+@pytest.fixture(scope="module")
+def hip_library():
+    """Every bfloat16 product of more than 16 rows in the BLAS library, without the one-time choice up to 64 rows."""
+    from ampere_kv_engine_amd.kernels.hip import HipKernels
+    return HipKernels("cuda:0", tune_products=False)
+
+
+@pytest.fixture(params=["own", "library", "chosen"])
+def hip_either(request, hip, hip_own, hip_library):
+    return {"own": hip_own, "library": hip_library, "chosen": hip}[request.param]
 
 
 @pytest.fixture(scope="module")
@@ -205,6 +212,26 @@ def test_gated_linear_rows_do_not_depend_on_the_batch_and_other_sizes_stay_stack
             assert torch.equal(part, whole[first:first + n])
     assert hip.prepare_gated_linear(torch.zeros(40, 64, dtype=torch.bfloat16), torch.zeros(40, 64, dtype=torch.bfloat16)) is None
     assert hip.prepare_gated_linear(torch.zeros(48, 64), torch.zeros(48, 64)) is None
+
+
+def test_products_of_17_to_64_rows_choose_once(hip, ref):
+    """Between 17 and 64 rows the engine's own product and the library's are timed at the first call with a matrix
+    shape and number of row tiles; the choice is remembered, every call gives the product, and other row counts do
+    not ask."""
+    from ampere_kv_engine_amd.kernels.hip import HipKernels
+    kernels = HipKernels("cuda:0")
+    w = rand(320, 256, dtype=torch.bfloat16, seed=41, scale=0.05)
+    packed = kernels.prepare_linear(w.cuda())
+    for rows, known in ((8, 0), (20, 1), (31, 1), (65, 1), (64, 2), (50, 2)):
+        x = rand(rows, 256, dtype=torch.bfloat16, seed=42)
+        want = torch.empty(rows, 320, dtype=torch.bfloat16)
+        ref.linear(x, w, want)
+        got = torch.empty(rows, 320, dtype=torch.bfloat16, device="cuda")
+        kernels.linear(x.cuda(), packed, got)
+        torch.testing.assert_close(got.cpu().float(), want.float(), **tol(torch.bfloat16))
+        assert len(kernels._tuned) == known
+    assert set(kernels._tuned) == {("linear", 320, 256, 2), ("linear", 320, 256, 4)}
+    assert set(kernels._tuned.values()) <= {"own", "library"}
 
 
 def test_linear_keeps_other_weights_row_major(hip):
