@@ -231,102 +231,138 @@ __global__ void kv_write_kernel(const T* __restrict__ k, long k_stride, const T*
 }
 
 // ---- fused: per-head RMSNorm of q and k, rotation of q and k, q out, k and v into the token's cache slot -------
-// One wave per (token, group of `heads_per_wave` heads) of the q_heads + 2 * kv_heads heads of a qkv row (many
-// heads per wave when there are many tokens, one when there are few and latency counts).  A lane owns
-// the rotation pairs (j, j + dim/2) for j = lane, lane + 64, ...: both members of a pair sit in its registers, so
-// the rotation needs no exchange, and the token's position, cache slot and the pair's cos/sin are fetched once for
-// all the heads of the group.  Any step can be switched off: q_weight/k_weight null (no norm), table null (no
-// rotation), slot_map null (no cache write).
-constexpr int kMaxPairsPerLane = 2;  // head sizes up to 256
+// A head of a qkv row belongs to dim / 16 neighbouring lanes; a lane owns 8 consecutive rotation pairs
+// (j, j + dim/2), j = 8 * part .. + 7, read and written as two pieces of 8 elements (16 bytes of bfloat16), so the
+// rotation needs no exchange between lanes and a wave works on 64 / (dim / 16) heads of one token at once.  The sum
+// of squares of a head is formed in the same order in every lane of the head.  Any step can be switched off:
+// q_weight/k_weight null (no norm), table null (no rotation), slot_map null (no cache write).
+template <typename T> __device__ __forceinline__ void load8(const T* p, float (&v)[8]);
+template <> __device__ __forceinline__ void load8<float>(const float* p, float (&v)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+template <> __device__ __forceinline__ void load8<bf16_t>(const bf16_t* p, float (&v)[8]) {
+  const uint4 u = *reinterpret_cast<const uint4*>(p);
+  const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = __uint_as_float(w[i] << 16);
+    v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+template <typename T> __device__ __forceinline__ void store8(T* p, const float (&v)[8]);
+template <> __device__ __forceinline__ void store8<float>(float* p, const float (&v)[8]) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+template <> __device__ __forceinline__ void store8<bf16_t>(bf16_t* p, const float (&v)[8]) {
+  uint4 u;
+  u.x = bf16_bits(v[0]) | (static_cast<uint32_t>(bf16_bits(v[1])) << 16);
+  u.y = bf16_bits(v[2]) | (static_cast<uint32_t>(bf16_bits(v[3])) << 16);
+  u.z = bf16_bits(v[4]) | (static_cast<uint32_t>(bf16_bits(v[5])) << 16);
+  u.w = bf16_bits(v[6]) | (static_cast<uint32_t>(bf16_bits(v[7])) << 16);
+  *reinterpret_cast<uint4*>(p) = u;
+}
 
 template <typename T>
 __global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
     const T* __restrict__ qkv, const float* __restrict__ q_weight, const float* __restrict__ k_weight, float eps,
     const float* __restrict__ table, int table_positions, const int* __restrict__ positions,
     const int* __restrict__ slot_map, T* __restrict__ k_pages, T* __restrict__ v_pages, T* __restrict__ q_out,
-    long tokens, int q_heads, int kv_heads, int dim, int page_size, long num_slots, int heads_per_wave) {
+    long tokens, int q_heads, int kv_heads, int dim, int page_size, long num_slots) {
   const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const int lanes_per_head = dim / 16, heads_per_wave = kWave / lanes_per_head;
   const int heads = q_heads + 2 * kv_heads, groups = (heads + heads_per_wave - 1) / heads_per_wave;
   const long item = static_cast<long>(blockIdx.x) * waves + wave;
   if (item >= tokens * groups) return;
   const long n = item / groups;
-  const int first_head = static_cast<int>(item % groups) * heads_per_wave;
-  const int half = dim / 2;
+  const int sub = lane / lanes_per_head, part = lane % lanes_per_head;
+  const int h = static_cast<int>(item % groups) * heads_per_wave + sub;
+  const bool active = sub < heads_per_wave && h < heads;
+  const bool is_q = h < q_heads, is_v = h >= q_heads + kv_heads;
+  const int half = dim / 2, j0 = part * 8;
   const float nan = __uint_as_float(0x7fc00000u);
+  const bool normed = q_weight != nullptr;
 
-  // per token: the pair's cos/sin, the cache slot
-  float cs[kMaxPairsPerLane], sn[kMaxPairsPerLane];
-  float wq_lo[kMaxPairsPerLane], wq_hi[kMaxPairsPerLane], wk_lo[kMaxPairsPerLane], wk_hi[kMaxPairsPerLane];
-#pragma unroll
-  for (int p = 0; p < kMaxPairsPerLane; ++p) {
-    const int j = lane + p * kWave;
-    cs[p] = 1.f;
-    sn[p] = 0.f;
-    wq_lo[p] = wq_hi[p] = wk_lo[p] = wk_hi[p] = 1.f;
-    if (j < half) {
-      if (table != nullptr) {
-        const int pos = positions[n];
-        if (pos < 0 || pos >= table_positions) {
-          cs[p] = sn[p] = nan;
-        } else {
-          cs[p] = table[(static_cast<long>(pos) * half + j) * 2];
-          sn[p] = table[(static_cast<long>(pos) * half + j) * 2 + 1];
-        }
-      }
-      if (q_weight != nullptr) {
-        wq_lo[p] = q_weight[j];
-        wq_hi[p] = q_weight[j + half];
-        wk_lo[p] = k_weight[j];
-        wk_hi[p] = k_weight[j + half];
-      }
-    }
-  }
   long slot = -1;
   if (slot_map != nullptr) {
     slot = slot_map[n];
     if (slot < 0 || slot >= num_slots) slot = -1;  // host checks the map; never write outside the pool
   }
   const long page = slot >= 0 ? slot / page_size : 0, offset = slot >= 0 ? slot % page_size : 0;
+  const bool works = active && (is_q || slot >= 0);  // keys and values of a token without a slot go nowhere
 
-  for (int h = first_head; h < min(first_head + heads_per_wave, heads); ++h) {
+  float lo[8], hi[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) lo[e] = hi[e] = 0.f;
+  if (works) {
     const T* src = qkv + (n * heads + h) * dim;
-    if (h >= q_heads + kv_heads) {  // value: copied as it is, into the [dim, page_size] layout
-      if (slot < 0) continue;
-      const long at = (page * kv_heads + (h - q_heads - kv_heads)) * dim * page_size + offset;
-      for (int i = lane; i < dim; i += kWave) v_pages[at + static_cast<long>(i) * page_size] = src[i];
-      continue;
-    }
-    const bool is_q = h < q_heads;
-    if (!is_q && slot < 0) continue;
-    T* dst = is_q ? q_out + (n * q_heads + h) * dim
-                  : k_pages + ((page * kv_heads + (h - q_heads)) * page_size + offset) * dim;
-    float lo[kMaxPairsPerLane], hi[kMaxPairsPerLane];
-    float acc = 0.f;
+    load8<T>(src + j0, lo);
+    load8<T>(src + half + j0, hi);
+  }
+  if (works && is_v) {  // value: copied as it is, into the [dim, page_size] layout
+    T* dst = v_pages + (page * kv_heads + (h - q_heads - kv_heads)) * dim * page_size + offset;
 #pragma unroll
-    for (int p = 0; p < kMaxPairsPerLane; ++p) {
-      const int j = lane + p * kWave;
-      lo[p] = hi[p] = 0.f;
-      if (j < half) {
-        lo[p] = to_float(src[j]);
-        hi[p] = to_float(src[j + half]);
-        acc += lo[p] * lo[p] + hi[p] * hi[p];
-      }
-    }
-    const bool normed = q_weight != nullptr;
-    const float scale = normed ? rsqrtf(wave_sum(acc) / static_cast<float>(dim) + eps) : 1.f;
-#pragma unroll
-    for (int p = 0; p < kMaxPairsPerLane; ++p) {
-      const int j = lane + p * kWave;
-      if (j >= half) continue;
-      float a = lo[p], b = hi[p];
-      if (normed) {  // normalise, round to the activation type, times the weight, round again
-        a = rounded<T>(rounded<T>(a * scale) * (is_q ? wq_lo[p] : wk_lo[p]));
-        b = rounded<T>(rounded<T>(b * scale) * (is_q ? wq_hi[p] : wk_hi[p]));
-      }
-      dst[j] = from_float<T>(a * cs[p] - b * sn[p]);
-      dst[j + half] = from_float<T>(b * cs[p] + a * sn[p]);
+    for (int e = 0; e < 8; ++e) {
+      dst[static_cast<long>(j0 + e) * page_size] = from_float<T>(lo[e]);
+      dst[static_cast<long>(half + j0 + e) * page_size] = from_float<T>(hi[e]);
     }
   }
+  // the head's sum of squares: every lane of the head adds the parts up in the same order
+  float own = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) own += lo[e] * lo[e] + hi[e] * hi[e];
+  float total = 0.f;
+  if (normed) {
+    for (int p = 0; p < lanes_per_head; ++p) total += __shfl(own, sub * lanes_per_head + p, kWave);
+  }
+  if (!works || is_v) return;
+
+  float cs[8], sn[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    cs[e] = 1.f;
+    sn[e] = 0.f;
+  }
+  if (table != nullptr) {
+    const int pos = positions[n];
+    if (pos < 0 || pos >= table_positions) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) cs[e] = sn[e] = nan;
+    } else {
+      const float* at = table + (static_cast<long>(pos) * half + j0) * 2;  // (cos, sin) pairs of 8 consecutive j
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float4 pair = *reinterpret_cast<const float4*>(at + 4 * q);
+        cs[2 * q] = pair.x;
+        sn[2 * q] = pair.y;
+        cs[2 * q + 1] = pair.z;
+        sn[2 * q + 1] = pair.w;
+      }
+    }
+  }
+  if (normed) {  // normalise, round to the activation type, times the weight, round again
+    const float scale = rsqrtf(total / static_cast<float>(dim) + eps);
+    const float* w = is_q ? q_weight : k_weight;
+    float w_lo[8], w_hi[8];
+    load8<float>(w + j0, w_lo);
+    load8<float>(w + half + j0, w_hi);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      lo[e] = rounded<T>(rounded<T>(lo[e] * scale) * w_lo[e]);
+      hi[e] = rounded<T>(rounded<T>(hi[e] * scale) * w_hi[e]);
+    }
+  }
+  float out_lo[8], out_hi[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    out_lo[e] = lo[e] * cs[e] - hi[e] * sn[e];
+    out_hi[e] = hi[e] * cs[e] + lo[e] * sn[e];
+  }
+  T* dst = is_q ? q_out + (n * q_heads + h) * dim
+                : k_pages + ((page * kv_heads + (h - q_heads)) * page_size + offset) * dim;
+  store8<T>(dst + j0, out_lo);
+  store8<T>(dst + half + j0, out_hi);
 }
 
 inline unsigned blocks_for(long items, int per_block) { return static_cast<unsigned>((items + per_block - 1) / per_block); }
@@ -428,14 +464,14 @@ int akv_qk_norm_rope_write(const void* qkv, const float* q_weight, const float* 
                            void* k_pages, void* v_pages, void* q_out, int dtype, long tokens, int q_heads,
                            int kv_heads, int dim, int page_size, long num_pages, hipStream_t stream) {
   if (tokens <= 0) return 0;
-  if (dim > 2 * kMaxPairsPerLane * kWave || (dim & 1) != 0) return -2;
-  const int heads_per_wave = tokens >= 512 ? 8 : (tokens >= 64 ? 2 : 1);
+  if ((dim & 15) != 0 || dim > 16 * kWave) return -2;  // a head is dim / 16 lanes of one wave
+  const int heads_per_wave = kWave / (dim / 16);
   const long items = tokens * ((q_heads + 2 * kv_heads + heads_per_wave - 1) / heads_per_wave);
   AKV_DISPATCH(dtype, T,
                qk_norm_rope_write_kernel<T><<<blocks_for(items, 4), 256, 0, stream>>>(
                    static_cast<const T*>(qkv), q_weight, k_weight, eps, table, table_positions, positions, slot_map,
                    static_cast<T*>(k_pages), static_cast<T*>(v_pages), static_cast<T*>(q_out), tokens, q_heads,
-                   kv_heads, dim, page_size, num_pages * page_size, heads_per_wave));
+                   kv_heads, dim, page_size, num_pages * page_size));
   return AKV_LAUNCH_STATUS();
 }
 
