@@ -48,6 +48,7 @@ class Engine:
                                          dtype=torch.float32, device=self.device)
         self.loaded = False
         self._graphs: dict[tuple[int, int], tuple] = {}     # (requests, table width) -> recorded decode step
+        self._graph_logits = None                            # [max_seqs, vocab] float32, where recorded steps write
         self._recordable = (engine_config.decode_graphs and self.device.type == "cuda" and all(
             part.graph_safe for block in self.model.blocks for part in (block, block.mixer, block.feed_forward)))
 
@@ -112,7 +113,7 @@ class Engine:
         the metadata in the step's device buffer differs.  Such a step is run once as it is, then recorded into a
         HIP graph, then replayed - which takes the launches' host time out of decoding.  Launch sizes that depend on
         the requests' lengths are taken from the table width's bound, so one recording serves all lengths under it.
-        The returned logits live in the recording's own buffer: the next replay of it overwrites them."""
+        The returned logits live in a buffer that all recordings share: the next such step overwrites them."""
         ctx, _ = self.builder.build(entries, width_multiple=self.GRAPH_WIDTH_MULTIPLE)
         ctx.stream_buffer = self.stream_buffer
         width = ctx.paged[0].width if ctx.paged else 0
@@ -122,8 +123,11 @@ class Engine:
         ctx.max_seq_len = bound
         ctx.host_seq_lens = [bound] * ctx.num_seqs
         recorded = self._graphs.get(key)
+        if self._graph_logits is None:  # one buffer for every recording: a recorded step's logits are its first rows
+            self._graph_logits = torch.empty((self.config.max_seqs, self.spec.vocab_size), dtype=torch.float32,
+                                             device=self.device)
         if recorded is None:
-            logits = torch.empty((ctx.num_seqs, self.spec.vocab_size), dtype=torch.float32, device=self.device)
+            logits = self._graph_logits[:ctx.num_seqs]
             self.model.forward(ctx, self.cache.layer_cache, logits)        # settles the arenas; also this step's result
             self._graphs[key] = (None, logits)
             return logits
