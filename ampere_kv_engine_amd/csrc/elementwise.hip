@@ -292,39 +292,20 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
   const long page = slot >= 0 ? slot / page_size : 0, offset = slot >= 0 ? slot % page_size : 0;
   const bool works = active && (is_q || slot >= 0);  // keys and values of a token without a slot go nowhere
 
-  float lo[8], hi[8];
+  // every load goes out before anything waits: the row's pieces, the pair's cos/sin, the norm weights
+  float lo[8], hi[8], cs[8], sn[8], w_lo[8], w_hi[8];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) lo[e] = hi[e] = 0.f;
+  for (int e = 0; e < 8; ++e) {
+    lo[e] = hi[e] = sn[e] = 0.f;
+    cs[e] = w_lo[e] = w_hi[e] = 1.f;
+  }
+  const bool turns = works && !is_v;  // a query or key head: normed and rotated
   if (works) {
     const T* src = qkv + (n * heads + h) * dim;
     load8<T>(src + j0, lo);
     load8<T>(src + half + j0, hi);
   }
-  if (works && is_v) {  // value: copied as it is, into the [dim, page_size] layout
-    T* dst = v_pages + (page * kv_heads + (h - q_heads - kv_heads)) * dim * page_size + offset;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      dst[static_cast<long>(j0 + e) * page_size] = from_float<T>(lo[e]);
-      dst[static_cast<long>(half + j0 + e) * page_size] = from_float<T>(hi[e]);
-    }
-  }
-  // the head's sum of squares: every lane of the head adds the parts up in the same order
-  float own = 0.f;
-#pragma unroll
-  for (int e = 0; e < 8; ++e) own += lo[e] * lo[e] + hi[e] * hi[e];
-  float total = 0.f;
-  if (normed) {
-    for (int p = 0; p < lanes_per_head; ++p) total += __shfl(own, sub * lanes_per_head + p, kWave);
-  }
-  if (!works || is_v) return;
-
-  float cs[8], sn[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    cs[e] = 1.f;
-    sn[e] = 0.f;
-  }
-  if (table != nullptr) {
+  if (turns && table != nullptr) {
     const int pos = positions[n];
     if (pos < 0 || pos >= table_positions) {
 #pragma unroll
@@ -341,12 +322,36 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
       }
     }
   }
-  if (normed) {  // normalise, round to the activation type, times the weight, round again
-    const float scale = rsqrtf(total / static_cast<float>(dim) + eps);
+  if (turns && normed) {
     const float* w = is_q ? q_weight : k_weight;
-    float w_lo[8], w_hi[8];
     load8<float>(w + j0, w_lo);
     load8<float>(w + half + j0, w_hi);
+  }
+  if (works && is_v) {  // value: copied as it is, into the [dim, page_size] layout
+    T* dst = v_pages + (page * kv_heads + (h - q_heads - kv_heads)) * dim * page_size + offset;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      dst[static_cast<long>(j0 + e) * page_size] = from_float<T>(lo[e]);
+      dst[static_cast<long>(half + j0 + e) * page_size] = from_float<T>(hi[e]);
+    }
+  }
+  // the head's sum of squares; every lane of the head ends with the same bits (a butterfly adds the same two numbers
+  // on both sides; otherwise the parts are added in the same order by every lane)
+  float total = 0.f;
+  if (normed) {
+    float own = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) own += lo[e] * lo[e] + hi[e] * hi[e];
+    if ((lanes_per_head & (lanes_per_head - 1)) == 0) {
+      total = own;
+      for (int step = 1; step < lanes_per_head; step <<= 1) total += __shfl_xor(total, step, kWave);
+    } else {
+      for (int p = 0; p < lanes_per_head; ++p) total += __shfl(own, sub * lanes_per_head + p, kWave);
+    }
+  }
+  if (!turns) return;
+  if (normed) {  // normalise, round to the activation type, times the weight, round again
+    const float scale = rsqrtf(total / static_cast<float>(dim) + eps);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       lo[e] = rounded<T>(rounded<T>(lo[e] * scale) * w_lo[e]);
