@@ -104,6 +104,7 @@ class HipKernels:
         self.decode_min_segment = 128   # but into segments no shorter than this many keys
         self.decode_max_splits = 32     # and no more than this many (the merge walks them one after the other)
         self.share_prompt_tiles = True  # prompt portions: blocks of four waves share keys and values through LDS
+        self.one_wave_per_head = False  # True: every attention goes to the plain kernel, a wave per (token, head)
         for name in ("akv_embed", "akv_add_rmsnorm", "akv_rmsnorm_rows", "akv_copy_rows", "akv_gather_rows",
                      "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
                      "akv_linear_tiled", "akv_linear_packed", "akv_linear_packed_swiglu", "akv_attention_rows", "akv_sample"):
@@ -441,7 +442,8 @@ class HipKernels:
         self._dense(meta.block_table, "block_table", torch.int32, (ctx.num_seqs, meta.width))
         if ctx.max_seq_len > meta.width * page_size:
             raise KernelError(f"a request of {ctx.max_seq_len} tokens does not fit a block table of {meta.width} pages")
-        if q.dtype == torch.bfloat16 and page_size >= 4 and page_size & (page_size - 1) == 0:
+        if (q.dtype == torch.bfloat16 and page_size >= 4 and page_size & (page_size - 1) == 0
+                and not self.one_wave_per_head):
             self._dense(ctx.q_start, "q_start", torch.int32, (ctx.num_seqs + 1,))
             self._dense(ctx.seq_lens, "seq_lens", torch.int32, (ctx.num_seqs,))
             if ctx.host_q_start[ctx.num_seqs] != tokens or len(ctx.host_seq_lens) != ctx.num_seqs:

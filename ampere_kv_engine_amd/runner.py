@@ -5,7 +5,8 @@ one prompt, one model, `--mode` chooses what is done with it.
 
 Options the reference has keep their names and meanings: `--mode` (check | generate | benchmark), `--repeats`
 (benchmark repetitions after one warm-up), `--cache` (only `paged` exists here), `--kv-dtype` (bf16; the cache
-follows `--dtype`).  The reference reads a text and tokenizes it; this engine takes token ids in and gives token
+follows `--dtype`), `--decode-kernel` (v1: one query head per wave; v3: the query heads of a group share every key
+and value load - here the MFMA kernels, and the default).  The reference reads a text and tokenizes it; this engine takes token ids in and gives token
 ids out, so the prompt is a line of integers on standard input (or `--prompt-ids`, or a seeded random prompt with
 `--prompt-len`).  `check` replaces the reference's comparison with a borrowed model by a comparison of the serving
 arithmetic with the engine's own true 32-bit path, step by step on the same tokens.
@@ -50,6 +51,9 @@ def build_parser() -> argparse.ArgumentParser:
     parser.add_argument("--cache", choices=("paged",), default="paged", help="the cache is paged; nothing else exists")
     parser.add_argument("--kv-dtype", choices=("bf16", "fp32"), default=None,
                         help="must agree with --dtype: the cache holds what the arithmetic produces")
+    parser.add_argument("--decode-kernel", choices=("v1", "v3"), default="v3",
+                        help="attention kernel of the bfloat16 path: v1 one query head per wave (the plain kernel), "
+                             "v3 the query heads of a group share every key and value load (MFMA kernels)")
     parser.add_argument("--dtype", choices=("bfloat16", "float32"), default="bfloat16")
     parser.add_argument("--prompt-ids", help="token ids separated by commas or blanks (default: read a line from stdin)")
     parser.add_argument("--prompt-len", type=int, help="use a seeded random prompt of this length")
@@ -70,7 +74,9 @@ def _engine(folder: str, dtype: str, args, capacity: int) -> Engine:
     config = EngineConfig(dtype=dtype, page_size=args.page_size, num_pages=pages, max_seqs=2,
                           max_batched_tokens=max(min(capacity, 8192), 1), max_seq_len=pages * args.page_size,
                           device=args.device)
-    return Engine.from_folder(folder, config)
+    engine = Engine.from_folder(folder, config)
+    engine.kernels.one_wave_per_head = args.decode_kernel == "v1"
+    return engine
 
 
 def check(folder: str, prompt: list[int], args) -> list[int]:

@@ -242,6 +242,10 @@ def test_command_line(model_folders):
     result = run("--model", model_folders["A"], "--mode", "benchmark", "--repeats", "2", "--max-new-tokens", "6",
                  "--prompt-len", "20")
     assert result.returncode == 0 and '"tpot_ms"' in result.stdout, result.stderr[-2000:]
+    for kernel in ("v1", "v3"):          # bfloat16: a query head per wave, or the heads of a group sharing the loads
+        result = run("--model", model_folders["A"], "--mode", "generate", "--decode-kernel", kernel, "--max-new-tokens",
+                     "6", "--ignore-eos", "--prompt-ids", ",".join(map(str, prompt)))
+        assert result.returncode == 0 and f"generated_token_ids = {want}" in result.stdout, result.stderr[-2000:]
     result = run("--model", model_folders["A"], "--mode", "generate", "--cache", "contiguous", "--prompt-ids", "1")
     assert result.returncode != 0
 
