@@ -741,19 +741,24 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
 }
 
 // Merge of the segments' partial results: out = sum_z 2^(m_z - M) O_z / sum_z 2^(m_z - M) l_z, M = max_z m_z
-// (csrc/paged_decode.cu:528-544 of the reference has the same rule in base e).  One wave per (tile, head group,
-// column); a lane owns dims lane, lane + 64, ...; the segments are summed in ascending order.
+// (csrc/paged_decode.cu:528-544 of the reference has the same rule in base e).  One block of kMergeWaves waves per
+// (tile, head group, column); a lane owns dims lane, lane + 64, ...; wave w sums the segments w, w + kMergeWaves, ...
+// in ascending order, and the waves' sums are added in the order of the waves: the order of the whole sum is fixed.
+constexpr int kMergeWaves = 4;
+
 template <int NQ>
-__global__ __launch_bounds__(64) void attention_merge_kernel(const Args a) {
+__global__ __launch_bounds__(64 * kMergeWaves) void attention_merge_kernel(const Args a) {
+  constexpr int PER = (D + 63) / 64;
+  __shared__ float sums[kMergeWaves][PER * 64 + 1];  // per wave: the weighted sum per dim, then the denominator
   const Tile t = find_tile(a, blockIdx.x, a.tokens_per_tile);
   if (!t.found) return;
   const int kvh = blockIdx.y / a.head_groups, hg = blockIdx.y % a.head_groups;
-  const int c = blockIdx.z, lane = threadIdx.x;
+  const int c = blockIdx.z, lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int token = c / a.heads_per_tile, head_in_group = hg * a.heads_per_tile + c % a.heads_per_tile;
   if (token >= t.tokens || head_in_group >= a.group) return;
   const float* src = a.partial + (((static_cast<long>(blockIdx.x) * gridDim.y + blockIdx.y) * a.num_splits) * (16 * NQ) + c) * PSTRIDE;
   const long split_stride = static_cast<long>(16 * NQ) * PSTRIDE;
-  // first the segments' maxima (a lane per segment), then the weighted sums
+  // every wave finds the maximum over all segments (a lane per segment)
   float top = -INFINITY;
   bool poisoned = false;
   for (int z0 = 0; z0 < a.num_splits; z0 += 64) {
@@ -764,41 +769,56 @@ __global__ __launch_bounds__(64) void attention_merge_kernel(const Args a) {
   }
   top = wave_max(top);
   poisoned = __any(poisoned);
-  constexpr int PER = (D + 63) / 64;
+  // this wave's segments: z = wave + kMergeWaves * i
+  const int mine = (a.num_splits - wave + kMergeWaves - 1) / kMergeWaves;
   float denom = 0.f, acc[PER];
 #pragma unroll
   for (int i = 0; i < PER; ++i) acc[i] = 0.f;
-  for (int z0 = 0; z0 < a.num_splits; z0 += 64) {
-    const int z = z0 + lane;
+  for (int i0 = 0; i0 < mine; i0 += 64) {
+    const int i = i0 + lane;
     float w = 0.f;
-    if (z < a.num_splits) {
+    if (i < mine) {
+      const long z = wave + static_cast<long>(kMergeWaves) * i;
       const float mz = src[z * split_stride + D];
       w = (mz == -INFINITY || mz != mz) ? 0.f : __builtin_amdgcn_exp2f(mz - top);
       denom += w * src[z * split_stride + D + 1];
     }
-    const int count = min(64, a.num_splits - z0);
-    for (int zz0 = 0; zz0 < count; zz0 += 8) {  // ascending segments: the order of the sum is fixed
-      float v[8][PER];                            // eight segments' loads go out together
+    const int count = min(64, mine - i0);
+    for (int ii0 = 0; ii0 < count; ii0 += 8) {  // ascending segments; eight segments' loads go out together
+      float v[8][PER];
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float* p = src + (z0 + min(zz0 + j, count - 1)) * split_stride;
+        const float* p = src + (wave + static_cast<long>(kMergeWaves) * (i0 + min(ii0 + j, count - 1))) * split_stride;
 #pragma unroll
-        for (int i = 0; i < PER; ++i) v[j][i] = lane + i * 64 < D ? p[lane + i * 64] : 0.f;
+        for (int e = 0; e < PER; ++e) v[j][e] = lane + e * 64 < D ? p[lane + e * 64] : 0.f;
       }
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float wz = zz0 + j < count ? __shfl(w, zz0 + j, 64) : 0.f;
+        const float wz = ii0 + j < count ? __shfl(w, ii0 + j, 64) : 0.f;
 #pragma unroll
-        for (int i = 0; i < PER; ++i) acc[i] = fmaf(wz, v[j][i], acc[i]);
+        for (int e = 0; e < PER; ++e) acc[e] = fmaf(wz, v[j][e], acc[e]);
       }
     }
   }
   denom = wave_sum(denom);
-  bf16_t* dst = a.out + (static_cast<long>(t.first_row + token) * a.q_heads + kvh * a.group + head_in_group) * D;
-  const float inv = poisoned ? __uint_as_float(0x7fc00000u) : 1.f / denom;
 #pragma unroll
-  for (int i = 0; i < PER; ++i)
-    if (lane + i * 64 < D) dst[lane + i * 64] = from_float<bf16_t>(acc[i] * inv);
+  for (int e = 0; e < PER; ++e) sums[wave][e * 64 + lane] = acc[e];
+  if (lane == 0) sums[wave][PER * 64] = denom;
+  __syncthreads();
+  if (wave != 0) return;
+  float total = 0.f;
+#pragma unroll
+  for (int e = 0; e < PER; ++e) acc[e] = 0.f;
+  for (int w = 0; w < kMergeWaves; ++w) {
+    total += sums[w][PER * 64];
+#pragma unroll
+    for (int e = 0; e < PER; ++e) acc[e] += sums[w][e * 64 + lane];
+  }
+  bf16_t* dst = a.out + (static_cast<long>(t.first_row + token) * a.q_heads + kvh * a.group + head_in_group) * D;
+  const float inv = poisoned ? __uint_as_float(0x7fc00000u) : 1.f / total;
+#pragma unroll
+  for (int e = 0; e < PER; ++e)
+    if (lane + e * 64 < D) dst[lane + e * 64] = from_float<bf16_t>(acc[e] * inv);
 }
 
 template <int NQ>
@@ -815,7 +835,7 @@ int launch(const Args& a, int tiles, bool shared, hipStream_t stream) {
   if (a.num_splits > 1) {
     attention_mfma_kernel<NQ, true, true><<<grid, 64, 0, stream>>>(a);
     grid.z = a.heads_per_tile * a.tokens_per_tile;  // the columns that can be (token, head) pairs
-    attention_merge_kernel<NQ><<<grid, 64, 0, stream>>>(a);
+    attention_merge_kernel<NQ><<<grid, 64 * kMergeWaves, 0, stream>>>(a);
   } else {
     attention_mfma_kernel<NQ, false, true><<<grid, 64, 0, stream>>>(a);
   }
