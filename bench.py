@@ -3,7 +3,9 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--context S] [--layers L]
 
 A "step" is one decode step of the whole batch: every live request feeds its last token through the engine's
-step function and the sampler chooses the next one (greedy), exactly as generation does.  The requests' caches
+step function and the sampler chooses the next one (greedy), exactly as generation does.  Three untimed steps come
+before the W warm-up steps (the engine runs a batch shape once as it is, records it, then replays the recording), so
+the K timed steps are replays whatever W is.  The requests' caches
 are brought to the context length beforehand (pages filled with random keys and values: what they hold does
 not change the time a step takes).  One JSON line is printed:
   value     decoded tokens per second at the default batch
@@ -38,6 +40,7 @@ QWEN3_8B = dict(architectures=["Qwen3ForCausalLM"], num_hidden_layers=36, hidden
 QWEN3_14B = dict(QWEN3_8B, num_hidden_layers=40, hidden_size=5120, num_attention_heads=40, intermediate_size=17408)
 QWEN3_32B = dict(QWEN3_8B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, intermediate_size=25600)
 PAGE_SIZE, CONTEXT, PREFILL_TOKENS = 16, 8192, 2048
+PRIMING = 3   # untimed steps before the warm-up steps: the first runs eagerly, the second is recorded, the third replays
 HBM_PEAK_GBS, BF16_PEAK_FLOPS = 8000.0, 2.5e15
 
 
@@ -124,7 +127,7 @@ def main() -> int:
     max_batch = max([args.batch] + points)
     raw = dict(QWEN3_8B, num_hidden_layers=args.layers)
     config = Qwen3Config.from_dict(raw)
-    tokens_per_request = args.context + args.warmup + args.steps + 1
+    tokens_per_request = args.context + PRIMING + args.warmup + args.steps + 1
     pages = max_batch * ((tokens_per_request + PAGE_SIZE - 1) // PAGE_SIZE) + PREFILL_TOKENS // PAGE_SIZE + 2
     engine_config = EngineConfig(dtype="bfloat16", page_size=PAGE_SIZE, num_pages=pages, max_seqs=max_batch,
                                  max_batched_tokens=PREFILL_TOKENS, max_seq_len=tokens_per_request + PAGE_SIZE,
@@ -149,7 +152,7 @@ def main() -> int:
             logits = engine.step([StepEntry(seq, [token], [0]) for seq, token in zip(seqs, tokens)])
             tokens = sampler.sample(logits, greedy, draws)
 
-        for _ in range(warmup):
+        for _ in range(PRIMING + warmup):
             one_step()
         sync()
         started = time.perf_counter()
@@ -187,7 +190,7 @@ def main() -> int:
     ms_per_step = elapsed / args.steps * 1000
     value = args.batch * args.steps / elapsed
     weight_bytes = engine.model.weight_bytes_per_step()
-    kv_bytes = args.batch * (args.context + args.warmup + args.steps // 2) * engine.cache.bytes_per_token()
+    kv_bytes = args.batch * (args.context + PRIMING + args.warmup + args.steps // 2) * engine.cache.bytes_per_token()
     achieved = (weight_bytes + kv_bytes) / (ms_per_step / 1000) / 1e9
     record = {
         "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2,048 tokens (Qwen3-8B bf16)",
