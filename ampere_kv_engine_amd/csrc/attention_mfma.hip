@@ -523,7 +523,7 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
 #pragma unroll
   for (int p = 0; p < PK; ++p) {
     const int c = p * 256 + tid, key = c / (D / 8);
-    k_mine[p] = c < kKeyPieces;
+    k_mine[p] = kKeyPieces % 256 == 0 || c < kKeyPieces;  // (known when compiling for the usual head sizes)
     k_sel[p] = step_pages == 1 ? 0 : key >> a.page_shift;
     k_from[p] = head_bytes + (c % (D / 8)) * 16u + static_cast<uint32_t>(key & page_mask) * (D * 2u);
     k_to[p] = (((key >> 2) & 1) * 16 + (key >> 3) * 4 + (key & 3)) * KROW + (c % (D / 8)) * 8;  // tile j, row rho
@@ -533,7 +533,7 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
     const int c = p * 256 + tid;
     const int run = (c / D) >> run_shift, within = c - ((run * D) << run_shift);
     const int dim = within >> run_shift, piece = (run << run_shift) + (within & ((1 << run_shift) - 1));
-    v_mine[p] = c < kValuePieces;
+    v_mine[p] = kValuePieces % 256 == 0 || c < kValuePieces;
     v_sel[p] = step_pages == 1 ? 0 : (piece * 8) >> a.page_shift;
     v_from[p] = head_bytes + (static_cast<uint32_t>(dim) << (a.page_shift + 1)) + static_cast<uint32_t>((piece * 8) & page_mask) * 2u;
     v_to[p] = dim * VROW + piece * 8;
