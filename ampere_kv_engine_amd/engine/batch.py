@@ -40,6 +40,8 @@ class Arena:
     of a given size no device memory is allocated and addresses repeat from step to step."""
 
     ALIGN = 256
+    ELEMENT_BYTES = {torch.float32: 4, torch.bfloat16: 2, torch.int32: 4, torch.int64: 8, torch.uint8: 1,
+                     torch.float16: 2}
 
     def __init__(self, device, chunk_bytes: int = 64 << 20):
         self.device = device
@@ -56,14 +58,15 @@ class Arena:
         count = 1
         for s in shape:
             count *= int(s)
-        nbytes = max(count * torch.empty((), dtype=dtype).element_size(), 1)
+        size = self.ELEMENT_BYTES.get(dtype) or torch.empty((), dtype=dtype).element_size()
+        nbytes = max(count * size, 1)
         nbytes = (nbytes + self.ALIGN - 1) // self.ALIGN * self.ALIGN
         while True:
             if self.chunk_index >= len(self.chunks):
                 self.chunks.append(torch.empty(max(nbytes, self.chunk_bytes), dtype=torch.uint8, device=self.device))
             chunk = self.chunks[self.chunk_index]
             if self.offset + nbytes <= chunk.numel():
-                raw = chunk[self.offset:self.offset + count * torch.empty((), dtype=dtype).element_size()]
+                raw = chunk[self.offset:self.offset + count * size]
                 self.offset += nbytes
                 return raw.view(dtype).view(*shape)
             self.chunk_index += 1

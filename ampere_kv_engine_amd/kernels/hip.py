@@ -17,6 +17,9 @@ _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 MAX_HEAD_DIM = 256
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 class KernelError(RuntimeError):
     pass
 
@@ -112,6 +115,9 @@ class HipKernels:
 
     # ---- helpers -----------------------------------------------------------------------------------------
     def _stream(self):
+        """The current stream's handle (the raw getter spares the construction of a Stream object per launch)."""
+        if _raw_stream is not None:
+            return ctypes.c_void_p(_raw_stream(self.device.index))
         return ctypes.c_void_p(torch.cuda.current_stream(self.device).cuda_stream)
 
     def _check(self, status: int, what: str) -> None:
@@ -286,8 +292,9 @@ class HipKernels:
     def gated_scratch(self, weight: GatedWeight, rows: int, dtype: torch.dtype):
         """Shape of the buffer `gated_linear` wants for this many rows (the stacked product of the library path),
         or None."""
-        probe = torch.empty((), dtype=dtype)
-        return (rows, 2 * weight.inter) if self._library_product(rows, weight.stacked, probe) else None
+        wanted = (weight.stacked is not None and self.library_products_above is not None
+                  and rows > self.library_products_above and dtype == torch.bfloat16)
+        return (rows, 2 * weight.inter) if wanted else None
 
     def gated_linear(self, x, weight: GatedWeight, out, scratch=None):
         """out [rows, inter] = silu(x Wgate^T) * (x Wup^T): one kernel, from float32 accumulators; with many rows the
