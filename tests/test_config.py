@@ -80,3 +80,30 @@ def test_engine_config_checks_its_numbers():
     with pytest.raises(ValueError):
         EngineConfig(page_size=0)
     assert EngineConfig(page_size=16, max_seq_len=100).max_pages_per_seq == 7
+
+
+def test_plan_memory_counts_weights_copies_and_pages():
+    """Pages that fit beside a model, from its specification alone (no device)."""
+    from ampere_kv_engine_amd.config import EngineConfig, Qwen3Config
+    from ampere_kv_engine_amd.engine import plan_memory
+    raw = dict(architectures=["Qwen3ForCausalLM"], vocab_size=1000, hidden_size=64, num_hidden_layers=3,
+               num_attention_heads=4, num_key_value_heads=2, head_dim=16, intermediate_size=128, rope_theta=1e4,
+               rms_norm_eps=1e-6, tie_word_embeddings=False, hidden_act="silu")
+    spec = Qwen3Config.from_dict(raw).to_model_spec()
+    layer = (4 + 2 + 2) * 16 * 64 + 64 * 64 + 3 * 128 * 64          # q/k/v, o, gate/up/down
+    norms = 3 * (2 * 64 + 2 * 16) + 64
+    config = EngineConfig(dtype="bfloat16", page_size=8, num_pages=1, max_seqs=2, max_batched_tokens=16, max_seq_len=64)
+    plan = plan_memory(spec, config, 1 << 30)
+    assert plan.weight_bytes == 2 * (3 * layer + norms + 2 * 1000 * 64)
+    assert plan.second_copy_bytes == 2 * (3 * layer + 1000 * 64)        # every matrix but the embedding table
+    assert plan.page_bytes == 3 * 2 * 2 * 16 * 8 * 2                     # layers x (k, v) x kv heads x dim x page x bytes
+    assert plan.num_pages == ((1 << 30) - plan.weight_bytes - plan.second_copy_bytes - plan.fixed_bytes) // plan.page_bytes
+    assert plan.tokens == plan.num_pages * 8
+    own = plan_memory(spec, EngineConfig(dtype="bfloat16", page_size=8, num_pages=1, max_seqs=2, max_batched_tokens=16,
+                                         max_seq_len=64, library_products_above=None), 1 << 30)
+    assert own.second_copy_bytes == 0 and own.num_pages > plan.num_pages
+    full = plan_memory(spec, EngineConfig(dtype="float32", page_size=8, num_pages=1, max_seqs=2, max_batched_tokens=16,
+                                          max_seq_len=64), 1 << 30)
+    assert full.weight_bytes == 2 * plan.weight_bytes and full.second_copy_bytes == 0 and full.page_bytes == 2 * plan.page_bytes
+    with pytest.raises(ValueError, match="not a page"):
+        plan_memory(spec, config, plan.weight_bytes + plan.second_copy_bytes + plan.fixed_bytes + plan.page_bytes)
