@@ -20,7 +20,7 @@ class EngineConfig:
     max_batched_tokens: int = 2048   # most tokens one step may carry
     max_seq_len: int = 8192          # longest sequence a request may reach (block-table width, rotary table)
     device: str = "cuda:0"
-    decode_graphs: bool = True       # replay a recorded HIP graph for steps in which every request brings one token
+    decode_graphs: bool = True       # replay recorded HIP graphs: decode steps, and small mixed steps whose shape repeats
     # bfloat16 products of more rows than this go to the BLAS library, which reads the matrices row-major: they are
     # then kept twice (row-major and packed for the engine's own kernels).  None: one copy, own kernels only.
     library_products_above: int | None = 16

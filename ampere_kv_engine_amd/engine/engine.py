@@ -47,7 +47,7 @@ class Engine:
         self.stream_buffer = torch.empty((engine_config.max_batched_tokens, spec.hidden_size),
                                          dtype=torch.float32, device=self.device)
         self.loaded = False
-        self._graphs: dict[tuple[int, int], tuple] = {}     # (requests, table width) -> recorded decode step
+        self._graphs: dict[tuple, object] = {}               # (tokens per request, wanted rows, table width) -> graph
         self._graph_logits = None                            # [max_seqs, vocab] float32, where recorded steps write
         self._recordable = (engine_config.decode_graphs and self.device.type == "cuda" and all(
             part.graph_safe for block in self.model.blocks for part in (block, block.mixer, block.feed_forward)))
@@ -98,46 +98,64 @@ class Engine:
                 if not 0 <= int(token) < vocab:
                     raise ValueError(f"token id {token} of request {e.seq.request_id!r} is outside the vocabulary "
                                      f"of {vocab}")
-        if self._recordable and all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries):
-            return self._decode_step_recorded(entries)
+        if self._recordable:
+            shape = self._recordable_shape(entries)
+            if shape is not None:
+                return self._step_recorded(entries, shape)
         ctx, _ = self.builder.build(entries)
         ctx.stream_buffer = self.stream_buffer
         return self.model.forward(ctx, self.cache.layer_cache)
 
-    # ---- decode steps as recorded graphs ----------------------------------------------------------------------
+    # ---- steps as recorded graphs -----------------------------------------------------------------------------
     GRAPH_WIDTH_MULTIPLE = 64     # block tables of a recorded step are this many pages wide, or a multiple
+    RECORD_MAX_TOKENS = 512       # steps with prompt portions are recorded up to this many tokens: beyond it the
+                                  # device works longer on a step than the host needs to launch it
+    MAX_RECORDINGS = 512          # shapes met after this many are run as they are
 
-    def _decode_step_recorded(self, entries: list[StepEntry]) -> torch.Tensor:
-        """A step in which every request brings one token and wants its logits launches the same kernels with the
-        same arguments every time, as long as the number of requests and the width of the block tables stay: only
-        the metadata in the step's device buffer differs.  Such a step is run once as it is, then recorded into a
-        HIP graph, then replayed - which takes the launches' host time out of decoding.  Launch sizes that depend on
-        the requests' lengths are taken from the table width's bound, so one recording serves all lengths under it.
-        The returned logits live in a buffer that all recordings share: the next such step overwrites them."""
+    def _recordable_shape(self, entries: list[StepEntry]):
+        """(tokens per request in the step's order - single tokens first -, wanted rows), or None for a step that
+        is run as it is: nothing wanted, more wanted rows than the shared logits buffer has, or long portions."""
+        counts = tuple(sorted((len(e.tokens) for e in entries), key=lambda count: count != 1))
+        wanted = sum(len(e.want) for e in entries)
+        if wanted == 0 or wanted > self.config.max_seqs:
+            return None
+        if counts[-1] != 1 and sum(counts) > self.RECORD_MAX_TOKENS:
+            return None
+        return counts, wanted
+
+    def _step_recorded(self, entries: list[StepEntry], shape) -> torch.Tensor:
+        """A step launches the same kernels with the same arguments every time, as long as the requests bring the
+        same numbers of tokens, as many rows are wanted and the width of the block tables stays: only the metadata in
+        the step's device buffer differs.  A step of such a shape is run once as it is, then recorded into a HIP
+        graph, then replayed - which takes the launches' host time out of decoding and out of small mixed steps.
+        Launch sizes that depend on the requests' lengths are taken from the table width's bound, so one recording
+        serves all lengths under it.  The returned logits live in a buffer that all recordings share: the next
+        recorded step overwrites them."""
+        counts, wanted = shape
         ctx, _ = self.builder.build(entries, width_multiple=self.GRAPH_WIDTH_MULTIPLE)
         ctx.stream_buffer = self.stream_buffer
         width = ctx.paged[0].width if ctx.paged else 0
-        key = (ctx.num_seqs, width)
+        key = (counts, wanted, width)
         # sizes of launches come from the bound, not from this step's lengths
         bound = max(width * self.config.page_size, 1)
         ctx.max_seq_len = bound
         ctx.host_seq_lens = [bound] * ctx.num_seqs
-        recorded = self._graphs.get(key)
         if self._graph_logits is None:  # one buffer for every recording: a recorded step's logits are its first rows
             self._graph_logits = torch.empty((self.config.max_seqs, self.spec.vocab_size), dtype=torch.float32,
                                              device=self.device)
-        if recorded is None:
-            logits = self._graph_logits[:ctx.num_seqs]
-            self.model.forward(ctx, self.cache.layer_cache, logits)        # settles the arenas; also this step's result
-            self._graphs[key] = (None, logits)
+        logits = self._graph_logits[:wanted]
+        graph = self._graphs.get(key, False)
+        if graph is False:              # first met: run as it is (this also settles the arenas)
+            self.model.forward(ctx, self.cache.layer_cache, logits)
+            if len(self._graphs) < self.MAX_RECORDINGS or counts[-1] == 1:   # (decode steps are always remembered)
+                self._graphs[key] = None
             return logits
-        graph, logits = recorded
-        if graph is None:
+        if graph is None:               # met again: record
             graph = torch.cuda.CUDAGraph()
             torch.cuda.synchronize(self.device)
             with torch.cuda.graph(graph, stream=self._capture_stream()):
                 self.model.forward(ctx, self.cache.layer_cache, logits)
-            self._graphs[key] = (graph, logits)
+            self._graphs[key] = graph
         graph.replay()
         return logits
 

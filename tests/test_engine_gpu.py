@@ -86,6 +86,6 @@ def test_recorded_decode_steps_of_many_requests(case):
             expected = want[i][len(tokens) - decoded + step]
             torch.testing.assert_close(got[i], expected, **tolerance("bfloat16", want[i]), msg=lambda m: f"step {step} request {i}: {m}")
         torch.cuda.synchronize()
-    assert sum(graph is not None for graph, _ in engine._graphs.values()) == 1
+    assert sum(graph is not None for graph in engine._graphs.values()) == 1
     for seq in seqs:
         engine.close(seq)
