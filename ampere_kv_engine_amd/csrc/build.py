@@ -14,6 +14,7 @@ import shutil
 import subprocess
 import sys
 import tempfile
+import threading
 import time
 from concurrent.futures import ThreadPoolExecutor
 
@@ -46,20 +47,28 @@ def source_stamp(sources=None) -> str:
     return digest.hexdigest()
 
 
+_BUILD_DIR: str | None = None
+_BUILD_DIR_LOCK = threading.Lock()
+
+
 def _build_dir() -> str:
-    """`_build/` beside the sources; a per-user temporary folder when the tree cannot be written."""
-    local = os.path.join(HERE, "_build")
-    try:
-        os.makedirs(local, exist_ok=True)
-        probe = os.path.join(local, f".probe{os.getpid()}")
-        with open(probe, "w"):
-            pass
-        os.remove(probe)
-        return local
-    except OSError:
-        fallback = os.path.join(tempfile.gettempdir(), f"akv_build_{os.getuid()}_{source_stamp()[:12]}")
-        os.makedirs(fallback, exist_ok=True)
-        return fallback
+    """`_build/` beside the sources; a per-user temporary folder when the tree cannot be written.  Decided once
+    (several head sizes are compiled by threads of one process)."""
+    global _BUILD_DIR
+    with _BUILD_DIR_LOCK:
+        if _BUILD_DIR is None:
+            local = os.path.join(HERE, "_build")
+            try:
+                os.makedirs(local, exist_ok=True)
+                probe = os.path.join(local, f".probe{os.getpid()}")
+                with open(probe, "w"):
+                    pass
+                os.remove(probe)
+                _BUILD_DIR = local
+            except OSError:
+                _BUILD_DIR = os.path.join(tempfile.gettempdir(), f"akv_build_{os.getuid()}_{source_stamp()[:12]}")
+                os.makedirs(_BUILD_DIR, exist_ok=True)
+        return _BUILD_DIR
 
 
 def library_path() -> str | None:
