@@ -31,9 +31,10 @@ int akv_qk_norm_rope_write(const void* qkv, const float* q_weight, const float* 
 int akv_linear_tiled(const void* x, int x_dtype, const void* w, int w_dtype, void* y, int y_dtype, int rows, int outs,
                      int k, hipStream_t stream);
 int akv_linear_packed(const void* x, const void* wp, void* y, int y_dtype, int rows, int outs, int k, int n_tiles,
-                      int k_tiles, hipStream_t stream);
+                      int k_tiles, int x_packed, hipStream_t stream);
 int akv_linear_packed_swiglu(const void* x, const void* wp, void* y, int y_dtype, int rows, int inter, int k,
-                             int n_tiles, int k_tiles, hipStream_t stream);
+                             int n_tiles, int k_tiles, int x_packed, hipStream_t stream);
+int akv_pack_rows(const void* x, void* xp, int rows, int k, hipStream_t stream);
 int akv_attention_rows(const void* q, const void* k_pages, const void* v_pages, const int* seq_of_token,
                        const int* positions, const int* block_table, int table_width, void* out, int dtype,
                        long tokens, int q_heads, int kv_heads, int dim, int page_size, long num_pages, float scale,

@@ -77,7 +77,7 @@ template <int MT, int RT> constexpr bool kSkinnyOwnSets = RT * MT <= 8;
 template <int MT, int RT, typename TY, bool GATED>
 __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __restrict__ x, const uintx4* __restrict__ wp,
                                                             TY* __restrict__ y, int rows, int outs, int k,
-                                                            int k_tiles, int n_tiles, int k_split) {
+                                                            int k_tiles, int n_tiles, int k_split, int x_packed) {
   constexpr int U = 8 / RT;  // k-tiles per group: 8 weight tiles (8 KB) per group and wave; two groups are in flight
   extern __shared__ float red[];  // [wave, or group of waves with the same row tiles][RT][MT][4][64]
   const int lane = threadIdx.x & 63, waves = blockDim.x >> 6;
@@ -99,12 +99,16 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
     const char* w_wave = reinterpret_cast<const char*>(wp) + static_cast<size_t>(row_tile) * w_tile_row;
     const uint32_t w_lane = lane * 16u;
     const char* x_bytes = reinterpret_cast<const char*>(x);
+    const uint32_t x_step = x_packed ? 1024u : 64u;  // bytes from a k-tile's operand to the next
     uint32_t x_lane[MT];
     bool x_row[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       x_row[mt] = mt * 16 + r < rows;
-      x_lane[mt] = static_cast<uint32_t>(mt * 16 + r) * static_cast<uint32_t>(k) * 2u + g * 16u;
+      // row-major x: row mt * 16 + r, 16 bytes at k = g * 8 of the k-tile.  Packed x ([row tile][k / 8][16 rows][8]):
+      // the k-tile's operand is 1 KB of consecutive bytes, lane after lane, as the weights' is.
+      x_lane[mt] = x_packed ? static_cast<uint32_t>(mt) * static_cast<uint32_t>(k) * 32u + lane * 16u
+                            : static_cast<uint32_t>(mt * 16 + r) * static_cast<uint32_t>(k) * 2u + g * 16u;
     }
     const bool ragged = (k & 31) != 0;  // the last k-tile reaches beyond x's row
     const uintx4 zero = {0u, 0u, 0u, 0u};
@@ -114,7 +118,7 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
     uintx4 a0[RT][U], a1[RT][U], b0[MT][U], b1[MT][U];
     auto fetch = [&](int kt, uintx4 (&a)[RT][U], uintx4 (&b)[MT][U]) {
       const char* w_at = w_wave + static_cast<size_t>(kt) * 1024;
-      const char* x_at = x_bytes + static_cast<size_t>(kt) * 64;
+      const char* x_at = x_bytes + static_cast<size_t>(kt) * x_step;
       if (kt + U <= kt1 && row_tile + RT <= n_tiles) {  // the whole group exists: no test per load
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
@@ -136,7 +140,7 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
           for (int u = 0; u < U; ++u) b[mt][u] = zero;
           if (x_row[mt]) {
 #pragma unroll
-            for (int u = 0; u < U; ++u) b[mt][u] = *reinterpret_cast<const uintx4*>(x_at + x_lane[mt] + u * 64u);
+            for (int u = 0; u < U; ++u) b[mt][u] = *reinterpret_cast<const uintx4*>(x_at + x_lane[mt] + u * x_step);
           }
         }
       } else {
@@ -146,7 +150,7 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
           for (int u = 0; u < U; ++u) {
             const bool inside = !ragged || (kt + u) * 32 + g * 8 < k;
             b[mt][u] = (kt + u < kt1 && x_row[mt] && inside)
-                           ? *reinterpret_cast<const uintx4*>(x_at + x_lane[mt] + u * 64u) : zero;
+                           ? *reinterpret_cast<const uintx4*>(x_at + x_lane[mt] + u * x_step) : zero;
           }
       }
     };
@@ -237,7 +241,7 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
 
 template <int MT, int RT, typename TY, bool GATED>
 int launch_skinny(const void* x, const void* wp, void* y, int rows, int outs, int k, int k_tiles, int n_tiles,
-                  hipStream_t stream) {
+                  int x_packed, hipStream_t stream) {
   // Enough waves to keep every CU's memory pipe full: k is split over the waves of a block when there are few row
   // tiles - down to short parts of k while the waves are very few, and further only while a wave keeps enough k-tiles
   // for two rounds of its double-buffered loop (measured: 1,536 waves of 32 k-tiles beat 3,072 of 16).
@@ -256,28 +260,28 @@ int launch_skinny(const void* x, const void* wp, void* y, int rows, int outs, in
   const size_t lds = k_split > 1 ? sets * RT * MT * 4 * 64 * sizeof(float) : 0;
   linear_skinny_kernel<MT, RT, TY, GATED><<<blocks, waves * 64, lds, stream>>>(
       static_cast<const bf16_t*>(x), static_cast<const uintx4*>(wp), static_cast<TY*>(y), rows, outs, k, k_tiles,
-      n_tiles, k_split);
+      n_tiles, k_split, x_packed);
   return AKV_LAUNCH_STATUS();
 }
 
 template <typename TY, bool GATED>
 int dispatch_skinny(const void* x, const void* wp, void* y, int rows, int outs, int k, int k_tiles, int n_tiles,
-                    hipStream_t stream) {
+                    int x_packed, hipStream_t stream) {
   switch ((rows + 15) / 16) {
     case 1:
       // two row tiles per wave halve the activation loads per weight byte; that pays with several rows of x and
       // enough row tiles that the waves stay many (measured at 384 row tiles: 12.7 -> 11.5 us at 8 rows)
       if (GATED || (rows >= 4 && n_tiles >= 384 && n_tiles < 2048))
-        return launch_skinny<1, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
-      return launch_skinny<1, GATED ? 2 : 1, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
-    case 2: return launch_skinny<2, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+        return launch_skinny<1, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
+      return launch_skinny<1, GATED ? 2 : 1, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
+    case 2: return launch_skinny<2, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
     // four row tiles per wave where that still leaves a thousand waves, two otherwise
     case 3:
-      return n_tiles >= 512 ? launch_skinny<3, 4, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream)
-                            : launch_skinny<3, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+      return n_tiles >= 512 ? launch_skinny<3, 4, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream)
+                            : launch_skinny<3, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
     case 4:
-      return n_tiles >= 512 ? launch_skinny<4, 4, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream)
-                            : launch_skinny<4, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+      return n_tiles >= 512 ? launch_skinny<4, 4, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream)
+                            : launch_skinny<4, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
     default: return -2;
   }
 }
@@ -469,17 +473,36 @@ int launch_wide(const void* x, const void* wp, void* y, int rows, int outs, int 
   return AKV_LAUNCH_STATUS();
 }
 
+// x [rows, k] row-major -> [tile of 16 rows][k / 8][16 rows][8]: a thread moves 16 bytes; consecutive threads read
+// consecutive pieces of a row.  Rows beyond `rows` of the last tile are not written (their lanes never load them).
+__global__ void pack_rows_kernel(const uintx4* __restrict__ x, uintx4* __restrict__ xp, int rows, int pieces) {
+  const long index = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (index >= static_cast<long>(rows) * pieces) return;
+  const int row = static_cast<int>(index / pieces), piece = static_cast<int>(index % pieces);
+  xp[(static_cast<long>(row / 16) * pieces + piece) * 16 + row % 16] = x[index];
+}
+
 }  // namespace
+
+extern "C" int akv_pack_rows(const void* x, void* xp, int rows, int k, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if ((k & 7) != 0) return -2;
+  const long pieces = static_cast<long>(rows) * (k / 8);
+  pack_rows_kernel<<<static_cast<unsigned>((pieces + 255) / 256), 256, 0, stream>>>(
+      static_cast<const uintx4*>(x), static_cast<uintx4*>(xp), rows, k / 8);
+  return AKV_LAUNCH_STATUS();
+}
 
 namespace {
 template <bool GATED>
 int linear_packed(const void* x, const void* wp, void* y, int y_dtype, int rows, int outs, int k, int n_tiles,
-                  int k_tiles, hipStream_t stream) {
+                  int k_tiles, int x_packed, hipStream_t stream) {
   if (rows <= 64) {
-    if (y_dtype == kF32) return dispatch_skinny<float, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
-    if (y_dtype == kBF16) return dispatch_skinny<bf16_t, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+    if (y_dtype == kF32) return dispatch_skinny<float, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
+    if (y_dtype == kBF16) return dispatch_skinny<bf16_t, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
     return -1;
   }
+  if (x_packed) return -2;  // only the products of up to 64 rows read packed activations
   if (y_dtype == kF32) return launch_wide<float, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
   if (y_dtype == kBF16) return launch_wide<bf16_t, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
   return -1;
@@ -488,18 +511,19 @@ int linear_packed(const void* x, const void* wp, void* y, int y_dtype, int rows,
 
 // x [rows, k] bfloat16 row-major; wp the packed weight of `n_tiles` x `k_tiles` tiles; y [rows, outs] bfloat16 or
 // float32.  k must be a multiple of 8 (a lane's 16-byte read of x must lie inside or outside the row as a whole).
+// `x_packed` (rows <= 64 only): x is not row-major but [tile of 16 rows][k / 8][16 rows][8], what akv_pack_rows writes.
 extern "C" int akv_linear_packed(const void* x, const void* wp, void* y, int y_dtype, int rows, int outs, int k,
-                                 int n_tiles, int k_tiles, hipStream_t stream) {
+                                 int n_tiles, int k_tiles, int x_packed, hipStream_t stream) {
   if (rows <= 0 || outs <= 0) return 0;
   if ((k & 7) != 0 || n_tiles * 16 < outs || k_tiles * 32 < k) return -2;
-  return linear_packed<false>(x, wp, y, y_dtype, rows, outs, k, n_tiles, k_tiles, stream);
+  return linear_packed<false>(x, wp, y, y_dtype, rows, outs, k, n_tiles, k_tiles, x_packed, stream);
 }
 
 // The gated pair in one pass: wp holds 2 * inter / 16 row tiles, gate tile t at 2t and up tile t at 2t + 1;
 // y [rows, inter] = silu(x Wgate^T) * (x Wup^T).  inter must be a multiple of 16.
 extern "C" int akv_linear_packed_swiglu(const void* x, const void* wp, void* y, int y_dtype, int rows, int inter,
-                                        int k, int n_tiles, int k_tiles, hipStream_t stream) {
+                                        int k, int n_tiles, int k_tiles, int x_packed, hipStream_t stream) {
   if (rows <= 0 || inter <= 0) return 0;
   if ((k & 7) != 0 || (inter & 15) != 0 || n_tiles * 8 != inter || k_tiles * 32 < k) return -2;
-  return linear_packed<true>(x, wp, y, y_dtype, rows, inter, k, n_tiles, k_tiles, stream);
+  return linear_packed<true>(x, wp, y, y_dtype, rows, inter, k, n_tiles, k_tiles, x_packed, stream);
 }

@@ -89,6 +89,7 @@ class HipKernels:
         self.tune_products = tune_products     # 17..64 rows: own kernel or library, whichever is faster for the shape
         self._tuned = {}                       # (kind, outs, k, row tiles) -> "own" | "library"
         self._spacer = None                    # the buffer whose fill precedes every timed run
+        self._packed_rows = None               # where activations are repacked for the engine's own product
         self.device = torch.device(device)
         if self.device.type == "cuda" and self.device.index is None:
             self.device = torch.device("cuda", 0)
@@ -110,7 +111,8 @@ class HipKernels:
         self.one_wave_per_head = False  # True: every attention goes to the plain kernel, a wave per (token, head)
         for name in ("akv_embed", "akv_add_rmsnorm", "akv_rmsnorm_rows", "akv_copy_rows", "akv_gather_rows",
                      "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
-                     "akv_linear_tiled", "akv_linear_packed", "akv_linear_packed_swiglu", "akv_attention_rows", "akv_sample"):
+                     "akv_linear_tiled", "akv_linear_packed", "akv_linear_packed_swiglu", "akv_pack_rows",
+                     "akv_attention_rows", "akv_sample"):
             getattr(self.lib, name).restype = ctypes.c_int
 
     # ---- helpers -----------------------------------------------------------------------------------------
@@ -223,6 +225,21 @@ class HipKernels:
         return (row_major is not None and self.library_products_above is not None
                 and rows > self.library_products_above and out.dtype == torch.bfloat16)
 
+    PACK_ROWS_ABOVE = 16            # the engine's own product of more rows than this reads repacked activations
+    PACKED_ROWS_ELEMENTS = 64 * 65536
+
+    def _operand_rows(self, x, rows: int, k: int):
+        """What the engine's own product of up to 64 rows reads as x, and whether that is the repacked form.  With
+        several tiles of 16 rows the 16-byte gathers of a row-major x keep the vector memory pipe busier than the
+        weights do; one small kernel lays x out [tile of 16 rows][k / 8][16 rows][8] first (into one buffer that all
+        products on the stream share in turn), and an operand of the product is then 1 KB of consecutive bytes."""
+        if not self.PACK_ROWS_ABOVE < rows <= self.OWN_SKINNY_ROWS or (rows + 15) // 16 * 16 * k > self.PACKED_ROWS_ELEMENTS:
+            return x, 0
+        if self._packed_rows is None:
+            self._packed_rows = torch.empty(self.PACKED_ROWS_ELEMENTS, dtype=torch.bfloat16, device=self.device)
+        self._check(self.lib.akv_pack_rows(_ptr(x), _ptr(self._packed_rows), rows, k, self._stream()), "pack_rows")
+        return self._packed_rows, 1
+
     def _own_or_library(self, key: tuple, rows: int, own, library) -> None:
         """A product that may go to the library.  More than 64 rows: it does.  Up to 64 rows (the range of the skinny
         kernel, where neither side wins for every shape): whichever of the two is faster for a matrix of this shape
@@ -264,9 +281,10 @@ class HipKernels:
             self._dense(weight.data, "packed weight", torch.bfloat16)
 
             def own():
-                self._check(self.lib.akv_linear_packed(_ptr(x), _ptr(weight.data), _ptr(out), _code(out), rows,
+                operand, packed_rows = self._operand_rows(x, rows, weight.k)
+                self._check(self.lib.akv_linear_packed(_ptr(operand), _ptr(weight.data), _ptr(out), _code(out), rows,
                                                        weight.outs, weight.k, weight.n_tiles, weight.k_tiles,
-                                                       self._stream()), "linear")
+                                                       packed_rows, self._stream()), "linear")
             if self._library_product(rows, weight.row_major, out):
                 self._own_or_library(("linear", weight.outs, weight.k), rows, own,
                                      lambda: torch.mm(x, weight.row_major.t(), out=out))
@@ -311,18 +329,21 @@ class HipKernels:
             self._dense(scratch, "scratch", torch.bfloat16, (rows, 2 * weight.inter))
 
             def own():
-                self._check(self.lib.akv_linear_packed_swiglu(_ptr(x), _ptr(packed.data), _ptr(out), _code(out), rows,
-                                                              weight.inter, weight.k, packed.n_tiles, packed.k_tiles,
-                                                              self._stream()), "gated_linear")
+                operand, packed_rows = self._operand_rows(x, rows, weight.k)
+                self._check(self.lib.akv_linear_packed_swiglu(_ptr(operand), _ptr(packed.data), _ptr(out), _code(out),
+                                                              rows, weight.inter, weight.k, packed.n_tiles,
+                                                              packed.k_tiles, packed_rows, self._stream()),
+                            "gated_linear")
 
             def library():
                 torch.mm(x, weight.stacked.t(), out=scratch)
                 self.swiglu(scratch, out)
             self._own_or_library(("gated", weight.inter, weight.k), rows, own, library)
             return
-        self._check(self.lib.akv_linear_packed_swiglu(_ptr(x), _ptr(packed.data), _ptr(out), _code(out), rows,
+        operand, packed_rows = self._operand_rows(x, rows, weight.k)
+        self._check(self.lib.akv_linear_packed_swiglu(_ptr(operand), _ptr(packed.data), _ptr(out), _code(out), rows,
                                                       weight.inter, weight.k, packed.n_tiles, packed.k_tiles,
-                                                      self._stream()), "gated_linear")
+                                                      packed_rows, self._stream()), "gated_linear")
 
     def swiglu(self, gate_up, out):
         tokens, inter = out.shape
