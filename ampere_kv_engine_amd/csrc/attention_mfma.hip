@@ -44,6 +44,20 @@ __device__ __forceinline__ floatx4 mfma16(uintx4 a, uintx4 b, floatx4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
+// The maximum over the four lanes r, r + 16, r + 32 and r + 48, in all four of them: two lane swaps inside the vector
+// unit (halves of the wave, then rows of 16 lanes) instead of two trips through LDS.
+__device__ __forceinline__ float max_over_halves(float v) {
+  const uint32_t bits = __float_as_uint(v);
+  const auto swapped = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+  return fmaxf(__uint_as_float(swapped[0]), __uint_as_float(swapped[1]));
+}
+__device__ __forceinline__ float max_over_row_pairs(float v) {
+  const uint32_t bits = __float_as_uint(v);
+  const auto swapped = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+  return fmaxf(__uint_as_float(swapped[0]), __uint_as_float(swapped[1]));
+}
+__device__ __forceinline__ float max_over_groups(float v) { return max_over_row_pairs(max_over_halves(v)); }
+
 struct Args {
   const bf16_t* q;            // [tokens, q_heads * D]
   const bf16_t* k_pages;      // [pages, kv_heads, page_size, D]
@@ -309,8 +323,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
       }
       float top = fmaxf(fmaxf(fmaxf(s[nq][0][0], s[nq][0][1]), fmaxf(s[nq][0][2], s[nq][0][3])),
                         fmaxf(fmaxf(s[nq][1][0], s[nq][1][1]), fmaxf(s[nq][1][2], s[nq][1][3])));
-      top = fmaxf(top, __shfl_xor(top, 16, 64));
-      top = fmaxf(top, __shfl_xor(top, 32, 64));
+      top = max_over_groups(top);
       const float m_new = fmaxf(m[nq], top * a.scale_log2);   // the scale is positive: max commutes with it
       const float m_safe = m_new == -INFINITY ? 0.f : m_new;  // nothing seen yet: every weight is 0, no NaN
       correction[nq] = __builtin_amdgcn_exp2f(m[nq] - m_safe);
@@ -427,12 +440,18 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
 // lanes of a group then fall into different banks.  Pages must hold at least 8 tokens (an aligned run of 8 keys of a
 // value row is one 16-byte piece).
 constexpr int kSharedWaves = 4;
-constexpr int KROW = D + 8;   // bfloat16 per key row in LDS
-constexpr int VROW = 32 + 8;  // bfloat16 per value row in LDS
+// Rows in LDS, in bfloat16.  16 lanes read 16 bytes each from 16 consecutive rows; such a read runs at full rate when
+// the rows are 2 (mod 4) pieces of 16 bytes apart (measured: 1.5 times slower with an odd number of pieces, worse
+// with a multiple of 4), so rows are padded up to that: keys 2 * D bytes + 0 or 32, values 64 bytes + 32.
+constexpr int KROW = D + ((D / 8) % 4 == 2 ? 0 : 16);
+constexpr int VROW = 32 + 16;
 constexpr float kLazy = 8.f;  // the exponentials' reference point trails the maximum by at most 2^kLazy
 
-template <int NQ>
-__global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) void attention_shared_kernel(const Args a) {
+// SP: pages per step of 32 keys (4: pages of 8 tokens, 2: of 16, 1: of 32 or more) - with it the page arithmetic of a
+// step is known when compiling.
+template <int NQ, int SP>
+__global__ __launch_bounds__(64 * kSharedWaves, D <= 128 ? (NQ == 1 ? 3 : 2) : 1) void attention_shared_kernel(const Args a) {
+  const int page_shift = SP == 4 ? 3 : (SP == 2 ? 4 : a.page_shift);
   __shared__ __align__(16) bf16_t k_lds[2][32 * KROW];
   __shared__ __align__(16) bf16_t v_lds[2][D * VROW];
   __shared__ int bad_page;
@@ -454,7 +473,7 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
   t.first_pos = __builtin_amdgcn_readfirstlane(t.first_pos);
   const int kvh = (rank % heads) / a.head_groups, hg = (rank % heads) % a.head_groups;
   const uintx4 zero = uintx4{0u, 0u, 0u, 0u};
-  const int page_mask = (1 << a.page_shift) - 1;
+  const int page_mask = (1 << page_shift) - 1;
   if (tid == 0) bad_page = 0;
 
   // this wave's tile inside the block's, and this lane's columns
@@ -492,7 +511,7 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
   floatx4 l[NQ], o[NQ][DT];
 #pragma unroll
   for (int nq = 0; nq < NQ; ++nq) {
-    m[nq] = -INFINITY;
+    m[nq] = col_valid[nq] ? -INFINITY : 1e30f;  // (a column that is no (token, head) pair: all its weights are 0)
     l[nq] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[nq][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -502,11 +521,11 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
   const int* table = a.block_table + static_cast<long>(t.request) * a.table_width;
   const char* k_bytes = reinterpret_cast<const char*>(a.k_pages);
   const char* v_bytes = reinterpret_cast<const char*>(a.v_pages);
-  const uint32_t page_bytes = static_cast<uint32_t>(a.kv_heads) * D * 2u << a.page_shift;
-  const uint32_t head_bytes = static_cast<uint32_t>(kvh) * D * 2u << a.page_shift;
+  const uint32_t page_bytes = static_cast<uint32_t>(a.kv_heads) * D * 2u << page_shift;
+  const uint32_t head_bytes = static_cast<uint32_t>(kvh) * D * 2u << page_shift;
   constexpr int kKeyPieces = 32 * (D / 8), kValuePieces = D * 4;
   constexpr int PK = (kKeyPieces + 255) / 256, PV = (kValuePieces + 255) / 256;
-  const int run_shift = min(2, a.page_shift - 3);  // aligned runs of 8 keys of this step in one page row: 1, 2 or 4
+  const int run_shift = min(2, page_shift - 3);  // aligned runs of 8 keys of this step in one page row: 1, 2 or 4
   const std::true_type checked{};
   const std::false_type unchecked{};
   bool bad = false;
@@ -515,7 +534,7 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
   // in LDS.  What changes - the step's 1, 2 or 4 page ids - is the same for every thread: it is read and checked with
   // scalar instructions, one step before the loads that need it are issued, so no load waits for the table entry
   // that addresses it and no lane spends arithmetic on it.
-  const int step_pages = max(1, 32 >> a.page_shift), span = min(32, 1 << a.page_shift);
+  constexpr int step_pages = SP, span = 32 / SP;  // (span: keys of a step in one page)
   int k_sel[PK], v_sel[PV];             // which of the step's pages holds the piece
   uint32_t k_from[PK], v_from[PV];      // byte offset inside the page, without what the step's first key adds
   uint32_t k_to[PK], v_to[PV];          // element offset in the LDS buffer
@@ -524,7 +543,7 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
   for (int p = 0; p < PK; ++p) {
     const int c = p * 256 + tid, key = c / (D / 8);
     k_mine[p] = kKeyPieces % 256 == 0 || c < kKeyPieces;  // (known when compiling for the usual head sizes)
-    k_sel[p] = step_pages == 1 ? 0 : key >> a.page_shift;
+    k_sel[p] = step_pages == 1 ? 0 : key >> page_shift;
     k_from[p] = head_bytes + (c % (D / 8)) * 16u + static_cast<uint32_t>(key & page_mask) * (D * 2u);
     k_to[p] = (((key >> 2) & 1) * 16 + (key >> 3) * 4 + (key & 3)) * KROW + (c % (D / 8)) * 8;  // tile j, row rho
   }
@@ -534,10 +553,26 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
     const int run = (c / D) >> run_shift, within = c - ((run * D) << run_shift);
     const int dim = within >> run_shift, piece = (run << run_shift) + (within & ((1 << run_shift) - 1));
     v_mine[p] = kValuePieces % 256 == 0 || c < kValuePieces;
-    v_sel[p] = step_pages == 1 ? 0 : (piece * 8) >> a.page_shift;
-    v_from[p] = head_bytes + (static_cast<uint32_t>(dim) << (a.page_shift + 1)) + static_cast<uint32_t>((piece * 8) & page_mask) * 2u;
+    v_sel[p] = step_pages == 1 ? 0 : (piece * 8) >> page_shift;
+    v_from[p] = head_bytes + (static_cast<uint32_t>(dim) << (page_shift + 1)) + static_cast<uint32_t>((piece * 8) & page_mask) * 2u;
     v_to[p] = dim * VROW + piece * 8;
   }
+  // With the usual sizes (a head of 128 and pages of 16 or more, say) all pieces that the wave moves in one turn p
+  // come from the same page of the step.  Then the page's address stays in scalar registers and a load takes the
+  // thread's constant 32-bit offset beside it: no address arithmetic per lane and step.
+  int k_page[PK], v_page[PV];
+  bool same_page = true;
+#pragma unroll
+  for (int p = 0; p < PK; ++p) {
+    k_page[p] = __builtin_amdgcn_readfirstlane(k_sel[p]);
+    same_page = same_page && (k_sel[p] == k_page[p] || !k_mine[p]);
+  }
+#pragma unroll
+  for (int p = 0; p < PV; ++p) {
+    v_page[p] = __builtin_amdgcn_readfirstlane(v_sel[p]);
+    same_page = same_page && (v_sel[p] == v_page[p] || !v_mine[p]);
+  }
+  same_page = __all(same_page);
   // key of a piece relative to the step's first: only steps at the edge of the range ask, so it is not kept
   auto k_key = [&](int p) { return (p * 256 + tid) / (D / 8); };
   auto v_key = [&](int p) {
@@ -547,14 +582,14 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
   // The page ids of the step at `base`.  CHECK: the step may reach outside [range_lo, range_hi]; pages wholly
   // outside are not looked up (their entries may lie beyond the table).
   auto page_wanted = [&](int base, int i) {
-    const int first = base + (i << a.page_shift);
+    const int first = base + (i << page_shift);
     return first <= range_hi && first + span - 1 >= range_lo;
   };
   auto lookup = [&](int base, int (&pages)[4], auto check) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       pages[i] = 0;
-      if (i < step_pages && (!decltype(check)::value || page_wanted(base, i))) pages[i] = table[(base >> a.page_shift) + i];
+      if (i < step_pages && (!decltype(check)::value || page_wanted(base, i))) pages[i] = table[(base >> page_shift) + i];
     }
   };
   auto fetch = [&](int base, const int (&pages)[4], uintx4 (&kst)[PK], uintx4 (&vst)[PV], auto check) {
@@ -578,7 +613,10 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
         wanted = wanted && key >= range_lo && key <= range_hi;
       }
       kst[p] = zero;
-      if (wanted) kst[p] = *reinterpret_cast<const uintx4*>(k_bytes + of(k_sel[p]) + in_page * (D * 2u) + k_from[p]);
+      if (wanted) {
+        if (same_page) kst[p] = *reinterpret_cast<const uintx4*>(k_bytes + of(k_page[p]) + in_page * (D * 2u) + k_from[p]);
+        else kst[p] = *reinterpret_cast<const uintx4*>(k_bytes + of(k_sel[p]) + in_page * (D * 2u) + k_from[p]);
+      }
     }
 #pragma unroll
     for (int p = 0; p < PV; ++p) {
@@ -591,7 +629,8 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
       }
       uintx4 v = zero;
       if (wanted) {
-        v = *reinterpret_cast<const uintx4*>(v_bytes + of(v_sel[p]) + in_page * 2u + v_from[p]);
+        if (same_page) v = *reinterpret_cast<const uintx4*>(v_bytes + of(v_page[p]) + in_page * 2u + v_from[p]);
+        else v = *reinterpret_cast<const uintx4*>(v_bytes + of(v_sel[p]) + in_page * 2u + v_from[p]);
         if (decltype(check)::value && live < 8) {  // slots beyond the last key were never written: anything, NaN included
           uint32_t keep[4];
 #pragma unroll
@@ -600,6 +639,36 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
         }
       }
       vst[p] = v;
+    }
+  };
+  // The same for a step that lies inside the range as a whole, when every turn's pieces come from one page: the
+  // page's address is scalar, a load adds the thread's constant offset, and nothing is tested per piece.
+  auto fetch_inside = [&](int base, const int (&pages)[4], uintx4 (&kst)[PK], uintx4 (&vst)[PV]) {
+    size_t at[SP];
+#pragma unroll
+    for (int i = 0; i < SP; ++i) {
+      int page = pages[i];
+      if (static_cast<uint32_t>(page) >= static_cast<uint32_t>(a.num_pages)) {
+        bad = true;
+        page = 0;
+      }
+      at[i] = static_cast<size_t>(page) * page_bytes;
+    }
+    auto of = [&](int sel) {
+      if constexpr (SP == 1) return at[0];
+      else if constexpr (SP == 2) return sel == 0 ? at[0] : at[1];
+      else return sel == 0 ? at[0] : (sel == 1 ? at[1] : (sel == 2 ? at[2] : at[3]));
+    };
+    const uint32_t in_page = SP == 1 ? static_cast<uint32_t>(base & page_mask) : 0u;
+#pragma unroll
+    for (int p = 0; p < PK; ++p) {
+      kst[p] = zero;
+      if (k_mine[p]) kst[p] = *reinterpret_cast<const uintx4*>(k_bytes + of(k_page[p]) + in_page * (D * 2u) + k_from[p]);
+    }
+#pragma unroll
+    for (int p = 0; p < PV; ++p) {
+      vst[p] = zero;
+      if (v_mine[p]) vst[p] = *reinterpret_cast<const uintx4*>(v_bytes + of(v_page[p]) + in_page * 2u + v_from[p]);
     }
   };
   auto stash = [&](int buffer, const uintx4 (&kst)[PK], const uintx4 (&vst)[PV]) {
@@ -611,9 +680,9 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
       if (v_mine[p]) *reinterpret_cast<uintx4*>(&v_lds[buffer][v_to[p]]) = vst[p];
   };
 
-  // One step of 32 keys from LDS.  MASK: some column does not see the whole step.
-  auto step = [&](int base, int buffer, auto mask) {
-    floatx4 s[NQ][2];
+  // ---- the parts of a step of 32 keys -----------------------------------------------------------------------------------
+  // scores: S^T = K . Q^T from the keys in LDS
+  auto scores = [&](int buffer, floatx4 (&s)[NQ][2]) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
 #pragma unroll
@@ -627,28 +696,31 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
         for (int nq = 0; nq < NQ; ++nq) s[nq][j] = mfma16(keys, qreg[nq][kt], s[nq][j]);
       }
     }
-    uintx4 preg[NQ], plow[NQ];
-    float correction[NQ];
+  };
+  // keys that a column does not see count as -inf
+  auto hide = [&](int base, floatx4 (&s)[NQ][2]) {
+#pragma unroll
+    for (int nq = 0; nq < NQ; ++nq)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = base + g * 8 + j * 4 + i;
+          const bool seen = col_valid[nq] && key <= col_pos[nq] && key >= col_low[nq];
+          if (!seen) s[nq][j][i] = -INFINITY;
+        }
+  };
+  // The reference point of the exponentials follows the maximum lazily: it moves only when the maximum has grown by
+  // more than 2^kLazy, so weights stay below 2^kLazy (harmless in float32 sums, and bfloat16 keeps its relative
+  // precision) and the accumulators are rescaled a few times per row instead of at every step.  Returns whether
+  // some column's reference moved; `correction` is what its accumulators are to be multiplied by then.
+  auto follow = [&](const floatx4 (&s)[NQ][2], float (&correction)[NQ]) {
     bool rescale = false;
 #pragma unroll
     for (int nq = 0; nq < NQ; ++nq) {
-      if (decltype(mask)::value) {
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int key = base + g * 8 + j * 4 + i;
-            const bool seen = col_valid[nq] && key <= col_pos[nq] && key >= col_low[nq];
-            if (!seen) s[nq][j][i] = -INFINITY;
-          }
-      }
       float top = fmaxf(fmaxf(fmaxf(s[nq][0][0], s[nq][0][1]), fmaxf(s[nq][0][2], s[nq][0][3])),
                         fmaxf(fmaxf(s[nq][1][0], s[nq][1][1]), fmaxf(s[nq][1][2], s[nq][1][3])));
-      top = fmaxf(top, __shfl_xor(top, 16, 64));
-      top = fmaxf(top, __shfl_xor(top, 32, 64));
-      // The reference point of the exponentials follows the maximum lazily: it moves only when the maximum has grown
-      // by more than 2^kLazy, so weights stay below 2^kLazy (harmless in float32 sums, and bfloat16 keeps its relative
-      // precision) and the accumulators are rescaled a few times per row instead of at every step.
+      top = max_over_groups(top);
       const float scaled = top * a.scale_log2;                 // the scale is positive: max commutes with it
       const bool moved = scaled > m[nq] + kLazy;               // also the first keys seen: m is -inf
       const float m_new = moved ? scaled : m[nq];
@@ -656,14 +728,35 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
       correction[nq] = moved ? __builtin_amdgcn_exp2f(m[nq] - m_safe) : 1.f;
       rescale = rescale || moved;
       m[nq] = m_new;
-      // A weight enters the second product as two bfloat16 numbers (p = high + low, 16 bits of mantissa together),
-      // so that the weighted sum does not carry the 2^-9 relative error of a single bfloat16.
+    }
+    return __any(rescale);
+  };
+  auto rescale = [&](const float (&correction)[NQ]) {
+#pragma unroll
+    for (int nq = 0; nq < NQ; ++nq) {
+      l[nq] *= correction[nq];
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o[nq][dt] *= correction[nq];
+    }
+  };
+  // Exponents of the weights, base 2, relative to the reference point.
+  auto exponents = [&](const floatx4 (&s)[NQ][2], float (&t)[NQ][8]) {
+#pragma unroll
+    for (int nq = 0; nq < NQ; ++nq) {
+      const float m_safe = m[nq] == -INFINITY ? 0.f : m[nq];   // nothing seen yet: every weight is 0, no NaN
+#pragma unroll
+      for (int e = 0; e < 8; ++e) t[nq][e] = fmaf(s[nq][e >> 2][e & 3], a.scale_log2, -m_safe);
+    }
+  };
+  // A weight enters the second product as two bfloat16 numbers (p = high + low, 16 bits of mantissa together), so
+  // that the weighted sum does not carry the 2^-9 relative error of a single bfloat16.
+  auto weights = [&](const float (&t)[NQ][8], uintx4 (&preg)[NQ], uintx4 (&plow)[NQ]) {
+#pragma unroll
+    for (int nq = 0; nq < NQ; ++nq) {
       uint32_t high[4], low[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        floatx2 p;
-        p[0] = __builtin_amdgcn_exp2f(fmaf(s[nq][e >> 1][(e & 1) * 2], a.scale_log2, -m_safe));
-        p[1] = __builtin_amdgcn_exp2f(fmaf(s[nq][e >> 1][(e & 1) * 2 + 1], a.scale_log2, -m_safe));
+        const floatx2 p = {__builtin_amdgcn_exp2f(t[nq][2 * e]), __builtin_amdgcn_exp2f(t[nq][2 * e + 1])};
         high[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(p, bf16x2));
         const floatx2 rest = {p[0] - __uint_as_float(high[e] << 16), p[1] - __uint_as_float(high[e] & 0xffff0000u)};
         low[e] = __builtin_bit_cast(uint32_t, __builtin_convertvector(rest, bf16x2));
@@ -671,15 +764,9 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
       preg[nq] = uintx4{high[0], high[1], high[2], high[3]};
       plow[nq] = uintx4{low[0], low[1], low[2], low[3]};
     }
-    if (__any(rescale)) {
-#pragma unroll
-      for (int nq = 0; nq < NQ; ++nq) {
-        l[nq] *= correction[nq];
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) o[nq][dt] *= correction[nq];
-      }
-    }
-    // O^T += V^T . P^T, and the weights' sums from the same two-part weights: a row of ones beside the value rows
+  };
+  // O^T += V^T . P^T, and the weights' sums from the same two-part weights: a row of ones beside the value rows
+  auto accumulate = [&](int buffer, const uintx4 (&preg)[NQ], const uintx4 (&plow)[NQ]) {
 #pragma unroll
     for (int nq = 0; nq < NQ; ++nq) l[nq] = mfma16(ones, plow[nq], mfma16(ones, preg[nq], l[nq]));
 #pragma unroll
@@ -688,6 +775,37 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
 #pragma unroll
       for (int nq = 0; nq < NQ; ++nq) o[nq][dt] = mfma16(values, plow[nq], mfma16(values, preg[nq], o[nq][dt]));
     }
+  };
+  // One step.  MASK: some column does not see the whole step.
+  // Without a mask the maximum is not looked for at all as long as no exponent of the wave exceeds kLazy: then no
+  // reference point would move, and the exponents are the ones the weights need.  (A column that has seen nothing
+  // yet has the reference -inf and asks for the search; columns that are no (token, head) pair start with a huge
+  // reference and never ask.)
+  auto step = [&](int base, int buffer, auto mask) {
+    floatx4 s[NQ][2];
+    float t[NQ][8], correction[NQ];
+    uintx4 preg[NQ], plow[NQ];
+    scores(buffer, s);
+    if (decltype(mask)::value) {
+      hide(base, s);
+      if (follow(s, correction)) rescale(correction);
+      exponents(s, t);
+    } else {
+      exponents(s, t);
+      bool search = false;
+#pragma unroll
+      for (int nq = 0; nq < NQ; ++nq) {
+        const float top = fmaxf(fmaxf(fmaxf(t[nq][0], t[nq][1]), fmaxf(t[nq][2], t[nq][3])),
+                                fmaxf(fmaxf(t[nq][4], t[nq][5]), fmaxf(t[nq][6], t[nq][7])));
+        search = search || top > kLazy || m[nq] == -INFINITY;
+      }
+      if (__any(search)) {
+        if (follow(s, correction)) rescale(correction);
+        exponents(s, t);
+      }
+    }
+    weights(t, preg, plow);
+    accumulate(buffer, preg, plow);
   };
 
   uintx4 kst[PK], vst[PV];
@@ -707,8 +825,22 @@ __global__ __launch_bounds__(64 * kSharedWaves, (NQ == 1 && D <= 128) ? 3 : 1) v
   if (first_base + 32 <= range_hi) lookup_step(first_base + 32);
   stash(0, kst, vst);
   __syncthreads();
+  // Steps before `calm_to` (and from `calm_from` on, with a window) are calm: the step, the next one that is
+  // fetched meanwhile and the one after it whose pages are looked up all lie inside the range, and every wave sees
+  // all 32 keys - nothing is tested in them.
+  const int calm_from = a.window > 0 ? (max(range_lo, last_pos - a.window + 1) + 31) & ~31 : first_base;
+  // base < calm_to: base + 95 <= range_hi, and base + 31 <= the block's first position
+  const int calm_to = same_page ? min(range_hi - 94, t.first_pos - 30) : first_base;
   int buffer = 0;
   for (int base = first_base; base <= range_hi; base += 32, buffer ^= 1) {
+    if (base >= calm_from && base < calm_to) {
+      fetch_inside(base + 32, pages, kst, vst);
+      lookup(base + 64, pages, unchecked);
+      if (wave_active) step(base, buffer, unchecked);
+      stash(buffer ^ 1, kst, vst);
+      __syncthreads();
+      continue;
+    }
     const bool more = base + 32 <= range_hi;
     if (more) fetch_step(base + 32);
     if (base + 64 <= range_hi) lookup_step(base + 64);
@@ -825,11 +957,12 @@ template <int NQ>
 int launch(const Args& a, int tiles, bool shared, hipStream_t stream) {
   dim3 grid(tiles, a.kv_heads * a.head_groups, a.num_splits);
   if (shared) {
-    if constexpr (NQ == 1) {  // one tile of 16 columns per wave: three blocks fit a compute unit
-      attention_shared_kernel<1><<<dim3(tiles * a.kv_heads * a.head_groups), 64 * kSharedWaves, 0, stream>>>(a);
-      return AKV_LAUNCH_STATUS();
-    }
-    return -2;
+    const dim3 blocks(tiles * a.kv_heads * a.head_groups);
+    if (a.page_shift >= 5) attention_shared_kernel<NQ, 1><<<blocks, 64 * kSharedWaves, 0, stream>>>(a);
+    else if (a.page_shift == 4) attention_shared_kernel<NQ, 2><<<blocks, 64 * kSharedWaves, 0, stream>>>(a);
+    else if (a.page_shift == 3) attention_shared_kernel<NQ, 4><<<blocks, 64 * kSharedWaves, 0, stream>>>(a);
+    else return -2;
+    return AKV_LAUNCH_STATUS();
   }
   if (a.num_splits == 1) grid.x = (tiles + 1) / 2;  // a block takes a late tile and an early one
   if (a.num_splits > 1) {
@@ -863,7 +996,7 @@ extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
   while ((1 << page_shift) < page_size) ++page_shift;
   if (page_size < 4 || (1 << page_shift) != page_size || q_heads % kv_heads != 0 ||
       heads_per_tile * tokens_per_tile > 16 * nq || kv_heads * head_groups > 65535 || num_splits > 65535 ||
-      num_splits < 1 || (single_tokens && tiles != seq_count) || (shared && (page_size < 8 || num_splits != 1 || nq != 1)))
+      num_splits < 1 || (single_tokens && tiles != seq_count) || (shared && (page_size < 8 || num_splits != 1)))
     return -2;
   Args a;
   a.q = static_cast<const bf16_t*>(q);

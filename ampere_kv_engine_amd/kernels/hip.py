@@ -109,6 +109,8 @@ class HipKernels:
         self.decode_max_splits = 128    # and no more than this many (four waves of the merge share them)
         self.share_prompt_tiles = True  # prompt portions: blocks of four waves share keys and values through LDS
         self.one_wave_per_head = False  # True: every attention goes to the plain kernel, a wave per (token, head)
+        self.wide_prompt_tiles = None   # such blocks with 32 columns per wave instead of 16: None = by the step's size
+        self.compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
         for name in ("akv_embed", "akv_add_rmsnorm", "akv_rmsnorm_rows", "akv_copy_rows", "akv_gather_rows",
                      "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
                      "akv_linear_tiled", "akv_linear_packed", "akv_linear_packed_swiglu", "akv_pack_rows",
@@ -462,6 +464,21 @@ class HipKernels:
             self._stream()),
             "attention")
 
+    def _wide_shared_tiles(self, ctx, first, q_heads, kv_heads) -> bool:
+        """Whether the prompt portions of the step go to blocks of 4 x 32 columns rather than 4 x 16.  The wide
+        blocks do a step of 32 keys for twice the columns with the same loads and bookkeeping (a fifth to a quarter
+        faster where they fill the device), but there are half as many of them, and two per compute unit instead of
+        three: they are taken when there are two or more per compute unit and the keys are many (measured on
+        prompts of 512 to 8,192 tokens after histories of 0 to 15,360)."""
+        group = q_heads // kv_heads
+        heads_per_tile = min(group, 32)
+        per_block = 4 * (32 // heads_per_tile)
+        starts = ctx.host_q_start
+        blocks = sum((starts[r + 1] - starts[r] + per_block - 1) // per_block for r in range(first, ctx.num_seqs))
+        blocks *= kv_heads * ((group + heads_per_tile - 1) // heads_per_tile)
+        units = self.compute_units
+        return blocks >= 2 * units and (ctx.max_seq_len >= 4096 or 2 * blocks >= 5 * units)
+
     def attention(self, q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out):
         tokens = q.shape[0]
         self._dense(q, "q", None, (tokens, q_heads * head_dim))
@@ -483,7 +500,12 @@ class HipKernels:
                 self._attention_mfma(*common, 0, decodes, 1, True)
             if ctx.num_seqs > decodes:
                 shared = page_size >= 8 and self.share_prompt_tiles
-                nq = 1 if shared or head_dim > 128 else 2
+                nq = 2 if head_dim <= 128 else 1
+                if shared and nq == 2:
+                    wide = self.wide_prompt_tiles
+                    if wide is None:
+                        wide = self._wide_shared_tiles(ctx, decodes, q_heads, kv_heads)
+                    nq = 2 if wide else 1
                 self._attention_mfma(*common, decodes, ctx.num_seqs - decodes, nq, False, shared=shared)
             return
         self._dense(ctx.seq_of_token, "seq_of_token", torch.int32, (tokens,))

@@ -410,26 +410,26 @@ def test_attention(hip, ref, dtype, q_heads, kv_heads, dim, page_size, portions,
     torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(dtype))
 
 
-@pytest.mark.parametrize("shared", [True, False])
+@pytest.mark.parametrize("shared", ["narrow", "wide", False])
 @pytest.mark.parametrize("q_heads,kv_heads,dim,page_size", [(8, 2, 128, 16), (6, 1, 32, 8), (8, 4, 64, 64), (3, 1, 256, 32),
                                                             (5, 5, 80, 16), (40, 2, 64, 8), (4, 2, 16, 128)])
 @pytest.mark.parametrize("portions", [[(0, 700)], [(100, 300), (0, 45), (511, 2)]])
 @pytest.mark.parametrize("window", [None, 100])
 def test_attention_prompt_portions(hip, ref, shared, q_heads, kv_heads, dim, page_size, portions, window):
-    """Long portions on both bfloat16 prompt kernels: blocks of four waves that share keys and values through LDS
-    (several blocks per request, steps inside one page and across four, groups of more heads than a tile), and one
-    wave per tile."""
+    """Long portions on the bfloat16 prompt kernels: blocks of four waves that share keys and values through LDS, with
+    16 and with 32 columns per wave (several blocks per request, steps inside one page and across four, groups of
+    more heads than a tile), and one wave per tile."""
     q, k_pages, v_pages, ctx, meta, _, _ = _attention_case(torch.bfloat16, q_heads, kv_heads, dim, page_size, portions,
                                                            window, 28)
     want = torch.empty_like(q)
     ref.attention(q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, dim, dim ** -0.5, window, want)
     cctx, cmeta = _to_cuda(ctx, meta)
     got = torch.full_like(q, float("nan"), device="cuda")
-    hip.share_prompt_tiles = shared
+    hip.share_prompt_tiles, hip.wide_prompt_tiles = bool(shared), shared == "wide"
     try:
         hip.attention(q.cuda(), k_pages.cuda(), v_pages.cuda(), cctx, cmeta, q_heads, kv_heads, dim, dim ** -0.5, window, got)
     finally:
-        hip.share_prompt_tiles = True
+        hip.share_prompt_tiles, hip.wide_prompt_tiles = True, None
     torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(torch.bfloat16))
 
 
