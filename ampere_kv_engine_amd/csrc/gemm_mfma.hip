@@ -73,12 +73,15 @@ __device__ __forceinline__ floatx4 silu_times(floatx4 gate, floatx4 up) {
 // tiles, so the traffic from the caches stays near the traffic from memory.
 // whether every wave of a block gets LDS for its own accumulators in the sum over the parts of k (8 waves, <= 64 KB)
 template <int MT, int RT> constexpr bool kSkinnyOwnSets = RT * MT <= 8;
+// k-tiles per group of loads: 8 weight tiles (8 KB) per group and wave - fewer where the activations' operands of a
+// group (MT per k-tile) would not fit the registers beside them
+template <int MT, int RT> constexpr int kSkinnyGroup = (RT == 1 && MT >= 3) ? 4 : 8 / RT;
 
 template <int MT, int RT, typename TY, bool GATED>
 __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __restrict__ x, const uintx4* __restrict__ wp,
                                                             TY* __restrict__ y, int rows, int outs, int k,
                                                             int k_tiles, int n_tiles, int k_split, int x_packed) {
-  constexpr int U = 8 / RT;  // k-tiles per group: 8 weight tiles (8 KB) per group and wave; two groups are in flight
+  constexpr int U = kSkinnyGroup<MT, RT>;  // k-tiles per group; two groups are in flight
   extern __shared__ float red[];  // [wave, or group of waves with the same row tiles][RT][MT][4][64]
   const int lane = threadIdx.x & 63, waves = blockDim.x >> 6;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // the same in every lane: keeps addresses scalar
@@ -245,7 +248,7 @@ int launch_skinny(const void* x, const void* wp, void* y, int rows, int outs, in
   // Enough waves to keep every CU's memory pipe full: k is split over the waves of a block when there are few row
   // tiles - down to short parts of k while the waves are very few, and further only while a wave keeps enough k-tiles
   // for two rounds of its double-buffered loop (measured: 1,536 waves of 32 k-tiles beat 3,072 of 16).
-  constexpr int U = 8 / RT;
+  constexpr int U = kSkinnyGroup<MT, RT>;
   const int wave_rows = (n_tiles + RT - 1) / RT;
   int k_split = 1;
   while (k_split < 8) {
@@ -274,14 +277,26 @@ int dispatch_skinny(const void* x, const void* wp, void* y, int rows, int outs, 
       if (GATED || (rows >= 4 && n_tiles >= 384 && n_tiles < 2048))
         return launch_skinny<1, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
       return launch_skinny<1, GATED ? 2 : 1, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
-    case 2: return launch_skinny<2, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
-    // four row tiles per wave where that still leaves a thousand waves, two otherwise
+    // Several tiles of x rows.  Two tiles: a wave takes 2 row tiles of the weights, or 1 where there are so few that
+    // the blocks would not even cover the compute units (4,096 outputs: 15.6 -> 13.1 us at k = 4,096).  Three and
+    // four: 4 row tiles where that still leaves a thousand waves (the gated product is measured better with 2 up to
+    // 2,048 row tiles: 68.7 -> 51.8 us at 64 rows), 2 otherwise.
+    case 2:
+      if (!GATED && n_tiles <= 256)
+        return launch_skinny<2, GATED ? 2 : 1, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
+      return launch_skinny<2, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
     case 3:
-      return n_tiles >= 512 ? launch_skinny<3, 4, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream)
-                            : launch_skinny<3, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
+      if (!GATED && n_tiles <= 256)
+        return launch_skinny<3, GATED ? 2 : 1, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
+      return n_tiles >= (GATED ? 2048 : 512)
+                 ? launch_skinny<3, 4, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream)
+                 : launch_skinny<3, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
     case 4:
-      return n_tiles >= 512 ? launch_skinny<4, 4, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream)
-                            : launch_skinny<4, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
+      if (!GATED && n_tiles <= 256)
+        return launch_skinny<4, GATED ? 2 : 1, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
+      return n_tiles >= (GATED ? 2048 : 512)
+                 ? launch_skinny<4, 4, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream)
+                 : launch_skinny<4, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
     default: return -2;
   }
 }
