@@ -15,7 +15,7 @@ Everything here except the tensors is host bookkeeping and runs without a GPU (`
 
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 
 import torch
 

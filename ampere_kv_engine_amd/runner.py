@@ -145,7 +145,6 @@ def main(argv=None) -> int:
     scratch = None
     folder = args.model
     if args.random_config is not None:
-        from .config.registry import register_architecture  # noqa: F401  (registry is filled on import)
         from .config import registry
         from .weights.random import write_random_model
         with open(args.random_config) as handle:

@@ -3,11 +3,10 @@ Qwen3-32B layer sizes (hidden 5120, 64 query heads, feed-forward 25600) with few
 serving arithmetic against it within bfloat16's reach.  Also inputs made so that a fault shows: a window's edge."""
 
 import pytest
-import torch
 
 import schedules
 from ampere_kv_engine_amd.config import EngineConfig, Qwen3Config
-from ampere_kv_engine_amd.engine import Engine, StepEntry
+from ampere_kv_engine_amd.engine import Engine
 from ampere_kv_engine_amd.weights import write_random_model
 from conftest import random_ids
 from plain.qwen3_plain import PlainQwen3

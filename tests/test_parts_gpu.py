@@ -1,7 +1,6 @@
 """Each part alone on the GPU against the plain function of the same part, at sizes that are not the tiny
 models'; and the entry points: greedy generation through `generate_tokens`, the scheduler and the command line."""
 
-import json
 import os
 import subprocess
 import sys
