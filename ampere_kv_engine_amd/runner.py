@@ -3,13 +3,15 @@ one prompt, one model, `--mode` chooses what is done with it.
 
     python -m ampere_kv_engine_amd.runner --model DIR --mode generate --cache paged < prompt_ids.txt
 
-Options the reference has keep their names and meanings: `--mode` (check | generate | benchmark), `--repeats`
+Options the reference has keep their names and meanings: `--mode` (check | generate | benchmark | cuda-check), `--repeats`
 (benchmark repetitions after one warm-up), `--cache` (only `paged` exists here), `--kv-dtype` (bf16; the cache
 follows `--dtype`), `--decode-kernel` (v1: one query head per wave; v3: the query heads of a group share every key
 and value load - here the MFMA kernels, and the default).  The reference reads a text and tokenizes it; this engine takes token ids in and gives token
 ids out, so the prompt is a line of integers on standard input (or `--prompt-ids`, or a seeded random prompt with
 `--prompt-len`).  `check` replaces the reference's comparison with a borrowed model by a comparison of the serving
-arithmetic with the engine's own true 32-bit path, step by step on the same tokens.
+arithmetic with the engine's own true 32-bit path, step by step on the same tokens.  `cuda-check` is the reference's
+lock-step run of two cache sets (ampere_kv/runner.py:471-550): the decode attention kernels of `--decode-kernel`
+beside the plain kernel that takes one query head per wave, each generating from its own choices.
 """
 
 from __future__ import annotations
@@ -44,7 +46,7 @@ def build_parser() -> argparse.ArgumentParser:
     parser.add_argument("--random-config", help="config.json of a model to be filled with random weights "
                         "(written to a temporary model folder with --weights-seed)")
     parser.add_argument("--weights-seed", type=int, default=0)
-    parser.add_argument("--mode", choices=("check", "generate", "benchmark"), default="check",
+    parser.add_argument("--mode", choices=("check", "generate", "benchmark", "cuda-check"), default="check",
                         help="check: serving arithmetic against the 32-bit path; generate: generation only; "
                              "benchmark: timed generation")
     parser.add_argument("--repeats", type=int, default=3, help="benchmark: measured runs after one warm-up")
@@ -109,6 +111,78 @@ def check(folder: str, prompt: list[int], args) -> list[int]:
     return generated
 
 
+def check_decode_kernels(folder: str, prompt: list[int], args) -> list[int]:
+    """Two engines with caches of their own generate greedily side by side, each from its own choices: one decodes
+    with the attention kernels that `--decode-kernel` names, the other with the plain kernel (one query head per
+    wave, no split of the keys, no matrix cores).  Both run the prompt through the same kernels, so their first
+    logits must be equal bit for bit; the logits of decode steps are only observed (largest difference, relative
+    L2); the first step at which the two choose different tokens ends the run with an error - the other's token is
+    never fed in (ampere_kv/runner.py:471-550)."""
+    from .engine.batch import StepEntry
+    capacity = len(prompt) + args.max_new_tokens
+    actual, reference = _engine(folder, args.dtype, args, capacity), _engine(folder, args.dtype, args, capacity)
+    a, b = actual.open("actual"), reference.open("reference")
+    eos = actual.spec.eos_token_ids
+    actual_ids, reference_ids, used = [], [], 0
+    print(f"at most {args.max_new_tokens} new tokens, prompt of {len(prompt)}, capacity "
+          f"{actual.config.num_pages * args.page_size} per layer, decode kernel {args.decode_kernel}")
+    try:
+        actual_input = reference_input = prompt
+        for step in range(args.max_new_tokens):
+            want = [len(actual_input) - 1]
+            if step == 0:    # the prompt: the same kernels on both sides
+                reference.kernels.one_wave_per_head = actual.kernels.one_wave_per_head
+            else:
+                reference.kernels.one_wave_per_head = True
+            la = actual.step([StepEntry(a, actual_input, want)]).clone()
+            lb = reference.step([StepEntry(b, reference_input, want)]).clone()
+            if not (torch.isfinite(la).all() and torch.isfinite(lb).all()):
+                raise AssertionError(f"step {step}: logits are not finite")
+            used = len(prompt) + step
+            if a.length != used or b.length != used:
+                raise AssertionError(f"step {step}: cache lengths {a.length} and {b.length}, expected {used}")
+            actual_id, reference_id = int(la[0].argmax()), int(lb[0].argmax())
+            if step == 0:
+                torch.testing.assert_close(la, lb, rtol=0, atol=0)
+                print(f"[PASS] prompt logits of both cache sets are identical: first token {actual_id}, "
+                      f"cache length {used}")
+            else:
+                difference = la - lb
+                norm = float(torch.linalg.vector_norm(lb))
+                relative = f"{float(torch.linalg.vector_norm(difference)) / norm:.8g}" if norm else "n/a"
+                print(f"[observed] decode step {step}: largest |difference| {float(difference.abs().max()):.8g}, "
+                      f"relative L2 {relative}")
+            actual_ids.append(actual_id)
+            reference_ids.append(reference_id)
+            if actual_id != reference_id:
+                print(f"[diverged] token {step + 1}: {args.decode_kernel} chose {actual_id}, plain chose "
+                      f"{reference_id}, cache length {used}")
+                for label, logits in ((args.decode_kernel, la), ("plain", lb)):
+                    scores, ids = logits[0].topk(2)
+                    print(f"  {label}: best two ids {ids.tolist()}, logits {scores.tolist()}, "
+                          f"margin {float(scores[0] - scores[1]):.8g}")
+                print(f"{args.decode_kernel}: {actual_ids}\nplain: {reference_ids}")
+                raise AssertionError("the two kernels chose different tokens; generation stopped there")
+            if (not args.ignore_eos and actual_id in eos) or step + 1 == args.max_new_tokens:
+                break
+            actual_input, reference_input = [actual_id], [reference_id]
+        crossed = (used - 1) // args.page_size > (len(prompt) - 1) // args.page_size
+        reason = "EOS" if (not args.ignore_eos and actual_ids[-1] in eos) else "reached limit"
+        print(f"{args.decode_kernel}: {actual_ids}\nplain: {reference_ids}")
+        print(f"stop reason {reason}, {len(actual_ids)} tokens, {len(actual_ids) - 1} decode steps, final cache length "
+              f"{used}, decode crossed a page: {crossed}")
+        if len(actual_ids) == 1:
+            print("[not covered] the first token ended the request: no decode step ran")
+        elif not crossed:
+            print("[not covered] no decode step crossed into a new page")
+    finally:
+        actual.close(a)
+        reference.close(b)
+        print("both cache sets were given back")
+    print("[PASS] both kernels generated the same tokens")
+    return actual_ids
+
+
 def benchmark(engine: Engine, prompt: list[int], args) -> list[int]:
     """One warm-up, then `--repeats` timed generations of fixed length (end-of-sequence ids ignored); medians of
     time to first token, time per output token, total and tokens per second (ampere_kv/runner.py:409-468)."""
@@ -165,6 +239,8 @@ def main(argv=None) -> int:
     print(f"model={folder} mode={args.mode} cache={args.cache} dtype={args.dtype} prompt_tokens={len(prompt)}")
     if args.mode == "check":
         generated = check(folder, prompt, args)
+    elif args.mode == "cuda-check":
+        generated = check_decode_kernels(folder, prompt, args)
     else:
         engine = _engine(folder, args.dtype, args, len(prompt) + args.max_new_tokens)
         if args.mode == "benchmark":
@@ -174,7 +250,7 @@ def main(argv=None) -> int:
                                         ignore_eos=args.ignore_eos, temperature=args.temperature,
                                         seed=args.sample_seed, prefill_chunk_size=args.prefill_chunk)
         eos = engine.spec.eos_token_ids
-    if args.mode == "check":
+    if args.mode in ("check", "cuda-check"):
         from .config.registry import load_config
         eos = load_config(folder).to_model_spec().eos_token_ids
     reason = "EOS" if (generated[-1] in eos and not args.ignore_eos) else "reached the limit of new tokens"

@@ -245,6 +245,18 @@ def test_command_line(model_folders):
         result = run("--model", model_folders["A"], "--mode", "generate", "--decode-kernel", kernel, "--max-new-tokens",
                      "6", "--ignore-eos", "--prompt-ids", ",".join(map(str, prompt)))
         assert result.returncode == 0 and f"generated_token_ids = {want}" in result.stdout, result.stderr[-2000:]
+    # two cache sets in lock step: the decode kernels of the matrix cores beside the plain one
+    result = run("--model", model_folders["A"], "--mode", "cuda-check", "--max-new-tokens", "24", "--ignore-eos",
+                 "--prompt-ids", ",".join(map(str, prompt)))
+    assert result.returncode == 0, result.stdout[-1500:] + result.stderr[-1500:]
+    assert "[PASS] prompt logits of both cache sets are identical" in result.stdout
+    assert "[PASS] both kernels generated the same tokens" in result.stdout and "[not covered]" not in result.stdout
+    assert result.stdout.count("[observed] decode step") == 23
+    # a model from a configuration file alone, with random weights
+    config_file = os.path.join(model_folders["A"], "config.json")
+    result = run("--random-config", config_file, "--weights-seed", "3", "--mode", "generate", "--max-new-tokens", "4",
+                 "--ignore-eos", "--prompt-len", "9")
+    assert result.returncode == 0 and "generated_token_ids" in result.stdout, result.stderr[-2000:]
     result = run("--model", model_folders["A"], "--mode", "generate", "--cache", "contiguous", "--prompt-ids", "1")
     assert result.returncode != 0
 
