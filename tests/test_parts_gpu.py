@@ -261,6 +261,25 @@ def test_command_line(model_folders):
     assert result.returncode != 0
 
 
+def test_scheduler_measurements_run(model_folders):
+    """`python -m ampere_kv_engine_amd.bench_scheduler` with the reference's option names, on a tiny model: both
+    experiments run, the batch of more than four is checked against single runs first, and every sample ends with
+    the pool whole (the program asserts it)."""
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    page = str(TINY["A"][2])
+    result = subprocess.run([sys.executable, "-m", "ampere_kv_engine_amd.bench_scheduler", "--model", model_folders["A"],
+                             "--history", "40", "--steps", "6", "--repeats", "1", "--batches", "1", "5", "--insert-at",
+                             "3", "--insert-history", "30", "--chunks", "0", "7", "--page-size", page,
+                             "--max-batched-tokens", "64"], env=env, capture_output=True, text=True, timeout=300)
+    assert result.returncode == 0, result.stdout[-1500:] + result.stderr[-1500:]
+    assert "[before] B=5: the batch generates the same 6 tokens as each request alone" in result.stdout
+    assert result.stdout.count("[decode] B=") == 2 and result.stdout.count("time to the late request's first token") == 2
+    result = subprocess.run([sys.executable, "-m", "ampere_kv_engine_amd.bench_scheduler", "--model", model_folders["A"],
+                             "--only", "insert", "--steps", "4", "--insert-at", "9"], env=env, capture_output=True,
+                            text=True, timeout=300)
+    assert result.returncode != 0 and "--insert-at" in result.stderr
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_recorded_mixed_steps_equal_eager_ones(dtype, model_folders):
     """Small steps with prompt portions are recorded too, once their shape (tokens per request, wanted rows) comes
