@@ -435,10 +435,10 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
 // values of a step of 32 keys are fetched from the pages ONCE per block - every thread moves a few 16-byte pieces into
 // LDS, double-buffered, one barrier per step - and each wave reads its MFMA A operands from there.  Against one wave
 // per tile this takes three quarters of the traffic off the vector memory pipe and the address arithmetic off the
-// waves, and leaves registers for two blocks per compute unit.  In LDS a key row is padded by 16 bytes and stored at the
-// MFMA row it feeds (tile j, row rho), a value row (one dim, 32 keys) is padded by 16 bytes: operand reads of the 16
-// lanes of a group then fall into different banks.  Pages must hold at least 8 tokens (an aligned run of 8 keys of a
-// value row is one 16-byte piece).
+// waves.  With 16 columns per wave (NQ = 1) three blocks fit a compute unit; with 32 (NQ = 2) two, which do a step for
+// twice the columns with the same loads, barriers and bookkeeping - the host takes them where they still fill the
+// device.  In LDS a key row is stored at the MFMA row it feeds (tile j, row rho); a value row is one dim's 32 keys.
+// Pages must hold at least 8 tokens (an aligned run of 8 keys of a value row is one 16-byte piece).
 constexpr int kSharedWaves = 4;
 // Rows in LDS, in bfloat16.  16 lanes read 16 bytes each from 16 consecutive rows; such a read runs at full rate when
 // the rows are 2 (mod 4) pieces of 16 bytes apart (measured: 1.5 times slower with an odd number of pieces, worse
@@ -985,7 +985,7 @@ int launch(const Args& a, int tiles, bool shared, hipStream_t stream) {
 // with num_splits > 1 `partial` must hold tiles * kv_heads * head_groups * num_splits * 16 * nq * (D + 4) floats.
 // page_size must be a power of two, at least 4.  `single_tokens` says that every request brings exactly one token.
 // `shared`: blocks of four waves that share keys and values through LDS; `tiles` then counts tiles of
-// 4 * tokens_per_tile tokens, nq and num_splits must be 1 and pages hold at least 8 tokens.
+// 4 * tokens_per_tile tokens, num_splits must be 1 and pages hold at least 8 tokens.
 extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
     const void* q, const void* k_pages, const void* v_pages, void* out, float* partial, const int* q_start,
     const int* seq_lens, const int* block_table, int table_width, int seq_first, int seq_count, int tiles, int nq,
