@@ -130,7 +130,8 @@ def main() -> int:
     tokens_per_request = args.context + PRIMING + args.warmup + args.steps + 1
     pages = max_batch * ((tokens_per_request + PAGE_SIZE - 1) // PAGE_SIZE) + PREFILL_TOKENS // PAGE_SIZE + 2
     engine_config = EngineConfig(dtype="bfloat16", page_size=PAGE_SIZE, num_pages=pages, max_seqs=max_batch,
-                                 max_batched_tokens=PREFILL_TOKENS, max_seq_len=tokens_per_request + PAGE_SIZE,
+                                 max_batched_tokens=PREFILL_TOKENS,
+                                 max_seq_len=max(tokens_per_request, PREFILL_TOKENS) + PAGE_SIZE,
                                  device="cuda:0", library_products_above=library_above)
     engine = Engine.from_random(config, seed=0, engine_config=engine_config)
     for group in engine.cache.groups:       # any finite keys and values: their content does not change the timing

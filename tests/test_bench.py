@@ -1,0 +1,44 @@
+"""The measurement program's contract: one GPU only, one JSON line with the agreed keys."""
+
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+from conftest import ROOT
+
+BENCH = os.path.join(ROOT, "bench.py")
+
+
+def test_more_than_one_gpu_is_refused_with_one_line():
+    result = subprocess.run([sys.executable, BENCH, "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert result.returncode == 2
+    assert len(result.stdout.strip().splitlines()) == 1 and "one GPU" in result.stdout
+
+
+@pytest.mark.gpu
+def test_the_line_of_a_short_run():
+    """Two layers of the benchmark's sizes, a few steps: the line holds the metric, the flat configuration with both
+    layer counts, the decode roofline, the prefill and the further batch sizes."""
+    result = subprocess.run([sys.executable, BENCH, "--layers", "2", "--steps", "3", "--warmup", "1", "--points", "1",
+                             "--context", "512"], capture_output=True, text=True, timeout=600, cwd=ROOT)
+    assert result.returncode == 0, result.stderr[-2000:]
+    line = json.loads(result.stdout.strip().splitlines()[-1])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "prefill", "roofline", "points"):
+        assert key in line, key
+    assert line["n_gpus"] == 1 and line["steps"] == 3 and line["warmup"] == 1 and line["higher_is_better"] is True
+    config = line["config"]
+    assert len(config) <= 20 and all(not isinstance(v, (dict, list)) for v in config.values())
+    assert config["layers"] == 2 and config["layers_of_config"] == 36 and config["global_batch"] == 8
+    assert config["seq_len"] == 512 and config["hidden"] == 4096 and config["vocab"] == 151936
+    assert abs(line["value"] - 8 / (line["ms_per_step"] / 1e3)) < 1e-2 * line["value"]
+    roofline = line["roofline"]
+    assert roofline["bound"] == "hbm" and roofline["peak"] == 8000.0 and roofline["unit"] == "GB/s"
+    assert abs(roofline["frac"] - roofline["achieved"] / roofline["peak"]) < 1e-3
+    prefill = line["prefill"]
+    assert prefill["tokens"] == 2048 and prefill["ms"] > 0 and 0 < prefill["frac"] < 1
+    assert abs(prefill["value"] - 2048 / (prefill["ms"] / 1e3)) < 1e-2 * prefill["value"]
+    assert line["points"]["decode_b1"] > 0
