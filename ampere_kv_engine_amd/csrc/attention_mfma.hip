@@ -78,6 +78,13 @@ struct Args {
   int window;                 // 0: none
   int seg_keys, num_splits;
   int units;                  // compute units of the device (block order of the shared kernel)
+  // FRESH launches (single tokens whose projections have not been normed, rotated or written to the cache yet):
+  const bf16_t* qkv;          // [tokens, (q_heads + 2 * kv_heads) * D]: query, key and value heads of a token in a row
+  const float* q_weight;      // [D] weights of the per-head norm of queries and of keys; both null: no norm
+  const float* k_weight;
+  const float* rope_table;    // [table_positions, D / 2, 2] (cos, sin) per position and rotation pair; null: no rotation
+  int table_positions;
+  float eps;
 };
 
 // Which request and which of its tiles this block works on.
@@ -134,12 +141,98 @@ __device__ __forceinline__ Tile find_tile(const Args& a, int slot, int per_tile)
   return t;
 }
 
+// A head as a lane's operand pieces (piece kt: dims kt * 32 + g * 8 .. + 7), normed over the head and rotated in place:
+// x * rsqrt(mean(x^2) + eps), rounded, times the weight, rounded; then the pairs (j, j + D / 2) are turned by the
+// position's angles (ampere_kv/runner.py:48-57, :88-98 of the reference).  With D a multiple of 64 the partner of
+// piece kt is piece kt + KT / 2 of the same lane, and the head's sum of squares is the sum over the four lanes that
+// share r16.  What it needs from memory is fetched apart (`HeadWeights`, `HeadAngles`), so that a kernel can have
+// these loads and others on their way before any arithmetic waits for them.  All 64 lanes call `encode_head` together.
+constexpr int KH = (KT + 1) / 2;  // pieces of the first half of a head
+struct HeadWeights {
+  floatx2 w[KT][4];
+};
+struct HeadAngles {
+  floatx2 cs[KH][4], sn[KH][4];
+};
+__device__ __forceinline__ void fetch_weights(HeadWeights& to, const float* weight, int g) {
+#pragma unroll
+  for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const float4 v = *reinterpret_cast<const float4*>(weight + kt * 32 + g * 8 + h * 4);
+      to.w[kt][2 * h] = floatx2{v.x, v.y};
+      to.w[kt][2 * h + 1] = floatx2{v.z, v.w};
+    }
+}
+// `angles`: a row of the table (cos, sin per rotation pair); `poison`: the position has no row - every angle is NaN
+__device__ __forceinline__ void fetch_angles(HeadAngles& to, const float* angles, bool poison, int g) {
+  const float nan = __uint_as_float(0x7fc00000u);
+#pragma unroll
+  for (int kt = 0; kt < KT / 2; ++kt)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float4 v = *reinterpret_cast<const float4*>(angles + (kt * 32 + g * 8) * 2 + 4 * q);
+      to.cs[kt][q] = floatx2{poison ? nan : v.x, poison ? nan : v.z};
+      to.sn[kt][q] = floatx2{poison ? nan : v.y, poison ? nan : v.w};
+    }
+}
+
+// rounding of two floats to bfloat16 (nearest, ties to even) in one conversion instruction, and back
+__device__ __forceinline__ floatx2 rounded2(floatx2 v) {
+  const uint32_t bits = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+  return floatx2{__uint_as_float(bits << 16), __uint_as_float(bits & 0xffff0000u)};
+}
+
+__device__ __forceinline__ void encode_head(uintx4 (&reg)[KT], bool normed, float eps, const HeadWeights& weights,
+                                            bool rotated, const HeadAngles& angles) {
+  static_assert(KT % 2 == 0 || D % 64 != 0, "pieces pair up when the head size is a multiple of 64");
+  floatx2 x[KT][4];
+#pragma unroll
+  for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+    for (int w = 0; w < 4; ++w) x[kt][w] = floatx2{__uint_as_float(reg[kt][w] << 16), __uint_as_float(reg[kt][w] & 0xffff0000u)};
+  if (normed) {
+    float squares = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int w = 0; w < 4; ++w) squares += x[kt][w][0] * x[kt][w][0] + x[kt][w][1] * x[kt][w][1];
+    squares += __shfl_xor(squares, 16, 64);
+    squares += __shfl_xor(squares, 32, 64);
+    const float scale = rsqrtf(squares / static_cast<float>(D) + eps);
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) {
+#pragma unroll
+      for (int w = 0; w < 4; ++w) x[kt][w] = rounded2(rounded2(x[kt][w] * scale) * weights.w[kt][w]);
+    }
+  }
+  if (rotated) {
+#pragma unroll
+    for (int kt = 0; kt < KT / 2; ++kt)
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const floatx2 cs = angles.cs[kt][w], sn = angles.sn[kt][w];
+        const floatx2 lo = x[kt][w], hi = x[kt + KT / 2][w];
+        x[kt][w] = lo * cs - hi * sn;
+        x[kt + KT / 2][w] = hi * cs + lo * sn;
+      }
+  }
+#pragma unroll
+  for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+    for (int w = 0; w < 4; ++w) reg[kt][w] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x[kt][w], bf16x2));
+}
+
 // Inside a step of 32 keys starting at `base`, MFMA tile j (0 or 1), row rho (0..15) is key
 //     base + (rho / 4) * 8 + j * 4 + rho % 4.
 // With this order the 8 score elements a lane holds (rows 4g .. 4g + 3 of both tiles) are the 8 CONSECUTIVE keys
 // base + 8g .. + 7, so the value operand of lane group g is one 16-byte read of a value page row.
 // PIPE: the next step's keys are fetched while this step computes (costs registers: used where they are there).
-template <int NQ, bool SPLIT, bool PIPE>
+// FRESH (single tokens, D a multiple of 64): query, key and value of the token come raw from the stacked projection
+// `a.qkv`.  Every block norms and rotates its own query heads in registers; the block whose keys include the token's
+// own position does the same for the new key, puts it and the new value into its operands in place of what the page
+// holds there, and writes both to the page for later steps.  No other block reads that slot in this launch.
+template <int NQ, bool SPLIT, bool PIPE, bool FRESH>
 __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
   const int lane = threadIdx.x, r16 = lane & 15, g = lane >> 4;
   // Without SPLIT a block works on two tiles, one after the other: tile `tiles - 1 - x` and tile `x`.  Under the
@@ -168,10 +261,26 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
     col_pos[nq] = t.first_pos + token;
     col_low[nq] = a.window > 0 ? max(0, col_pos[nq] - a.window + 1) : 0;
     col_at[nq] = (static_cast<long>(t.first_row + token) * a.q_heads + kvh * a.group + head_in_group) * D;
+    // FRESH: the raw query head of the stacked row (a single token: row t.first_row)
+    const bf16_t* q_from = FRESH ? a.qkv + (static_cast<long>(t.first_row) * (a.q_heads + 2 * a.kv_heads) + kvh * a.group + head_in_group) * D
+                                 : a.q + col_at[nq];
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt) {
       const int dim = kt * 32 + g * 8;
-      qreg[nq][kt] = (col_valid[nq] && dim < D) ? *reinterpret_cast<const uintx4*>(a.q + col_at[nq] + dim) : zero;
+      qreg[nq][kt] = (col_valid[nq] && dim < D) ? *reinterpret_cast<const uintx4*>(q_from + dim) : zero;
+    }
+  }
+  // FRESH: what the encoding of queries and the new key needs from memory is asked for here, and used only after
+  // the first keys have been asked for too.
+  const int new_pos = t.first_pos;
+  const bool normed = FRESH && a.q_weight != nullptr, rotated = FRESH && a.rope_table != nullptr;
+  HeadWeights q_weights, k_weights;
+  HeadAngles head_angles;
+  if constexpr (FRESH) {
+    if (normed) fetch_weights(q_weights, a.q_weight, g);
+    if (rotated) {
+      const bool known = new_pos >= 0 && new_pos < a.table_positions;
+      fetch_angles(head_angles, a.rope_table + (known ? static_cast<long>(new_pos) * D : 0L), !known, g);
     }
   }
 
@@ -206,6 +315,55 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
   const uint32_t k_lane = head_bytes + g * 16u;                         // + key row * D * 2 + kt * 64
   const uint32_t v_lane = head_bytes + (static_cast<uint32_t>(r16) << (a.page_shift + 1));  // + dt * 16 rows + key * 2
   const uint32_t v_tile = 32u << a.page_shift;                          // 16 value rows
+
+  // FRESH: the block whose keys include the token's own position holds the new key as operand pieces (the same in
+  // every r16) and the new value per dim row, and writes both to the token's slot (one block per kv head does).
+  bool owns_new = false;
+  uintx4 knew[KT];
+  uint32_t vnew[DT] = {};
+  if constexpr (FRESH) {
+    owns_new = new_pos >= range_lo && new_pos <= range_hi;
+    if (owns_new) {
+      const bf16_t* row = a.qkv + static_cast<long>(t.first_row) * (a.q_heads + 2 * a.kv_heads) * D;
+      const bf16_t* k_from = row + static_cast<long>(a.q_heads + kvh) * D;
+      const bf16_t* v_from = row + static_cast<long>(a.q_heads + a.kv_heads + kvh) * D;
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) knew[kt] = *reinterpret_cast<const uintx4*>(k_from + kt * 32 + g * 8);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) vnew[dt] = v_from[dt * 16 + r16].bits;
+      if (normed) fetch_weights(k_weights, a.k_weight, g);
+    }
+  }
+  auto encode_fresh = [&]() {
+#pragma unroll
+    for (int nq = 0; nq < NQ; ++nq) {
+      encode_head(qreg[nq], normed, a.eps, q_weights, rotated, head_angles);
+      if (!col_valid[nq]) {
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) qreg[nq][kt] = zero;
+      }
+    }
+    if (!owns_new) return;
+    encode_head(knew, normed, a.eps, k_weights, rotated, head_angles);
+    if (hg != 0) return;
+    const int page = table[new_pos >> a.page_shift];
+    if (page < 0 || page >= a.num_pages) {
+      poisoned = true;
+      return;
+    }
+    const size_t slot_k = static_cast<size_t>(page) * page_bytes + (k_lane + static_cast<uint32_t>(new_pos & page_mask) * (D * 2u));
+    const size_t slot_v = static_cast<size_t>(page) * page_bytes + (v_lane + static_cast<uint32_t>(new_pos & page_mask) * 2u);
+    char* k_out = const_cast<char*>(k_bytes);  // the pages are this launch's to write at this one slot
+    char* v_out = const_cast<char*>(v_bytes);
+    if (r16 == 0) {
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<uintx4*>(k_out + slot_k + kt * 64u) = knew[kt];
+    }
+    if (g == 0) {
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<uint16_t*>(v_out + slot_v + dt * v_tile) = static_cast<uint16_t>(vnew[dt]);
+    }
+  };
 
   // Keys of the step at `base` into A operands.  CHECK: the step may reach outside [range_lo, range_hi]; rows outside
   // are zero and never looked up.
@@ -379,6 +537,25 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
         else load_keys(base + 32, next, checked);
       }
     }
+    if constexpr (FRESH) {
+      if (owns_new && base == (new_pos & ~31)) {  // the new key and value take the place of what the page holds
+        const int at = new_pos - base;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          if (key_in_step + j * 4 == at) {
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) cur[j][kt] = knew[kt];
+          }
+        if (g == (at >> 3)) {
+          const int word = (at & 7) >> 1, shift = (at & 1) * 16;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int w = 0; w < 4; ++w)
+              if (w == word) vreg[dt][w] = (vreg[dt][w] & ~(0xffffu << shift)) | (vnew[dt] << shift);
+        }
+      }
+    }
     // every valid column sees the whole step: below the diagonal, inside window and segment
     const bool whole = here && base + 31 <= t.first_pos && (a.window == 0 || base >= last_pos - a.window + 1);
     if (whole) step(base, cur, unchecked);
@@ -390,12 +567,14 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
       if (inside(first_base)) load_keys(first_base, kreg, unchecked);
       else load_keys(first_base, kreg, checked);
     }
+    if constexpr (FRESH) encode_fresh();  // while the first keys are on their way
     for (int base = first_base; base <= range_hi; base += 64) {  // two turns: the key registers swap roles
       turn(base, kreg, knext);
       if (base + 32 > range_hi) break;
       turn(base + 32, knext, kreg);
     }
   } else {
+    if constexpr (FRESH) encode_fresh();
     for (int base = first_base; base <= range_hi; base += 32) turn(base, kreg, knext);
   }
 
@@ -965,12 +1144,27 @@ int launch(const Args& a, int tiles, bool shared, hipStream_t stream) {
     return AKV_LAUNCH_STATUS();
   }
   if (a.num_splits == 1) grid.x = (tiles + 1) / 2;  // a block takes a late tile and an early one
+  if (a.qkv != nullptr) {
+    if constexpr (NQ == 1 && D % 64 == 0) {
+      if (!a.single_tokens) return -2;
+      if (a.num_splits > 1) {
+        attention_mfma_kernel<NQ, true, true, true><<<grid, 64, 0, stream>>>(a);
+        grid.z = a.heads_per_tile * a.tokens_per_tile;
+        attention_merge_kernel<NQ><<<grid, 64 * kMergeWaves, 0, stream>>>(a);
+      } else {
+        attention_mfma_kernel<NQ, false, true, true><<<grid, 64, 0, stream>>>(a);
+      }
+      return AKV_LAUNCH_STATUS();
+    } else {
+      return -2;
+    }
+  }
   if (a.num_splits > 1) {
-    attention_mfma_kernel<NQ, true, true><<<grid, 64, 0, stream>>>(a);
+    attention_mfma_kernel<NQ, true, true, false><<<grid, 64, 0, stream>>>(a);
     grid.z = a.heads_per_tile * a.tokens_per_tile;  // the columns that can be (token, head) pairs
     attention_merge_kernel<NQ><<<grid, 64 * kMergeWaves, 0, stream>>>(a);
   } else {
-    attention_mfma_kernel<NQ, false, true><<<grid, 64, 0, stream>>>(a);
+    attention_mfma_kernel<NQ, false, true, false><<<grid, 64, 0, stream>>>(a);
   }
   return AKV_LAUNCH_STATUS();
 }
@@ -986,17 +1180,24 @@ int launch(const Args& a, int tiles, bool shared, hipStream_t stream) {
 // page_size must be a power of two, at least 4.  `single_tokens` says that every request brings exactly one token.
 // `shared`: blocks of four waves that share keys and values through LDS; `tiles` then counts tiles of
 // 4 * tokens_per_tile tokens, num_splits must be 1 and pages hold at least 8 tokens.
+// `qkv` (not null: single tokens, nq 1, head sizes that are multiples of 64): the tokens' stacked raw projections
+// [tokens, (q_heads + 2 * kv_heads) * D]; `q` is not read, the kernel norms (q_weight, k_weight, eps; both weights
+// null: no norm) and rotates (rope_table [table_positions, D / 2, 2], null: no rotation) queries and the new keys
+// itself and writes the new keys and values to the tokens' slots, which the block tables must already name.
 extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
     const void* q, const void* k_pages, const void* v_pages, void* out, float* partial, const int* q_start,
     const int* seq_lens, const int* block_table, int table_width, int seq_first, int seq_count, int tiles, int nq,
     int q_heads, int kv_heads, int heads_per_tile, int head_groups, int tokens_per_tile, int page_size, long num_pages,
-    float scale, int window, int seg_keys, int num_splits, int single_tokens, int shared, hipStream_t stream) {
+    float scale, int window, int seg_keys, int num_splits, int single_tokens, int shared, const void* qkv,
+    const float* q_weight, const float* k_weight, float eps, const float* rope_table, int table_positions,
+    hipStream_t stream) {
   if (tiles <= 0 || seq_count <= 0) return 0;
   int page_shift = 0;
   while ((1 << page_shift) < page_size) ++page_shift;
   if (page_size < 4 || (1 << page_shift) != page_size || q_heads % kv_heads != 0 ||
       heads_per_tile * tokens_per_tile > 16 * nq || kv_heads * head_groups > 65535 || num_splits > 65535 ||
-      num_splits < 1 || (single_tokens && tiles != seq_count) || (shared && (page_size < 8 || num_splits != 1)))
+      num_splits < 1 || (single_tokens && tiles != seq_count) || (shared && (page_size < 8 || num_splits != 1)) ||
+      (qkv != nullptr && (shared || !single_tokens || nq != 1 || D % 64 != 0 || (q_weight == nullptr) != (k_weight == nullptr))))
     return -2;
   Args a;
   a.q = static_cast<const bf16_t*>(q);
@@ -1025,6 +1226,12 @@ extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
   a.seg_keys = seg_keys;
   a.num_splits = num_splits;
   a.units = 1;
+  a.qkv = static_cast<const bf16_t*>(qkv);
+  a.q_weight = q_weight;
+  a.k_weight = k_weight;
+  a.rope_table = rope_table;
+  a.table_positions = table_positions;
+  a.eps = eps;
   if (shared) {
     static int units_of[64] = {0};  // compute units per device, asked once
     int device = 0;

@@ -23,7 +23,7 @@ SOURCES = ("elementwise.hip", "gemm.hip", "gemm_mfma.hip", "attention.hip", "sam
 HEADERS = ("common.h", "api.h")
 LIBRARY = "libakv_kernels.so"
 ATTENTION_SOURCE = "attention_mfma.hip"        # compiled once per head size, into its own small library
-DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 128, 256)
+DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 128, 192, 256)
 ARCH = "gfx950"
 # packed-fp32 instructions are switched off for all device code of this library
 FLAGS = ("-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",

@@ -78,6 +78,7 @@ def _ptr(t: torch.Tensor | None):
 class HipKernels:
     name = "hip-gfx950"
     OWN_SKINNY_ROWS = 64            # the most rows the engine's own decode product takes
+    _tuned_by_device: dict = {}     # device index -> the choices between own and library products made so far
 
     def __init__(self, device: torch.device | str = "cuda:0", library_products_above: int | None = 16,
                  tune_products: bool = True):
@@ -87,7 +88,6 @@ class HipKernels:
         once per matrix shape; False sends every product above the limit to the library."""
         self.library_products_above = library_products_above
         self.tune_products = tune_products     # 17..64 rows: own kernel or library, whichever is faster for the shape
-        self._tuned = {}                       # (kind, outs, k, row tiles) -> "own" | "library"
         self._spacer = None                    # the buffer whose fill precedes every timed run
         self._packed_rows = None               # where activations are repacked for the engine's own product
         self.device = torch.device(device)
@@ -97,6 +97,9 @@ class HipKernels:
             raise KernelError(f"the HIP kernels run on a GPU; device {self.device} is not one")
         if not torch.cuda.is_available():
             raise KernelError("no GPU is visible: the engine computes with HIP kernels only and has no CPU path")
+        # (kind, outs, k, row tiles) -> "own" | "library": one table per device for the whole process, so that two
+        # engines of a process, whose results may be compared bit for bit, send a product of one shape the same way
+        self._tuned = HipKernels._tuned_by_device.setdefault(self.device.index, {})
         path = ensure_built()
         try:
             self.lib = ctypes.CDLL(path)
@@ -109,6 +112,7 @@ class HipKernels:
         self.decode_max_splits = 128    # and no more than this many (four waves of the merge share them)
         self.share_prompt_tiles = True  # prompt portions: blocks of four waves share keys and values through LDS
         self.one_wave_per_head = False  # True: every attention goes to the plain kernel, a wave per (token, head)
+        self.fresh_decode_tokens = True  # single tokens: norm, rotation and cache write inside the attention kernel
         self.wide_prompt_tiles = None   # such blocks with 32 columns per wave instead of 16: None = by the step's size
         self.compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
         for name in ("akv_embed", "akv_add_rmsnorm", "akv_rmsnorm_rows", "akv_copy_rows", "akv_gather_rows",
@@ -429,11 +433,12 @@ class HipKernels:
         return self._attention_entry[head_dim]
 
     def _attention_mfma(self, q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out,
-                        page_size, num_pages, seq_first, seq_count, nq, split, shared=False):
+                        page_size, num_pages, seq_first, seq_count, nq, split, shared=False, fresh=None):
         """Requests seq_first .. seq_first + seq_count - 1 of the step on the MFMA kernel, in tiles of 16 * nq
         (token, head-of-group) columns; `split` says that each of them brings one token (decode) and cuts the keys
         over several waves; `shared` (prompt portions, pages of 8 tokens and more) lets blocks of four waves, four
-        tiles, fetch every key and value once into LDS."""
+        tiles, fetch every key and value once into LDS; `fresh` (with `split`): (qkv, q_weight, k_weight, eps, table),
+        the raw projections that the kernel norms, rotates and writes to the cache itself."""
         group = q_heads // kv_heads
         heads_per_tile = min(group, 16 * nq)
         head_groups = (group + heads_per_tile - 1) // heads_per_tile
@@ -456,12 +461,14 @@ class HipKernels:
                 arena = getattr(ctx, "arena", None)
                 partial = (arena.take((count,), torch.float32) if arena is not None
                            else torch.empty(count, dtype=torch.float32, device=self.device))
+        qkv, q_weight, k_weight, eps, table = fresh if fresh is not None else (None, None, None, 0.0, None)
         self._check(self._attention_mfma_entry(head_dim)(
             _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial), _ptr(ctx.q_start), _ptr(ctx.seq_lens),
             _ptr(meta.block_table), meta.width, seq_first, seq_count, tiles, nq, q_heads, kv_heads, heads_per_tile,
             head_groups, tokens_per_tile, page_size, ctypes.c_long(num_pages), ctypes.c_float(scale),
             int(window) if window is not None else 0, seg_keys, num_splits, 1 if split else 0, 1 if shared else 0,
-            self._stream()),
+            _ptr(qkv), _ptr(q_weight), _ptr(k_weight), ctypes.c_float(eps), _ptr(table),
+            table.shape[0] if table is not None else 0, self._stream()),
             "attention")
 
     def _wide_shared_tiles(self, ctx, first, q_heads, kv_heads) -> bool:
@@ -479,7 +486,45 @@ class HipKernels:
         units = self.compute_units
         return blocks >= 2 * units and (ctx.max_seq_len >= 4096 or 2 * blocks >= 5 * units)
 
-    def attention(self, q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out):
+    def _matrix_core_attention(self, dtype, page_size) -> bool:
+        return (dtype == torch.bfloat16 and page_size >= 4 and page_size & (page_size - 1) == 0
+                and not self.one_wave_per_head)
+
+    def encode_and_attend(self, qkv, q_weight, k_weight, eps, table, positions, slot_map, k_pages, v_pages, q, ctx,
+                          meta, q_heads, kv_heads, head_dim, scale, window, out):
+        """`qk_norm_rope_write` followed by `attention`, as one call: out[tokens, q_heads * head_dim] from the raw
+        stacked projections qkv.  `slot_map` must name, for every token, the slot that the request's block table
+        names for the token's position.  `q` is where encoded queries are kept between the two kernels.
+        The requests that bring a single token (the first `ctx.num_decode_seqs`; their tokens are the step's first
+        rows) need no kernel of their own for the first half where the attention kernel takes raw projections:
+        it norms and rotates their queries and new keys in registers and writes the new keys and values itself."""
+        tokens = qkv.shape[0]
+        decodes = ctx.num_decode_seqs
+        fresh = (self.fresh_decode_tokens and decodes > 0 and slot_map is not None and head_dim % 64 == 0
+                 and self._matrix_core_attention(qkv.dtype, k_pages.shape[2] if k_pages.dim() == 4 else 0))
+        if not fresh:
+            self.qk_norm_rope_write(qkv, q_weight, k_weight, eps, table, positions, slot_map, k_pages, v_pages, q,
+                                    q_heads, kv_heads, head_dim)
+            self.attention(q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out)
+            return
+        if ctx.host_q_start[decodes] != decodes:
+            raise KernelError("the single tokens of a step must be its first rows")
+        self._dense(qkv, "qkv", torch.bfloat16, (tokens, (q_heads + 2 * kv_heads) * head_dim))
+        if (q_weight is None) != (k_weight is None):
+            raise KernelError("q and k are normed together or not at all")
+        if q_weight is not None:
+            self._dense(q_weight, "q_weight", torch.float32, (head_dim,))
+            self._dense(k_weight, "k_weight", torch.float32, (head_dim,))
+        if table is not None:
+            self._dense(table, "table", torch.float32, (table.shape[0], head_dim // 2, 2))
+        if decodes < tokens:    # prompt portions: the kernel of the first half, on their rows alone
+            self.qk_norm_rope_write(qkv[decodes:], q_weight, k_weight, eps, table, positions[decodes:],
+                                    slot_map[decodes:], k_pages, v_pages, q[decodes:], q_heads, kv_heads, head_dim)
+        self.attention(q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out,
+                       fresh=(qkv, q_weight, k_weight, float(eps), table))
+
+    def attention(self, q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out, fresh=None):
+        """`fresh` is `encode_and_attend`'s: the raw projections of the step and what encodes them."""
         tokens = q.shape[0]
         self._dense(q, "q", None, (tokens, q_heads * head_dim))
         self._dense(out, "out", q.dtype, (tokens, q_heads * head_dim))
@@ -487,8 +532,9 @@ class HipKernels:
         self._dense(meta.block_table, "block_table", torch.int32, (ctx.num_seqs, meta.width))
         if ctx.max_seq_len > meta.width * page_size:
             raise KernelError(f"a request of {ctx.max_seq_len} tokens does not fit a block table of {meta.width} pages")
-        if (q.dtype == torch.bfloat16 and page_size >= 4 and page_size & (page_size - 1) == 0
-                and not self.one_wave_per_head):
+        if fresh is not None and not self._matrix_core_attention(q.dtype, page_size):
+            raise KernelError("raw projections are taken by the matrix-core attention alone")
+        if self._matrix_core_attention(q.dtype, page_size):
             self._dense(ctx.q_start, "q_start", torch.int32, (ctx.num_seqs + 1,))
             self._dense(ctx.seq_lens, "seq_lens", torch.int32, (ctx.num_seqs,))
             if ctx.host_q_start[ctx.num_seqs] != tokens or len(ctx.host_seq_lens) != ctx.num_seqs:
@@ -497,7 +543,7 @@ class HipKernels:
                       num_pages)
             decodes = ctx.num_decode_seqs
             if decodes:      # single tokens against long histories: one small tile each, keys split over waves
-                self._attention_mfma(*common, 0, decodes, 1, True)
+                self._attention_mfma(*common, 0, decodes, 1, True, fresh=fresh)
             if ctx.num_seqs > decodes:
                 shared = page_size >= 8 and self.share_prompt_tiles
                 nq = 2 if head_dim <= 128 else 1

@@ -80,18 +80,19 @@ class Attention(Part):
         qkv = ctx.arena.take((tokens, self.q_size + 2 * self.kv_size), self.rt.dtype)
         self.qkv.forward(x, qkv)
         q = ctx.arena.take((tokens, self.q_size), self.rt.dtype)
+        merged = ctx.arena.take((tokens, self.q_size), self.rt.dtype)
         if self.fused:
-            k.qk_norm_rope_write(
+            k.encode_and_attend(
                 qkv, self.q_norm.weight if self.q_norm is not None else None,
                 self.k_norm.weight if self.k_norm is not None else None,
                 self.q_norm.eps if self.q_norm is not None else 0.0,
                 self.position.table, ctx.positions, meta.slot_map if writes_cache else None,
-                cache.k, cache.v, q, self.q_heads, self.kv_heads, self.head_dim)
+                cache.k, cache.v, q, ctx, meta, self.q_heads, self.kv_heads, self.head_dim,
+                self.scale, self.window, merged)
         else:
             self._encode_with_parts(qkv, q, ctx, meta, cache, writes_cache)
-        merged = ctx.arena.take((tokens, self.q_size), self.rt.dtype)
-        k.attention(q, cache.k, cache.v, ctx, meta, self.q_heads, self.kv_heads, self.head_dim,
-                    self.scale, self.window, merged)
+            k.attention(q, cache.k, cache.v, ctx, meta, self.q_heads, self.kv_heads, self.head_dim,
+                        self.scale, self.window, merged)
         out = ctx.arena.take((tokens, self.hidden), self.rt.dtype)
         return self.out.forward(merged, out)
 

@@ -216,8 +216,8 @@ def test_gated_linear_rows_do_not_depend_on_the_batch_and_other_sizes_stay_stack
 
 def test_products_of_17_to_64_rows_choose_once(hip, ref):
     """Between 17 and 64 rows the engine's own product and the library's are timed at the first call with a matrix
-    shape and number of row tiles; the choice is remembered, every call gives the product, and other row counts do
-    not ask."""
+    shape and number of row tiles; the choice is remembered for the process, every call gives the product, and other
+    row counts do not ask."""
     from ampere_kv_engine_amd.kernels.hip import HipKernels
     kernels = HipKernels("cuda:0")
     w = rand(320, 256, dtype=torch.bfloat16, seed=41, scale=0.05)
@@ -229,9 +229,12 @@ def test_products_of_17_to_64_rows_choose_once(hip, ref):
         got = torch.empty(rows, 320, dtype=torch.bfloat16, device="cuda")
         kernels.linear(x.cuda(), packed, got)
         torch.testing.assert_close(got.cpu().float(), want.float(), **tol(torch.bfloat16))
-        assert len(kernels._tuned) == known
-    assert set(kernels._tuned) == {("linear", 320, 256, 2), ("linear", 320, 256, 4)}
-    assert set(kernels._tuned.values()) <= {"own", "library"}
+        assert sum(key[1:3] == (320, 256) for key in kernels._tuned) == known
+    mine = {key: choice for key, choice in kernels._tuned.items() if key[1:3] == (320, 256)}
+    assert set(mine) == {("linear", 320, 256, 2), ("linear", 320, 256, 4)}
+    assert set(mine.values()) <= {"own", "library"}
+    # the kernel sets of a process share the choices: two engines send a product of one shape the same way
+    assert HipKernels("cuda:0")._tuned is kernels._tuned
 
 
 def test_linear_keeps_other_weights_row_major(hip):
@@ -463,6 +466,96 @@ def test_attention_decodes_beside_portions(hip, ref):
     got = torch.full_like(q, float("nan"), device="cuda")
     hip.attention(q.cuda(), k_pages.cuda(), v_pages.cuda(), cctx, cmeta, 8, 2, 128, 128 ** -0.5, None, got)
     torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(torch.bfloat16))
+
+
+def _raw_projection_case(q_heads, kv_heads, dim, page_size, portions, window, seed, decodes):
+    """An attention case whose new tokens are not in the cache yet: their slots hold NaN, their stacked raw
+    projections come beside, with the slot of every token as the block tables name it."""
+    _, k_pages, v_pages, ctx, meta, _, _ = _attention_case(torch.bfloat16, q_heads, kv_heads, dim, page_size, portions,
+                                                           window, seed)
+    ctx.num_decode_seqs = decodes
+    slots = []
+    for r, (history, new) in enumerate(portions):
+        for pos in range(history, history + new):
+            page = int(meta.block_table[r, pos // page_size])
+            slots.append(page * page_size + pos % page_size)
+            k_pages[page, :, pos % page_size] = float("nan")
+            v_pages[page, :, :, pos % page_size] = float("nan")
+    qkv = rand(ctx.num_tokens, (q_heads + 2 * kv_heads) * dim, dtype=torch.bfloat16, seed=seed + 1)
+    exponent = torch.arange(0, dim, 2, dtype=torch.int64).float() / dim
+    table = torch.empty(ctx.max_seq_len + 1, dim // 2, 2)
+    TorchKernels().rope_table(1.0 / (1e4 ** exponent), table)
+    return qkv, table, torch.tensor(slots, dtype=torch.int32), k_pages, v_pages, ctx, meta
+
+
+def _check_encode_and_attend(hip, ref, q_heads, kv_heads, dim, page_size, portions, window, decodes, normed=True,
+                             rotated=True, seed=31):
+    qkv, table, slots, k_pages, v_pages, ctx, meta = _raw_projection_case(q_heads, kv_heads, dim, page_size, portions,
+                                                                          window, seed, decodes)
+    qw, kw = (1 + rand(dim, seed=18, scale=0.1), 1 + rand(dim, seed=19, scale=0.1)) if normed else (None, None)
+    sizes = (q_heads, kv_heads, dim, dim ** -0.5, window)
+    k_ref, v_ref = k_pages.clone(), v_pages.clone()
+    want = torch.empty(ctx.num_tokens, q_heads * dim, dtype=torch.bfloat16)
+    ref.encode_and_attend(qkv, qw, kw, 1e-6, table if rotated else None, ctx.positions, slots, k_ref, v_ref,
+                          torch.empty_like(want), ctx, meta, *sizes, want)
+    cctx, cmeta = _to_cuda(ctx, meta)
+    cu = lambda t: t.cuda() if t is not None else None
+    k_hip, v_hip = k_pages.cuda(), v_pages.cuda()
+    got = torch.full_like(want, float("nan"), device="cuda")
+    hip.encode_and_attend(qkv.cuda(), cu(qw), cu(kw), 1e-6, cu(table) if rotated else None, cctx.positions, slots.cuda(),
+                          k_hip, v_hip, torch.empty_like(got), cctx, cmeta, *sizes, got)
+    assert not torch.isnan(got).any()
+    torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(torch.bfloat16))
+    torch.testing.assert_close(k_hip.cpu().float(), k_ref.float(), equal_nan=True, **tol(torch.bfloat16))
+    torch.testing.assert_close(v_hip.cpu().float(), v_ref.float(), equal_nan=True, rtol=0, atol=0)
+    assert torch.isnan(k_hip.cpu().float()).sum() == torch.isnan(k_ref.float()).sum()   # nothing else was written
+
+
+@pytest.mark.parametrize("q_heads,kv_heads,dim,page_size", [(8, 2, 128, 16), (4, 4, 64, 4), (40, 2, 64, 8), (3, 1, 256, 32),
+                                                            (6, 2, 192, 16), (6, 1, 32, 8), (5, 5, 80, 16)])
+@pytest.mark.parametrize("histories", [[0], [31, 32, 63, 64, 15, 16, 1], [1500, 2, 700, 255, 1023], [4000] * 9])
+@pytest.mark.parametrize("window", [None, 100])
+def test_encode_and_attend_single_tokens(hip, ref, q_heads, kv_heads, dim, page_size, histories, window):
+    """Single tokens whose projections are raw: head sizes that are multiples of 64 go through the attention kernel
+    that norms, rotates and writes them itself (positions at the first and last key of a step, of a page and of a
+    segment; more heads per group than a tile holds), the others through the two kernels."""
+    _check_encode_and_attend(hip, ref, q_heads, kv_heads, dim, page_size, [(h, 1) for h in histories], window,
+                             len(histories))
+
+
+@pytest.mark.parametrize("normed,rotated", [(False, True), (True, False), (False, False)])
+def test_encode_and_attend_without_norm_or_rotation(hip, ref, normed, rotated):
+    _check_encode_and_attend(hip, ref, 8, 2, 128, 16, [(h, 1) for h in (300, 0, 77)], None, 3, normed, rotated)
+
+
+@pytest.mark.parametrize("dim", [128, 80])
+def test_encode_and_attend_mixed_step(hip, ref, dim):
+    """Three single tokens first, then two portions: the portions' rows alone go through the encoding kernel."""
+    _check_encode_and_attend(hip, ref, 8, 2, dim, 16, [(300, 1), (15, 1), (0, 1), (40, 37), (0, 130)], None, 3)
+
+
+def test_encode_and_attend_is_the_two_kernels(hip, ref):
+    """The attention kernel's own encoding gives what the encoding kernel followed by the attention gives, to the
+    rounding of the head's sum of squares (another order of the same sum)."""
+    portions = [(h, 1) for h in (2000, 33, 0, 640)]
+    qkv, table, slots, k_pages, v_pages, ctx, meta = _raw_projection_case(8, 2, 128, 16, portions, None, 35, 4)
+    qw, kw = 1 + rand(128, seed=18, scale=0.1), 1 + rand(128, seed=19, scale=0.1)
+    cctx, cmeta = _to_cuda(ctx, meta)
+    outs = []
+    for fresh in (True, False):
+        hip.fresh_decode_tokens = fresh
+        try:
+            k_hip, v_hip = k_pages.cuda(), v_pages.cuda()
+            got = torch.empty(4, 8 * 128, dtype=torch.bfloat16, device="cuda")
+            hip.encode_and_attend(qkv.cuda(), qw.cuda(), kw.cuda(), 1e-6, table.cuda(), cctx.positions, slots.cuda(),
+                                  k_hip, v_hip, torch.empty_like(got), cctx, cmeta, 8, 2, 128, 128 ** -0.5, None, got)
+            outs.append((got.float().cpu(), k_hip.float().cpu(), v_hip.float().cpu()))
+        finally:
+            hip.fresh_decode_tokens = True
+    torch.testing.assert_close(outs[0][0], outs[1][0], rtol=0.01, atol=0.002)
+    torch.testing.assert_close(outs[0][1], outs[1][1], equal_nan=True, rtol=1e-2, atol=1e-3)
+    assert (outs[0][1].nan_to_num() != outs[1][1].nan_to_num()).float().mean() < 0.01   # nearly every key bit for bit
+    torch.testing.assert_close(outs[0][2], outs[1][2], equal_nan=True, rtol=0, atol=0)
 
 
 def test_attention_over_a_pool_of_more_than_4_gb(hip, ref):

@@ -117,6 +117,12 @@ class TorchKernels:
         if slot_map is not None:
             self.kv_write(k.to(dtype), v, slot_map, k_pages, v_pages)
 
+    def encode_and_attend(self, qkv, q_weight, k_weight, eps, table, positions, slot_map, k_pages, v_pages, q, ctx,
+                          meta, q_heads, kv_heads, head_dim, scale, window, out):
+        self.qk_norm_rope_write(qkv, q_weight, k_weight, eps, table, positions, slot_map, k_pages, v_pages, q,
+                                q_heads, kv_heads, head_dim)
+        self.attention(q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out)
+
     def attention(self, q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out):
         page_size = k_pages.shape[2]
         group = q_heads // kv_heads
