@@ -135,7 +135,7 @@ class CacheManager:
     def can_reserve(self, seq: Sequence, num_tokens: int) -> bool:
         for table, group in zip(seq.tables, self.groups):
             required = (table.length + num_tokens + self.page_size - 1) // self.page_size
-            additional = max(0, required - len(table.pages))
+            additional = max(0, required - table.num_pages)
             if additional > group.allocator.num_free + table._passed_pages(table.length):
                 return False
         return True
@@ -174,9 +174,10 @@ class CacheManager:
         view = self.layer_cache[layer]
         table = seq.tables[view.group]
         keys, values = [], []
+        pages = table.pages
         for position in range(table.length):
             index, offset = divmod(position, self.page_size)
-            page = table.pages[index]
+            page = pages[index]
             if page < 0:
                 continue
             keys.append(view.k[page, :, offset])

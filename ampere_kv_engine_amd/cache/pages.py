@@ -9,6 +9,8 @@ reference: a table can give back the pages that a window has passed while the re
 
 from __future__ import annotations
 
+import numpy as np
+
 RELEASED = -1  # table entry of a page that was given back mid-request; no kernel may read it
 
 
@@ -53,6 +55,7 @@ class BlockTable:
         self.page_size = page_size
         self.window = window
         self._pages: list[int] = []
+        self._mirror = np.empty(16, dtype=np.int32)   # the same ids as an array, for the step's metadata
         self._length = 0
         self._first_live = 0      # logical index of the first page not yet given back
 
@@ -63,6 +66,16 @@ class BlockTable:
     @property
     def pages(self) -> tuple[int, ...]:
         return tuple(self._pages)
+
+    @property
+    def num_pages(self) -> int:
+        """Entries of the table, given-back ones included."""
+        return len(self._pages)
+
+    @property
+    def page_array(self) -> np.ndarray:
+        """The page ids as an int32 array (a view that the next `append_tokens` or `release` may change)."""
+        return self._mirror[:len(self._pages)]
 
     @property
     def num_held(self) -> int:
@@ -90,9 +103,16 @@ class BlockTable:
         for index in range(self._first_live, self._first_live + passed):
             self._allocator.free(self._pages[index])
             self._pages[index] = RELEASED
+            self._mirror[index] = RELEASED
         self._first_live += passed
+        if required > len(self._mirror):
+            grown = np.empty(max(required, 2 * len(self._mirror)), dtype=np.int32)
+            grown[:len(self._pages)] = self._mirror[:len(self._pages)]
+            self._mirror = grown
         for _ in range(additional):
-            self._pages.append(self._allocator.allocate())
+            page = self._allocator.allocate()
+            self._mirror[len(self._pages)] = page
+            self._pages.append(page)
         self._length = start + num_tokens
         return start
 

@@ -148,7 +148,7 @@ class BatchBuilder:
         starts = [self.cache.reserve(e.seq, len(e.tokens)) for e in ordered]
 
         n, r = total, len(ordered)
-        width = max(max((len(t.pages) for t in e.seq.tables), default=1) for e in ordered)
+        width = max(max((t.num_pages for t in e.seq.tables), default=1) for e in ordered)
         width = max(width, 1)
         width = min((width + width_multiple - 1) // width_multiple * width_multiple, max(self.max_width, width))
         self._turn ^= 1
@@ -181,22 +181,30 @@ class BatchBuilder:
 
         row = 0
         first_row_of = [0] * len(entries)
+        page_size = self.cache.page_size
         for index, (e, start) in enumerate(zip(ordered, starts)):
             count = len(e.tokens)
-            token_ids[row:row + count] = np.asarray(e.tokens, dtype=np.int64)
-            positions[row:row + count] = np.arange(start, start + count)
-            seq_of_token[row:row + count] = index
+            if count == 1:      # a decode token: scalars, no temporary arrays
+                token_ids[row] = e.tokens[0]
+                positions[row] = start
+                seq_of_token[row] = index
+            else:
+                token_ids[row:row + count] = np.asarray(e.tokens, dtype=np.int64)
+                positions[row:row + count] = np.arange(start, start + count)
+                seq_of_token[row:row + count] = index
             q_start[index] = row
             seq_lens[index] = start + count
             seq_slots[index] = e.seq.slot
             first_row_of[order[index]] = row
             for g, (slot_map, _, table, _) in zip(self.cache.groups, group_spans):
-                pages = e.seq.tables[g.index].pages
+                pages = e.seq.tables[g.index].page_array
                 table[index, :len(pages)] = pages
                 table[index, len(pages):] = -1
-                pos = np.arange(start, start + count)
-                page_of = np.asarray(pages, dtype=np.int64)[pos // self.cache.page_size]
-                slot_map[row:row + count] = page_of * self.cache.page_size + pos % self.cache.page_size
+                if count == 1:
+                    slot_map[row] = int(pages[start // page_size]) * page_size + start % page_size
+                else:
+                    pos = np.arange(start, start + count)
+                    slot_map[row:row + count] = pages[pos // page_size].astype(np.int64) * page_size + pos % page_size
             row += count
         # wanted rows in the caller's order of entries and places, whatever the layout above
         want_cursor = 0
@@ -235,7 +243,7 @@ class BatchBuilder:
             for e in entries:
                 table = e.seq.tables[g.index]
                 required = (table.length + len(e.tokens) + self.cache.page_size - 1) // self.cache.page_size
-                available += table._passed_pages(table.length) - max(0, required - len(table.pages))
+                available += table._passed_pages(table.length) - max(0, required - table.num_pages)
             if available < 0:
                 raise PagePoolExhausted(f"the step needs {-available} more page(s) than the pool of cache group "
                                         f"{g.index} has free; no token of the step was registered")

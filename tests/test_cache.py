@@ -133,6 +133,7 @@ def test_no_page_lost_held_twice_or_freed_twice_under_random_orders(seed):
             assert all(group.allocator.is_held(p) for p in held)
         for s in live.values():
             assert all(t.length == s.length for t in s.tables)
+            assert all(tuple(t.page_array.tolist()) == t.pages and t.num_pages == len(t.pages) for t in s.tables)
             full, windowed = s.tables
             assert full.num_held == -(-s.length // 4)
             assert windowed.num_held <= -(-(12 + 13) // 4) + 1
