@@ -108,7 +108,7 @@ class HipKernels:
         self.library_path = path
         self._attention_entry = {}      # head size -> entry point of that head size's attention library
         self.decode_wave_target = 2048  # decode attention cuts the keys until about this many waves are at work,
-        self.decode_min_segment = 64    # but into segments no shorter than this many keys
+        self.decode_min_segment = 128   # but into segments no shorter than this many keys (measured: 64 and 256 are slower)
         self.decode_max_splits = 128    # and no more than this many (four waves of the merge share them)
         self.share_prompt_tiles = True  # prompt portions: blocks of four waves share keys and values through LDS
         self.one_wave_per_head = False  # True: every attention goes to the plain kernel, a wave per (token, head)
