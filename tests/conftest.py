@@ -23,7 +23,12 @@ TINY_A = dict(architectures=["Qwen3ForCausalLM"], vocab_size=256, hidden_size=64
 TINY_B = dict(architectures=["Qwen3ForCausalLM"], vocab_size=379, hidden_size=96, num_hidden_layers=3,
               num_attention_heads=6, num_key_value_heads=1, head_dim=32, intermediate_size=200, rope_theta=1000000.0,
               rms_norm_eps=1e-5, tie_word_embeddings=False, hidden_act="silu")
-TINY = {"A": (TINY_A, 0, 16), "B": (TINY_B, 1, 8)}   # config, weight seed, page size
+# A third one with heads of 64: the size from which the decode attention kernel norms, rotates and writes a single
+# token's heads itself (a rotation pair then lies in one lane); pages of 4 tokens put several pages into every step.
+TINY_C = dict(architectures=["Qwen3ForCausalLM"], vocab_size=211, hidden_size=72, num_hidden_layers=2,
+              num_attention_heads=6, num_key_value_heads=3, head_dim=64, intermediate_size=104, rope_theta=500000.0,
+              rms_norm_eps=1e-6, tie_word_embeddings=False, hidden_act="silu")
+TINY = {"A": (TINY_A, 0, 16), "B": (TINY_B, 1, 8), "C": (TINY_C, 2, 4)}   # config, weight seed, page size
 
 
 @pytest.fixture(scope="session")

@@ -17,7 +17,7 @@ from engine_cases import PROMPTS, tolerance
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module", params=["A", "B"])
+@pytest.fixture(scope="module", params=["A", "B", "C"])
 def case(request, model_folders):
     return cases.make_case(request.param, model_folders)
 
@@ -40,7 +40,7 @@ def test_trace_run_program(case, dtype, tmp_path):
     """bin/trace_run as a user runs it: JSON steps on stdin, <step>.f32 files out, `done <step>` lines."""
     import numpy as np
     requests = {k: case["requests"][k] for k in ("a", "b", "e")}
-    schedule = schedules.mixed(requests, PROMPTS, case["page_size"], 192 // 16, seed=9)
+    schedule = schedules.mixed(requests, PROMPTS, 16, 192 // 16, seed=9)      # the program's own pages hold 16 tokens
     records = schedules.to_trace(requests, schedule)
     out = tmp_path / "out"
     result = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", case["folder"], "--dtype", dtype,
