@@ -36,6 +36,7 @@ class Sampler:
         self._host_t = torch.empty(max_rows, dtype=torch.float32, pin_memory=pin)
         self._host_s = torch.empty(max_rows, dtype=torch.int64, pin_memory=pin)
         self._host_d = torch.empty(max_rows, dtype=torch.int32, pin_memory=pin)
+        self._host_out = torch.empty(max_rows, dtype=torch.int32, pin_memory=pin)   # the chosen ids land here
 
     def sample(self, logits: torch.Tensor, params: list[SamplingParams], draws: list[int]) -> list[int]:
         """logits float32 [rows, vocab]; `draws[i]` is how many tokens request i has drawn before.  Returns the
@@ -56,4 +57,9 @@ class Sampler:
             self._seeds[:rows].copy_(self._host_s[:rows])
             self._draws[:rows].copy_(self._host_d[:rows])
             self.kernels.sample(logits, self._temperature[:rows], self._seeds[:rows], self._draws[:rows], out)
-        return out.tolist()
+        if self.device.type != "cuda":
+            return out.tolist()
+        # into pinned memory, then one wait for the stream: no staging copy on the way
+        self._host_out[:rows].copy_(out, non_blocking=True)
+        torch.cuda.current_stream(self.device).synchronize()
+        return self._host_out[:rows].tolist()
