@@ -238,10 +238,12 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
   // Without SPLIT a block works on two tiles, one after the other: tile `tiles - 1 - x` and tile `x`.  Under the
   // causal mask the late tiles of a prompt see many keys and the early ones few; a pair sees about the same number
   // as every other pair, so the blocks finish together instead of waiting for the longest.
-  for (int pass = 0; pass < (SPLIT ? 1 : 2); ++pass) {
-  const int slot = SPLIT ? static_cast<int>(blockIdx.x)
-                         : (pass == 0 ? a.tiles - 1 - static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x));
-  if (!SPLIT && pass == 1 && slot >= a.tiles - 1 - slot) break;  // the middle tile was the first pass's
+  // (FRESH launches hold single tokens, whose tiles have nothing to balance: one tile per block, like SPLIT.)
+  constexpr bool kOneTile = SPLIT || FRESH;
+  for (int pass = 0; pass < (kOneTile ? 1 : 2); ++pass) {
+  const int slot = kOneTile ? static_cast<int>(blockIdx.x)
+                            : (pass == 0 ? a.tiles - 1 - static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x));
+  if (!kOneTile && pass == 1 && slot >= a.tiles - 1 - slot) break;  // the middle tile was the first pass's
   const Tile t = find_tile(a, slot, a.tokens_per_tile);
   if (!t.found) continue;
   const int kvh = blockIdx.y / a.head_groups, hg = blockIdx.y % a.head_groups;
@@ -1143,7 +1145,7 @@ int launch(const Args& a, int tiles, bool shared, hipStream_t stream) {
     else return -2;
     return AKV_LAUNCH_STATUS();
   }
-  if (a.num_splits == 1) grid.x = (tiles + 1) / 2;  // a block takes a late tile and an early one
+  if (a.num_splits == 1 && a.qkv == nullptr) grid.x = (tiles + 1) / 2;  // a block takes a late tile and an early one
   if (a.qkv != nullptr) {
     if constexpr (NQ == 1 && D % 64 == 0) {
       if (!a.single_tokens) return -2;

@@ -114,6 +114,7 @@ class HipKernels:
         self.one_wave_per_head = False  # True: every attention goes to the plain kernel, a wave per (token, head)
         self.fresh_decode_tokens = True  # single tokens: norm, rotation and cache write inside the attention kernel
         self.wide_prompt_tiles = None   # such blocks with 32 columns per wave instead of 16: None = by the step's size
+        self.split_prompt_keys = None   # prompt portions on one wave per tile and key segment: None = by the step's size
         self.compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
         for name in ("akv_embed", "akv_add_rmsnorm", "akv_rmsnorm_rows", "akv_copy_rows", "akv_gather_rows",
                      "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
@@ -433,12 +434,15 @@ class HipKernels:
         return self._attention_entry[head_dim]
 
     def _attention_mfma(self, q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out,
-                        page_size, num_pages, seq_first, seq_count, nq, split, shared=False, fresh=None):
+                        page_size, num_pages, seq_first, seq_count, nq, split, shared=False, fresh=None, single=None):
         """Requests seq_first .. seq_first + seq_count - 1 of the step on the MFMA kernel, in tiles of 16 * nq
-        (token, head-of-group) columns; `split` says that each of them brings one token (decode) and cuts the keys
-        over several waves; `shared` (prompt portions, pages of 8 tokens and more) lets blocks of four waves, four
-        tiles, fetch every key and value once into LDS; `fresh` (with `split`): (qkv, q_weight, k_weight, eps, table),
-        the raw projections that the kernel norms, rotates and writes to the cache itself."""
+        (token, head-of-group) columns; `split` cuts the keys over several waves whose partial results a second
+        kernel merges; `single` (default: as `split`) says that each request brings one token (decode); `shared`
+        (prompt portions, pages of 8 tokens and more) lets blocks of four waves, four tiles, fetch every key and
+        value once into LDS; `fresh` (single tokens): (qkv, q_weight, k_weight, eps, table), the raw projections that
+        the kernel norms, rotates and writes to the cache itself."""
+        if single is None:
+            single = split
         group = q_heads // kv_heads
         heads_per_tile = min(group, 16 * nq)
         head_groups = (group + heads_per_tile - 1) // heads_per_tile
@@ -466,10 +470,24 @@ class HipKernels:
             _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial), _ptr(ctx.q_start), _ptr(ctx.seq_lens),
             _ptr(meta.block_table), meta.width, seq_first, seq_count, tiles, nq, q_heads, kv_heads, heads_per_tile,
             head_groups, tokens_per_tile, page_size, ctypes.c_long(num_pages), ctypes.c_float(scale),
-            int(window) if window is not None else 0, seg_keys, num_splits, 1 if split else 0, 1 if shared else 0,
+            int(window) if window is not None else 0, seg_keys, num_splits, 1 if single else 0, 1 if shared else 0,
             _ptr(qkv), _ptr(q_weight), _ptr(k_weight), ctypes.c_float(eps), _ptr(table),
             table.shape[0] if table is not None else 0, self._stream()),
             "attention")
+
+    def _few_portion_blocks(self, ctx, first, q_heads, kv_heads) -> bool:
+        """Whether the prompt portions of the step are so short, and their histories so long, that blocks of four
+        tiles would leave most compute units idle while each walks thousands of keys: then a wave takes a tile and a
+        segment of the keys, as in decoding.  Measured at Qwen3-8B sizes, blocks of four tiles against cut keys:
+        128 tokens after 4,096: 114 / 63 us; 64 after 8,192: 221 / 65; 32 after 16,384: 437 / 70; but 256 after
+        2,048: 67 / 77, 128 after 1,024: 37 / 41, 512 after 4,096: 128 / 195."""
+        group = q_heads // kv_heads
+        heads_per_tile = min(group, 16)
+        per_block = 4 * (16 // heads_per_tile)
+        starts = ctx.host_q_start
+        blocks = sum((starts[r + 1] - starts[r] + per_block - 1) // per_block for r in range(first, ctx.num_seqs))
+        blocks *= kv_heads * ((group + heads_per_tile - 1) // heads_per_tile)
+        return 4 * blocks <= self.compute_units and ctx.max_seq_len >= 2048
 
     def _wide_shared_tiles(self, ctx, first, q_heads, kv_heads) -> bool:
         """Whether the prompt portions of the step go to blocks of 4 x 32 columns rather than 4 x 16.  The wide
@@ -547,6 +565,12 @@ class HipKernels:
             if ctx.num_seqs > decodes:
                 shared = page_size >= 8 and self.share_prompt_tiles
                 nq = 2 if head_dim <= 128 else 1
+                cut = self.split_prompt_keys
+                if cut is None:
+                    cut = self._few_portion_blocks(ctx, decodes, q_heads, kv_heads)
+                if cut:     # short portions after long histories: too few blocks to fill the device, so the keys are cut
+                    self._attention_mfma(*common, decodes, ctx.num_seqs - decodes, nq, True, single=False)
+                    return
                 if shared and nq == 2:
                     wide = self.wide_prompt_tiles
                     if wide is None:

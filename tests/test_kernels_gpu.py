@@ -413,7 +413,7 @@ def test_attention(hip, ref, dtype, q_heads, kv_heads, dim, page_size, portions,
     torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(dtype))
 
 
-@pytest.mark.parametrize("shared", ["narrow", "wide", False])
+@pytest.mark.parametrize("shared", ["narrow", "wide", False, "cut"])
 @pytest.mark.parametrize("q_heads,kv_heads,dim,page_size", [(8, 2, 128, 16), (6, 1, 32, 8), (8, 4, 64, 64), (3, 1, 256, 32),
                                                             (5, 5, 80, 16), (40, 2, 64, 8), (4, 2, 16, 128)])
 @pytest.mark.parametrize("portions", [[(0, 700)], [(100, 300), (0, 45), (511, 2)]])
@@ -421,18 +421,20 @@ def test_attention(hip, ref, dtype, q_heads, kv_heads, dim, page_size, portions,
 def test_attention_prompt_portions(hip, ref, shared, q_heads, kv_heads, dim, page_size, portions, window):
     """Long portions on the bfloat16 prompt kernels: blocks of four waves that share keys and values through LDS, with
     16 and with 32 columns per wave (several blocks per request, steps inside one page and across four, groups of
-    more heads than a tile), and one wave per tile."""
+    more heads than a tile), one wave per tile, and one wave per tile and segment of the keys (what short portions
+    after long histories get)."""
     q, k_pages, v_pages, ctx, meta, _, _ = _attention_case(torch.bfloat16, q_heads, kv_heads, dim, page_size, portions,
                                                            window, 28)
     want = torch.empty_like(q)
     ref.attention(q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, dim, dim ** -0.5, window, want)
     cctx, cmeta = _to_cuda(ctx, meta)
     got = torch.full_like(q, float("nan"), device="cuda")
-    hip.share_prompt_tiles, hip.wide_prompt_tiles = bool(shared), shared == "wide"
+    hip.share_prompt_tiles, hip.wide_prompt_tiles, hip.split_prompt_keys = bool(shared), shared == "wide", shared == "cut"
+    hip.decode_min_segment = 32 if shared == "cut" else hip.decode_min_segment    # several segments at these lengths
     try:
         hip.attention(q.cuda(), k_pages.cuda(), v_pages.cuda(), cctx, cmeta, q_heads, kv_heads, dim, dim ** -0.5, window, got)
     finally:
-        hip.share_prompt_tiles, hip.wide_prompt_tiles = True, None
+        hip.share_prompt_tiles, hip.wide_prompt_tiles, hip.split_prompt_keys, hip.decode_min_segment = True, None, None, 128
     torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(torch.bfloat16))
 
 
@@ -452,6 +454,23 @@ def test_attention_decode_batch(hip, ref, q_heads, kv_heads, dim, page_size, his
     got = torch.empty_like(q, device="cuda")
     hip.attention(q.cuda(), k_pages.cuda(), v_pages.cuda(), cctx, cmeta, q_heads, kv_heads, dim, dim ** -0.5, window, got)
     assert not torch.isnan(got).any()
+    torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(torch.bfloat16))
+
+
+def test_short_portion_after_a_long_history_has_its_keys_cut(hip, ref):
+    """16 tokens after 2,500: blocks of four tiles would be 16 on the whole device, so the keys are cut over waves
+    (the same request beside a single token of another; the rule is asked directly too)."""
+    portions = [(700, 1), (2500, 16)]
+    q, k_pages, v_pages, ctx, meta, _, _ = _attention_case(torch.bfloat16, 8, 2, 128, 16, portions, None, 33)
+    ctx.num_decode_seqs = 1
+    assert hip._few_portion_blocks(ctx, 1, 8, 2)
+    long_portion = SimpleNamespace(host_q_start=[0, 1, 2049], num_seqs=2, max_seq_len=4096)
+    assert not hip._few_portion_blocks(long_portion, 1, 8, 2)
+    want = torch.empty_like(q)
+    ref.attention(q, k_pages, v_pages, ctx, meta, 8, 2, 128, 128 ** -0.5, None, want)
+    cctx, cmeta = _to_cuda(ctx, meta)
+    got = torch.full_like(q, float("nan"), device="cuda")
+    hip.attention(q.cuda(), k_pages.cuda(), v_pages.cuda(), cctx, cmeta, 8, 2, 128, 128 ** -0.5, None, got)
     torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(torch.bfloat16))
 
 
