@@ -89,3 +89,26 @@ def test_recorded_decode_steps_of_many_requests(case):
     assert sum(graph is not None for graph in engine._graphs.values()) == 1
     for seq in seqs:
         engine.close(seq)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_short_portions_and_single_tokens_after_a_long_history(model_folders, dtype):
+    """2,100 tokens in one step, then portions of 24 and 2 tokens and single tokens: at that history the bfloat16
+    attention of a short portion cuts its keys over waves as decoding does (heads of 64: the single tokens' own
+    encoding too).  Every fed position against the plain implementation."""
+    from conftest import TINY, random_ids
+    from ampere_kv_engine_amd.config import EngineConfig
+    from ampere_kv_engine_amd.engine import Engine
+    from plain.qwen3_plain import PlainQwen3
+    raw, _, _ = TINY["C"]
+    folder = model_folders["C"]
+    ids = random_ids(raw["vocab_size"], 2140, seed=77)
+    want = PlainQwen3(folder).logits(ids)
+    engine = Engine.from_folder(folder, EngineConfig(dtype=dtype, page_size=16, num_pages=140, max_seqs=2,
+                                                     max_batched_tokens=2112, max_seq_len=2240, device="cuda:0"))
+    schedule = [([("r", 2100)], []), ([("r", 24)], []), ([("r", 2)], [])] + [([("r", 1)], [])] * 13 + [([("r", 1)], ["r"])]
+    got, _ = schedules.run(engine, {"r": ids}, schedule)
+    error = (got["r"] - want).abs().max(dim=1).values
+    limit = tolerance(dtype, want)["atol"]
+    assert float(error.max()) <= limit, f"first wrong position {int((error > limit).nonzero()[0])}, error {float(error.max()):.3g}"
+    assert engine.cache.num_free_pages == [140]
