@@ -39,6 +39,8 @@ int akv_attention_rows(const void* q, const void* k_pages, const void* v_pages, 
                        const int* positions, const int* block_table, int table_width, void* out, int dtype,
                        long tokens, int q_heads, int kv_heads, int dim, int page_size, long num_pages, float scale,
                        int window, hipStream_t stream);
+int akv_decode_plan(const int* seq_lens, int seq_first, int seq_count, int window, int items_wanted, int min_segment,
+                    int items_grid, int* plan, hipStream_t stream);
 int akv_sample(const float* logits, const float* temperature, const unsigned long long* seeds,
                const unsigned int* draws, int* out, int rows, int vocab, hipStream_t stream);
 }

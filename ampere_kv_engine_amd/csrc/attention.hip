@@ -97,6 +97,64 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(
 
 }  // namespace
 
+// ---- the cut of single tokens' keys for the matrix-core decode attention ----------------------------------------------
+// The decode attention works on (request, segment of its keys) items.  Segments have ONE size for all requests of a
+// launch, worked out here from the lengths on the device: a long request among short ones gets as many segments as its
+// keys need, no block is started for a segment that holds nothing, and a step that was recorded once and is replayed
+// with other lengths is cut as the same step run eagerly would be.  One wave; lane r looks at request seq_first + r
+// (at most 64).  A request's keys span from `first` (the start of its window, down to a multiple of 32) to its token's
+// position; the size is the sum of the spans over items_wanted, up to a multiple of 32, at least min_segment; items
+// are numbered request by request.  The cut depends on the lengths only, so one plan serves every layer of a step.
+//   plan[0] = items in all, plan[1] = keys per segment
+//   plan[4 + 2 r] = items before request r's, plan[5 + 2 r] = its items                          (r < 64)
+//   plan[132 + 4 i] = request of item i (counted from seq_first), its first key, the token's position, its last key
+namespace {
+__global__ __launch_bounds__(64) void decode_plan_kernel(const int* __restrict__ seq_lens, int seq_first, int seq_count,
+                                                        int window, int items_wanted, int min_segment, int items_grid,
+                                                        int* __restrict__ plan) {
+  const int lane = threadIdx.x;
+  int pos = -1, first = 0, span = 0;
+  if (lane < seq_count) {
+    pos = seq_lens[seq_first + lane] - 1;
+    first = (window > 0 ? max(0, pos - window + 1) : 0) & ~31;
+    span = max(pos - first + 1, 0);
+  }
+  int total_span = span;
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1) total_span += __shfl_xor(total_span, offset, kWave);
+  const int size = max(min_segment, ((total_span + items_wanted - 1) / items_wanted + 31) & ~31);
+  const int count = (span + size - 1) / size;
+  int upto = count;  // inclusive prefix sum over the wave
+#pragma unroll
+  for (int step = 1; step < kWave; step <<= 1) {
+    const int other = __shfl_up(upto, step, kWave);
+    if (lane >= step) upto += other;
+  }
+  const int before = upto - count;
+  if (lane == kWave - 1) {
+    plan[0] = min(upto, items_grid);
+    plan[1] = size;
+  }
+  plan[4 + 2 * lane] = before;
+  plan[5 + 2 * lane] = count;
+  for (int z = 0; z < count; ++z) {
+    const int item = before + z;
+    if (item >= items_grid) break;  // (cannot happen with the host's bound; never write beyond the buffer)
+    const int lo = first + z * size;
+    *reinterpret_cast<int4*>(plan + 132 + 4 * item) = make_int4(lane, lo, pos, min(pos, lo + size - 1));
+  }
+}
+}  // namespace
+
+extern "C" int akv_decode_plan(const int* seq_lens, int seq_first, int seq_count, int window, int items_wanted,
+                               int min_segment, int items_grid, int* plan, hipStream_t stream) {
+  if (seq_count <= 0) return 0;
+  if (seq_count > 64 || items_wanted < 1 || min_segment < 32 || (min_segment & 31) != 0 || items_grid < 1) return -2;
+  decode_plan_kernel<<<1, 64, 0, stream>>>(seq_lens, seq_first, seq_count, window, items_wanted, min_segment, items_grid,
+                                           plan);
+  return AKV_LAUNCH_STATUS();
+}
+
 extern "C" int akv_attention_rows(const void* q, const void* k_pages, const void* v_pages, const int* seq_of_token,
                                   const int* positions, const int* block_table, int table_width, void* out, int dtype,
                                   long tokens, int q_heads, int kv_heads, int dim, int page_size, long num_pages,

@@ -77,6 +77,13 @@ struct Args {
   float scale_log2;           // softmax scale * log2(e)
   int window;                 // 0: none
   int seg_keys, num_splits;
+  // PLAN (single tokens, at most 64 requests per launch, instead of seg_keys / num_splits): the requests' keys were
+  // cut into (request, segment) items by `akv_decode_plan`, which wrote `plan`: [0] items in all, [4 + 2 r] the items
+  // before request r's and [5 + 2 r] their number, [132 + 4 i] item i's request (from seq_first), first key, token
+  // position and last key.  Such a launch has grid (kv_heads * head_groups, items_grid): the items that exist come
+  // first; `items_grid` is a bound the host knows.
+  const int* plan;
+  int items_grid;
   int units;                  // compute units of the device (block order of the shared kernel)
   // FRESH launches (single tokens whose projections have not been normed, rotated or written to the cache yet):
   const bf16_t* qkv;          // [tokens, (q_heads + 2 * kv_heads) * D]: query, key and value heads of a token in a row
@@ -232,8 +239,10 @@ __device__ __forceinline__ void encode_head(uintx4 (&reg)[KT], bool normed, floa
 // `a.qkv`.  Every block norms and rotates its own query heads in registers; the block whose keys include the token's
 // own position does the same for the new key, puts it and the new value into its operands in place of what the page
 // holds there, and writes both to the page for later steps.  No other block reads that slot in this launch.
+// (Split launches of head sizes up to 128 are held to the registers of two waves per SIMD: decoding lives on the
+// number of waves that wait for memory at the same time.)
 template <int NQ, bool SPLIT, bool PIPE, bool FRESH>
-__global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
+__global__ __launch_bounds__(64, (SPLIT && NQ == 1 && D <= 128) ? 2 : 1) void attention_mfma_kernel(const Args a) {
   const int lane = threadIdx.x, r16 = lane & 15, g = lane >> 4;
   // Without SPLIT a block works on two tiles, one after the other: tile `tiles - 1 - x` and tile `x`.  Under the
   // causal mask the late tiles of a prompt see many keys and the early ones few; a pair sees about the same number
@@ -244,9 +253,32 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
   const int slot = kOneTile ? static_cast<int>(blockIdx.x)
                             : (pass == 0 ? a.tiles - 1 - static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x));
   if (!kOneTile && pass == 1 && slot >= a.tiles - 1 - slot) break;  // the middle tile was the first pass's
-  const Tile t = find_tile(a, slot, a.tokens_per_tile);
-  if (!t.found) continue;
-  const int kvh = blockIdx.y / a.head_groups, hg = blockIdx.y % a.head_groups;
+  Tile t{};
+  int seg_lo = 0, seg_hi = 0x7fffffff;     // SPLIT: the keys of this block's segment
+  long part = 0;                           // SPLIT: index of its partial result's tile
+  if (SPLIT && a.plan != nullptr) {        // item blockIdx.y of the plan: a request and a segment of its keys
+    const int item = static_cast<int>(blockIdx.y);
+    if (item >= a.plan[0]) return;
+    const int4 record = *reinterpret_cast<const int4*>(a.plan + 132 + 4 * item);
+    t.request = a.seq_first + record.x;
+    t.first_row = a.q_start[a.seq_first] + record.x;   // one row per request
+    t.tokens = 1;
+    t.first_pos = record.z;
+    t.found = true;
+    seg_lo = record.y;
+    seg_hi = record.w;
+    part = static_cast<long>(item) * gridDim.x + blockIdx.x;
+  } else {
+    t = find_tile(a, slot, a.tokens_per_tile);
+    if (!t.found) continue;
+    if (SPLIT) {
+      seg_lo = static_cast<int>(blockIdx.z) * a.seg_keys;
+      seg_hi = seg_lo + a.seg_keys - 1;
+      part = (static_cast<long>(blockIdx.x) * gridDim.y + blockIdx.y) * a.num_splits + blockIdx.z;
+    }
+  }
+  const int head_block = (SPLIT && a.plan != nullptr) ? blockIdx.x : blockIdx.y;  // (kv head, group of its query heads)
+  const int kvh = head_block / a.head_groups, hg = head_block % a.head_groups;
   const uintx4 zero = uintx4{0u, 0u, 0u, 0u};
   const int page_size = 1 << a.page_shift, page_mask = page_size - 1;
 
@@ -291,8 +323,8 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
   int range_lo = a.window > 0 ? max(0, t.first_pos - a.window + 1) : 0;
   int range_hi = last_pos;
   if (SPLIT) {
-    range_lo = max(range_lo, static_cast<int>(blockIdx.z) * a.seg_keys);
-    range_hi = min(range_hi, (static_cast<int>(blockIdx.z) + 1) * a.seg_keys - 1);
+    range_lo = max(range_lo, seg_lo);
+    range_hi = min(range_hi, seg_hi);
   }
 
   float m[NQ], l[NQ];
@@ -590,7 +622,7 @@ __global__ __launch_bounds__(64) void attention_mfma_kernel(const Args a) {
     if (SPLIT) {
       if (!col_valid[nq]) continue;  // (next column) the merge never reads columns that are no (token, head) pair
       const int c = nq * 16 + r16;
-      float* dst = a.partial + ((((static_cast<long>(blockIdx.x) * gridDim.y + blockIdx.y) * a.num_splits + blockIdx.z) * (16 * NQ)) + c) * PSTRIDE;
+      float* dst = a.partial + (part * (16 * NQ) + c) * PSTRIDE;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<floatx4*>(dst + dt * 16 + g * 4) = o[nq][dt];
       if (g == 0) {
@@ -1069,21 +1101,28 @@ __global__ __launch_bounds__(64 * kMergeWaves) void attention_merge_kernel(const
   const int c = blockIdx.z, lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int token = c / a.heads_per_tile, head_in_group = hg * a.heads_per_tile + c % a.heads_per_tile;
   if (token >= t.tokens || head_in_group >= a.group) return;
+  // the request's partial results: `splits` tiles, `split_stride` floats apart
   const float* src = a.partial + (((static_cast<long>(blockIdx.x) * gridDim.y + blockIdx.y) * a.num_splits) * (16 * NQ) + c) * PSTRIDE;
-  const long split_stride = static_cast<long>(16 * NQ) * PSTRIDE;
+  long split_stride = static_cast<long>(16 * NQ) * PSTRIDE;
+  int splits = a.num_splits;
+  if (a.plan != nullptr) {  // the plan's items of request blockIdx.x follow each other
+    splits = a.plan[5 + 2 * blockIdx.x];
+    src = a.partial + ((static_cast<long>(a.plan[4 + 2 * blockIdx.x]) * gridDim.y + blockIdx.y) * (16 * NQ) + c) * PSTRIDE;
+    split_stride *= gridDim.y;
+  }
   // every wave finds the maximum over all segments (a lane per segment)
   float top = -INFINITY;
   bool poisoned = false;
-  for (int z0 = 0; z0 < a.num_splits; z0 += 64) {
+  for (int z0 = 0; z0 < splits; z0 += 64) {
     const int z = z0 + lane;
-    const float mz = z < a.num_splits ? src[z * split_stride + D] : -INFINITY;
+    const float mz = z < splits ? src[z * split_stride + D] : -INFINITY;
     poisoned = poisoned || mz != mz;
     top = fmaxf(top, mz);
   }
   top = wave_max(top);
   poisoned = __any(poisoned);
   // this wave's segments: z = wave + kMergeWaves * i
-  const int mine = (a.num_splits - wave + kMergeWaves - 1) / kMergeWaves;
+  const int mine = (splits - wave + kMergeWaves - 1) / kMergeWaves;
   float denom = 0.f, acc[PER];
 #pragma unroll
   for (int i = 0; i < PER; ++i) acc[i] = 0.f;
@@ -1145,14 +1184,16 @@ int launch(const Args& a, int tiles, bool shared, hipStream_t stream) {
     else return -2;
     return AKV_LAUNCH_STATUS();
   }
-  if (a.num_splits == 1 && a.qkv == nullptr) grid.x = (tiles + 1) / 2;  // a block takes a late tile and an early one
+  const bool items = a.plan != nullptr;  // single tokens whose keys were cut on the device: always with the merge
+  if (items) grid = dim3(a.kv_heads * a.head_groups, a.items_grid, 1);
+  const dim3 merge_grid(items ? a.seq_count : tiles, a.kv_heads * a.head_groups, a.heads_per_tile * a.tokens_per_tile);
+  if (a.num_splits == 1 && a.qkv == nullptr && !items) grid.x = (tiles + 1) / 2;  // a block takes a late tile and an early one
   if (a.qkv != nullptr) {
     if constexpr (NQ == 1 && D % 64 == 0) {
       if (!a.single_tokens) return -2;
-      if (a.num_splits > 1) {
+      if (items || a.num_splits > 1) {
         attention_mfma_kernel<NQ, true, true, true><<<grid, 64, 0, stream>>>(a);
-        grid.z = a.heads_per_tile * a.tokens_per_tile;
-        attention_merge_kernel<NQ><<<grid, 64 * kMergeWaves, 0, stream>>>(a);
+        attention_merge_kernel<NQ><<<merge_grid, 64 * kMergeWaves, 0, stream>>>(a);
       } else {
         attention_mfma_kernel<NQ, false, true, true><<<grid, 64, 0, stream>>>(a);
       }
@@ -1161,10 +1202,9 @@ int launch(const Args& a, int tiles, bool shared, hipStream_t stream) {
       return -2;
     }
   }
-  if (a.num_splits > 1) {
+  if (items || a.num_splits > 1) {
     attention_mfma_kernel<NQ, true, true, false><<<grid, 64, 0, stream>>>(a);
-    grid.z = a.heads_per_tile * a.tokens_per_tile;  // the columns that can be (token, head) pairs
-    attention_merge_kernel<NQ><<<grid, 64 * kMergeWaves, 0, stream>>>(a);
+    attention_merge_kernel<NQ><<<merge_grid, 64 * kMergeWaves, 0, stream>>>(a);  // a block per column that can be a (token, head) pair
   } else {
     attention_mfma_kernel<NQ, false, true, false><<<grid, 64, 0, stream>>>(a);
   }
@@ -1182,6 +1222,9 @@ int launch(const Args& a, int tiles, bool shared, hipStream_t stream) {
 // page_size must be a power of two, at least 4.  `single_tokens` says that every request brings exactly one token.
 // `shared`: blocks of four waves that share keys and values through LDS; `tiles` then counts tiles of
 // 4 * tokens_per_tile tokens, num_splits must be 1 and pages hold at least 8 tokens.
+// `plan` (not null: single tokens, at most 64 requests): seg_keys and num_splits are not used; the requests' keys were
+// cut into items by akv_decode_plan with the same seq_first, seq_count and window; `items_grid` is the bound given
+// there, and `partial` must hold items_grid * kv_heads * head_groups * 16 * nq * (D + 4) floats.
 // `qkv` (not null: single tokens, nq 1, head sizes that are multiples of 64): the tokens' stacked raw projections
 // [tokens, (q_heads + 2 * kv_heads) * D]; `q` is not read, the kernel norms (q_weight, k_weight, eps; both weights
 // null: no norm) and rotates (rope_table [table_positions, D / 2, 2], null: no rotation) queries and the new keys
@@ -1192,14 +1235,15 @@ extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
     int q_heads, int kv_heads, int heads_per_tile, int head_groups, int tokens_per_tile, int page_size, long num_pages,
     float scale, int window, int seg_keys, int num_splits, int single_tokens, int shared, const void* qkv,
     const float* q_weight, const float* k_weight, float eps, const float* rope_table, int table_positions,
-    hipStream_t stream) {
+    const int* plan, int items_grid, hipStream_t stream) {
   if (tiles <= 0 || seq_count <= 0) return 0;
   int page_shift = 0;
   while ((1 << page_shift) < page_size) ++page_shift;
   if (page_size < 4 || (1 << page_shift) != page_size || q_heads % kv_heads != 0 ||
       heads_per_tile * tokens_per_tile > 16 * nq || kv_heads * head_groups > 65535 || num_splits > 65535 ||
       num_splits < 1 || (single_tokens && tiles != seq_count) || (shared && (page_size < 8 || num_splits != 1)) ||
-      (qkv != nullptr && (shared || !single_tokens || nq != 1 || D % 64 != 0 || (q_weight == nullptr) != (k_weight == nullptr))))
+      (qkv != nullptr && (shared || !single_tokens || nq != 1 || D % 64 != 0 || (q_weight == nullptr) != (k_weight == nullptr))) ||
+      (plan != nullptr && (shared || !single_tokens || seq_count > 64 || items_grid < 1 || items_grid > 65535)))
     return -2;
   Args a;
   a.q = static_cast<const bf16_t*>(q);
@@ -1227,6 +1271,8 @@ extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
   a.window = window;
   a.seg_keys = seg_keys;
   a.num_splits = num_splits;
+  a.plan = plan;
+  a.items_grid = items_grid;
   a.units = 1;
   a.qkv = static_cast<const bf16_t*>(qkv);
   a.q_weight = q_weight;

@@ -113,13 +113,15 @@ class HipKernels:
         self.share_prompt_tiles = True  # prompt portions: blocks of four waves share keys and values through LDS
         self.one_wave_per_head = False  # True: every attention goes to the plain kernel, a wave per (token, head)
         self.fresh_decode_tokens = True  # single tokens: norm, rotation and cache write inside the attention kernel
+        self.cut_keys_on_device = True  # single tokens: segments of one size for all requests, worked out from the lengths
+        self._plan_buffers = []         # where such cuts are written: one buffer per plan of a step
         self.wide_prompt_tiles = None   # such blocks with 32 columns per wave instead of 16: None = by the step's size
         self.split_prompt_keys = None   # prompt portions on one wave per tile and key segment: None = by the step's size
         self.compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
         for name in ("akv_embed", "akv_add_rmsnorm", "akv_rmsnorm_rows", "akv_copy_rows", "akv_gather_rows",
                      "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
                      "akv_linear_tiled", "akv_linear_packed", "akv_linear_packed_swiglu", "akv_pack_rows",
-                     "akv_attention_rows", "akv_sample"):
+                     "akv_attention_rows", "akv_decode_plan", "akv_sample"):
             getattr(self.lib, name).restype = ctypes.c_int
 
     # ---- helpers -----------------------------------------------------------------------------------------
@@ -451,8 +453,17 @@ class HipKernels:
         per_tile = tokens_per_tile * (4 if shared else 1)
         tiles = sum((starts[r + 1] - starts[r] + per_tile - 1) // per_tile
                     for r in range(seq_first, seq_first + seq_count))
-        num_splits, seg_keys, partial = 1, 0, None
-        if split:
+        num_splits, seg_keys, partial, plan, items_grid = 1, 0, None, None, 0
+        arena = getattr(ctx, "arena", None)
+        take = lambda count: (arena.take((count,), torch.float32) if arena is not None
+                              else torch.empty(count, dtype=torch.float32, device=self.device))
+        if (split and single and self.cut_keys_on_device and seq_count <= 64
+                and max(ctx.host_seq_lens[seq_first:seq_first + seq_count]) > self.decode_min_segment):
+            # single tokens: their keys are cut on the device, from the lengths there (requests of 128 keys or
+            # fewer are not cut: then the kernel without merge)
+            plan, items_grid = self._decode_plan(ctx, seq_first, seq_count, window, kv_heads * head_groups)
+            partial = take(items_grid * kv_heads * head_groups * 16 * nq * (head_dim + 4))
+        elif split:
             longest = max(ctx.host_seq_lens[seq_first:seq_first + seq_count])
             pairs = tiles * kv_heads * head_groups
             num_splits = max(1, min((self.decode_wave_target + pairs - 1) // pairs,
@@ -461,10 +472,7 @@ class HipKernels:
             seg_keys = ((longest + num_splits - 1) // num_splits + 31) // 32 * 32
             num_splits = (longest + seg_keys - 1) // seg_keys
             if num_splits > 1:
-                count = tiles * kv_heads * head_groups * num_splits * 16 * nq * (head_dim + 4)
-                arena = getattr(ctx, "arena", None)
-                partial = (arena.take((count,), torch.float32) if arena is not None
-                           else torch.empty(count, dtype=torch.float32, device=self.device))
+                partial = take(tiles * kv_heads * head_groups * num_splits * 16 * nq * (head_dim + 4))
         qkv, q_weight, k_weight, eps, table = fresh if fresh is not None else (None, None, None, 0.0, None)
         self._check(self._attention_mfma_entry(head_dim)(
             _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial), _ptr(ctx.q_start), _ptr(ctx.seq_lens),
@@ -472,8 +480,50 @@ class HipKernels:
             head_groups, tokens_per_tile, page_size, ctypes.c_long(num_pages), ctypes.c_float(scale),
             int(window) if window is not None else 0, seg_keys, num_splits, 1 if single else 0, 1 if shared else 0,
             _ptr(qkv), _ptr(q_weight), _ptr(k_weight), ctypes.c_float(eps), _ptr(table),
-            table.shape[0] if table is not None else 0, self._stream()),
+            table.shape[0] if table is not None else 0, _ptr(plan), items_grid, self._stream()),
             "attention")
+
+    PLAN_ENTRIES = 132          # ints of a plan before its items (4 per item)
+
+    def _decode_plan(self, ctx, seq_first, seq_count, window, head_blocks):
+        """The cut of the keys of requests seq_first .. + seq_count - 1 (single tokens) into (request, segment) items:
+        segments of one size for all requests - about `decode_wave_target` waves in all, no segment shorter than
+        `decode_min_segment` unless it is a request's only one - worked out by a one-wave kernel from the lengths on
+        the device.  The cut depends on the lengths alone, so the layers of a step share one plan: it is remembered on
+        the step's context.  Returns the plan and the bound on the number of items that sizes grids and buffers."""
+        items = max(1, self.decode_wave_target // head_blocks)
+        key = (seq_first, seq_count, int(window) if window is not None else 0, items, self.decode_min_segment)
+        plans = getattr(ctx, "decode_plans", None)
+        if plans is None:
+            plans = {}
+            try:
+                ctx.decode_plans = plans
+            except AttributeError:
+                pass
+        if key in plans:
+            return plans[key]
+        smallest = self.decode_min_segment
+        items_grid = min(items + seq_count, sum((length + smallest - 1) // smallest
+                                                for length in ctx.host_seq_lens[seq_first:seq_first + seq_count]))
+        if items_grid > 65535:
+            raise KernelError(f"{items_grid} segments of keys in one launch; the grid holds 65,535")
+        # plans live in buffers of the kernel set (a step's arenas are handed on from layer to layer), one per plan
+        # of a step; a step's plans are made before any later step's, on the same stream
+        index = len(plans)
+        while len(self._plan_buffers) <= index:
+            self._plan_buffers.append(None)
+        need = self.PLAN_ENTRIES + 4 * items_grid
+        if self._plan_buffers[index] is None or self._plan_buffers[index].numel() < need:
+            if torch.cuda.is_current_stream_capturing() and self._plan_buffers[index] is not None:
+                raise KernelError("a recorded step needs a larger plan of its keys than the steps before it")
+            self._plan_buffers[index] = torch.empty(max(need, self.PLAN_ENTRIES + 4 * 4096), dtype=torch.int32,
+                                                    device=self.device)
+        plan = self._plan_buffers[index]
+        self._dense(ctx.seq_lens, "seq_lens", torch.int32, (ctx.num_seqs,))
+        self._check(self.lib.akv_decode_plan(_ptr(ctx.seq_lens), seq_first, seq_count, key[2], items, smallest,
+                                             items_grid, _ptr(plan), self._stream()), "decode_plan")
+        plans[key] = (plan, items_grid)
+        return plans[key]
 
     def _few_portion_blocks(self, ctx, first, q_heads, kv_heads) -> bool:
         """Whether the prompt portions of the step are so short, and their histories so long, that blocks of four
@@ -560,8 +610,9 @@ class HipKernels:
             common = (q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out, page_size,
                       num_pages)
             decodes = ctx.num_decode_seqs
-            if decodes:      # single tokens against long histories: one small tile each, keys split over waves
-                self._attention_mfma(*common, 0, decodes, 1, True, fresh=fresh)
+            # single tokens against long histories: one small tile each, keys split over waves; 64 requests a launch
+            for first in range(0, decodes, 64):
+                self._attention_mfma(*common, first, min(64, decodes - first), 1, True, fresh=fresh)
             if ctx.num_seqs > decodes:
                 shared = page_size >= 8 and self.share_prompt_tiles
                 nq = 2 if head_dim <= 128 else 1

@@ -457,6 +457,54 @@ def test_attention_decode_batch(hip, ref, q_heads, kv_heads, dim, page_size, his
     torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("lengths,window", [([9000, 130, 129, 4000], None), ([300] * 64, None), ([70000, 33, 512], None),
+                                            ([5000, 200, 1000], 300), ([1], None)])
+def test_decode_plan(hip, lengths, window):
+    """The cut of single tokens' keys into items, as the one-wave kernel writes it, against the rule in plain
+    arithmetic: one segment size for all requests from the sum of their spans, items numbered request by request."""
+    items_wanted, smallest, first_request = 256, 128, 2
+    seq_lens = torch.tensor([7, 7] + lengths, dtype=torch.int32, device="cuda")        # two requests before the launch's
+    ctx = SimpleNamespace(seq_lens=seq_lens, num_seqs=len(lengths) + 2, host_seq_lens=[7, 7] + lengths)
+    hip.decode_wave_target, kept = items_wanted * 4, hip.decode_wave_target
+    try:
+        plan, grid = hip._decode_plan(ctx, first_request, len(lengths), window, 4)
+    finally:
+        hip.decode_wave_target = kept
+    plan = plan.cpu().tolist()
+    spans, firsts = [], []
+    for length in lengths:
+        pos = length - 1
+        first = (max(0, pos - window + 1) if window else 0) // 32 * 32
+        firsts.append(first)
+        spans.append(pos - first + 1)
+    size = max(smallest, (-(-sum(spans) // items_wanted) + 31) // 32 * 32)
+    counts = [-(-span // size) for span in spans]
+    assert plan[0] == sum(counts) <= grid and plan[1] == size
+    item = 0
+    for r, (length, first, count) in enumerate(zip(lengths, firsts, counts)):
+        assert plan[4 + 2 * r:6 + 2 * r] == [item, count]
+        for z in range(count):
+            lo = first + z * size
+            assert plan[132 + 4 * item:136 + 4 * item] == [r, lo, length - 1, min(length - 1, lo + size - 1)]
+            item += 1
+
+
+def test_attention_of_many_single_tokens_of_very_different_lengths(hip, ref):
+    """70 requests in one step (two launches of at most 64), one of them a hundred times longer than most: every
+    request's keys are cut into segments of the same size."""
+    histories = [6000] + [40 + 13 * i for i in range(69)]
+    portions = [(h, 1) for h in histories]
+    q, k_pages, v_pages, ctx, meta, _, _ = _attention_case(torch.bfloat16, 8, 2, 128, 16, portions, None, 36)
+    ctx.num_decode_seqs = len(portions)
+    want = torch.empty_like(q)
+    ref.attention(q, k_pages, v_pages, ctx, meta, 8, 2, 128, 128 ** -0.5, None, want)
+    cctx, cmeta = _to_cuda(ctx, meta)
+    got = torch.full_like(q, float("nan"), device="cuda")
+    hip.attention(q.cuda(), k_pages.cuda(), v_pages.cuda(), cctx, cmeta, 8, 2, 128, 128 ** -0.5, None, got)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(torch.bfloat16))
+    assert len(cctx.decode_plans) == 2
+
+
 def test_short_portion_after_a_long_history_has_its_keys_cut(hip, ref):
     """16 tokens after 2,500: blocks of four tiles would be 16 on the whole device, so the keys are cut over waves
     (the same request beside a single token of another; the rule is asked directly too)."""
