@@ -264,15 +264,84 @@ template <> __device__ __forceinline__ void store8<bf16_t>(bf16_t* p, const floa
   *reinterpret_cast<uint4*>(p) = u;
 }
 
+// Values of eight consecutive rows of the step and one kv head, written by one wave.  A value page lies
+// [dim, page_size]: a token's value is `dim` elements that are page_size apart, and written token by token that is
+// `dim` two-byte stores per head.  Here a lane takes two dims of eight tokens (eight 4-byte reads, each token's row
+// read by the wave as one piece); when the eight tokens' slots follow each other from a multiple of eight inside one
+// page - portions of prompts mostly do - it writes each dim's eight tokens as ONE 16-byte store.  Otherwise, and for
+// storage that is not 2 bytes wide, element by element.
+template <typename T>
+__device__ __forceinline__ void write_values_by_eights(const T* __restrict__ qkv, const int* __restrict__ slot_map,
+                                                       T* __restrict__ v_pages, long tokens, int q_heads, int kv_heads,
+                                                       int dim, int page_size, long num_slots, long item, int lane) {
+  const long groups = (tokens + 7) / 8;
+  if (item >= groups * kv_heads) return;
+  const long n0 = (item / kv_heads) * 8;
+  const int h = static_cast<int>(item % kv_heads);
+  const long row = static_cast<long>(q_heads + 2 * kv_heads) * dim;
+  long slot[8];
+  bool together = (page_size & 7) == 0 && sizeof(T) == 2;
+#pragma unroll
+  for (int t = 0; t < 8; ++t) {
+    slot[t] = n0 + t < tokens ? slot_map[n0 + t] : -1;
+    if (slot[t] < 0 || slot[t] >= num_slots) slot[t] = -1;  // host checks the map; never write outside the pool
+    together = together && slot[t] >= 0 && slot[t] == slot[0] + t;
+  }
+  together = together && (slot[0] & 7) == 0;
+  const T* src = qkv + n0 * row + static_cast<long>(q_heads + kv_heads + h) * dim;
+  for (int d = 2 * lane; d < dim; d += 2 * kWave) {
+    T pair[8][2];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      if (slot[t] >= 0) {
+        pair[t][0] = src[t * row + d];
+        pair[t][1] = src[t * row + d + 1];
+      } else {
+        pair[t][0] = pair[t][1] = T{};
+      }
+    }
+    if constexpr (sizeof(T) == 2) {
+      if (together) {
+        const long page = slot[0] / page_size, offset = slot[0] % page_size;
+        T* dst = v_pages + ((page * kv_heads + h) * dim + d) * page_size + offset;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          T line[8];
+#pragma unroll
+          for (int t = 0; t < 8; ++t) line[t] = pair[t][e];
+          *reinterpret_cast<uint4*>(dst + static_cast<long>(e) * page_size) = *reinterpret_cast<const uint4*>(line);
+        }
+        continue;
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      if (slot[t] < 0) continue;
+      const long page = slot[t] / page_size, offset = slot[t] % page_size;
+      T* dst = v_pages + ((page * kv_heads + h) * dim + d) * page_size + offset;
+      dst[0] = pair[t][0];
+      dst[page_size] = pair[t][1];
+    }
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
     const T* __restrict__ qkv, const float* __restrict__ q_weight, const float* __restrict__ k_weight, float eps,
     const float* __restrict__ table, int table_positions, const int* __restrict__ positions,
     const int* __restrict__ slot_map, T* __restrict__ k_pages, T* __restrict__ v_pages, T* __restrict__ q_out,
-    long tokens, int q_heads, int kv_heads, int dim, int page_size, long num_slots) {
+    long tokens, int q_heads, int kv_heads, int dim, int page_size, long num_slots, unsigned value_blocks_from) {
   const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  if (blockIdx.x >= value_blocks_from) {  // the blocks that write values, eight tokens at a time (see below)
+    write_values_by_eights<T>(qkv, slot_map, v_pages, tokens, q_heads, kv_heads, dim, page_size, num_slots,
+                              static_cast<long>(blockIdx.x - value_blocks_from) * waves + wave, lane);
+    return;
+  }
   const int lanes_per_head = dim / 16, heads_per_wave = kWave / lanes_per_head;
-  const int heads = q_heads + 2 * kv_heads, groups = (heads + heads_per_wave - 1) / heads_per_wave;
+  // with blocks of their own for the values, the heads of this part are the query and key heads alone
+  const int row_heads = q_heads + 2 * kv_heads;
+  const int heads = value_blocks_from == 0xffffffffu ? row_heads : q_heads + kv_heads;
+  const int groups = (heads + heads_per_wave - 1) / heads_per_wave;
   const long item = static_cast<long>(blockIdx.x) * waves + wave;
   if (item >= tokens * groups) return;
   const long n = item / groups;
@@ -301,7 +370,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
   }
   const bool turns = works && !is_v;  // a query or key head: normed and rotated
   if (works) {
-    const T* src = qkv + (n * heads + h) * dim;
+    const T* src = qkv + (n * row_heads + h) * dim;
     load8<T>(src + j0, lo);
     load8<T>(src + half + j0, hi);
   }
@@ -471,12 +540,17 @@ int akv_qk_norm_rope_write(const void* qkv, const float* q_weight, const float* 
   if (tokens <= 0) return 0;
   if ((dim & 15) != 0 || dim > 16 * kWave) return -2;  // a head is dim / 16 lanes of one wave
   const int heads_per_wave = kWave / (dim / 16);
-  const long items = tokens * ((q_heads + 2 * kv_heads + heads_per_wave - 1) / heads_per_wave);
+  // With a cache to write and several tokens, the values get blocks of their own after those of queries and keys.
+  const bool values_apart = slot_map != nullptr && tokens >= 8;
+  const int heads = values_apart ? q_heads + kv_heads : q_heads + 2 * kv_heads;
+  const long items = tokens * ((heads + heads_per_wave - 1) / heads_per_wave);
+  const long value_items = values_apart ? (tokens + 7) / 8 * kv_heads : 0;
+  const unsigned first = blocks_for(items, 4), more = values_apart ? blocks_for(value_items, 4) : 0u;
   AKV_DISPATCH(dtype, T,
-               qk_norm_rope_write_kernel<T><<<blocks_for(items, 4), 256, 0, stream>>>(
+               qk_norm_rope_write_kernel<T><<<first + more, 256, 0, stream>>>(
                    static_cast<const T*>(qkv), q_weight, k_weight, eps, table, table_positions, positions, slot_map,
                    static_cast<T*>(k_pages), static_cast<T*>(v_pages), static_cast<T*>(q_out), tokens, q_heads,
-                   kv_heads, dim, page_size, num_pages * page_size));
+                   kv_heads, dim, page_size, num_pages * page_size, values_apart ? first : 0xffffffffu));
   return AKV_LAUNCH_STATUS();
 }
 

@@ -320,6 +320,39 @@ def test_qk_norm_rope_write(hip, ref, dtype, q_heads, kv_heads, dim, page_size, 
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("q_heads,kv_heads,dim,page_size", [(4, 2, 16, 16), (6, 1, 32, 8), (8, 8, 128, 4), (5, 5, 80, 32),
+                                                             (2, 1, 256, 16), (32, 8, 128, 16)])
+def test_qk_norm_rope_write_of_many_tokens(hip, ref, dtype, q_heads, kv_heads, dim, page_size):
+    """From eight tokens on the values get blocks of their own that take eight rows at a time: eight slots that follow
+    each other from a multiple of eight (one 16-byte store per dim), the same run shifted by three (it crosses into
+    another page where pages are small), slots in falling order, a run cut by the end of the step."""
+    starts = [4 * 64, 2 * 64 + 3, None, 5 * 64 + 8, 1 * 64]            # first slot of each group of eight rows
+    slots = []
+    for group, start in enumerate(starts):
+        slots += [6 * 64 + 40 - 3 * i for i in range(8)] if start is None else [start + i for i in range(8)]
+    slots = slots[:37]                                                   # the last group has five rows
+    tokens, num_pages = len(slots), 8 * 64 // page_size
+    qkv = rand(tokens, (q_heads + 2 * kv_heads) * dim, dtype=dtype, seed=51)
+    qw, kw = 1 + rand(dim, seed=18, scale=0.1), 1 + rand(dim, seed=19, scale=0.1)
+    exponent = torch.arange(0, dim, 2, dtype=torch.int64).float() / dim
+    table = torch.empty(64, dim // 2, 2)
+    ref.rope_table(1.0 / (1e4 ** exponent), table)
+    positions = torch.arange(tokens, dtype=torch.int32) + 11
+    slots = torch.tensor(slots, dtype=torch.int32)
+    k_ref, v_ref = _pages(num_pages, kv_heads, page_size, dim, dtype)
+    q_ref = torch.empty(tokens, q_heads * dim, dtype=dtype)
+    ref.qk_norm_rope_write(qkv, qw, kw, 1e-6, table, positions, slots, k_ref, v_ref, q_ref, q_heads, kv_heads, dim)
+    k_hip, v_hip = (t.cuda() for t in _pages(num_pages, kv_heads, page_size, dim, dtype))
+    q_hip = torch.empty(tokens, q_heads * dim, dtype=dtype, device="cuda")
+    hip.qk_norm_rope_write(qkv.cuda(), qw.cuda(), kw.cuda(), 1e-6, table.cuda(), positions.cuda(), slots.cuda(), k_hip,
+                           v_hip, q_hip, q_heads, kv_heads, dim)
+    torch.testing.assert_close(q_hip.cpu().float(), q_ref.float(), **tol(dtype))
+    torch.testing.assert_close(k_hip.cpu().float(), k_ref.float(), equal_nan=True, **tol(dtype))
+    torch.testing.assert_close(v_hip.cpu().float(), v_ref.float(), equal_nan=True, rtol=0, atol=0)   # v: bitwise copy
+    assert torch.isnan(v_hip.cpu().float()).sum() == torch.isnan(v_ref.float()).sum()   # nothing else was written
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_kv_write(hip, ref, dtype):
     tokens, kv_heads, dim, page_size = 5, 3, 48, 8
     k = rand(tokens, kv_heads, dim, dtype=dtype, seed=20)
