@@ -34,6 +34,9 @@ int akv_linear_packed(const void* x, const void* wp, void* y, int y_dtype, int r
                       int k_tiles, int x_packed, hipStream_t stream);
 int akv_linear_packed_swiglu(const void* x, const void* wp, void* y, int y_dtype, int rows, int inter, int k,
                              int n_tiles, int k_tiles, int x_packed, hipStream_t stream);
+int akv_linear_packed_normed(const float* stream_in, const void* delta, const float* norm_weight, float eps,
+                             float* stream_out, const void* wp, void* y, int rows, int outs, int k, int n_tiles,
+                             int k_tiles, int gated, hipStream_t stream);
 int akv_pack_rows(const void* x, void* xp, int rows, int k, hipStream_t stream);
 int akv_attention_rows(const void* q, const void* k_pages, const void* v_pages, const int* seq_of_token,
                        const int* positions, const int* block_table, int table_width, void* out, int dtype,

@@ -77,10 +77,24 @@ template <int MT, int RT> constexpr bool kSkinnyOwnSets = RT * MT <= 8;
 // group (MT per k-tile) would not fit the registers beside them
 template <int MT, int RT> constexpr int kSkinnyGroup = (RT == 1 && MT >= 3) ? 4 : 8 / RT;
 
-template <int MT, int RT, typename TY, bool GATED>
+// NORMED (a few rows): x is not read.  The rows are the residual sum `stream_in` (+ `delta`) normed as the norm
+// kernel norms them - x * rsqrt(mean(x^2) + eps), rounded, times the weight, rounded - by every block for itself into
+// LDS, while its first weights are on their way; block 0 also writes the new residual sum to `stream_out` (another
+// buffer: the other blocks still read the old one).  That spares the step the norm's own launch.
+struct NormIn {
+  const float* stream_in;   // [rows, k]
+  const bf16_t* delta;      // [rows, k] or null
+  const float* weight;      // [k]
+  float* stream_out;        // [rows, k], not stream_in
+  float eps;
+  int red_floats;           // floats of `red` before the rows in LDS
+};
+
+template <int MT, int RT, typename TY, bool GATED, bool NORMED = false>
 __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __restrict__ x, const uintx4* __restrict__ wp,
                                                             TY* __restrict__ y, int rows, int outs, int k,
-                                                            int k_tiles, int n_tiles, int k_split, int x_packed) {
+                                                            int k_tiles, int n_tiles, int k_split, int x_packed,
+                                                            const NormIn norm) {
   constexpr int U = kSkinnyGroup<MT, RT>;  // k-tiles per group; two groups are in flight
   extern __shared__ float red[];  // [wave, or group of waves with the same row tiles][RT][MT][4][64]
   const int lane = threadIdx.x & 63, waves = blockDim.x >> 6;
@@ -96,7 +110,76 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  if (row_tile < n_tiles && kt0 < kt1) {
+  const bool works = row_tile < n_tiles && kt0 < kt1;
+  // NORMED: the first group of weights is asked for before the rows are normed (every thread of the block takes part in
+  // that, also those of waves without work), and handed to the loop below.
+  constexpr int UN = NORMED ? U : 1;
+  uintx4 early[NORMED ? RT : 1][UN];
+  if constexpr (NORMED) {
+    const uintx4 none = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        early[rt][u] = (works && kt0 + u < kt1 && row_tile + rt < n_tiles)
+                           ? load_once(wp + (static_cast<size_t>(row_tile + rt) * k_tiles + kt0 + u) * 64 + lane) : none;
+    uint16_t* rows_lds = reinterpret_cast<uint16_t*>(red + norm.red_floats);
+    // the waves share the rows: waves / rows of them take a row, each its own stride of the row's pieces of 8
+    const int waves_per_row = max(1, waves / rows);
+    const int row = wave / waves_per_row, part = wave % waves_per_row;
+    const bool has_row = row < rows;
+    const float* from = norm.stream_in + static_cast<size_t>(has_row ? row : 0) * k;
+    const bf16_t* add = norm.delta != nullptr ? norm.delta + static_cast<size_t>(has_row ? row : 0) * k : nullptr;
+    auto eight = [&](int i, float (&v)[8]) {
+      const float4 lo = *reinterpret_cast<const float4*>(from + i), hi = *reinterpret_cast<const float4*>(from + i + 4);
+      v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+      if (add != nullptr) {
+        const uintx4 d = *reinterpret_cast<const uintx4*>(add + i);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          v[2 * w] += __uint_as_float(d[w] << 16);
+          v[2 * w + 1] += __uint_as_float(d[w] & 0xffff0000u);
+        }
+      }
+    };
+    const int first = (part * 64 + lane) * 8, stride = waves_per_row * 64 * 8;
+    float squares = 0.f;
+    if (has_row) {
+      for (int i = first; i < k; i += stride) {
+        float v[8];
+        eight(i, v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) squares += v[e] * v[e];
+      }
+    }
+    squares = wave_sum(squares);
+    if (lane == 0) red[wave] = squares;
+    __syncthreads();
+    if (has_row) {
+      float total = 0.f;
+      for (int p = 0; p < waves_per_row; ++p) total += red[row * waves_per_row + p];  // the same order in every wave
+      const float scale = rsqrtf(total / static_cast<float>(k) + norm.eps);
+      for (int i = first; i < k; i += stride) {  // (the row comes from the caches the second time)
+        float v[8];
+        eight(i, v);
+        if (blockIdx.x == 0) {
+          float* to = norm.stream_out + static_cast<size_t>(row) * k + i;
+          *reinterpret_cast<float4*>(to) = make_float4(v[0], v[1], v[2], v[3]);
+          *reinterpret_cast<float4*>(to + 4) = make_float4(v[4], v[5], v[6], v[7]);
+        }
+        const float4 g0 = *reinterpret_cast<const float4*>(norm.weight + i), g1 = *reinterpret_cast<const float4*>(norm.weight + i + 4);
+        const float gain[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+        uintx4 packed;
+#pragma unroll
+        for (int w = 0; w < 4; ++w)
+          packed[w] = bf16_bits(rounded<bf16_t>(v[2 * w] * scale) * gain[2 * w]) |
+                      (static_cast<uint32_t>(bf16_bits(rounded<bf16_t>(v[2 * w + 1] * scale) * gain[2 * w + 1])) << 16);
+        *reinterpret_cast<uintx4*>(rows_lds + static_cast<size_t>(row) * k + i) = packed;
+      }
+    }
+    __syncthreads();  // the rows are in LDS; `red` is free again
+  }
+  if (works) {
     // Addresses: a scalar base per wave plus a 32-bit lane offset, so that a load is one instruction.
     const size_t w_tile_row = static_cast<size_t>(k_tiles) * 1024;  // bytes of one row tile
     const char* w_wave = reinterpret_cast<const char*>(wp) + static_cast<size_t>(row_tile) * w_tile_row;
@@ -136,7 +219,18 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
             a[rt][u] = (kt + u < kt1 && row_tile + rt < n_tiles)
                            ? load_once(reinterpret_cast<const uintx4*>(w_at + rt * w_tile_row + w_lane + u * 1024u)) : zero;
       }
-      if (kt + U <= kt1 && !ragged) {  // one test per row tile of x instead of one per load
+      if constexpr (NORMED) {  // the rows lie in LDS, normed: lane (r, g) reads row r, 16 bytes at k = g * 8 of the k-tile
+        const char* rows_lds = reinterpret_cast<const char*>(red + norm.red_floats);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int u = 0; u < U; ++u) {
+            const bool inside = !ragged || (kt + u) * 32 + g * 8 < k;
+            b[mt][u] = (kt + u < kt1 && x_row[mt] && inside)
+                           ? *reinterpret_cast<const uintx4*>(rows_lds + (static_cast<size_t>(mt * 16 + r) * k + (kt + u) * 32 + g * 8) * 2)
+                           : zero;
+          }
+      } else if (kt + U <= kt1 && !ragged) {  // one test per row tile of x instead of one per load
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
@@ -166,6 +260,12 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
           for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = mfma16(a[rt][u], b[mt][u], acc[rt][mt]);
     };
     fetch(kt0, a0, b0);
+    if constexpr (NORMED) {  // (the weights of the first group were asked for before the rows were normed)
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int u = 0; u < U; ++u) a0[rt][u] = early[rt][u];
+    }
     for (int kt = kt0; kt < kt1; kt += 2 * U) {
       fetch(kt + U, a1, b1);      // beyond kt1 this fills zeros
       multiply(a0, b0);
@@ -242,9 +342,9 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
   }
 }
 
-template <int MT, int RT, typename TY, bool GATED>
+template <int MT, int RT, typename TY, bool GATED, bool NORMED = false>
 int launch_skinny(const void* x, const void* wp, void* y, int rows, int outs, int k, int k_tiles, int n_tiles,
-                  int x_packed, hipStream_t stream) {
+                  int x_packed, hipStream_t stream, NormIn norm = NormIn{}) {
   // Enough waves to keep every CU's memory pipe full: k is split over the waves of a block when there are few row
   // tiles - down to short parts of k while the waves are very few, and further only while a wave keeps enough k-tiles
   // for two rounds of its double-buffered loop (measured: 1,536 waves of 32 k-tiles beat 3,072 of 16).
@@ -260,10 +360,16 @@ int launch_skinny(const void* x, const void* wp, void* y, int rows, int outs, in
   const int rows_per_block = waves / k_split;
   const int blocks = (wave_rows + rows_per_block - 1) / rows_per_block;
   const size_t sets = kSkinnyOwnSets<MT, RT> ? waves : rows_per_block;
-  const size_t lds = k_split > 1 ? sets * RT * MT * 4 * 64 * sizeof(float) : 0;
-  linear_skinny_kernel<MT, RT, TY, GATED><<<blocks, waves * 64, lds, stream>>>(
+  size_t lds = k_split > 1 ? sets * RT * MT * 4 * 64 * sizeof(float) : 0;
+  if constexpr (NORMED) {  // room for the block's sums, then the normed rows
+    lds = lds < 64 ? 64 : lds;
+    norm.red_floats = static_cast<int>(lds / sizeof(float));
+    lds += static_cast<size_t>(rows) * k * 2;
+    if (lds > 64 * 1024) return -2;
+  }
+  linear_skinny_kernel<MT, RT, TY, GATED, NORMED><<<blocks, waves * 64, lds, stream>>>(
       static_cast<const bf16_t*>(x), static_cast<const uintx4*>(wp), static_cast<TY*>(y), rows, outs, k, k_tiles,
-      n_tiles, k_split, x_packed);
+      n_tiles, k_split, x_packed, norm);
   return AKV_LAUNCH_STATUS();
 }
 
@@ -541,4 +647,23 @@ extern "C" int akv_linear_packed_swiglu(const void* x, const void* wp, void* y, 
   if (rows <= 0 || inter <= 0) return 0;
   if ((k & 7) != 0 || (inter & 15) != 0 || n_tiles * 8 != inter || k_tiles * 32 < k) return -2;
   return linear_packed<true>(x, wp, y, y_dtype, rows, inter, k, n_tiles, k_tiles, x_packed, stream);
+}
+
+
+// The product of a few rows that are not computed yet: rows = norm(stream_in (+ delta)) as akv_add_rmsnorm norms them
+// (bfloat16 activations), normed by every block of the product for itself; stream_out [rows, k] receives
+// stream_in + delta and must be another buffer than stream_in.  `gated`: akv_linear_packed_swiglu's packing and result.
+// At most 4 rows; k a multiple of 8; -2 where the rows do not fit the block's LDS beside its sums.
+extern "C" int akv_linear_packed_normed(const float* stream_in, const void* delta, const float* norm_weight, float eps,
+                                        float* stream_out, const void* wp, void* y, int rows, int outs, int k,
+                                        int n_tiles, int k_tiles, int gated, hipStream_t stream) {
+  if (rows <= 0 || outs <= 0) return 0;
+  if (rows > 4 || (k & 7) != 0 || k_tiles * 32 < k || stream_in == stream_out ||
+      (gated ? ((outs & 15) != 0 || n_tiles * 8 != outs) : n_tiles * 16 < outs))
+    return -2;
+  NormIn norm{stream_in, static_cast<const bf16_t*>(delta), norm_weight, stream_out, eps, 0};
+  if (gated) return launch_skinny<1, 2, bf16_t, true, true>(nullptr, wp, y, rows, outs, k, k_tiles, n_tiles, 0, stream, norm);
+  if (rows >= 4 && n_tiles >= 384 && n_tiles < 2048)
+    return launch_skinny<1, 2, bf16_t, false, true>(nullptr, wp, y, rows, outs, k, k_tiles, n_tiles, 0, stream, norm);
+  return launch_skinny<1, 1, bf16_t, false, true>(nullptr, wp, y, rows, outs, k, k_tiles, n_tiles, 0, stream, norm);
 }

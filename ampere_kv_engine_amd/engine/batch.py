@@ -96,6 +96,9 @@ class StepContext:
     max_new_tokens: int = 0        # longest portion of the step
     arenas: tuple = ()             # two arenas used by alternate layers (a layer's output outlives its own arena's reset)
     stream_buffer: torch.Tensor | None = None   # float32 [max tokens, hidden]: the residual sum
+    spare_buffer: torch.Tensor | None = None    # float32 [a few rows, hidden]: where a small step may move it
+    stream: torch.Tensor | None = None          # the step's residual sum, wherever it is now
+    spare_stream: torch.Tensor | None = None    # the other buffer's rows, or None where the step has too many
 
 
 class BatchBuilder:

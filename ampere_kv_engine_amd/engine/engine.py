@@ -46,6 +46,10 @@ class Engine:
                                     engine_config.max_seqs, engine_config.max_pages_per_seq)
         self.stream_buffer = torch.empty((engine_config.max_batched_tokens, spec.hidden_size),
                                          dtype=torch.float32, device=self.device)
+        # a second place for the residual sum of steps of a few rows: a product that norms its rows itself reads the
+        # old sum in every block while one block writes the new one
+        self.spare_buffer = torch.empty((self.SPARE_STREAM_ROWS, spec.hidden_size), dtype=torch.float32,
+                                        device=self.device)
         self.loaded = False
         self._graphs: dict[tuple, object] = {}               # (tokens per request, wanted rows, table width) -> graph
         self._graph_logits = None                            # [max_seqs, vocab] float32, where recorded steps write
@@ -103,10 +107,11 @@ class Engine:
             if shape is not None:
                 return self._step_recorded(entries, shape)
         ctx, _ = self.builder.build(entries)
-        ctx.stream_buffer = self.stream_buffer
+        ctx.stream_buffer, ctx.spare_buffer = self.stream_buffer, self.spare_buffer
         return self.model.forward(ctx, self.cache.layer_cache)
 
     # ---- steps as recorded graphs -----------------------------------------------------------------------------
+    SPARE_STREAM_ROWS = 1         # steps of up to this many tokens may move the residual sum between two buffers
     GRAPH_WIDTH_MULTIPLE = 64     # block tables of a recorded step are this many pages wide, or a multiple
     RECORD_MAX_TOKENS = 512       # steps with prompt portions are recorded up to this many tokens: beyond it the
                                   # device works longer on a step than the host needs to launch it
@@ -133,7 +138,7 @@ class Engine:
         recorded step overwrites them."""
         counts, wanted = shape
         ctx, _ = self.builder.build(entries, width_multiple=self.GRAPH_WIDTH_MULTIPLE)
-        ctx.stream_buffer = self.stream_buffer
+        ctx.stream_buffer, ctx.spare_buffer = self.stream_buffer, self.spare_buffer
         width = ctx.paged[0].width if ctx.paged else 0
         key = (counts, wanted, width)
         # sizes of launches come from the bound, not from this step's lengths

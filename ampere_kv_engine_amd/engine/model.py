@@ -81,14 +81,18 @@ class Model:
         rt, k = self.rt, self.rt.kernels
         hidden = self.spec.hidden_size
         arenas = ctx.arenas
-        stream = ctx.stream_buffer[:ctx.num_tokens]
-        self.embedding.forward(ctx.token_ids, stream)
+        # the residual sum; a block may move it to the step's spare buffer (`ctx.spare_stream`) and says so in `ctx.stream`
+        ctx.stream = ctx.stream_buffer[:ctx.num_tokens]
+        spare = getattr(ctx, "spare_buffer", None)
+        ctx.spare_stream = spare[:ctx.num_tokens] if spare is not None and ctx.num_tokens <= spare.shape[0] else None
+        self.embedding.forward(ctx.token_ids, ctx.stream)
         pending = None
         for step_index, entry in enumerate(self.spec.run_order):
             ctx.arena = arenas[step_index & 1]
             ctx.arena.reset()
-            pending = self.blocks[entry.layer].forward(stream, pending, ctx, layer_cache[entry.cache_layer],
+            pending = self.blocks[entry.layer].forward(ctx.stream, pending, ctx, layer_cache[entry.cache_layer],
                                                        entry.writes_cache)
+        stream = ctx.stream
         wanted = ctx.logit_rows.shape[0]
         if wanted == 0:
             return None

@@ -115,12 +115,14 @@ class HipKernels:
         self.fresh_decode_tokens = True  # single tokens: norm, rotation and cache write inside the attention kernel
         self.cut_keys_on_device = True  # single tokens: segments of one size for all requests, worked out from the lengths
         self._plan_buffers = []         # where such cuts are written: one buffer per plan of a step
+        self.norm_in_products = True    # steps of a few rows: the products that follow a norm compute it themselves
         self.wide_prompt_tiles = None   # such blocks with 32 columns per wave instead of 16: None = by the step's size
         self.split_prompt_keys = None   # prompt portions on one wave per tile and key segment: None = by the step's size
         self.compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
         for name in ("akv_embed", "akv_add_rmsnorm", "akv_rmsnorm_rows", "akv_copy_rows", "akv_gather_rows",
                      "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
-                     "akv_linear_tiled", "akv_linear_packed", "akv_linear_packed_swiglu", "akv_pack_rows",
+                     "akv_linear_tiled", "akv_linear_packed", "akv_linear_packed_swiglu", "akv_linear_packed_normed",
+                     "akv_pack_rows",
                      "akv_attention_rows", "akv_decode_plan", "akv_sample"):
             getattr(self.lib, name).restype = ctypes.c_int
 
@@ -307,6 +309,43 @@ class HipKernels:
         self._dense(out, "out", None, (rows, outs))
         self._check(self.lib.akv_linear_tiled(_ptr(x), _code(x), _ptr(weight), _code(weight), _ptr(out), _code(out),
                                               rows, outs, k, self._stream()), "linear")
+
+    # The most rows whose norm the product's blocks compute for themselves.  Every block reads the rows again (24 KB a
+    # row at 4,096 wide): measured at Qwen3-8B sizes, a step of one row gains 0.16 ms of 4.09, two rows lose 0.04 ms,
+    # four lose 0.21 ms - so it is one.  (The kernel takes up to four.)
+    NORM_IN_PRODUCT_ROWS = 1
+
+    def norm_in_product(self, rows: int, weight, dtype) -> bool:
+        """Whether `linear_after_norm` takes this product: a few bfloat16 rows, a packed matrix, rows that fit the
+        block's LDS beside its sums."""
+        packed = weight.packed if isinstance(weight, GatedWeight) else weight
+        return (self.norm_in_products and 0 < rows <= self.NORM_IN_PRODUCT_ROWS and dtype == torch.bfloat16
+                and isinstance(packed, PackedWeight) and packed.k % 8 == 0 and rows * packed.k * 2 <= 48 * 1024)
+
+    def linear_after_norm(self, stream, delta, norm_weight, eps, stream_out, weight, out):
+        """out = norm(stream (+ delta)) W^T (a `GatedWeight`: silu(. Wgate^T) * (. Wup^T)) without a kernel for the
+        norm: every block of the product adds, norms and rounds the few rows itself, as `add_rmsnorm` would, while its
+        first weights are on their way.  stream [rows, k] float32 is not changed; stream_out [rows, k], another
+        buffer, receives stream + delta."""
+        gated = isinstance(weight, GatedWeight)
+        packed = weight.packed if gated else weight
+        rows, k = stream.shape
+        if not self.norm_in_product(rows, weight, out.dtype):
+            raise KernelError("this product does not take rows that are still to be normed")
+        self._dense(stream, "stream", torch.float32, (rows, packed.k))
+        self._dense(stream_out, "stream_out", torch.float32, (rows, k))
+        if stream_out.data_ptr() == stream.data_ptr():
+            raise KernelError("stream_out must be another buffer than stream")
+        if delta is not None:
+            self._dense(delta, "delta", torch.bfloat16, (rows, k))
+        self._dense(norm_weight, "norm weight", torch.float32, (k,))
+        outs = weight.inter if gated else packed.outs
+        self._dense(out, "out", torch.bfloat16, (rows, outs))
+        self._dense(packed.data, "packed weight", torch.bfloat16)
+        self._check(self.lib.akv_linear_packed_normed(
+            _ptr(stream), _ptr(delta), _ptr(norm_weight), ctypes.c_float(eps), _ptr(stream_out), _ptr(packed.data),
+            _ptr(out), rows, outs, k, packed.n_tiles, packed.k_tiles, 1 if gated else 0, self._stream()),
+            "linear_after_norm")
 
     def prepare_gated_linear(self, gate: torch.Tensor, up: torch.Tensor):
         """The packing for `gated_linear`, or None where the two matrices have to stay a stacked product followed by

@@ -17,6 +17,7 @@ from .position import NoPosition, RotaryHalf
 
 class Attention(Part):
     graph_safe = True
+    takes_pending_norm = True       # x is read once, by the stacked q/k/v product
 
     def __init__(self, spec, runtime):
         self.rt = runtime

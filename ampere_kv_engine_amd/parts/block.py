@@ -38,13 +38,34 @@ class PreNormBlock(Part):
     def forward(self, stream, pending, ctx, cache, writes_cache=True):
         """stream [tokens, hidden] float32 (updated in place); pending: the previous branch's output, not
         yet added, or None.  Returns this block's own pending output."""
-        tokens = stream.shape[0]
-        normed = ctx.arena.take((tokens, self.hidden), self.rt.dtype)
-        self.mixer_norm.forward_residual(stream, pending, normed)
+        normed, unnormed = self._normed(self.mixer_norm, self.mixer, stream, pending, ctx)
         mixed = self.mixer.forward(normed, ctx, cache, writes_cache)
-        normed2 = ctx.arena.take((tokens, self.hidden), self.rt.dtype)
-        self.feed_forward_norm.forward_residual(stream, mixed, normed2)
-        return self.feed_forward.forward(normed2, ctx)
+        stream = self._after(unnormed, stream, ctx)
+        normed, unnormed = self._normed(self.feed_forward_norm, self.feed_forward, stream, mixed, ctx)
+        out = self.feed_forward.forward(normed, ctx)
+        self._after(unnormed, stream, ctx)
+        return out
+
+    def _normed(self, norm, reader, stream, delta, ctx):
+        """norm(stream + delta) for `reader`: computed now - or, in steps of few rows (the context then has a spare
+        buffer for the residual sum), handed on unnormed to a reader that can take that, whose first product may
+        norm the rows itself: one launch less."""
+        spare = getattr(ctx, "spare_stream", None)
+        if spare is not None and getattr(reader, "takes_pending_norm", False) and hasattr(norm, "pending"):
+            unnormed = norm.pending(stream, delta, spare, ctx.arena)
+            return unnormed, unnormed
+        normed = ctx.arena.take((stream.shape[0], self.hidden), self.rt.dtype)
+        norm.forward_residual(stream, delta, normed)
+        return normed, None
+
+    @staticmethod
+    def _after(unnormed, stream, ctx):
+        """Where the residual sum is after the reader ran: in the spare buffer if its product normed the rows - the two
+        buffers then change roles, and the context is told - else where it was."""
+        if unnormed is None or not unnormed.moved:
+            return stream
+        ctx.stream, ctx.spare_stream = unnormed.stream_out, stream
+        return unnormed.stream_out
 
 
 def _build_prenorm(spec, runtime, mixer=None, feed_forward=None):

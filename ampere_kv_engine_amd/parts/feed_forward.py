@@ -13,6 +13,7 @@ from .linear import Linear
 
 class SwiGLU(Part):
     graph_safe = True
+    takes_pending_norm = True       # x is read once, by the first product
 
     def __init__(self, spec, runtime):
         self.rt = runtime
@@ -46,7 +47,11 @@ class SwiGLU(Part):
         """x [tokens, hidden] -> [tokens, hidden], both in the activation dtype."""
         tokens = x.shape[0]
         act = ctx.arena.take((tokens, self.inter), self.rt.dtype)
-        if self.gated is not None:
+        if self.gated is not None and hasattr(x, "product") and x.product(self.gated, act):
+            pass                    # the product normed the rows itself
+        elif self.gated is not None:
+            if hasattr(x, "rows"):
+                x = x.rows()
             shape = self.rt.kernels.gated_scratch(self.gated, tokens, self.rt.dtype)
             scratch = ctx.arena.take(shape, self.rt.dtype) if shape is not None else None
             self.rt.kernels.gated_linear(x, self.gated, act, scratch)

@@ -48,6 +48,11 @@ class Linear(Part):
     def weight_bytes(self):
         return self._bytes
 
-    def forward(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    def forward(self, x, out: torch.Tensor) -> torch.Tensor:
+        """x: [rows, in] in the activation dtype, or rows that are still to be normed (`PendingNorm`)."""
+        if hasattr(x, "product"):
+            if x.product(self.weight, out):
+                return out
+            x = x.rows()
         self.rt.kernels.linear(x, self.weight, out)
         return out

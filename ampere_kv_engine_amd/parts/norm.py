@@ -38,4 +38,46 @@ class RMSNorm(Part):
         return out
 
 
+    def pending(self, stream: torch.Tensor, delta: torch.Tensor | None, stream_out: torch.Tensor, arena) -> "PendingNorm":
+        """`forward_residual` not yet computed: for a consumer whose first product can compute it itself."""
+        return PendingNorm(self, stream, delta, stream_out, arena)
+
+
+class PendingNorm:
+    """The rows norm(stream + delta) before anybody has computed them.  A part that `takes_pending_norm` reads them
+    exactly once, through a `Linear` or the kernel set's gated product: where the kernel set's product can norm a few
+    rows itself (`norm_in_product`), it does, and the new residual sum is then in `stream_out` (`moved` tells the
+    block); otherwise the rows are normed here first, in place as `forward_residual` does."""
+
+    def __init__(self, norm: RMSNorm, stream, delta, stream_out, arena):
+        self.norm, self.stream, self.delta, self.stream_out, self.arena = norm, stream, delta, stream_out, arena
+        self.shape = (stream.shape[0], norm.size)
+        self.dtype = norm.rt.dtype
+        self.moved = False          # the residual sum now lives in stream_out
+        self._used = False
+
+    def _once(self):
+        if self._used:
+            raise RuntimeError("rows that were handed on unnormed can be read once")
+        self._used = True
+
+    def product(self, weight, out: torch.Tensor) -> bool:
+        """out = these rows times `weight` (a packed matrix or a gated pair) if the kernel set computes the norm inside
+        that product; False if the caller has to ask for `rows()` and multiply itself."""
+        kernels = self.norm.rt.kernels
+        can = getattr(kernels, "norm_in_product", None)
+        if can is None or not can(self.shape[0], weight, out.dtype):
+            return False
+        self._once()
+        kernels.linear_after_norm(self.stream, self.delta, self.norm.weight, self.norm.eps, self.stream_out, weight, out)
+        self.moved = True
+        return True
+
+    def rows(self) -> torch.Tensor:
+        """The rows, normed now by the norm's own kernel (the residual sum is updated in place)."""
+        self._once()
+        out = self.arena.take(self.shape, self.dtype)
+        return self.norm.forward_residual(self.stream, self.delta, out)
+
+
 register_part("norm", "rmsnorm", RMSNorm)

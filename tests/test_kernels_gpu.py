@@ -214,6 +214,57 @@ def test_gated_linear_rows_do_not_depend_on_the_batch_and_other_sizes_stay_stack
     assert hip.prepare_gated_linear(torch.zeros(48, 64), torch.zeros(48, 64)) is None
 
 
+@pytest.mark.parametrize("rows", [1, 3, 4])
+@pytest.mark.parametrize("outs,k", [(320, 256), (6144, 4096), (48, 520), (4096, 5120)])
+@pytest.mark.parametrize("with_delta", [True, False])
+def test_linear_after_norm(hip, ref, rows, outs, k, with_delta):
+    """The product whose blocks norm the rows themselves against the norm kernel followed by the product; the new
+    residual sum goes to the other buffer, the old one stays."""
+    stream = rand(rows, k, seed=61, scale=2.0)
+    delta = rand(rows, k, dtype=torch.bfloat16, seed=62) if with_delta else None
+    gain = 1 + rand(k, seed=63, scale=0.1)
+    w = rand(outs, k, dtype=torch.bfloat16, seed=64, scale=0.05)
+    want_stream, normed = stream.clone(), torch.empty(rows, k, dtype=torch.bfloat16)
+    ref.add_rmsnorm(want_stream, delta, gain, 1e-5, normed)
+    want = torch.empty(rows, outs, dtype=torch.bfloat16)
+    ref.linear(normed, w, want)
+    packed = hip.prepare_linear(w.cuda())
+    assert hip.norm_in_product(1, packed, torch.bfloat16) and not hip.norm_in_product(2, packed, torch.bfloat16)
+    old, new = stream.cuda(), torch.full((rows, k), float("nan"), device="cuda")
+    got = torch.full((rows, outs), float("nan"), dtype=torch.bfloat16, device="cuda")
+    hip.NORM_IN_PRODUCT_ROWS = 4         # what the kernel takes; the engine uses it for one row
+    try:
+        hip.linear_after_norm(old, delta.cuda() if with_delta else None, gain.cuda(), 1e-5, new, packed, got)
+    finally:
+        del hip.NORM_IN_PRODUCT_ROWS
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(torch.bfloat16))
+    torch.testing.assert_close(new.cpu(), want_stream, rtol=0, atol=0)
+    torch.testing.assert_close(old.cpu(), stream, rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("rows", [1, 4])
+def test_gated_linear_after_norm(hip, ref, rows):
+    inter, k = 208, 264
+    stream = rand(rows, k, seed=65, scale=2.0)
+    delta = rand(rows, k, dtype=torch.bfloat16, seed=66)
+    gain = 1 + rand(k, seed=67, scale=0.1)
+    gate, up = (rand(inter, k, dtype=torch.bfloat16, seed=68 + i, scale=0.05) for i in range(2))
+    want_stream, normed = stream.clone(), torch.empty(rows, k, dtype=torch.bfloat16)
+    ref.add_rmsnorm(want_stream, delta, gain, 1e-6, normed)
+    want = torch.empty(rows, inter, dtype=torch.bfloat16)
+    ref.gated_linear(normed, ref.prepare_gated_linear(gate, up), want)
+    weight = hip.prepare_gated_linear(gate.cuda(), up.cuda())
+    new = torch.empty(rows, k, device="cuda")
+    got = torch.full((rows, inter), float("nan"), dtype=torch.bfloat16, device="cuda")
+    hip.NORM_IN_PRODUCT_ROWS = 4
+    try:
+        hip.linear_after_norm(stream.cuda(), delta.cuda(), gain.cuda(), 1e-6, new, weight, got)
+    finally:
+        del hip.NORM_IN_PRODUCT_ROWS
+    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(torch.bfloat16))
+    torch.testing.assert_close(new.cpu(), want_stream, rtol=0, atol=0)
+
+
 def test_products_of_17_to_64_rows_choose_once(hip, ref):
     """Between 17 and 64 rows the engine's own product and the library's are timed at the first call with a matrix
     shape and number of row tiles; the choice is remembered for the process, every call gives the product, and other
