@@ -102,6 +102,8 @@ def main() -> int:
     parser.add_argument("--layers", type=int, default=QWEN3_8B["num_hidden_layers"],
                         help="fewer layers than the configuration has, where memory or time needs it")
     parser.add_argument("--points", default="1,64", help="further batch sizes to time (comma separated, '' for none)")
+    parser.add_argument("--contexts", default="", help="requests of different context lengths in one batch, e.g. "
+                        "'32768,512x63' (overrides --batch and --context; no further points, no prefill)")
     parser.add_argument("--no-prefill", action="store_true")
     parser.add_argument("--prefill-only", action="store_true", help="time the prefill alone (for kernel profiles)")
     parser.add_argument("--workload", choices=["decode", "serving-14b", "batch-32b"], default="decode",
@@ -123,12 +125,22 @@ def main() -> int:
     from ampere_kv_engine_amd.engine import Engine, StepEntry
     from ampere_kv_engine_amd.sampling import Sampler, SamplingParams
 
+    contexts = None
+    if args.contexts:
+        contexts = []
+        for piece in args.contexts.split(","):
+            length, _, count = piece.partition("x")
+            contexts += [int(length)] * (int(count) if count else 1)
+        args.batch, args.context, args.points, args.no_prefill = len(contexts), max(contexts), "", True
     points = [int(p) for p in args.points.split(",") if p]
     max_batch = max([args.batch] + points)
     raw = dict(QWEN3_8B, num_hidden_layers=args.layers)
     config = Qwen3Config.from_dict(raw)
     tokens_per_request = args.context + PRIMING + args.warmup + args.steps + 1
     pages = max_batch * ((tokens_per_request + PAGE_SIZE - 1) // PAGE_SIZE) + PREFILL_TOKENS // PAGE_SIZE + 2
+    if contexts is not None:
+        grown = PRIMING + args.warmup + args.steps + 1
+        pages = sum((length + grown + PAGE_SIZE - 1) // PAGE_SIZE for length in contexts) + PREFILL_TOKENS // PAGE_SIZE + 2
     engine_config = EngineConfig(dtype="bfloat16", page_size=PAGE_SIZE, num_pages=pages, max_seqs=max_batch,
                                  max_batched_tokens=PREFILL_TOKENS,
                                  max_seq_len=max(tokens_per_request, PREFILL_TOKENS) + PAGE_SIZE,
@@ -143,8 +155,8 @@ def main() -> int:
     def decode(batch: int, steps: int, warmup: int) -> float:
         """Seconds for `steps` decode steps of `batch` requests whose caches hold `context` tokens."""
         seqs = [engine.open(f"b{batch}_{i}") for i in range(batch)]
-        for seq in seqs:
-            engine.cache.reserve(seq, args.context - 1)
+        for index, seq in enumerate(seqs):
+            engine.cache.reserve(seq, (contexts[index] if contexts is not None else args.context) - 1)
         tokens = torch.randint(0, config.vocab_size, (batch,), generator=generator).tolist()
         greedy, draws = [SamplingParams() for _ in range(batch)], [0] * batch
 
@@ -191,7 +203,8 @@ def main() -> int:
     ms_per_step = elapsed / args.steps * 1000
     value = args.batch * args.steps / elapsed
     weight_bytes = engine.model.weight_bytes_per_step()
-    kv_bytes = args.batch * (args.context + PRIMING + args.warmup + args.steps // 2) * engine.cache.bytes_per_token()
+    held = sum(contexts) if contexts is not None else args.batch * args.context
+    kv_bytes = (held + args.batch * (PRIMING + args.warmup + args.steps // 2)) * engine.cache.bytes_per_token()
     achieved = (weight_bytes + kv_bytes) / (ms_per_step / 1000) / 1e9
     record = {
         "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2,048 tokens (Qwen3-8B bf16)",
@@ -205,7 +218,8 @@ def main() -> int:
                    "intermediate": config.intermediate_size, "vocab": config.vocab_size, "page_size": PAGE_SIZE,
                    "prefill_tokens": PREFILL_TOKENS, "rope_theta": config.rope_theta, "rms_norm_eps": config.rms_norm_eps,
                    "tied_embeddings": config.tie_word_embeddings,
-                   "library_products_above_rows": engine.config.library_products_above},
+                   "library_products_above_rows": engine.config.library_products_above,
+                   **({"contexts": args.contexts} if contexts is not None else {})},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
     }

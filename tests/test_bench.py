@@ -42,3 +42,17 @@ def test_the_line_of_a_short_run():
     assert prefill["tokens"] == 2048 and prefill["ms"] > 0 and 0 < prefill["frac"] < 1
     assert abs(prefill["value"] - 2048 / (prefill["ms"] / 1e3)) < 1e-2 * prefill["value"]
     assert line["points"]["decode_b1"] > 0
+
+
+@pytest.mark.gpu
+def test_a_batch_of_different_context_lengths():
+    """`--contexts 700,40x3`: four requests, one much longer than the others; the line names them and counts the
+    cache bytes of each."""
+    result = subprocess.run([sys.executable, BENCH, "--layers", "2", "--steps", "3", "--warmup", "1", "--contexts",
+                             "700,40x3"], capture_output=True, text=True, timeout=600, cwd=ROOT)
+    assert result.returncode == 0, result.stderr[-2000:]
+    line = json.loads(result.stdout.strip().splitlines()[-1])
+    config = line["config"]
+    assert config["global_batch"] == 4 and config["seq_len"] == 700 and config["contexts"] == "700,40x3"
+    assert len(config) <= 20 and "prefill" not in line and "points" not in line
+    assert abs(line["value"] - 4 / (line["ms_per_step"] / 1e3)) < 1e-2 * line["value"]
