@@ -10,8 +10,10 @@
 // order of the 32 key slots, exactly the B operand the second product needs; and O^T has the same column per lane
 // as the softmax statistics.  Nothing is transposed, nothing goes through LDS.
 // Scores, softmax (base 2, scale folded in) and the weighted sum are float32.  Keys are walked in steps of 32
-// aligned to absolute positions.  With SPLIT, grid.z cuts the keys into segments whose partial results (maximum,
-// sum, unnormalised output) a second kernel merges: decode has too few (request, head) pairs to fill the GPU otherwise.
+// aligned to absolute positions.  With SPLIT a block takes a segment of a request's keys, and a second kernel merges
+// the segments' partial results (maximum, sum, unnormalised output): decode has too few (request, head) pairs to fill
+// the GPU otherwise.  Single tokens' segments come from a plan made on the device from the requests' lengths (one
+// segment size for all of them); prompt portions that are cut get the same number of segments each (grid.z).
 
 #include <type_traits>
 
