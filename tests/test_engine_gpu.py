@@ -112,3 +112,29 @@ def test_short_portions_and_single_tokens_after_a_long_history(model_folders, dt
     limit = tolerance(dtype, want)["atol"]
     assert float(error.max()) <= limit, f"first wrong position {int((error > limit).nonzero()[0])}, error {float(error.max()):.3g}"
     assert engine.cache.num_free_pages == [140]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_long_and_a_short_request_decode_together(model_folders, dtype):
+    """A request of 2,100 tokens and one of 40 take their next 16 tokens in the same steps: the bfloat16 attention
+    cuts both requests' keys into segments of one size (many for the long one, one for the short one)."""
+    from conftest import TINY, random_ids
+    from ampere_kv_engine_amd.config import EngineConfig
+    from ampere_kv_engine_amd.engine import Engine
+    from plain.qwen3_plain import PlainQwen3
+    raw, _, _ = TINY["C"]
+    folder = model_folders["C"]
+    requests = {"long": random_ids(raw["vocab_size"], 2116, seed=78), "short": random_ids(raw["vocab_size"], 56, seed=79)}
+    plain = PlainQwen3(folder)
+    want = {name: plain.logits(ids) for name, ids in requests.items()}
+    engine = Engine.from_folder(folder, EngineConfig(dtype=dtype, page_size=16, num_pages=145, max_seqs=2,
+                                                     max_batched_tokens=2112, max_seq_len=2240, device="cuda:0"))
+    schedule = [([("long", 2100)], []), ([("short", 40)], [])] + [([("long", 1), ("short", 1)], [])] * 15
+    schedule.append(([("long", 1), ("short", 1)], ["long", "short"]))
+    got, _ = schedules.run(engine, requests, schedule)
+    for name in requests:
+        error = (got[name] - want[name]).abs().max(dim=1).values
+        limit = tolerance(dtype, want[name])["atol"]
+        assert float(error.max()) <= limit, (f"{name}: first wrong position {int((error > limit).nonzero()[0])}, "
+                                             f"error {float(error.max()):.3g}")
+    assert engine.cache.num_free_pages == [145]
