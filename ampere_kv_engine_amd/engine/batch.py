@@ -49,6 +49,9 @@ class Arena:
         self.chunks: list[torch.Tensor] = []
         self.chunk_index = 0
         self.offset = 0
+        # Steps ask for the same pieces in the same order again and again: the tensor made for (chunk, offset, shape,
+        # dtype) is kept and handed out again instead of slicing and viewing anew (chunks are never replaced).
+        self._views: dict[tuple, torch.Tensor] = {}
 
     def reset(self) -> None:
         self.chunk_index = 0
@@ -66,9 +69,14 @@ class Arena:
                 self.chunks.append(torch.empty(max(nbytes, self.chunk_bytes), dtype=torch.uint8, device=self.device))
             chunk = self.chunks[self.chunk_index]
             if self.offset + nbytes <= chunk.numel():
-                raw = chunk[self.offset:self.offset + count * size]
+                key = (self.chunk_index, self.offset, tuple(shape), dtype)
+                view = self._views.get(key)
+                if view is None:
+                    if len(self._views) >= 8192:     # shapes keep changing: do not keep them all
+                        self._views.clear()
+                    view = self._views[key] = chunk[self.offset:self.offset + count * size].view(dtype).view(*shape)
                 self.offset += nbytes
-                return raw.view(dtype).view(*shape)
+                return view
             self.chunk_index += 1
             self.offset = 0
 

@@ -143,13 +143,14 @@ class HipKernels:
         raise KernelError(f"{what}: launch failed with HIP error {status}")
 
     def _dense(self, t: torch.Tensor, name: str, dtype: torch.dtype | None = None, shape: tuple | None = None):
-        if not isinstance(t, torch.Tensor) or t.device != self.device:
+        # (called a thousand times in a step that is not replayed from a recording: the comparisons are the cheap ones)
+        if not isinstance(t, torch.Tensor) or not t.is_cuda or t.get_device() != self.device.index:
             raise KernelError(f"{name} must be a tensor on {self.device}, got {getattr(t, 'device', type(t))}")
         if not t.is_contiguous():
             raise KernelError(f"{name} must be contiguous")
         if dtype is not None and t.dtype != dtype:
             raise KernelError(f"{name} must be {dtype}, got {t.dtype}")
-        if shape is not None and tuple(t.shape) != tuple(shape):
+        if shape is not None and t.shape != (shape if type(shape) is tuple else tuple(shape)):
             raise KernelError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
         return t
 
