@@ -8,7 +8,8 @@ per request and one tensor `[layers, 2, pages, kv_heads, page_size * head_dim]`,
 every layer of its group.  Within a page, keys lie `[page_size, head_dim]` and values `[head_dim, page_size]`:
 scores contract over head_dim and the weighted sum over keys, and each reaches the matrix cores with its
 contracted axis contiguous.  Groups with a window give pages back while the request lives.  Mixers that ask
-for `SlotState` get a tensor `[slots, *shape]` per layer, zeroed when a request takes the slot.
+for `SlotState` get a tensor `[slots, *shape]` per layer, zeroed (or set by the mixer's own `init`) when a request
+takes the slot.
 
 Everything here except the tensors is host bookkeeping and runs without a GPU (`allocate_tensors=False`).
 """
@@ -66,7 +67,7 @@ class CacheManager:
         self.slots = SlotTable(max_seqs)
         self.groups: list[PagedGroup] = []
         self.layer_cache: dict[int, LayerCache] = {}
-        self._state_tensors: list[torch.Tensor] = []
+        self._state_tensors: list[tuple[torch.Tensor, SlotState]] = []
         self._live: dict[str, Sequence] = {}
         by_need: dict[PagedKV, PagedGroup] = {}
         for layer in sorted(needs):
@@ -94,7 +95,7 @@ class CacheManager:
                          if allocate_tensors else None)
                 self.layer_cache[layer] = LayerCache(state=state)
                 if state is not None:
-                    self._state_tensors.append(state)
+                    self._state_tensors.append((state, need))
             elif need is None:
                 self.layer_cache[layer] = LayerCache()
 
@@ -125,8 +126,11 @@ class CacheManager:
         if request_id in self._live:
             raise ValueError(f"request {request_id!r} already holds a sequence")
         slot = self.slots.take()
-        for state in self._state_tensors:
-            state[slot].zero_()
+        for state, need in self._state_tensors:     # a reused slot starts as a fresh one
+            if need.init is not None:
+                need.init(state[slot])
+            else:
+                state[slot].zero_()
         seq = Sequence(request_id, slot,
                        [BlockTable(g.allocator, self.page_size, g.need.window) for g in self.groups])
         self._live[request_id] = seq

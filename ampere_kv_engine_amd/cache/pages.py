@@ -117,7 +117,10 @@ class BlockTable:
         return start
 
     def locate(self, position: int) -> tuple[int, int]:
-        if type(position) is not int or not 0 <= position < self._length:
+        """(page id, offset in the page) of a registered position."""
+        if isinstance(position, bool) or not isinstance(position, int):
+            raise TypeError(f"a position is an integer, got {type(position).__name__}")
+        if position < 0 or position >= self._length:
             raise ValueError(f"position {position} is outside the registered length {self._length}")
         index, offset = divmod(position, self.page_size)
         page = self._pages[index]

@@ -24,6 +24,11 @@ class EngineConfig:
     # bfloat16 products of more rows than this go to the BLAS library, which reads the matrices row-major: they are
     # then kept twice (row-major and packed for the engine's own kernels).  None: one copy, own kernels only.
     library_products_above: int | None = 16
+    # Exceptions to that rule for products of 17..64 rows, where for some matrix shapes the engine's own kernel is the
+    # faster one.  "fixed": none (every run sends every product the same way).  "measure": both are timed once, when the
+    # weights have been loaded (never inside a step), each decision is logged and the table can be saved
+    # (`engine.kernels.save_product_choices(path)`).  Anything else: the path of such a saved table.
+    product_choices: str = "fixed"
 
     def __post_init__(self):
         if self.dtype not in DTYPES:
@@ -35,6 +40,9 @@ class EngineConfig:
         above = self.library_products_above
         if above is not None and (not isinstance(above, int) or above < 0):
             raise ValueError(f"library_products_above must be None or a non-negative integer, got {above!r}")
+
+        if not isinstance(self.product_choices, str) or not self.product_choices:
+            raise ValueError("product_choices must be 'fixed', 'measure' or the path of a saved table")
 
     @property
     def max_pages_per_seq(self) -> int:

@@ -4,6 +4,8 @@
 //                     argmax_i( logits[i] / temperature - log(-log(u_i)) ), u_i uniform in (0, 1).
 // u_i comes from Philox-4x32-10 keyed by the request's seed with counter (i, draw number), so a request's draws
 // depend on its own seed and draw count only, never on the batch it shares a step with.
+// A row that holds a NaN, or no logit above -infinity, has no next token: the result is -1 (the attention kernels
+// answer a block table that names a page outside the pool with NaN, and that must not turn into token 0).
 
 #include "common.h"
 #include "api.h"
@@ -36,6 +38,10 @@ __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ 
                                                       int vocab) {
   __shared__ float best_value[16];
   __shared__ int best_index[16];
+  __shared__ int any_nan;
+  if (threadIdx.x == 0) any_nan = 0;
+  __syncthreads();
+  bool saw_nan = false;
   const int row = blockIdx.x;
   const float* x = logits + static_cast<size_t>(row) * vocab;
   const float t = temperature != nullptr ? temperature[row] : 0.f;
@@ -58,6 +64,7 @@ __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ 
     for (int u = 0; u < kAhead; ++u) {
       const int i = i0 + u * blockDim.x;
       float score = fetched[u];
+      saw_nan |= score != score;
       if (t > 0.f && i < vocab) {
         const uint32_t bits = philox_first(static_cast<uint32_t>(i), draw, k0, k1);
         const float u01 = (static_cast<float>(bits >> 8) + 0.5f) * 0x1p-24f;
@@ -73,11 +80,12 @@ __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ 
   }
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   if (lane == 0) { best_value[wave] = value; best_index[wave] = index; }
+  if (__any(saw_nan) && lane == 0) any_nan = 1;      // (every writer stores the same value)
   __syncthreads();
   if (threadIdx.x == 0) {
     for (int w = 1; w < blockDim.x / kWave; ++w)
       if (best_value[w] > value || (best_value[w] == value && best_index[w] < index)) { value = best_value[w]; index = best_index[w]; }
-    out[row] = index < vocab ? index : 0;
+    out[row] = (index < vocab && any_nan == 0) ? index : -1;
   }
 }
 

@@ -151,10 +151,10 @@ class BatchBuilder:
             if e.seq.length + len(e.tokens) > self.max_width * self.cache.page_size:
                 raise ValueError(f"request {e.seq.request_id!r} would reach {e.seq.length + len(e.tokens)} tokens; "
                                  f"the engine was built for {self.max_width * self.cache.page_size}")
-        # all-or-nothing over the whole step: check every request before registering any
-        self._check_pages(entries)
         order = sorted(range(len(entries)), key=lambda i: (len(entries[i].tokens) != 1, i))
         ordered = [entries[i] for i in order]
+        # all-or-nothing over the whole step: check every request before registering any
+        self._check_pages(ordered)
         num_decode = sum(1 for e in ordered if len(e.tokens) == 1)
         starts = [self.cache.reserve(e.seq, len(e.tokens)) for e in ordered]
 
@@ -247,14 +247,18 @@ class BatchBuilder:
         )
         return ctx, first_wanted_of
 
-    def _check_pages(self, entries: list[StepEntry]) -> None:
+    def _check_pages(self, ordered: list[StepEntry]) -> None:
+        """Plays the step's registrations through in the order they will be made (a request first gives back the
+        pages its window has passed, then takes what it needs) and refuses the step if the pool would run dry at
+        any point of it - a sum over the whole step would let an early request count on pages a later one frees."""
         from ..cache.pages import PagePoolExhausted
         for g in self.cache.groups:
             available = g.allocator.num_free
-            for e in entries:
+            for e in ordered:
                 table = e.seq.tables[g.index]
                 required = (table.length + len(e.tokens) + self.cache.page_size - 1) // self.cache.page_size
                 available += table._passed_pages(table.length) - max(0, required - table.num_pages)
-            if available < 0:
-                raise PagePoolExhausted(f"the step needs {-available} more page(s) than the pool of cache group "
-                                        f"{g.index} has free; no token of the step was registered")
+                if available < 0:
+                    raise PagePoolExhausted(f"the step needs {-available} more page(s) than the pool of cache group "
+                                            f"{g.index} has free when request {e.seq.request_id!r} registers its "
+                                            "tokens; no token of the step was registered")

@@ -8,6 +8,7 @@ logits at the wanted places.  It replaces the reference's three forward function
 
 from __future__ import annotations
 
+import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, Sequence
@@ -34,7 +35,10 @@ class Engine:
         self.dtype = _TORCH_DTYPE[engine_config.dtype]
         if kernels is None:
             from ..kernels.hip import HipKernels
-            kernels = HipKernels(self.device, library_products_above=engine_config.library_products_above)
+            choices = engine_config.product_choices
+            table = HipKernels.load_product_choices(choices) if choices not in ("fixed", "measure") else None
+            kernels = HipKernels(self.device, library_products_above=engine_config.library_products_above,
+                                 product_choices=table)
         self.kernels = kernels
         self.runtime = Runtime(kernels=kernels, dtype=self.dtype, device=self.device,
                                max_seq_len=engine_config.max_seq_len, page_size=engine_config.page_size)
@@ -73,14 +77,20 @@ class Engine:
         engine.arch_config = arch_config
         source = RandomSource(seed, str(engine.device))
         engine.model.load(lambda spec: source.get_spec(spec, engine.dtype))
-        engine.loaded = True
+        engine._loaded()
         return engine
 
     def load_folder(self, folder: str) -> None:
         checkpoint = Checkpoint(folder)
         checkpoint.check(self.model.tensors())
         self.model.load(lambda spec: checkpoint.get(spec.name, self.dtype).to(self.device))
+        self._loaded()
+
+    def _loaded(self) -> None:
+        """The weights are in place: what is decided once per model is decided now, not inside a step."""
         self.loaded = True
+        if self.config.product_choices == "measure" and hasattr(self.kernels, "measure_products"):
+            self.kernels.measure_products()
 
     # ---- requests ---------------------------------------------------------------------------------
     def open(self, request_id: str) -> Sequence:
@@ -91,24 +101,40 @@ class Engine:
 
     # ---- the step ---------------------------------------------------------------------------------
     @torch.no_grad()
-    def step(self, entries: list[StepEntry]) -> torch.Tensor | None:
+    def step(self, entries: list[StepEntry], *, borrow_logits: bool = False) -> torch.Tensor | None:
         """Returns float32 logits `[wanted, vocab]` in the order of the entries and of each entry's `want`
-        (None if nothing is wanted).  The new tokens' keys and values are in the cache afterwards."""
+        (None if nothing is wanted).  The new tokens' keys and values are in the cache afterwards.
+
+        The returned tensor is the caller's own.  With `borrow_logits=True` a step that is replayed from a recording
+        returns a view of the one buffer all recordings write their logits to: it is valid until the next call of
+        `step` and spares a copy (the scheduler and `generate_tokens` sample from it at once)."""
         if not self.loaded:
             raise RuntimeError("the engine has no weights yet")
-        vocab = self.spec.vocab_size
-        for e in entries:
-            for token in e.tokens:
-                if not 0 <= int(token) < vocab:
-                    raise ValueError(f"token id {token} of request {e.seq.request_id!r} is outside the vocabulary "
-                                     f"of {vocab}")
+        self._check_token_ids(entries)
         if self._recordable:
             shape = self._recordable_shape(entries)
             if shape is not None:
-                return self._step_recorded(entries, shape)
+                logits = self._step_recorded(entries, shape)
+                return logits if borrow_logits else logits.clone()
         ctx, _ = self.builder.build(entries)
         ctx.stream_buffer, ctx.spare_buffer = self.stream_buffer, self.spare_buffer
         return self.model.forward(ctx, self.cache.layer_cache)
+
+    def _check_token_ids(self, entries: list[StepEntry]) -> None:
+        """Every token id must name a row of the embedding table; one comparison per entry, not one per token."""
+        vocab = self.spec.vocab_size
+        for e in entries:
+            if len(e.tokens) == 1:
+                bad = not 0 <= int(e.tokens[0]) < vocab
+            else:
+                ids = np.asarray(e.tokens)
+                if ids.dtype.kind not in "iu":
+                    raise ValueError(f"the token ids of request {e.seq.request_id!r} are not integers")
+                bad = ids.size and (int(ids.min()) < 0 or int(ids.max()) >= vocab)
+            if bad:
+                token = next(t for t in e.tokens if not 0 <= int(t) < vocab)
+                raise ValueError(f"token id {token} of request {e.seq.request_id!r} is outside the vocabulary "
+                                 f"of {vocab}")
 
     # ---- steps as recorded graphs -----------------------------------------------------------------------------
     SPARE_STREAM_ROWS = 1         # steps of up to this many tokens may move the residual sum between two buffers
@@ -134,8 +160,8 @@ class Engine:
         the step's device buffer differs.  A step of such a shape is run once as it is, then recorded into a HIP
         graph, then replayed - which takes the launches' host time out of decoding and out of small mixed steps.
         Launch sizes that depend on the requests' lengths are taken from the table width's bound, so one recording
-        serves all lengths under it.  The returned logits live in a buffer that all recordings share: the next
-        recorded step overwrites them."""
+        serves all lengths under it.  The logits are written to a buffer that all recordings share: the next
+        recorded step overwrites them (`step` hands out a copy unless the caller asked to borrow the buffer)."""
         counts, wanted = shape
         ctx, _ = self.builder.build(entries, width_multiple=self.GRAPH_WIDTH_MULTIPLE)
         ctx.stream_buffer, ctx.spare_buffer = self.stream_buffer, self.spare_buffer

@@ -7,7 +7,7 @@ import time
 
 import torch
 
-from ..sampling.sampler import Sampler, SamplingParams
+from ..sampling.sampler import NO_TOKEN, Sampler, SamplingParams
 from .batch import StepEntry
 
 MAX_NEW_TOKENS = 32  # the reference's default (ampere_kv/runner.py:17); it counts the token the prefill yields
@@ -43,9 +43,11 @@ def generate_tokens(engine, input_ids, *, max_new_tokens: int = MAX_NEW_TOKENS, 
         for start in range(0, len(prompt), chunk):
             portion = prompt[start:start + chunk]
             last = start + chunk >= len(prompt)
-            logits = engine.step([StepEntry(seq, portion, [len(portion) - 1] if last else [])])
+            logits = engine.step([StepEntry(seq, portion, [len(portion) - 1] if last else [])], borrow_logits=True)
         while True:
             token = sampler.sample(logits, [params], [len(generated)])[0]
+            if token == NO_TOKEN:
+                raise RuntimeError(f"the step gave request {request_id!r} no finite logit after {len(generated)} tokens")
             if timings is not None:
                 ready = time.perf_counter()
                 if not generated:
@@ -53,7 +55,7 @@ def generate_tokens(engine, input_ids, *, max_new_tokens: int = MAX_NEW_TOKENS, 
             generated.append(token)
             if token in eos or len(generated) >= max_new_tokens:
                 break
-            logits = engine.step([StepEntry(seq, [token], [0])])
+            logits = engine.step([StepEntry(seq, [token], [0])], borrow_logits=True)
         final_length = seq.length
     finally:
         engine.close(seq)

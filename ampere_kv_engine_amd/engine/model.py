@@ -45,9 +45,9 @@ class Model:
         specs += self.head.tensors()
         tied = self.spec.head.get("tied_to")
         if tied is not None:
-            # a file of a tied model may still carry the head's tensor; it must then be the same shape
+            # a file of a tied model may still carry the head's tensor; it must then hold the embedding's values
             specs.append(TensorSpec(self.spec.head["name"], (self.spec.vocab_size, self.spec.hidden_size),
-                                    optional=True))
+                                    optional=True, same_as=self.embedding.name))
         return specs
 
     def load(self, fetch) -> None:

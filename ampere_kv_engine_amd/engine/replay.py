@@ -50,7 +50,7 @@ def replay(engine, lines, out_dir: str, report=print) -> None:
                 live[name] = engine.open(name)
             entries.append(StepEntry(live[name], [int(t) for t in item["tokens"]], [int(w) for w in item.get("want", [])]))
         if entries:
-            logits = engine.step(entries)
+            logits = engine.step(entries, borrow_logits=True)       # copied to the host at once
             if logits is not None:
                 data = logits.detach().to("cpu").numpy().astype("<f4", copy=False)
                 path = os.path.join(out_dir, f"{step}.f32")

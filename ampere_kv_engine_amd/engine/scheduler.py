@@ -21,11 +21,12 @@ from __future__ import annotations
 
 import time
 
-from ..sampling.sampler import Sampler, SamplingParams
+from ..sampling.sampler import NO_TOKEN, Sampler, SamplingParams
 from .batch import StepEntry
 
 WAITING, PREFILLING, RUNNING, FINISHED = "waiting", "prefilling", "running", "finished"
 STOP_LIMIT, STOP_EOS, STOP_CANCELLED, STOP_EXPIRED = "reached limit", "EOS", "cancelled", "expired"
+STOP_NO_LOGITS = "error: no finite logits"      # the step gave this request NaN (or nothing above -infinity)
 
 
 class Request:
@@ -54,7 +55,9 @@ class Request:
 
 class Scheduler:
     def __init__(self, engine, *, max_batch: int | None = None, prefill_chunk_size: int = 0,
-                 max_batched_tokens: int | None = None, mixed: bool = True, clock=time.monotonic):
+                 max_batched_tokens: int | None = None, mixed: bool = True, clock=time.monotonic, on_token=None):
+        """`on_token(request, token)`, if given, is called whenever a request has been given a token (right after the
+        round's one synchronisation): measurements hang their clocks there; the scheduler itself keeps no history."""
         cfg = engine.config
         self.engine = engine
         self.max_batch = cfg.max_seqs if max_batch is None else max_batch
@@ -62,6 +65,7 @@ class Scheduler:
         self.max_batched_tokens = cfg.max_batched_tokens if max_batched_tokens is None else max_batched_tokens
         self.mixed = mixed
         self.clock = clock
+        self.on_token = on_token
         if self.max_batch < 1 or self.max_batch > cfg.max_seqs:
             raise ValueError(f"max_batch must be between 1 and the engine's {cfg.max_seqs} request slots")
         if prefill_chunk_size < 0:
@@ -108,8 +112,8 @@ class Scheduler:
     def cancel(self, request: Request) -> None:
         """Marks the request; it is retired at the start of the next round.  Work already issued is not
         interrupted, a stop reason already set is kept, a finished request is left alone."""
-        if request.status != FINISHED:
-            request.stop_reason = request.stop_reason or STOP_CANCELLED
+        if request.status != FINISHED and not request.stop_reason:
+            request.stop_reason = STOP_CANCELLED
 
     @property
     def idle(self) -> bool:
@@ -184,19 +188,29 @@ class Scheduler:
             entries.append(StepEntry(request.seq, request.input_ids[start:start + count], [count - 1] if last else []))
             if last:
                 takers.append(request)
-        logits = self.engine.step(entries)
+        logits = self.engine.step(entries, borrow_logits=True)     # sampled from at once, below
         if not takers:
             return
         tokens = self.sampler.sample(logits, [r.sampling for r in takers], [len(r.output_ids) for r in takers])
         for request, token in zip(takers, tokens):
-            self._commit(request, token)
+            self._give(request, token)
 
-    def _commit(self, request: Request, token: int) -> None:
-        request.output_ids.append(token)
-        if len(request.output_ids) >= request.max_new_tokens:
-            request.stop_reason = request.stop_reason or STOP_LIMIT
-        elif token in self.eos_ids and not request.ignore_eos:
-            request.stop_reason = request.stop_reason or STOP_EOS
+    def _give(self, request: Request, token: int) -> None:
+        """The request's next token has been chosen: it joins the output, and may be the last (a stop reason that
+        is already there - a cancellation during the round - stays)."""
+        ended = None
+        if token == NO_TOKEN:           # nothing to choose from: the request ends here, with what it has
+            ended = STOP_NO_LOGITS
+        else:
+            request.output_ids.append(token)
+            if self.on_token is not None:
+                self.on_token(request, token)
+            if len(request.output_ids) >= request.max_new_tokens:
+                ended = STOP_LIMIT
+            elif not request.ignore_eos and token in self.eos_ids:
+                ended = STOP_EOS
+        if ended is not None and not request.stop_reason:
+            request.stop_reason = ended
 
     def _admit(self) -> None:
         """First come, first served; the head waits (and holds the others back) until its budget fits."""

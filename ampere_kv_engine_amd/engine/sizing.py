@@ -61,6 +61,13 @@ def plan_memory(spec: ModelSpec, engine_config: EngineConfig, memory_bytes: int)
     return MemoryPlan(weight_bytes, second, page_bytes, fixed, int(num_pages), engine_config.page_size)
 
 
+def page_bytes(spec: ModelSpec, dtype: str, page_size: int) -> int:
+    """Bytes one page of every cache group and layer takes (what `--kv-gb` is divided by)."""
+    cache = CacheManager(Model(spec, dry_runtime()).cache_needs(), page_size=page_size, num_pages=1, max_seqs=1,
+                         allocate_tensors=False)
+    return sum(g.bytes_per_token(_ELEMENT_BYTES[dtype]) for g in cache.groups) * page_size
+
+
 def _count(shape) -> int:
     total = 1
     for s in shape:

@@ -78,17 +78,19 @@ def _ptr(t: torch.Tensor | None):
 class HipKernels:
     name = "hip-gfx950"
     OWN_SKINNY_ROWS = 64            # the most rows the engine's own decode product takes
-    _tuned_by_device: dict = {}     # device index -> the choices between own and library products made so far
 
     def __init__(self, device: torch.device | str = "cuda:0", library_products_above: int | None = 16,
-                 tune_products: bool = True):
-        """`library_products_above`: bfloat16 products of more rows than this may go to the BLAS library (torch.mm),
+                 product_choices: dict | None = None):
+        """`library_products_above`: bfloat16 products of more rows than this go to the BLAS library (torch.mm),
         which then needs the matrices row-major beside their packing; None keeps the packing alone and every
-        product in this library's own kernels.  `tune_products`: up to 64 rows the faster of the two is found out
-        once per matrix shape; False sends every product above the limit to the library."""
+        product in this library's own kernels.  `product_choices`: exceptions to that rule for products of up to 64
+        rows, `{(kind, outs, k, tiles of 16 rows): "own" | "library"}` - a table that was measured once
+        (`measure_products`) or loaded from a file.  Nothing is ever timed or decided inside a step, so two runs
+        with the same table send every product the same way and give the same bits."""
         self.library_products_above = library_products_above
-        self.tune_products = tune_products     # 17..64 rows: own kernel or library, whichever is faster for the shape
-        self._spacer = None                    # the buffer whose fill precedes every timed run
+        self.product_choices: dict = dict(product_choices or {})
+        self._products: dict = {}              # (kind, outs, k) -> a prepared weight of that shape, for measure_products
+        self._spacer = None                    # the buffer whose reads precede every timed run
         self._packed_rows = None               # where activations are repacked for the engine's own product
         self.device = torch.device(device)
         if self.device.type == "cuda" and self.device.index is None:
@@ -97,9 +99,6 @@ class HipKernels:
             raise KernelError(f"the HIP kernels run on a GPU; device {self.device} is not one")
         if not torch.cuda.is_available():
             raise KernelError("no GPU is visible: the engine computes with HIP kernels only and has no CPU path")
-        # (kind, outs, k, row tiles) -> "own" | "library": one table per device for the whole process, so that two
-        # engines of a process, whose results may be compared bit for bit, send a product of one shape the same way
-        self._tuned = HipKernels._tuned_by_device.setdefault(self.device.index, {})
         path = ensure_built()
         try:
             self.lib = ctypes.CDLL(path)
@@ -230,7 +229,9 @@ class HipKernels:
         """bfloat16 matrices whose k is a multiple of 8 are packed for the MFMA kernels; others stay row-major and
         go through the plain tiled kernel."""
         if matrix.dtype == torch.bfloat16 and matrix.shape[1] % 8 == 0:
-            return PackedWeight(matrix, keep_row_major=self.library_products_above is not None)
+            weight = PackedWeight(matrix, keep_row_major=self.library_products_above is not None)
+            self._products.setdefault(("linear", weight.outs, weight.k), weight)
+            return weight
         return matrix
 
     def _library_product(self, rows: int, row_major, out) -> bool:
@@ -253,37 +254,78 @@ class HipKernels:
         return self._packed_rows, 1
 
     def _own_or_library(self, key: tuple, rows: int, own, library) -> None:
-        """A product that may go to the library.  More than 64 rows: it does.  Up to 64 rows (the range of the skinny
-        kernel, where neither side wins for every shape): whichever of the two is faster for a matrix of this shape
-        and this many tiles of 16 rows, found out at the first such call (never while a graph is recorded) and
-        remembered.  Each is timed twice on the device; before every timed run reads of 256 MB empty the caches, as
-        the other layers' weights do in a real step, and keep the device busy while the host queues the run, so that
-        the host's launch time is not part of what is measured."""
-        if rows > self.OWN_SKINNY_ROWS or not self.tune_products:
+        """A product that may go to the library: it does, unless it has at most 64 rows (the range of the skinny
+        kernel) and the table of choices names the engine's own kernel for this matrix shape and number of row
+        tiles.  The table is fixed before the first step; a step being recorded reads the same table."""
+        if rows <= self.OWN_SKINNY_ROWS and self.product_choices.get((*key, (rows + 15) // 16)) == "own":
+            own()
+        else:
             library()
-            return
-        key = (*key, (rows + 15) // 16)
-        choice = self._tuned.get(key)
-        if choice is None:
-            if torch.cuda.is_current_stream_capturing():
-                library()
-                return
-            if self._spacer is None:
-                self._spacer = torch.zeros(64 << 20, dtype=torch.float32, device=self.device)
-            timed = {"own": [], "library": []}
-            for _ in range(2):
-                for name, run in (("own", own), ("library", library)):
-                    for _ in range(4):      # ~0.25 ms of device work: more than the host needs to queue what follows
-                        self._spacer.sum()  # (reads: nothing is left to be written back while the run is timed)
-                    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    start.record()
-                    run()
-                    end.record()
-                    timed[name].append((start, end))
-            torch.cuda.synchronize(self.device)
-            best = {name: min(a.elapsed_time(b) for a, b in pairs) for name, pairs in timed.items()}
-            choice = self._tuned[key] = "own" if best["own"] <= best["library"] else "library"
-        (own if choice == "own" else library)()
+
+    def measure_products(self, row_tiles=(2, 3, 4), log=None) -> dict:
+        """For every matrix shape prepared so far and 32, 48 and 64 rows: the engine's own product against the
+        library's, each timed twice on the device; the faster one enters `product_choices`.  Before every timed run
+        reads of 256 MB empty the caches, as the other layers' weights do in a real step, and keep the device busy
+        while the host queues the run, so that the host's launch time is not part of what is measured.  Meant to be
+        called once after loading (`EngineConfig.product_choices = "measure"`); returns the table, which
+        `save_product_choices` writes for later runs.  Every decision is reported through `log` (default: the
+        logger "ampere_kv_engine_amd.kernels")."""
+        import logging
+        report = log or logging.getLogger("ampere_kv_engine_amd.kernels").info
+        if self.library_products_above is None:
+            return self.product_choices
+        if self._spacer is None:
+            self._spacer = torch.zeros(64 << 20, dtype=torch.float32, device=self.device)
+        for (kind, outs, k), weight in sorted(self._products.items(), key=lambda item: item[0]):
+            for tiles in row_tiles:
+                rows = 16 * tiles
+                if rows <= self.library_products_above or rows > self.OWN_SKINNY_ROWS:
+                    continue
+                x = torch.randn(rows, k, device=self.device).to(torch.bfloat16)
+                out = torch.empty(rows, outs, dtype=torch.bfloat16, device=self.device)
+                scratch = torch.empty(rows, 2 * outs, dtype=torch.bfloat16, device=self.device) if kind == "gated" else None
+                run = (lambda: self.gated_linear(x, weight, out, scratch)) if kind == "gated" else (lambda: self.linear(x, weight, out))
+                best = {}
+                for choice in ("own", "library"):
+                    self.product_choices[kind, outs, k, tiles] = choice
+                    run()                                            # (the first call may load code)
+                    samples = []
+                    for _ in range(2):
+                        for _ in range(4):      # ~0.25 ms of device work: more than the host needs to queue what follows
+                            self._spacer.sum()  # (reads: nothing is left to be written back while the run is timed)
+                        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                        start.record()
+                        run()
+                        end.record()
+                        samples.append((start, end))
+                    torch.cuda.synchronize(self.device)
+                    best[choice] = min(a.elapsed_time(b) for a, b in samples)
+                choice = "own" if best["own"] <= best["library"] else "library"
+                self.product_choices[kind, outs, k, tiles] = choice
+                report(f"product {kind} {outs}x{k}, {rows} rows: own {best['own'] * 1000:.1f} us, library "
+                       f"{best['library'] * 1000:.1f} us -> {choice}")
+        return self.product_choices
+
+    def save_product_choices(self, path: str) -> None:
+        import json
+        with open(path, "w") as handle:
+            json.dump({f"{kind}:{outs}x{k}:{tiles}": choice
+                       for (kind, outs, k, tiles), choice in sorted(self.product_choices.items())}, handle, indent=1)
+
+    @staticmethod
+    def load_product_choices(path: str) -> dict:
+        """The table `save_product_choices` wrote: {"linear:6144x4096:2": "own", ...} -> {(kind, outs, k, tiles): choice}."""
+        import json
+        with open(path) as handle:
+            raw = json.load(handle)
+        table = {}
+        for name, choice in raw.items():
+            kind, shape, tiles = name.split(":")
+            outs, k = shape.split("x")
+            if choice not in ("own", "library"):
+                raise ValueError(f"{path}: the choice for {name} is {choice!r}, not 'own' or 'library'")
+            table[kind, int(outs), int(k), int(tiles)] = choice
+        return table
 
     def linear(self, x, weight, out):
         if isinstance(weight, PackedWeight):
@@ -353,7 +395,9 @@ class HipKernels:
         `swiglu` (float32 weights, sizes the packed kernels do not take)."""
         if (gate.dtype == torch.bfloat16 and up.dtype == torch.bfloat16 and gate.shape == up.shape
                 and gate.shape[1] % 8 == 0 and gate.shape[0] % 16 == 0):
-            return GatedWeight(gate, up, keep_row_major=self.library_products_above is not None)
+            weight = GatedWeight(gate, up, keep_row_major=self.library_products_above is not None)
+            self._products.setdefault(("gated", weight.inter, weight.k), weight)
+            return weight
         return None
 
     def gated_scratch(self, weight: GatedWeight, rows: int, dtype: torch.dtype):

@@ -72,9 +72,11 @@ class PagedKV:
 
 @dataclass(frozen=True)
 class SlotState:
-    """A per-request state of fixed size, zeroed when a request takes the slot."""
+    """A per-request state of fixed size.  When a request takes a slot its state is zeroed, or, if the mixer gives
+    `init`, set by `init(state_of_the_slot)` (a tensor of `shape`, to be filled in place)."""
     shape: tuple[int, ...]
     dtype: torch.dtype = torch.float32
+    init: Callable[[torch.Tensor], None] | None = None
 
 
 class Part:

@@ -25,6 +25,9 @@ class SamplingParams:
             raise ValueError("seed must fit in 63 bits")
 
 
+NO_TOKEN = -1       # what a row without a usable logit yields
+
+
 class Sampler:
     def __init__(self, kernels, device, max_rows: int):
         self.kernels, self.device, self.max_rows = kernels, torch.device(device), max_rows
@@ -40,7 +43,8 @@ class Sampler:
 
     def sample(self, logits: torch.Tensor, params: list[SamplingParams], draws: list[int]) -> list[int]:
         """logits float32 [rows, vocab]; `draws[i]` is how many tokens request i has drawn before.  Returns the
-        chosen ids (one device-to-host copy for the whole batch)."""
+        chosen ids (one device-to-host copy for the whole batch); `NO_TOKEN` (-1) for a row that holds a NaN or no
+        finite logit - the caller decides what becomes of that request."""
         rows = logits.shape[0]
         if rows != len(params) or rows != len(draws):
             raise ValueError("one SamplingParams and one draw count per row of logits")

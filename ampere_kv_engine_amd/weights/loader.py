@@ -20,12 +20,15 @@ from .spec import TensorSpec
 
 
 class WeightsError(ValueError):
-    """The checkpoint does not match the model: lists missing, unexpected and wrongly shaped tensors."""
+    """The checkpoint does not match the model: lists missing, unexpected and wrongly shaped tensors, tensors of a
+    dtype the engine does not keep, and tensors that must equal another one (a tied head) and do not."""
 
     def __init__(self, folder: str, missing: list[str], unexpected: list[str],
-                 wrong_shape: list[tuple[str, tuple, tuple]], wrong_dtype: list[tuple[str, str]]):
+                 wrong_shape: list[tuple[str, tuple, tuple]], wrong_dtype: list[tuple[str, str]],
+                 differing: list[tuple[str, str]] = ()):
         self.missing, self.unexpected = missing, unexpected
         self.wrong_shape, self.wrong_dtype = wrong_shape, wrong_dtype
+        self.differing = list(differing)
         lines = [f"weights in {folder} do not match the model:"]
         if missing:
             lines.append(f"  missing ({len(missing)}): " + ", ".join(missing))
@@ -35,6 +38,8 @@ class WeightsError(ValueError):
             lines.append(f"  wrong shape: {name} is {list(got)}, expected {list(want)}")
         for name, dtype in wrong_dtype:
             lines.append(f"  unsupported dtype: {name} is stored as {dtype}")
+        for name, other in self.differing:
+            lines.append(f"  differing values: {name} must equal {other} (the model ties them) and does not")
         super().__init__("\n".join(lines))
 
 
@@ -95,11 +100,22 @@ class Checkpoint:
                     wrong_shape.append((name, tuple(by_name[name].shape), shape))
                 if memory_dtype(dtype, torch.bfloat16) is None:
                     wrong_dtype.append((name, dtype))
-        if missing or unexpected or wrong_shape or wrong_dtype:
-            raise WeightsError(self.folder, missing, unexpected, wrong_shape, wrong_dtype)
+        differing = []
+        bad = {name for name, *_ in wrong_shape} | {name for name, _ in wrong_dtype}
+        for spec in expected:
+            other = spec.same_as
+            if other is None or spec.name not in self._meta or other not in self._meta or {spec.name, other} & bad:
+                continue
+            if not torch.equal(self._raw(spec.name), self._raw(other)):
+                differing.append((spec.name, other))
+        if missing or unexpected or wrong_shape or wrong_dtype or differing:
+            raise WeightsError(self.folder, missing, unexpected, wrong_shape, wrong_dtype, differing)
 
     def has(self, name: str) -> bool:
         return name in self._meta
+
+    def _raw(self, name: str) -> torch.Tensor:
+        return self._handles[self._file_of[name]].get_tensor(name)
 
     def get(self, name: str, engine_dtype: torch.dtype) -> torch.Tensor:
         """The tensor on the host, in the dtype it is kept in."""

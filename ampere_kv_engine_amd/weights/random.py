@@ -1,8 +1,10 @@
 """Random-weights mode: draw a model's tensors from a seed and write a model folder.
 
-Laws: matrices and embeddings N(0, 0.02); norm weights 1 + N(0, 0.1).  Every tensor is drawn in float32 on
-the host by its own generator, seeded from the folder's seed and the tensor's name, so a tensor's values
-depend on neither the order nor the presence of others; values are rounded to bfloat16 once and stored so.
+Laws, by the role a part gives its tensor: matrices and embeddings N(0, 0.02); norm weights 1 + N(0, 0.1); integer
+tables zero.  A part whose tensors follow another law names a role of its own and registers the law
+(`register_init_law`).  Every tensor is drawn in float32 on the host by its own generator, seeded from the folder's
+seed and the tensor's name, so a tensor's values depend on neither the order nor the presence of others; values are
+rounded to bfloat16 once and stored so.
 """
 
 from __future__ import annotations
@@ -14,7 +16,7 @@ import os
 import torch
 from safetensors.torch import save_file
 
-from .spec import EMBEDDING, INT_TABLE, MATRIX, NORM, TensorSpec
+from .spec import EMBEDDING, INT_TABLE, MATRIX, NORM, TensorSpec  # noqa: F401
 
 MATRIX_STD = 0.02
 NORM_STD = 0.1
@@ -25,16 +27,36 @@ def _generator(seed: int, name: str, device: str = "cpu") -> torch.Generator:
     return torch.Generator(device=device).manual_seed(int.from_bytes(digest[:8], "little") >> 1)
 
 
+def _normal(mean: float, std: float):
+    def law(shape, generator, device):
+        return mean + torch.randn(shape, generator=generator, dtype=torch.float32, device=device) * std
+    return law
+
+
+_INIT_LAWS = {
+    MATRIX: _normal(0.0, MATRIX_STD),
+    EMBEDDING: _normal(0.0, MATRIX_STD),
+    NORM: _normal(1.0, NORM_STD),
+    INT_TABLE: lambda shape, generator, device: torch.zeros(shape, dtype=torch.int32, device=device),
+}
+
+
+def register_init_law(role: str, law, *, replace: bool = False) -> None:
+    """`law(shape, generator, device)` returns the tensor (float32, or int32 for a table of integers) that random
+    weights give to tensors of `role`.  It must draw from `generator` alone, so that the seed fixes the values."""
+    if role in _INIT_LAWS and not replace:
+        raise ValueError(f"role {role!r} already has a law")
+    _INIT_LAWS[role] = law
+
+
 def draw(spec: TensorSpec, seed: int, device: str = "cpu") -> torch.Tensor:
-    """One tensor in float32 following its role's law."""
-    generator = _generator(seed, spec.name, device)
-    if spec.role in (MATRIX, EMBEDDING):
-        return torch.randn(spec.shape, generator=generator, dtype=torch.float32, device=device) * MATRIX_STD
-    if spec.role == NORM:
-        return 1.0 + torch.randn(spec.shape, generator=generator, dtype=torch.float32, device=device) * NORM_STD
-    if spec.role == INT_TABLE:
-        return torch.zeros(spec.shape, dtype=torch.int32, device=device)
-    raise ValueError(f"tensor {spec.name} has unknown role {spec.role!r}")
+    """One tensor following its role's law (float32; int32 for integer tables)."""
+    try:
+        law = _INIT_LAWS[spec.role]
+    except KeyError:
+        raise ValueError(f"tensor {spec.name} has role {spec.role!r}, for which no random law is registered; known: "
+                         f"{', '.join(sorted(_INIT_LAWS))}") from None
+    return law(tuple(spec.shape), _generator(seed, spec.name, device), device)
 
 
 def write_random_model(folder: str, config, seed: int, *, store_dtype: torch.dtype = torch.bfloat16) -> str:
@@ -48,7 +70,7 @@ def write_random_model(folder: str, config, seed: int, *, store_dtype: torch.dty
         if spec.optional:
             continue
         value = draw(spec, seed)
-        tensors[spec.name] = value if spec.role == INT_TABLE else value.to(store_dtype)
+        tensors[spec.name] = value.to(store_dtype) if value.is_floating_point() else value
     with open(os.path.join(folder, "config.json"), "w") as handle:
         json.dump(config.to_dict(), handle, indent=1)
     save_file(tensors, os.path.join(folder, "model.safetensors"), metadata={"format": "pt", "seed": str(seed)})
@@ -67,4 +89,4 @@ class RandomSource:
 
     def get_spec(self, spec: TensorSpec, engine_dtype: torch.dtype) -> torch.Tensor:
         value = draw(spec, self.seed, self.device)
-        return value if spec.role == INT_TABLE else value.to(engine_dtype)
+        return value.to(engine_dtype) if value.is_floating_point() else value

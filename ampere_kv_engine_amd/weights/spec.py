@@ -11,5 +11,6 @@ MATRIX, NORM, EMBEDDING, INT_TABLE = "matrix", "norm", "embedding", "int_table"
 class TensorSpec:
     name: str
     shape: tuple[int, ...]
-    role: str = MATRIX            # decides the random-init law: matrices and embeddings N(0, 0.02), norms 1 + N(0, 0.1)
+    role: str = MATRIX            # names the law random weights are drawn from (`weights.random.register_init_law`)
     optional: bool = False        # may be absent from the file (a head tied to the embedding)
+    same_as: str | None = None    # if the file holds it, it must hold the values of this other tensor (a tied head)

@@ -162,7 +162,7 @@ def main() -> int:
 
         def one_step():
             nonlocal tokens
-            logits = engine.step([StepEntry(seq, [token], [0]) for seq, token in zip(seqs, tokens)])
+            logits = engine.step([StepEntry(seq, [token], [0]) for seq, token in zip(seqs, tokens)], borrow_logits=True)
             tokens = sampler.sample(logits, greedy, draws)
 
         for _ in range(PRIMING + warmup):

@@ -12,11 +12,54 @@ PROMPTS = {"a": 40, "b": 45, "c": 90, "d": 20, "e": 1, "f": 30}     # tokens fed
 POOL_TOKENS = 320                                                   # < sum of lengths: pages must be used again
 
 
-def tolerance(dtype: str, want: torch.Tensor):
-    """float32: rounding of a few hundred float32 operations.  bfloat16: activations carry 8 bits, so a logit is
-    off by a few times 2^-8 of the largest one after a handful of layers."""
-    scale = max(float(want.abs().max()), 1.0)
-    return dict(rtol=0.0, atol=(2e-5 if dtype == "float32" else 0.03) * scale)
+# Limits on |engine - expectation|, as fractions of the expectation's size.  "max": the worst logit against the
+# largest |logit|; "rms": a position's root-mean-square error against the largest root-mean-square of a position's
+# logits.  float32: rounding of a few hundred float32 operations.  bfloat16: activations carry 8 bits and every branch
+# output is rounded; measured on the three tiny models over all cuttings, the engine lies within 0.008 (max) and 0.0084
+# (rms) of the plain float32 implementation and within 0.0055 and 0.006 of the torch double that rounds at the same
+# points, while keys or values of ONE page of ONE layer taken from another request move a position by 0.036 and 0.054
+# at the least - so the limits below separate the two by a factor of two and more on either side.
+LIMITS = {
+    ("float32", "plain"): dict(max=2e-5, rms=2e-5),
+    ("float32", "double"): dict(max=2e-5, rms=2e-5),
+    ("bfloat16", "plain"): dict(max=0.016, rms=0.025),
+    ("bfloat16", "double"): dict(max=0.012, rms=0.02),
+}
+
+
+def scales(want: torch.Tensor) -> tuple[float, float]:
+    """(largest |logit|, largest per-position root-mean-square) of an expectation [positions, vocab]."""
+    want = want.reshape(-1, want.shape[-1]).float()
+    return max(float(want.abs().max()), 0.25), max(float(want.pow(2).mean(dim=1).sqrt().max()), 0.05)
+
+
+def tolerance(dtype: str, want: torch.Tensor, against: str = "plain"):
+    """The "max" limit alone, in the form `torch.testing.assert_close` takes."""
+    return dict(rtol=0.0, atol=LIMITS[dtype, against]["max"] * scales(want)[0])
+
+
+def error_of(got: torch.Tensor, want: torch.Tensor, dtype: str, against: str = "plain"):
+    """(first position beyond a limit or None, worst max error / its limit, worst rms error / its limit) for logits
+    [positions, vocab] against an expectation of the same shape."""
+    got, want = got.reshape(-1, got.shape[-1]).float(), want.reshape(-1, want.shape[-1]).float()
+    assert got.shape == want.shape, f"{tuple(got.shape)} logits, {tuple(want.shape)} expected"
+    assert not torch.isnan(got).any(), "NaN logits"
+    limit = LIMITS[dtype, against]
+    top, rms = scales(want)
+    error = got - want
+    by_max = error.abs().max(dim=1).values / (limit["max"] * top)
+    by_rms = error.pow(2).mean(dim=1).sqrt() / (limit["rms"] * rms)
+    beyond = ((by_max > 1) | (by_rms > 1)).nonzero()
+    return (int(beyond[0]) if len(beyond) else None), float(by_max.max()), float(by_rms.max())
+
+
+def assert_logits_close(got, want, dtype: str, against: str = "plain", what: str = ""):
+    position, by_max, by_rms = error_of(got, want, dtype, against)
+    if position is not None:
+        raise AssertionError(f"{what}: first wrong position {position} of {want.reshape(-1, want.shape[-1]).shape[0]}; worst "
+                             f"max error {by_max:.2f} x its limit, worst rms error {by_rms:.2f} x its limit ({dtype} against "
+                             f"the {against} implementation)")
+    return by_max, by_rms
 
 
 def make_case(name, model_folders):
@@ -28,33 +71,45 @@ def make_case(name, model_folders):
     return dict(name=name, folder=folder, page_size=page_size, requests=requests, expected=expected, raw=raw)
 
 
-def make_engine(case, dtype, device, kernels=None):
+def make_engine(case, dtype, device, kernels=None, **engine_options):
     from ampere_kv_engine_amd.config import EngineConfig
     from ampere_kv_engine_amd.engine import Engine
     page = case["page_size"]
     config = EngineConfig(dtype=dtype, page_size=page, num_pages=POOL_TOKENS // page, max_seqs=4,
-                          max_batched_tokens=256, max_seq_len=512, device=device)
+                          max_batched_tokens=256, max_seq_len=512, device=device, **engine_options)
     return Engine.from_folder(case["folder"], config, kernels=kernels)
 
+
 def check(engine, case, schedule):
+    """Runs the schedule and compares every fed position with the plain implementation - and, in bfloat16, also with
+    the torch double of the kernel set run through the same schedule, which rounds where the kernels round."""
     got, pages = schedules.run(engine, case["requests"], schedule)
+    dtype = engine.config.dtype
     worst = 0.0
     for name, want in case["expected"].items():
-        assert got[name].shape == want.shape
-        assert not torch.isnan(got[name]).any(), f"request {name}: NaN logits"
-        error = (got[name] - want).abs()
-        worst = max(worst, float(error.max()))
-        limit = tolerance(engine.config.dtype, want)["atol"]
-        if float(error.max()) > limit:
-            position = int((error.max(dim=1).values > limit).nonzero()[0])
-            raise AssertionError(f"{case['name']}/{engine.config.dtype} request {name}: first wrong position {position} "
-                                 f"of {want.shape[0]} (page size {case['page_size']}), error {float(error[position].max()):.3g} "
-                                 f"> {limit:.3g}")
+        what = f"{case['name']}/{dtype} request {name} (page size {case['page_size']})"
+        worst = max(worst, *assert_logits_close(got[name], want, dtype, "plain", what))
+    if dtype == "bfloat16" and engine.device.type == "cuda":
+        same, _ = schedules.run(double_engine(case), case["requests"], schedule)
+        for name in case["expected"]:
+            what = f"{case['name']}/{dtype} request {name} (page size {case['page_size']})"
+            worst = max(worst, *assert_logits_close(got[name], same[name], dtype, "double", what))
     assert engine.cache.num_free_pages == [engine.config.num_pages], "pages were lost"
     assert engine.cache.slots.num_free == engine.config.max_seqs, "slots were lost"
-    print(f"[{case['name']} {engine.config.dtype}] worst |error| {worst:.3g}")
+    print(f"[{case['name']} {dtype}] worst error {worst:.2f} of its limit")
     return pages
 
+
+_DOUBLES = {}
+
+
+def double_engine(case, dtype="bfloat16"):
+    """The engine of `case` with the torch double of the kernel set, on the CPU (kept between tests)."""
+    from torch_kernels import TorchKernels
+    key = (case["name"], case["folder"], dtype)
+    if key not in _DOUBLES:
+        _DOUBLES[key] = make_engine(case, dtype, "cpu", kernels=TorchKernels())
+    return _DOUBLES[key]
 
 
 # ---- the cuttings, as functions of (engine, case) -----------------------------------------------------------------

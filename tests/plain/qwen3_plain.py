@@ -2,7 +2,7 @@
 
 It is the oracle of the test-suite: every function processes a whole sequence at once, keeps no cache,
 reads the model folder with its own few lines of safetensors code and shares nothing with the engine's
-packages.  Each function cites the lines of the reference (paths under /root/reference) whose formula it
+packages.  Each function cites the lines of the reference (paths relative to its checkout) whose formula it
 states.  Arithmetic runs in the dtype of the tensors it is given (float32 or float64); weights that are
 stored in bfloat16 are widened exactly.
 """
@@ -39,10 +39,11 @@ def rope(x: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor) -> to
     """Rotate x [T, H, d] by its tokens' absolute positions [T].  The angle of pair j is pos * inv_freq[j],
     the pairs are (j, j + d/2) (first half with second half), the whole head is rotated:
     out = x * cos + cat(-x[d/2:], x[:d/2]) * sin with cos/sin the angle table repeated twice along d.
-    ampere_kv/runner.py:86-98."""
-    angles = positions.to(torch.float32)[:, None] * inv_freq[None, :]          # [T, d/2], float32 angles
-    angles = torch.cat((angles, angles), dim=-1).to(x.dtype)                    # [T, d]
-    cos, sin = angles.cos()[:, None, :], angles.sin()[:, None, :]
+    Angles, cosines and sines are formed in float32 and only then cast to x's dtype.
+    ampere_kv/runner.py:86-98 (the cast: :92-93)."""
+    angles = positions.to(torch.float32)[:, None] * inv_freq[None, :].float()  # [T, d/2], float32 angles
+    angles = torch.cat((angles, angles), dim=-1)                                # [T, d]
+    cos, sin = angles.cos().to(x.dtype)[:, None, :], angles.sin().to(x.dtype)[:, None, :]
     half = x.shape[-1] // 2
     rotated = torch.cat((-x[..., half:], x[..., :half]), dim=-1)
     return x * cos + rotated * sin
@@ -57,16 +58,18 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, windo
     last `window` ones (j > history+i-window); None is the reference's behaviour."""
     q_heads, kv_heads = q.shape[1], k.shape[1]
     group = q_heads // kv_heads
-    k = k.repeat_interleave(group, dim=1)
-    v = v.repeat_interleave(group, dim=1)
-    scores = torch.einsum("ihd,jhd->hij", q, k) * (q.shape[-1] ** -0.5)
     q_pos = history + torch.arange(q.shape[0])
     k_pos = torch.arange(k.shape[0])
     visible = k_pos[None, :] <= q_pos[:, None]
     if window is not None:
         visible &= k_pos[None, :] > (q_pos[:, None] - window)
-    scores = scores.masked_fill(~visible[None], -math.inf)
-    return torch.einsum("hij,jhd->ihd", scores.softmax(dim=-1), v)
+    out = torch.empty_like(q)
+    for head in range(q_heads):              # one head at a time: a long sequence's scores of all heads need not fit
+        kv = head // group
+        scores = (q[:, head] @ k[:, kv].T) * (q.shape[-1] ** -0.5)
+        scores = scores.masked_fill(~visible, -math.inf)
+        out[:, head] = scores.softmax(dim=-1) @ v[:, kv]
+    return out
 
 
 def swiglu_feed_forward(x: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor) -> torch.Tensor:

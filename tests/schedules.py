@@ -113,14 +113,16 @@ def run(engine, requests: dict[str, list[int]], schedule, want_all: bool = True)
     return {name: torch.cat(parts) for name, parts in collected.items() if parts}, pages_held
 
 
-def to_trace(requests, schedule):
-    """The schedule as trace-replay JSON records, asking for every fed position."""
+def to_trace(requests, schedule, first_step: int = 0, prefix: str = ""):
+    """The schedule as trace-replay JSON records, asking for every fed position.  Steps are numbered from
+    `first_step` and request names get `prefix`, so that several schedules can follow each other in one trace."""
     fed = {name: 0 for name in requests}
     records = []
-    for number, (entries, ends) in enumerate(schedule):
+    for number, (entries, ends) in enumerate(schedule, start=first_step):
         items = []
         for name, count in entries:
-            items.append({"id": name, "tokens": requests[name][fed[name]:fed[name] + count], "want": list(range(count))})
+            items.append({"id": prefix + name, "tokens": requests[name][fed[name]:fed[name] + count],
+                          "want": list(range(count))})
             fed[name] += count
-        records.append({"step": number, "entries": items, "end": list(ends)})
+        records.append({"step": number, "entries": items, "end": [prefix + name for name in ends]})
     return records

@@ -151,3 +151,45 @@ def test_slot_table():
     with pytest.raises(ValueError):
         slots.give_back(a)
     assert slots.take() == a
+
+
+def test_a_mixer_may_say_how_its_state_starts():
+    """`SlotState(init=...)`: the slot of a new request is set by the mixer's own function, also when the slot was
+    used before; without it the state is zeroed."""
+    def ones_then_index(state):
+        state.fill_(1.0)
+        state[0] = 3.0
+    needs = {0: SlotState((4,), torch.float32, init=ones_then_index), 1: SlotState((2,))}
+    m = CacheManager(needs, page_size=4, num_pages=4, max_seqs=2, dtype=torch.float32)
+    a = m.open("a")
+    assert m.layer_cache[0].state[a.slot].tolist() == [3.0, 1.0, 1.0, 1.0] and m.layer_cache[1].state[a.slot].tolist() == [0.0, 0.0]
+    m.layer_cache[0].state[a.slot] = -5.0
+    m.layer_cache[1].state[a.slot] = -5.0
+    m.close(a)
+    b = m.open("b")
+    assert b.slot == a.slot
+    assert m.layer_cache[0].state[b.slot].tolist() == [3.0, 1.0, 1.0, 1.0] and m.layer_cache[1].state[b.slot].tolist() == [0.0, 0.0]
+
+
+def test_a_step_is_checked_in_the_order_its_requests_register():
+    """A windowed group: in one step a single-token request needs a new page while a portion of another request
+    gives pages back.  The single token registers first, so the pages the portion frees come too late for it: the
+    step must be refused as a whole, with nothing registered, and not fail half-way."""
+    from ampere_kv_engine_amd.engine.batch import BatchBuilder, StepEntry
+    needs = {0: PagedKV(1, 16, window=4)}
+    m = CacheManager(needs, page_size=4, num_pages=5, max_seqs=2, dtype=torch.float32, device="cpu")
+    builder = BatchBuilder(m, "cpu", 64, 2, 16)
+    old, young = m.open("old"), m.open("young")
+    builder.build([StepEntry(old, [0] * 16, [])])            # 4 pages; a later step of `old` frees 3 of them
+    builder.build([StepEntry(young, [0] * 4, [])])           # 1 page (none of it passed yet): the pool is empty
+    assert m.num_free_pages == [0]
+    before = (old.length, young.length, old.tables[0].pages, young.tables[0].pages)
+    # in caller order `old` would free 3 pages before `young` needs 1; in the step's order `young` (one token) is first
+    with pytest.raises(PagePoolExhausted, match="'young'"):
+        builder.build([StepEntry(old, [0, 0], []), StepEntry(young, [0], [0])])
+    assert (old.length, young.length, old.tables[0].pages, young.tables[0].pages) == before
+    assert m.num_free_pages == [0]
+    builder.build([StepEntry(old, [0, 0], [])])              # alone it fits: pages are given back first
+    builder.build([StepEntry(young, [0], [0])])
+    m.close(old), m.close(young)
+    assert m.num_free_pages == [5]

@@ -31,14 +31,14 @@ def hip_own():
 
 @pytest.fixture(scope="module")
 def hip_library():
-    """Every bfloat16 product of more than 16 rows in the BLAS library, without the one-time choice up to 64 rows."""
+    """Every bfloat16 product of more than 16 rows in the BLAS library (the rule without a table of exceptions)."""
     from ampere_kv_engine_amd.kernels.hip import HipKernels
-    return HipKernels("cuda:0", tune_products=False)
+    return HipKernels("cuda:0")
 
 
-@pytest.fixture(params=["own", "library", "chosen"])
-def hip_either(request, hip, hip_own, hip_library):
-    return {"own": hip_own, "library": hip_library, "chosen": hip}[request.param]
+@pytest.fixture(params=["own", "library"])
+def hip_either(request, hip_own, hip_library):
+    return {"own": hip_own, "library": hip_library}[request.param]
 
 
 @pytest.fixture(scope="module")
@@ -265,27 +265,40 @@ def test_gated_linear_after_norm(hip, ref, rows):
     torch.testing.assert_close(new.cpu(), want_stream, rtol=0, atol=0)
 
 
-def test_products_of_17_to_64_rows_choose_once(hip, ref):
-    """Between 17 and 64 rows the engine's own product and the library's are timed at the first call with a matrix
-    shape and number of row tiles; the choice is remembered for the process, every call gives the product, and other
-    row counts do not ask."""
+def test_products_of_17_to_64_rows_follow_a_table_that_is_measured_on_request(hip, ref, tmp_path):
+    """Between 17 and 64 rows a product goes to the library unless the table of choices names the engine's own kernel
+    for its matrix shape and number of row tiles.  Nothing is timed by a product call; `measure_products` fills the
+    table for the shapes prepared so far and reports every decision; the table can be saved and loaded; either choice
+    gives the product."""
     from ampere_kv_engine_amd.kernels.hip import HipKernels
     kernels = HipKernels("cuda:0")
     w = rand(320, 256, dtype=torch.bfloat16, seed=41, scale=0.05)
     packed = kernels.prepare_linear(w.cuda())
-    for rows, known in ((8, 0), (20, 1), (31, 1), (65, 1), (64, 2), (50, 2)):
-        x = rand(rows, 256, dtype=torch.bfloat16, seed=42)
-        want = torch.empty(rows, 320, dtype=torch.bfloat16)
-        ref.linear(x, w, want)
-        got = torch.empty(rows, 320, dtype=torch.bfloat16, device="cuda")
-        kernels.linear(x.cuda(), packed, got)
-        torch.testing.assert_close(got.cpu().float(), want.float(), **tol(torch.bfloat16))
-        assert sum(key[1:3] == (320, 256) for key in kernels._tuned) == known
-    mine = {key: choice for key, choice in kernels._tuned.items() if key[1:3] == (320, 256)}
-    assert set(mine) == {("linear", 320, 256, 2), ("linear", 320, 256, 4)}
-    assert set(mine.values()) <= {"own", "library"}
-    # the kernel sets of a process share the choices: two engines send a product of one shape the same way
-    assert HipKernels("cuda:0")._tuned is kernels._tuned
+    gate, up = (rand(64, 256, dtype=torch.bfloat16, seed=43 + i, scale=0.05) for i in range(2))
+    gated = kernels.prepare_gated_linear(gate.cuda(), up.cuda())
+
+    def products():
+        for rows in (8, 20, 31, 64, 65):
+            x = rand(rows, 256, dtype=torch.bfloat16, seed=42)
+            want = torch.empty(rows, 320, dtype=torch.bfloat16)
+            ref.linear(x, w, want)
+            got = torch.empty(rows, 320, dtype=torch.bfloat16, device="cuda")
+            kernels.linear(x.cuda(), packed, got)
+            torch.testing.assert_close(got.cpu().float(), want.float(), **tol(torch.bfloat16))
+    products()
+    assert kernels.product_choices == {}                       # calls decide nothing
+    lines = []
+    table = kernels.measure_products(log=lines.append)
+    assert set(table) == {(kind, outs, 256, tiles) for kind, outs in (("linear", 320), ("gated", 64)) for tiles in (2, 3, 4)}
+    assert set(table.values()) <= {"own", "library"} and len(lines) == 6 and all("->" in line for line in lines)
+    products()
+    for forced in ("own", "library"):
+        kernels.product_choices = {key: forced for key in table}
+        products()
+    path = str(tmp_path / "choices.json")
+    kernels.save_product_choices(path)
+    assert HipKernels.load_product_choices(path) == kernels.product_choices
+    assert HipKernels("cuda:0", product_choices=HipKernels.load_product_choices(path)).product_choices == kernels.product_choices
 
 
 def test_linear_keeps_other_weights_row_major(hip):

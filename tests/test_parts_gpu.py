@@ -1,6 +1,7 @@
 """Each part alone on the GPU against the plain function of the same part, at sizes that are not the tiny
 models'; and the entry points: greedy generation through `generate_tokens`, the scheduler and the command line."""
 
+import json
 import os
 import subprocess
 import sys
@@ -245,13 +246,15 @@ def test_command_line(model_folders):
         result = run("--model", model_folders["A"], "--mode", "generate", "--decode-kernel", kernel, "--max-new-tokens",
                      "6", "--ignore-eos", "--prompt-ids", ",".join(map(str, prompt)))
         assert result.returncode == 0 and f"generated_token_ids = {want}" in result.stdout, result.stderr[-2000:]
-    # two cache sets in lock step: the decode kernels of the matrix cores beside the plain one
+    # the decode kernels of the matrix cores beside the plain one, position by position on the same tokens
     result = run("--model", model_folders["A"], "--mode", "cuda-check", "--max-new-tokens", "24", "--ignore-eos",
                  "--prompt-ids", ",".join(map(str, prompt)))
     assert result.returncode == 0, result.stdout[-1500:] + result.stderr[-1500:]
-    assert "[PASS] prompt logits of both cache sets are identical" in result.stdout
-    assert "[PASS] both kernels generated the same tokens" in result.stdout and "[not covered]" not in result.stdout
-    assert result.stdout.count("[observed] decode step") == 23
+    records = [json.loads(line) for line in result.stdout.splitlines() if line.startswith("{")]
+    verdict = records[-1]
+    assert verdict["ok"] and verdict["covered"] and verdict["prompt_bit_identical"] and verdict["decode_steps"] == 23
+    assert len(records) == 25 and records[0]["largest_difference"] == 0.0
+    assert all(r["largest_difference"] <= r["limit"] for r in records[:-1])
     # a model from a configuration file alone, with random weights
     config_file = os.path.join(model_folders["A"], "config.json")
     result = run("--random-config", config_file, "--weights-seed", "3", "--mode", "generate", "--max-new-tokens", "4",
@@ -261,22 +264,59 @@ def test_command_line(model_folders):
     assert result.returncode != 0
 
 
+def test_command_line_with_several_prompts_and_the_engines_own_sizes(model_folders, tmp_path):
+    """`--prompts-file`: every line a request, all through the scheduler; `--max-seqs`, `--num-pages` / `--kv-gb`,
+    `--max-batched-tokens` and `--prefill-chunk` size the engine.  In float32 every request must generate what the
+    plain implementation generates for it alone, however few slots and pages there are."""
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    plain = P.PlainQwen3(model_folders["B"])
+    prompts = [random_ids(379, n, seed=80 + n) for n in (5, 17, 33, 1, 24)]
+    path = tmp_path / "prompts.txt"
+    path.write_text("\n".join(" ".join(map(str, p)) for p in prompts) + "\n")
+    want = [plain.greedy(p, 5) for p in prompts]
+    run = lambda *args: subprocess.run([sys.executable, "-m", "ampere_kv_engine_amd.runner", "--model", model_folders["B"],
+                                        "--mode", "generate", "--dtype", "float32", "--prompts-file", str(path),
+                                        "--max-new-tokens", "5", "--ignore-eos", "--page-size", "8", *args],
+                                       env=env, capture_output=True, text=True, timeout=300)
+    for sizes in (("--max-seqs", "2", "--num-pages", "12", "--max-batched-tokens", "16", "--prefill-chunk", "7"),
+                  ("--kv-gb", "0.001"), ()):
+        result = run(*sizes)
+        assert result.returncode == 0, result.stdout[-1500:] + result.stderr[-1500:]
+        records = [json.loads(line) for line in result.stdout.splitlines() if line.startswith("{")]
+        assert [r["generated_token_ids"] for r in records] == want, sizes
+        assert all(r["stop_reason"] == "reached limit" for r in records)
+    assert run("--num-pages", "3").returncode != 0                     # no room for the longest request
+
+
 def test_scheduler_measurements_run(model_folders):
-    """`python -m ampere_kv_engine_amd.bench_scheduler` with the reference's option names, on a tiny model: both
-    experiments run, the batch of more than four is checked against single runs first, and every sample ends with
-    the pool whole (the program asserts it)."""
+    """`python -m ampere_kv_engine_amd.bench_scheduler` with the reference's option names, on a tiny model: the three
+    experiments run and print one JSON line per result with raw samples, median and range; a batch of more than four
+    is first checked for independence of its neighbours; every sample ends with the pool whole (the program insists)."""
     env = dict(os.environ, PYTHONPATH=ROOT)
     page = str(TINY["A"][2])
-    result = subprocess.run([sys.executable, "-m", "ampere_kv_engine_amd.bench_scheduler", "--model", model_folders["A"],
-                             "--history", "40", "--steps", "6", "--repeats", "1", "--batches", "1", "5", "--insert-at",
-                             "3", "--insert-history", "30", "--chunks", "0", "7", "--page-size", page,
-                             "--max-batched-tokens", "64"], env=env, capture_output=True, text=True, timeout=300)
+    common = [sys.executable, "-m", "ampere_kv_engine_amd.bench_scheduler", "--model", model_folders["A"], "--page-size",
+              page, "--max-batched-tokens", "64"]
+    result = subprocess.run(common + ["--history", "40", "--steps", "6", "--repeats", "2", "--batches", "1", "5",
+                                      "--insert-at", "3", "--insert-history", "30", "--chunks", "0", "7", "--mixed"],
+                            env=env, capture_output=True, text=True, timeout=300)
     assert result.returncode == 0, result.stdout[-1500:] + result.stderr[-1500:]
-    assert "[before] B=5: the batch generates the same 6 tokens as each request alone" in result.stdout
-    assert result.stdout.count("[decode] B=") == 2 and result.stdout.count("time to the late request's first token") == 2
-    result = subprocess.run([sys.executable, "-m", "ampere_kv_engine_amd.bench_scheduler", "--model", model_folders["A"],
-                             "--only", "insert", "--steps", "4", "--insert-at", "9"], env=env, capture_output=True,
-                            text=True, timeout=300)
+    records = [json.loads(line) for line in result.stdout.splitlines()]
+    decode = [r for r in records if r.get("experiment") == "decode" and "round_ms" in r]
+    assert [r["batch"] for r in decode] == [1, 5] and all(len(r["round_ms"]["samples"]) == 2 for r in decode)
+    assert any(r.get("check") == "tokens do not depend on the neighbours" and r["batch"] == 5 for r in records)
+    insert = [r for r in records if r.get("experiment") == "insert"]
+    assert sorted((r["chunk"], r["rounds"]) for r in insert) == [(0, "decodes and portion apart"), (0, "one step"),
+                                                               (7, "decodes and portion apart"), (7, "one step")]
+    assert all(len(r["late_first_token_ms"]["samples"]) == 2 and r["largest_gap_after_ms"]["median"] > 0 for r in insert)
+    assert all((sum(r["shared_rounds"]) > 0) == (r["rounds"] == "one step") for r in insert)
+    result = subprocess.run(common + ["--only", "calibrate", "--history", "24", "--steps", "6", "--repeats", "1",
+                                      "--batches", "2", "--pending-history", "0", "16", "--chunks", "8"],
+                            env=env, capture_output=True, text=True, timeout=300)
+    assert result.returncode == 0, result.stdout[-1500:] + result.stderr[-1500:]
+    cells = [json.loads(line) for line in result.stdout.splitlines() if '"calibrate"' in line]
+    assert [c.get("fed_before") for c in cells] == [None, 0, 16] and all("feasible" in c for c in cells[1:])
+    result = subprocess.run(common + ["--only", "insert", "--steps", "4", "--insert-at", "9"], env=env,
+                            capture_output=True, text=True, timeout=300)
     assert result.returncode != 0 and "--insert-at" in result.stderr
 
 

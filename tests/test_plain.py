@@ -197,6 +197,62 @@ def test_logits_are_causal_and_tied_head_is_the_embedding(model_folders):
     assert "lm_head.weight" not in plain.w
 
 
+def _silenced(plain):
+    """The same model with every branch's last matrix zeroed: each block then adds nothing to the residual sum."""
+    for name in plain.w:
+        if name.endswith("o_proj.weight") or name.endswith("down_proj.weight"):
+            plain.w[name] = torch.zeros_like(plain.w[name])
+    return plain
+
+
+def test_the_embedding_is_a_row_gather_without_scaling(model_folders):
+    """With all branches silenced the hidden states ARE the embedding rows, bit for bit (ampere_kv/runner.py:282): a
+    multiplier (the square root of the width, say) or an added position embedding fails this."""
+    plain = _silenced(P.PlainQwen3(model_folders["B"], dtype=torch.float64))
+    ids = random_ids(379, 11, seed=3)
+    assert torch.equal(plain.hidden_states(ids), plain.w["model.embed_tokens.weight"][torch.tensor(ids)])
+
+
+def test_final_norm_then_head_is_the_library_routine(model_folders):
+    """logits = linear(rms_norm(h_L)) with the library's own norm and product (ampere_kv/runner.py:293-297), and the
+    norm is where it belongs: with the branches silenced h_L is the embedding row, so scaling the embedding table by 5
+    must leave the logits alone (eps next to nothing) - which fails if the final norm is dropped, if it is applied
+    after the head, or if the head reads the un-normed stream."""
+    import torch.nn.functional as F
+    plain = P.PlainQwen3(model_folders["B"], dtype=torch.float64)
+    ids = random_ids(379, 14, seed=4)
+    h = plain.hidden_states(ids)
+    want = F.linear(F.rms_norm(h, (h.shape[-1],), plain.w["model.norm.weight"], plain.eps), plain.w["lm_head.weight"])
+    torch.testing.assert_close(plain.logits(ids), want, rtol=1e-12, atol=1e-12)
+    assert want.shape == (14, 379)
+
+    quiet = _silenced(P.PlainQwen3(model_folders["B"], dtype=torch.float64))
+    quiet.eps = 1e-30
+    base = quiet.logits(ids)
+    quiet.w["model.embed_tokens.weight"] = 5.0 * quiet.w["model.embed_tokens.weight"]
+    torch.testing.assert_close(quiet.logits(ids), base, rtol=1e-10, atol=1e-12)
+    assert base.abs().max() > 1e-3
+    # the norm's weight multiplies after the normalisation: doubling it doubles the logits
+    quiet.w["model.norm.weight"] = 2.0 * quiet.w["model.norm.weight"]
+    torch.testing.assert_close(quiet.logits(ids), 2.0 * base, rtol=1e-10, atol=1e-12)
+
+
+def test_rope_forms_cosines_in_float32_and_casts_afterwards():
+    """ampere_kv/runner.py:92-93: the table is cos/sin of float32 angles, cast to the activations' dtype.  At a far
+    position the float64 cosine of the float32 angle differs from the float32 cosine by rounding only; a table formed
+    from angles in the activations' dtype (bfloat16 angles!) would be off by whole radians."""
+    f = P.rope_inverse_frequencies(8, 1e4)
+    x = torch.ones(1, 1, 8, dtype=torch.float64)
+    position = torch.tensor([4099])
+    out = P.rope(x, position, f)[0, 0]
+    angle = (position.float()[:, None] * f[None, :])[0]
+    cos, sin = angle.cos().double(), angle.sin().double()
+    torch.testing.assert_close(out[:4], cos - sin, rtol=0, atol=0)
+    torch.testing.assert_close(out[4:], cos + sin, rtol=0, atol=0)
+    low = P.rope(torch.ones(1, 1, 8, dtype=torch.bfloat16), position, f)[0, 0].float()
+    torch.testing.assert_close(low, out.float(), rtol=0, atol=2e-2)      # bfloat16 angles would miss by O(1)
+
+
 def test_greedy_continues_with_the_argmax(model_folders):
     plain = P.PlainQwen3(model_folders["B"])
     prompt = random_ids(379, 9, seed=6)

@@ -191,3 +191,31 @@ def test_scheduler_arguments():
         Scheduler(FakeEngine(), prefill_chunk_size=-1)
     with pytest.raises(ValueError):
         Scheduler(FakeEngine(), max_batched_tokens=2)
+
+
+def test_a_request_without_finite_logits_is_retired_with_an_error(model_folders):
+    """A step that answers one request with NaN (the attention kernels do so for a block table that names a page
+    outside the pool) must end that request with an error instead of feeding it token 0; its neighbour goes on."""
+    from ampere_kv_engine_amd.engine.scheduler import STOP_NO_LOGITS
+    raw, _, page = TINY["A"]
+    engine = make_engine(model_folders["A"], page, 32)
+    scheduler = Scheduler(engine)
+    good = scheduler.submit("good", random_ids(256, 6, seed=1), max_new_tokens=6, ignore_eos=True)
+    bad = scheduler.submit("bad", random_ids(256, 9, seed=2), max_new_tokens=6, ignore_eos=True)
+    scheduler.step()                                    # both prompts; first tokens
+    assert len(good.output_ids) == 1 and len(bad.output_ids) == 1
+    real_step = engine.step
+
+    def poisoned(entries, **kw):
+        logits = real_step(entries, **kw)
+        for row, entry in enumerate(entries):
+            if entry.seq.request_id == "bad":
+                logits[row] = float("nan")
+        return logits
+    engine.step = poisoned
+    finished, _ = scheduler.step()
+    assert finished == [bad] and bad.stop_reason == STOP_NO_LOGITS and bad.status == FINISHED
+    assert len(bad.output_ids) == 1 and len(good.output_ids) == 2
+    done, _ = drive(scheduler)
+    assert good in done and good.stop_reason == STOP_LIMIT and len(good.output_ids) == 6
+    assert engine.cache.num_free_pages == [32] and engine.cache.slots.num_free == 4

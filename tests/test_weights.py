@@ -103,6 +103,36 @@ def test_a_tied_model_may_carry_the_head_but_not_in_another_shape(tmp_path):
         Checkpoint(folder).check(expected_tensors(config.to_model_spec()))
 
 
+def test_a_tied_model_whose_head_differs_from_the_embedding_is_refused(tmp_path):
+    """Right shape, other values: the engine would silently use the embedding, so the file is refused by name."""
+    config = Qwen3Config.from_dict(TINY_A)
+    folder = write_random_model(str(tmp_path / "m"), config, seed=0)
+    path = os.path.join(folder, "model.safetensors")
+    tensors = load_file(path)
+    head = tensors["model.embed_tokens.weight"].clone()
+    head[17, 3] += 0.5
+    tensors["lm_head.weight"] = head
+    save_file(tensors, path)
+    with pytest.raises(WeightsError, match="differing values: lm_head.weight must equal model.embed_tokens.weight") as caught:
+        Checkpoint(folder).check(expected_tensors(config.to_model_spec()))
+    assert caught.value.differing == [("lm_head.weight", "model.embed_tokens.weight")]
+    assert not caught.value.missing and not caught.value.wrong_shape
+
+
+def test_a_role_of_its_own_brings_its_own_random_law():
+    """A part whose tensors follow another law than the three built in registers it under a role's name; nothing in
+    the package is edited."""
+    from ampere_kv_engine_amd.weights import TensorSpec, draw, register_init_law
+    with pytest.raises(ValueError, match="no random law is registered"):
+        draw(TensorSpec("x.decay", (4,), "toy_decay"), seed=0)
+    register_init_law("toy_decay", lambda shape, generator, device: torch.rand(shape, generator=generator, device=device) * 0.5 + 0.5)
+    value = draw(TensorSpec("x.decay", (64,), "toy_decay"), seed=0)
+    assert value.min() >= 0.5 and value.max() <= 1.0
+    assert torch.equal(value, draw(TensorSpec("x.decay", (64,), "toy_decay"), seed=0))
+    with pytest.raises(ValueError, match="already has a law"):
+        register_init_law("toy_decay", lambda *a: None)
+
+
 def test_sharded_checkpoints_are_read_through_the_index(tmp_path):
     config = Qwen3Config.from_dict(TINY_A)
     folder = write_random_model(str(tmp_path / "m"), config, seed=0)

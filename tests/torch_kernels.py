@@ -138,22 +138,26 @@ class TorchKernels:
             keys = k_pages[pages, :, key_pos % page_size].float()        # [S, kv_heads, d]
             values = v_pages[pages, :, :, key_pos % page_size].float()
             qs = q[first:last].reshape(last - first, q_heads, head_dim).float()
-            keys = keys.repeat_interleave(group, dim=1)
-            values = values.repeat_interleave(group, dim=1)
-            scores = torch.einsum("ihd,jhd->hij", qs, keys) * scale
             q_pos = history + torch.arange(last - first)
             visible = key_pos[None, :] <= q_pos[:, None]
             if window is not None:
                 visible &= key_pos[None, :] > q_pos[:, None] - window
-            scores = scores.masked_fill(~visible[None], -math.inf)
-            merged = torch.einsum("hij,jhd->ihd", scores.softmax(-1), values)
+            merged = torch.empty_like(qs)
+            for head in range(q_heads):          # a head at a time: long histories' scores of all heads need not fit
+                scores = (qs[:, head] @ keys[:, head // group].T) * scale
+                scores = scores.masked_fill(~visible, -math.inf)
+                merged[:, head] = scores.softmax(-1) @ values[:, head // group]
             out[first:last] = merged.reshape(last - first, q_heads * head_dim).to(out.dtype)
 
     # ---- sampling -----------------------------------------------------------------------------------------
     def sample(self, logits, temperature, seeds, draws, out):
         """temperature 0: the largest logit, ties to the lowest id.  Otherwise the Gumbel-max draw
-        argmax(logits / t - log(-log(u))), u from Philox-4x32-10 keyed by the seed with counter (id, draw)."""
+        argmax(logits / t - log(-log(u))), u from Philox-4x32-10 keyed by the seed with counter (id, draw).
+        A row with a NaN, or with nothing above -infinity, gives -1."""
         for row in range(logits.shape[0]):
+            if torch.isnan(logits[row]).any() or not (logits[row] > -math.inf).any():
+                out[row] = -1
+                continue
             t = float(temperature[row]) if temperature is not None else 0.0
             scores = logits[row].double()
             if t > 0:
