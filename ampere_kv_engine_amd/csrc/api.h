@@ -1,5 +1,5 @@
 // C entry points of the kernel library.  Every function enqueues on `stream` and returns 0, a hipError_t of the
-// launch, -1 for an unknown dtype code or -2 for sizes the kernel does not take.  dtype codes: 0 float32,
+// launch, -1 for an unknown dtype code, -2 for sizes the kernel does not take or -3 for sizes beyond a fixed buffer.  dtype codes: 0 float32,
 // 1 bfloat16.  Pointers are device pointers; shapes are checked by the caller on the host.
 #pragma once
 
@@ -38,6 +38,14 @@ int akv_linear_packed_normed(const float* stream_in, const void* delta, const fl
                              float* stream_out, const void* wp, void* y, int rows, int outs, int k, int n_tiles,
                              int k_tiles, int gated, hipStream_t stream);
 int akv_pack_rows(const void* x, void* xp, int rows, int k, hipStream_t stream);
+// No counterpart in the reference.  For callers that cannot allocate device memory (code under HIP graph capture,
+// tight serving loops, harnesses that forbid hipMalloc): akv_pack_rows + akv_linear_packed(x_packed = 1) as one call
+// that allocates nothing - the repacked activations live in 4 MiB of static device memory that each GPU holds from
+// the library's load to the end of the process.  Up to 64 rows with ceil(rows / 16) * 16 * k <= 2,097,152 elements;
+// -3 beyond that.  Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two
+// threads) race; calls that follow each other on a stream do not.
+int akv_linear_packed_static(const void* x, const void* wp, void* y, int y_dtype, int rows, int outs, int k,
+                             int n_tiles, int k_tiles, hipStream_t stream);
 int akv_attention_rows(const void* q, const void* k_pages, const void* v_pages, const int* seq_of_token,
                        const int* positions, const int* block_table, int table_width, void* out, int dtype,
                        long tokens, int q_heads, int kv_heads, int dim, int page_size, long num_pages, float scale,

@@ -16,10 +16,18 @@
 // rows with the tile of the 16 up rows of the same features, a wave always owns such pairs, and what it stores is
 // silu(gate) * up, taken from the float32 accumulators - the stacked product never goes to memory.
 
+#include <mutex>
+
 #include "common.h"
 #include "api.h"
 
 using namespace akv;
+
+// Where akv_linear_packed_static lays out its activations: device memory that exists from the moment the library is
+// loaded until the process ends, on every GPU the library runs on, so that entry point never has to ask for any.
+// In host code this name is only a handle for hipGetSymbolAddress; kernels are given the address that call returns.
+constexpr size_t kStaticRowsBytes = 64 * 32768 * sizeof(uint16_t);   // 64 rows of 32,768 bfloat16: 4 MiB
+static __device__ __align__(256) unsigned char scratch[kStaticRowsBytes];
 
 namespace {
 
@@ -638,6 +646,50 @@ extern "C" int akv_linear_packed(const void* x, const void* wp, void* y, int y_d
   if (rows <= 0 || outs <= 0) return 0;
   if ((k & 7) != 0 || n_tiles * 16 < outs || k_tiles * 32 < k) return -2;
   return linear_packed<false>(x, wp, y, y_dtype, rows, outs, k, n_tiles, k_tiles, x_packed, stream);
+}
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* scratch_of_device[kMaxDevices];   // the array's address on each device, asked for once
+std::mutex scratch_guard;
+
+// The address of `scratch` on the current device (every GPU holds its own copy at its own address).
+int static_rows(void** address) {
+  int device = -1;
+  hipError_t status = hipGetDevice(&device);
+  if (status != hipSuccess) return static_cast<int>(status);
+  if (device < 0 || device >= kMaxDevices) return -2;
+  std::lock_guard<std::mutex> lock(scratch_guard);
+  if (scratch_of_device[device] == nullptr) {
+    void* found = nullptr;
+    status = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+    if (status != hipSuccess) return static_cast<int>(status);
+    if (found == nullptr) return static_cast<int>(hipErrorInvalidSymbol);
+    scratch_of_device[device] = found;
+  }
+  *address = scratch_of_device[device];
+  return 0;
+}
+}  // namespace
+
+// akv_pack_rows followed by akv_linear_packed(x_packed = 1) without any allocation by anybody: the repacked
+// activations go to the library's own 4 MiB of static device memory instead of a buffer the caller brings.
+// Returns -3 where ceil(rows / 16) * 16 * k bfloat16 do not fit that memory or rows exceed 64.  Nothing needs clearing
+// between calls: a call writes every element that it reads (rows beyond `rows` of the last tile are neither).
+extern "C" int akv_linear_packed_static(const void* x, const void* wp, void* y, int y_dtype, int rows, int outs, int k,
+                                        int n_tiles, int k_tiles, hipStream_t stream) {
+  if (rows <= 0 || outs <= 0) return 0;
+  if ((k & 7) != 0 || n_tiles * 16 < outs || k_tiles * 32 < k) return -2;
+  if (rows > 64 || static_cast<size_t>((rows + 15) / 16 * 16) * k * sizeof(uint16_t) > kStaticRowsBytes) return -3;
+  void* packed = nullptr;
+  const int found = static_rows(&packed);
+  if (found != 0) return found;
+  const long pieces = static_cast<long>(rows) * (k / 8);
+  pack_rows_kernel<<<static_cast<unsigned>((pieces + 255) / 256), 256, 0, stream>>>(
+      static_cast<const uintx4*>(x), static_cast<uintx4*>(packed), rows, k / 8);
+  const int status = AKV_LAUNCH_STATUS();
+  if (status != 0) return status;
+  return linear_packed<false>(packed, wp, y, y_dtype, rows, outs, k, n_tiles, k_tiles, 1, stream);
 }
 
 // The gated pair in one pass: wp holds 2 * inter / 16 row tiles, gate tile t at 2t and up tile t at 2t + 1;

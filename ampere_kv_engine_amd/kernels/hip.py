@@ -121,7 +121,7 @@ class HipKernels:
         for name in ("akv_embed", "akv_add_rmsnorm", "akv_rmsnorm_rows", "akv_copy_rows", "akv_gather_rows",
                      "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
                      "akv_linear_tiled", "akv_linear_packed", "akv_linear_packed_swiglu", "akv_linear_packed_normed",
-                     "akv_pack_rows",
+                     "akv_pack_rows", "akv_linear_packed_static",
                      "akv_attention_rows", "akv_decode_plan", "akv_sample"):
             getattr(self.lib, name).restype = ctypes.c_int
 
@@ -352,6 +352,28 @@ class HipKernels:
         self._dense(out, "out", None, (rows, outs))
         self._check(self.lib.akv_linear_tiled(_ptr(x), _code(x), _ptr(weight), _code(weight), _ptr(out), _code(out),
                                               rows, outs, k, self._stream()), "linear")
+
+    STATIC_ROWS_ELEMENTS = 64 * 32768   # bfloat16 elements of the library's static device memory for repacked rows
+
+    def linear_without_allocation(self, x, weight: PackedWeight, out) -> None:
+        """out = x W^T for up to 64 bfloat16 rows through `akv_linear_packed_static`: the activations are repacked into
+        static device memory of the library instead of a buffer of this kernel set, so neither this call nor anything
+        under it allocates - for callers that must not (a graph being captured, a loop that may not touch the
+        allocator).  Calls that overlap on one GPU share that memory and race; calls on one stream do not."""
+        if not isinstance(weight, PackedWeight):
+            raise KernelError("the product without allocation takes a packed bfloat16 matrix")
+        rows = x.shape[0]
+        self._dense(x, "x", torch.bfloat16, (rows, weight.k))
+        self._dense(out, "out", None, (rows, weight.outs))
+        self._dense(weight.data, "packed weight", torch.bfloat16)
+        if rows > 64 or (rows + 15) // 16 * 16 * weight.k > self.STATIC_ROWS_ELEMENTS:
+            raise KernelError(f"{rows} rows of {weight.k} do not fit the static memory of the product without allocation: "
+                              f"at most 64 rows and {self.STATIC_ROWS_ELEMENTS} elements after rounding the rows up to 16")
+        status = self.lib.akv_linear_packed_static(_ptr(x), _ptr(weight.data), _ptr(out), _code(out), rows, weight.outs,
+                                                   weight.k, weight.n_tiles, weight.k_tiles, self._stream())
+        if status == -3:
+            raise KernelError("the product without allocation refused the sizes: they exceed its static memory")
+        self._check(status, "linear_without_allocation")
 
     # The most rows whose norm the product's blocks compute for themselves.  Every block reads the rows again (24 KB a
     # row at 4,096 wide): measured at Qwen3-8B sizes, a step of one row gains 0.16 ms of 4.09, two rows lose 0.04 ms,
