@@ -24,10 +24,10 @@ class EngineConfig:
     # bfloat16 products of more rows than this go to the BLAS library, which reads the matrices row-major: they are
     # then kept twice (row-major and packed for the engine's own kernels).  None: one copy, own kernels only.
     library_products_above: int | None = 16
-    # Exceptions to that rule for products of 17..64 rows, where for some matrix shapes the engine's own kernel is the
-    # faster one.  "fixed": none (every run sends every product the same way).  "measure": both are timed once, when the
-    # weights have been loaded (never inside a step), each decision is logged and the table can be saved
-    # (`engine.kernels.save_product_choices(path)`).  Anything else: the path of such a saved table.
+    # Which kernel takes a bfloat16 product of 17..512 rows: the engine's own skinny kernel, its mid-size kernel or the
+    # library.  "fixed": a rule from the sizes (every run sends every product the same way).  "measure": the candidates
+    # are timed once, when the weights have been loaded (never inside a step), each decision is logged and the table
+    # can be saved (`engine.kernels.save_product_choices(path)`).  Anything else: the path of such a saved table.
     product_choices: str = "fixed"
 
     def __post_init__(self):

@@ -46,6 +46,11 @@ int akv_pack_rows(const void* x, void* xp, int rows, int k, hipStream_t stream);
 // threads) race; calls that follow each other on a stream do not.
 int akv_linear_packed_static(const void* x, const void* wp, void* y, int y_dtype, int rows, int outs, int k,
                              int n_tiles, int k_tiles, hipStream_t stream);
+int akv_linear_mid_workspace(int rows, int n_tiles, int k_tiles, int gated, int along, int rt, int depth, int parts,
+                             long* partial_floats, long* counters);
+int akv_linear_mid(const void* x, const void* wp, void* y, int y_dtype, float* partial, unsigned* counters, int rows,
+                   int outs, int k, int n_tiles, int k_tiles, int gated, int along, int rt, int depth, int parts,
+                   hipStream_t stream);
 int akv_attention_rows(const void* q, const void* k_pages, const void* v_pages, const int* seq_of_token,
                        const int* positions, const int* block_table, int table_width, void* out, int dtype,
                        long tokens, int q_heads, int kv_heads, int dim, int page_size, long num_pages, float scale,

@@ -19,8 +19,8 @@ import time
 from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCES = ("elementwise.hip", "gemm.hip", "gemm_mfma.hip", "attention.hip", "sampling.hip")
-HEADERS = ("common.h", "api.h")
+SOURCES = ("elementwise.hip", "gemm.hip", "gemm_mfma.hip", "gemm_mid.hip", "attention.hip", "sampling.hip")
+HEADERS = ("common.h", "mfma_tiles.h", "api.h")
 LIBRARY = "libakv_kernels.so"
 ATTENTION_SOURCE = "attention_mfma.hip"        # compiled once per head size, into its own small library
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 128, 192, 256)

@@ -1,0 +1,374 @@
+// bfloat16 matrix products y = x W^T for some tens to some hundreds of rows (a decode step of many requests, a short
+// prompt, a small portion beside decoding requests) on the matrix cores, float32 accumulation.
+//
+// With so many rows the weights are still read once and memory still sets the pace, but a weight tile of 1 KB now
+// meets one activation operand of 1 KB per 16 rows.  If every wave fetched those operands for itself, the caches
+// would move several times what memory delivers.  Here the waves of a block share them:
+//   * a block owns a band of A * RT row tiles of the packed weight (see gemm_mfma.hip for the packing); 2 A of its
+//     waves multiply, A along the band x 2 along k (each half of the block's k);
+//   * per stage of S k-tiles the block's activations [16 * MT rows][S * 32 k] of either k half go through LDS,
+//     double-buffered, one barrier per stage, already in the lane order of the matrix-core operand (a tile of 16 rows
+//     x 32 k is 1 KB that lane l reads at l * 16: no bank conflicts).  Four further waves do nothing but fetch them,
+//     two stages ahead: a wave's loads come back in the order they were issued, so a multiplying wave that fetched
+//     activations between its weight loads would have to wait for ALL weights it has asked for before it could use
+//     the activations - which brings the weights' distance down to one stage (measured: 1.6 us per stage, whatever
+//     the depth of the ring);
+//   * every multiplying wave streams its own RT row tiles straight from memory into a ring of G operand register
+//     sets, G - 1 stages ahead.  A load takes about two microseconds to come back, so what sets the pace is how much
+//     is on its way: a product with few row tiles has few blocks, and each wave of them then keeps 12 KB and more in
+//     flight.
+// More than 16 * MT rows are taken by several blocks per band; these sit next to each other on one XCD, so that the
+// weights they share come from memory once (and are then not marked as read-once).
+//
+// GATED: the packed matrix alternates gate and up tiles (RT = 2 gives a wave one pair); what is stored is
+// silu(gate) * up from the float32 sums.
+
+#include "common.h"
+#include "mfma_tiles.h"
+#include "api.h"
+
+using namespace akv;
+
+namespace {
+
+constexpr int kHalves = 2;   // waves along k (A waves along the band of row tiles: 2, 3 or 4)
+constexpr int kXcds = 8;
+constexpr int kFetchers = 4;
+constexpr int kComputeUnits = 256;
+
+template <int MT> constexpr int kStage = MT <= 4 ? 4 : 2;     // k-tiles per stage and k half
+
+template <int A, int MT, int RT, int G, bool GATED, typename TY>
+__global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_kernel(const bf16_t* __restrict__ x, const uintx4* __restrict__ wp,
+                                                              TY* __restrict__ y, float* __restrict__ partial,
+                                                              unsigned* __restrict__ counters, int rows, int outs, int k,
+                                                              int k_tiles, int n_tiles, int bands, int parts,
+                                                              int part_tiles, int m_blocks) {
+  constexpr int S = kStage<MT>;
+  constexpr int kAlong = A, kMultipliers = A * kHalves;
+  constexpr int kTiles = kHalves * S * MT;        // activation tiles of one stage
+  constexpr int kLoads = kTiles / kFetchers;      // of which every fetching wave brings this many
+  static_assert(kTiles % kFetchers == 0, "the stage's tiles are dealt to the fetching waves");
+  static_assert(G % 2 == 0, "a ring position must always meet the same staging buffer");
+  extern __shared__ uintx4 staged[];              // [2][kTiles][64]; afterwards the sums of the second k half
+  __shared__ unsigned is_last;
+
+  // which work: blocks that share weights (same band and part of k, other rows) are neighbours on one XCD
+  const int xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
+  const int item = (slot / m_blocks) * kXcds + xcd, m_block = slot % m_blocks;
+  if (item >= bands * parts) return;
+  const int band = item / parts, part = item % parts;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r = lane & 15, g = lane >> 4;
+  const int row0 = m_block * MT * 16;
+  const int kb0 = part * part_tiles, kb1 = min(k_tiles, kb0 + part_tiles);   // the block's k-tiles
+  const int per_half = (kb1 - kb0 + kHalves - 1) / kHalves;
+  const int stages = (per_half + S - 1) / S;
+  const uintx4 zero = {0u, 0u, 0u, 0u};
+
+  if (wave >= kMultipliers) {
+    // ---- a fetching wave: activation tile i = (k half, k-tile of the stage, row tile); this wave brings
+    //      i = f, f + 4, ... of every stage, two stages ahead of the multiplying waves
+    const int f = wave - kMultipliers;
+    uintx4 fetched[2][kLoads];
+    auto fetch_rows = [&](int stage, uintx4 (&into)[kLoads]) {
+#pragma unroll
+      for (int j = 0; j < kLoads; ++j) {
+        const int i = f + kFetchers * j;
+        const int h = i / (S * MT), u = (i / MT) % S, mt = i % MT;
+        const int kt = kb0 + h * per_half + stage * S + u;
+        const int row = row0 + mt * 16 + r, col = kt * 32 + g * 8;
+        const bool there = kt < min(kb1, kb0 + (h + 1) * per_half) && row < rows && col < k;
+        into[j] = there ? *reinterpret_cast<const uintx4*>(x + static_cast<size_t>(row) * k + col) : zero;
+      }
+    };
+    fetch_rows(0, fetched[0]);
+    if (1 < stages) fetch_rows(1, fetched[1]);
+    for (int first = 0; first < stages; first += 2) {
+#pragma unroll
+      for (int d = 0; d < 2; ++d) {
+        const int stage = first + d;
+        if (stage < stages) {
+#pragma unroll
+          for (int j = 0; j < kLoads; ++j) staged[(d * kTiles + f + kFetchers * j) * 64 + lane] = fetched[d][j];
+          if (stage + 2 < stages) fetch_rows(stage + 2, fetched[d]);
+          __syncthreads();
+        }
+      }
+    }
+    return;
+  }
+
+  // ---- a multiplying wave
+  const int along = wave % kAlong, half = wave / kAlong;
+  const int tile0 = (band * kAlong + along) * RT;
+  const int mine0 = kb0 + half * per_half, mine1 = min(kb1, mine0 + per_half);
+  const bool shared_weights = m_blocks > 1;       // other blocks read the same tiles: let the caches keep them
+  floatx4 acc[RT][MT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  auto fetch_weights = [&](int stage, uintx4 (&a)[RT][S]) {
+    const int kt = mine0 + stage * S;
+    const uintx4* at = wp + (static_cast<size_t>(tile0) * k_tiles + kt) * 64 + lane;
+    if (kt + S <= mine1 && tile0 + RT <= n_tiles) {   // the whole group exists: no test per load
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int u = 0; u < S; ++u) {
+          const uintx4* from = at + (static_cast<size_t>(rt) * k_tiles + u) * 64;
+          a[rt][u] = shared_weights ? *from : load_once(from);
+        }
+    } else {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int u = 0; u < S; ++u) {
+          const uintx4* from = at + (static_cast<size_t>(rt) * k_tiles + u) * 64;
+          a[rt][u] = (kt + u < mine1 && tile0 + rt < n_tiles) ? (shared_weights ? *from : load_once(from)) : zero;
+        }
+    }
+  };
+  auto multiply = [&](int buffer, const uintx4 (&a)[RT][S]) {
+    const uintx4* tiles = staged + (buffer * kTiles + half * S * MT) * 64 + lane;
+#pragma unroll
+    for (int u = 0; u < S; ++u) {
+      uintx4 b[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) b[mt] = tiles[(u * MT + mt) * 64];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = mfma16(a[rt][u], b[mt], acc[rt][mt]);
+    }
+  };
+
+  uintx4 a[G][RT][S];
+#pragma unroll
+  for (int d = 0; d < G - 1; ++d)
+    if (d < stages) fetch_weights(d, a[d]);
+  for (int first = 0; first < stages; first += G) {
+#pragma unroll
+    for (int d = 0; d < G; ++d) {
+      const int stage = first + d;
+      if (stage < stages) {
+        __syncthreads();          // the stage's activations are in LDS
+        if (stage + G - 1 < stages) fetch_weights(stage + G - 1, a[(d + G - 1) % G]);
+        multiply(d & 1, a[d]);
+      }
+    }
+  }
+
+  // the two k halves: the second hands its sums over through LDS, the first adds them to its own
+  __syncthreads();
+  float* sums = reinterpret_cast<float*>(staged) + static_cast<size_t>(along) * RT * MT * 256;
+  if (half == 1) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        *reinterpret_cast<floatx4*>(sums + ((rt * MT + mt) * 64 + lane) * 4) = acc[rt][mt];
+  }
+  __syncthreads();
+  if (half == 0) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const floatx4 other = *reinterpret_cast<const floatx4*>(sums + ((rt * MT + mt) * 64 + lane) * 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[rt][mt][i] += other[i];
+      }
+  }
+  if (parts > 1) {
+    // k is cut over blocks as well: every block leaves its sums in `partial`; the block of a band that arrives last
+    // adds the parts in the order of their k ranges (whichever block that is, the bits are the same) and stores.
+    const size_t block_floats = static_cast<size_t>(kAlong) * RT * MT * 256;
+    float* band_parts = partial + (static_cast<size_t>(m_block) * bands + band) * parts * block_floats;
+    // No cache-wide write-back or invalidation is paid for this (a release and an acquire at device scope cost several
+    // microseconds per block here): the parts are stored and loaded with device scope themselves - such accesses go
+    // through to where all XCDs see them - and a wave's stores have been acknowledged when its vmcnt is back at zero.
+    if (half == 0) {
+      float* mine = band_parts + part * block_floats + static_cast<size_t>(along) * RT * MT * 256;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            __hip_atomic_store(mine + ((rt * MT + mt) * 4 + i) * 64 + lane, acc[rt][mt][i], __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+      __builtin_amdgcn_s_waitcnt(0);   // every counter at zero: the stores above have arrived
+    }
+    __syncthreads();                   // (the fetching waves have gone; all multiplying waves' stores have arrived)
+    if (threadIdx.x == 0) {
+      unsigned* counter = counters + m_block * bands + band;
+      const unsigned before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool last = before == static_cast<unsigned>(parts - 1);
+      if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+      is_last = last ? 1u : 0u;
+    }
+    __syncthreads();
+    if (is_last == 0u) return;
+    if (half == 0) {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
+      for (int p = 0; p < parts; ++p) {
+        const float* theirs = band_parts + p * block_floats + static_cast<size_t>(along) * RT * MT * 256;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              acc[rt][mt][i] += __hip_atomic_load(theirs + ((rt * MT + mt) * 4 + i) * 64 + lane, __ATOMIC_RELAXED,
+                                                  __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  }
+  if (half != 0) return;
+  if constexpr (GATED) {
+    static_assert(RT % 2 == 0, "a wave must own gate and up tiles in pairs");
+#pragma unroll
+    for (int rt = 0; rt < RT; rt += 2)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        if (tile0 + rt < n_tiles)
+          store_tile<TY>(y, silu_times(acc[rt][mt], acc[rt + 1][mt]), row0 + mt * 16 + r, ((tile0 + rt) >> 1) * 16 + g * 4,
+                         rows, outs);
+  } else {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        if (tile0 + rt < n_tiles) store_tile<TY>(y, acc[rt][mt], row0 + mt * 16 + r, (tile0 + rt) * 16 + g * 4, rows, outs);
+  }
+}
+
+struct MidPlan {
+  int along, mt, rt, depth, bands, parts, part_tiles, m_blocks;
+  size_t partial_floats, counters;
+};
+
+constexpr size_t kMostPartialFloats = 8u << 20;   // 32 MB: more than that is not worth a cut of k over blocks
+
+// How a product of `rows` rows is cut into blocks.  A compute unit draws little more than 20 GB/s from memory however
+// much its waves ask for, so a product streams at the device's rate only when every compute unit has a block, and
+// the blocks are equal: the cut (waves along the band, row tiles per wave, blocks along k) that keeps the busiest
+// compute unit's share smallest is taken, counted in weight tiles (measured at Qwen3-8B shapes: the best cut of every
+// product was one that gives each of the 256 compute units exactly one block).  `along`, `rt`, `depth` and `parts`
+// of 0 leave the choice to the sizes; others force it (for measurements).
+MidPlan plan_mid(int rows, int n_tiles, int k_tiles, bool gated, int along, int rt, int depth, int parts) {
+  MidPlan best{};
+  double best_cost = -1.0;
+  const int mt = rows > 64 ? 8 : (rows + 15) / 16 < 2 ? 2 : (rows + 15) / 16;
+  const int m_blocks = (rows + mt * 16 - 1) / (mt * 16);
+  for (int a = 2; a <= 4; ++a) {
+    if (along != 0 && a != along) continue;
+    for (int r = 1; r <= 2; ++r) {
+      if ((gated && r != 2) || (rt != 0 && r != rt)) continue;
+      for (int cut = 1; cut <= 16; cut *= 2) {
+        if (parts != 0 && cut != parts) continue;
+        if (parts == 0 && cut > 1 && k_tiles / cut < 2 * kHalves * 4) break;   // a block keeps a few stages of work
+        MidPlan p{};
+        p.along = a, p.mt = mt, p.rt = r, p.m_blocks = m_blocks;
+        p.bands = (n_tiles + a * r - 1) / (a * r);
+        p.part_tiles = (k_tiles + cut - 1) / cut;
+        p.parts = (k_tiles + p.part_tiles - 1) / p.part_tiles;
+        p.partial_floats = p.parts > 1 ? static_cast<size_t>(m_blocks) * p.bands * p.parts * a * r * mt * 256 : 0;
+        p.counters = p.parts > 1 ? static_cast<size_t>(m_blocks) * p.bands : 0;
+        if (parts == 0 && p.partial_floats > kMostPartialFloats) continue;
+        const long blocks = static_cast<long>(p.bands) * p.parts * m_blocks;
+        const long rounds = (blocks + kComputeUnits - 1) / kComputeUnits;
+        // tiles the busiest compute unit streams (+ a little per block, and what the exchange of partial sums moves:
+        // 4 bytes x parts per result against 1 KB per tile); of equal cuts the one with more waves along the band
+        // wins (they share the activations), then the one with fewer parts
+        double cost = static_cast<double>(rounds) * (static_cast<double>(a) * r * p.part_tiles + 8.0);
+        if (p.parts > 1) cost += static_cast<double>(a) * r * mt * p.parts / 8.0;
+        cost += 0.01 * (4 - a) + 0.001 * p.parts;
+        if (best_cost < 0.0 || cost < best_cost) best = p, best_cost = cost;
+      }
+    }
+  }
+  if (depth == 0) depth = best.rt == 2 ? 2 : 4;
+  if (best.rt == 2 && depth > 2) depth = 2;   // (two row tiles and a deeper ring do not fit the registers)
+  best.depth = depth;
+  return best;
+}
+
+template <int A, int MT, int RT, int G, bool GATED, typename TY>
+int launch_mid(const MidPlan& p, const void* x, const void* wp, void* y, float* partial, unsigned* counters, int rows,
+               int outs, int k, int k_tiles, int n_tiles, hipStream_t stream) {
+  constexpr size_t lds = 2 * kHalves * kStage<MT> * MT * 1024;
+  static_assert(lds >= static_cast<size_t>(A) * RT * MT * 1024, "the sums of a k half must fit the staging memory");
+  static_assert(lds <= 64 * 1024, "the staging memory is taken without asking for more than a block may have by default");
+  const long items = static_cast<long>(p.bands) * p.parts;
+  const long blocks = (items + kXcds - 1) / kXcds * kXcds * p.m_blocks;
+  if (blocks > 0x7fffffffL) return -2;
+  linear_mid_kernel<A, MT, RT, G, GATED, TY><<<static_cast<unsigned>(blocks), (A * kHalves + kFetchers) * 64, lds, stream>>>(
+      static_cast<const bf16_t*>(x), static_cast<const uintx4*>(wp), static_cast<TY*>(y), partial, counters, rows, outs,
+      k, k_tiles, n_tiles, p.bands, p.parts, p.part_tiles, p.m_blocks);
+  return AKV_LAUNCH_STATUS();
+}
+
+template <bool GATED, typename TY>
+int dispatch_mid(const MidPlan& p, const void* x, const void* wp, void* y, float* partial, unsigned* counters, int rows,
+                 int outs, int k, int k_tiles, int n_tiles, hipStream_t stream) {
+#define AKV_MID(A_, MT_, RT_, G_) \
+  if (p.along == A_ && p.mt == MT_ && p.rt == RT_ && p.depth == G_) \
+    return launch_mid<A_, MT_, RT_, G_, GATED, TY>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, stream)
+#define AKV_MID_ROWS(A_, RT_, G_) \
+  AKV_MID(A_, 2, RT_, G_); AKV_MID(A_, 3, RT_, G_); AKV_MID(A_, 4, RT_, G_); AKV_MID(A_, 8, RT_, G_)
+#define AKV_MID_ALONG(RT_, G_) AKV_MID_ROWS(2, RT_, G_); AKV_MID_ROWS(3, RT_, G_); AKV_MID_ROWS(4, RT_, G_)
+  AKV_MID_ALONG(2, 2);
+  if constexpr (!GATED) {
+    AKV_MID_ALONG(1, 2);
+    AKV_MID_ALONG(1, 4);
+  }
+#undef AKV_MID_ALONG
+#undef AKV_MID_ROWS
+#undef AKV_MID
+  return -2;
+}
+
+}  // namespace
+
+// What akv_linear_mid needs beside its operands for this product: floats of `partial` and unsigned integers of
+// `counters` (both 0 where k is not cut over blocks).  `counters` must be zero before the first launch that uses it;
+// every launch leaves it zero again.  Launches that may run at the same time must not share the two.
+extern "C" int akv_linear_mid_workspace(int rows, int n_tiles, int k_tiles, int gated, int along, int rt, int depth,
+                                        int parts, long* partial_floats, long* counters) {
+  const MidPlan p = plan_mid(rows, n_tiles, k_tiles, gated != 0, along, rt, depth, parts);
+  *partial_floats = static_cast<long>(p.partial_floats);
+  *counters = static_cast<long>(p.counters);
+  return 0;
+}
+
+// x [rows, k] bfloat16 row-major, 1 <= rows; wp the packed weight; y [rows, outs] (gated: [rows, inter], wp as for
+// akv_linear_packed_swiglu).  `along` (waves along a band: 2..4), `rt` (row tiles per wave, 1 or 2), `depth` (register
+// sets of the weight ring: 2, or 4 with rt = 1) and `parts` (blocks along k, a power of two) may be 0: chosen here.
+extern "C" int akv_linear_mid(const void* x, const void* wp, void* y, int y_dtype, float* partial, unsigned* counters,
+                              int rows, int outs, int k, int n_tiles, int k_tiles, int gated, int along, int rt,
+                              int depth, int parts, hipStream_t stream) {
+  if (rows <= 0 || outs <= 0) return 0;
+  if ((k & 7) != 0 || k_tiles * 32 < k) return -2;
+  if (gated ? ((outs & 15) != 0 || n_tiles * 8 != outs) : n_tiles * 16 < outs) return -2;
+  if (along < 0 || along == 1 || along > 4 || rt < 0 || rt > 2 || depth < 0 || parts < 0 || (parts & (parts - 1)) != 0) return -2;
+  const MidPlan p = plan_mid(rows, n_tiles, k_tiles, gated != 0, along, rt, depth, parts);
+  if (p.along == 0) return -2;
+  if (p.parts > 1 && (partial == nullptr || counters == nullptr)) return -2;
+  if (gated) {
+    if (y_dtype == kF32) return dispatch_mid<true, float>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, stream);
+    if (y_dtype == kBF16) return dispatch_mid<true, bf16_t>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, stream);
+    return -1;
+  }
+  if (y_dtype == kF32) return dispatch_mid<false, float>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, stream);
+  if (y_dtype == kBF16) return dispatch_mid<false, bf16_t>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, stream);
+  return -1;
+}

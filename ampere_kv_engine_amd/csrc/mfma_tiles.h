@@ -1,0 +1,53 @@
+// Pieces shared by the bfloat16 matrix-product kernels: operand vector types, the 16 x 16 x 32 matrix-core
+// instruction, the load of bytes that are used once, and the store of a 16 x 16 result tile.
+#pragma once
+
+#include "common.h"
+
+namespace akv {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float floatx4;
+typedef __attribute__((ext_vector_type(4))) unsigned int uintx4;  // 16 bytes of operand: 8 bfloat16 (a plain vector
+                                                                 // type: the compiler keeps it in registers)
+
+__device__ __forceinline__ floatx4 mfma16(uintx4 a, uintx4 b, floatx4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// A 16-byte read of data that is used once: it does not displace what others re-read from the caches.
+__device__ __forceinline__ uintx4 load_once(const uintx4* p) { return __builtin_nontemporal_load(p); }
+
+template <typename TY> __device__ __forceinline__ void store4(TY* p, floatx4 v);
+template <> __device__ __forceinline__ void store4<float>(float* p, floatx4 v) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, floatx4 v) {
+  uint2 packed;
+  packed.x = bf16_bits(v[0]) | (static_cast<uint32_t>(bf16_bits(v[1])) << 16);
+  packed.y = bf16_bits(v[2]) | (static_cast<uint32_t>(bf16_bits(v[3])) << 16);
+  *reinterpret_cast<uint2*>(p) = packed;
+}
+
+// Lane (r = l % 16, g = l / 16) owns outputs [feature0 + g * 4 + i][token r] of a 16 x 16 tile.
+template <typename TY>
+__device__ __forceinline__ void store_tile(TY* y, floatx4 acc, int token, int feature, int rows, int outs) {
+  if (token >= rows) return;
+  TY* dst = y + static_cast<size_t>(token) * outs + feature;
+  if (feature + 3 < outs && (outs & 3) == 0) {
+    store4<TY>(dst, acc);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (feature + i < outs) dst[i] = from_float<TY>(acc[i]);
+  }
+}
+
+__device__ __forceinline__ floatx4 silu_times(floatx4 gate, floatx4 up) {
+  floatx4 v;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v[i] = gate[i] / (1.f + expf(-gate[i])) * up[i];
+  return v;
+}
+
+}  // namespace akv

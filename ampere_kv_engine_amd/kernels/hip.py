@@ -83,15 +83,18 @@ class HipKernels:
                  product_choices: dict | None = None):
         """`library_products_above`: bfloat16 products of more rows than this go to the BLAS library (torch.mm),
         which then needs the matrices row-major beside their packing; None keeps the packing alone and every
-        product in this library's own kernels.  `product_choices`: exceptions to that rule for products of up to 64
-        rows, `{(kind, outs, k, tiles of 16 rows): "own" | "library"}` - a table that was measured once
-        (`measure_products`) or loaded from a file.  Nothing is ever timed or decided inside a step, so two runs
-        with the same table send every product the same way and give the same bits."""
+        product in this library's own kernels.  `product_choices`: which kernel takes a product of 17..512 rows,
+        `{(kind, outs, k, row bucket): "own" | "mid" | "library"}` - a table that was measured once
+        (`measure_products`) or loaded from a file; a fixed rule decides what the table does not name.  Nothing is
+        ever timed or decided inside a step, so two runs with the same table send every product the same way and
+        give the same bits."""
         self.library_products_above = library_products_above
         self.product_choices: dict = dict(product_choices or {})
         self._products: dict = {}              # (kind, outs, k) -> a prepared weight of that shape, for measure_products
         self._spacer = None                    # the buffer whose reads precede every timed run
         self._packed_rows = None               # where activations are repacked for the engine's own product
+        self._mid_partial = None               # the mid-size product's partial sums, where it cuts k over blocks
+        self._mid_counters = None              # and its arrival counters (zero between launches)
         self.device = torch.device(device)
         if self.device.type == "cuda" and self.device.index is None:
             self.device = torch.device("cuda", 0)
@@ -121,7 +124,7 @@ class HipKernels:
         for name in ("akv_embed", "akv_add_rmsnorm", "akv_rmsnorm_rows", "akv_copy_rows", "akv_gather_rows",
                      "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
                      "akv_linear_tiled", "akv_linear_packed", "akv_linear_packed_swiglu", "akv_linear_packed_normed",
-                     "akv_pack_rows", "akv_linear_packed_static",
+                     "akv_pack_rows", "akv_linear_packed_static", "akv_linear_mid", "akv_linear_mid_workspace",
                      "akv_attention_rows", "akv_decode_plan", "akv_sample"):
             getattr(self.lib, name).restype = ctypes.c_int
 
@@ -234,10 +237,6 @@ class HipKernels:
             return weight
         return matrix
 
-    def _library_product(self, rows: int, row_major, out) -> bool:
-        return (row_major is not None and self.library_products_above is not None
-                and rows > self.library_products_above and out.dtype == torch.bfloat16)
-
     PACK_ROWS_ABOVE = 16            # the engine's own product of more rows than this reads repacked activations
     PACKED_ROWS_ELEMENTS = 64 * 65536
 
@@ -253,41 +252,89 @@ class HipKernels:
         self._check(self.lib.akv_pack_rows(_ptr(x), _ptr(self._packed_rows), rows, k, self._stream()), "pack_rows")
         return self._packed_rows, 1
 
-    def _own_or_library(self, key: tuple, rows: int, own, library) -> None:
-        """A product that may go to the library: it does, unless it has at most 64 rows (the range of the skinny
-        kernel) and the table of choices names the engine's own kernel for this matrix shape and number of row
-        tiles.  The table is fixed before the first step; a step being recorded reads the same table."""
-        if rows <= self.OWN_SKINNY_ROWS and self.product_choices.get((*key, (rows + 15) // 16)) == "own":
-            own()
-        else:
-            library()
+    MID_ROWS = 512                  # the most rows the mid-size product takes
 
-    def measure_products(self, row_tiles=(2, 3, 4), log=None) -> dict:
-        """For every matrix shape prepared so far and 32, 48 and 64 rows: the engine's own product against the
-        library's, each timed twice on the device; the faster one enters `product_choices`.  Before every timed run
-        reads of 256 MB empty the caches, as the other layers' weights do in a real step, and keep the device busy
-        while the host queues the run, so that the host's launch time is not part of what is measured.  Meant to be
-        called once after loading (`EngineConfig.product_choices = "measure"`); returns the table, which
-        `save_product_choices` writes for later runs.  Every decision is reported through `log` (default: the
-        logger "ampere_kv_engine_amd.kernels")."""
+    @staticmethod
+    def _row_bucket(rows: int):
+        """Products of 17..512 rows are told apart by what the kernels make of the rows: tiles of 16 up to 64 rows
+        (2, 3, 4), then blocks of 128 rows (8: up to 128; 16: up to 256; 32: up to 512)."""
+        if rows <= 64:
+            return (rows + 15) // 16
+        return 8 if rows <= 128 else 16 if rows <= 256 else 32 if rows <= 512 else None
+
+    def _route(self, kind: str, outs: int, k: int, rows: int, has_row_major: bool, out_dtype) -> str:
+        """Which kernel takes a bfloat16 product of more than 16 rows: "own" (the skinny kernel up to 64 rows, the
+        wide one above), "mid" (17..512 rows: the block's waves share the activations through LDS) or "library".
+        The table of choices decides where it names the product; otherwise a fixed rule, from measurements at
+        Qwen3-8B shapes: the library where there is one, except for the gated product up to 64 rows and products
+        with a long k (k >= 2 outs) up to 128 rows, which the mid-size kernel streams a fifth to two fifths faster;
+        without the library, the skinny kernel up to 64 rows, the mid-size one up to 512, the wide one beyond."""
+        library = (has_row_major and self.library_products_above is not None and rows > self.library_products_above
+                   and out_dtype == torch.bfloat16)
+        bucket = self._row_bucket(rows)
+        if bucket is None:
+            return "library" if library else "own"
+        choice = self.product_choices.get((kind, outs, k, bucket))
+        if choice == "library" and not library:
+            choice = None
+        if choice is not None:
+            return choice
+        if not library:
+            return "own" if rows <= self.OWN_SKINNY_ROWS else "mid"
+        if kind == "gated":
+            return "mid" if rows <= 64 else "library"
+        return "mid" if (k >= 2 * outs and rows <= 128) else "library"
+
+    def _mid(self, x, packed: PackedWeight, out, rows: int, outs: int, gated: bool) -> None:
+        """The mid-size product (`csrc/gemm_mid.hip`).  Where it cuts k over blocks it needs room for partial sums
+        and a few counters; both belong to this kernel set and serve one launch at a time (one stream)."""
+        partial_floats, counters = ctypes.c_long(0), ctypes.c_long(0)
+        self.lib.akv_linear_mid_workspace(rows, packed.n_tiles, packed.k_tiles, 1 if gated else 0, 0, 0, 0, 0,
+                                          ctypes.byref(partial_floats), ctypes.byref(counters))
+        if partial_floats.value:
+            if self._mid_partial is None or self._mid_partial.numel() < partial_floats.value:
+                if torch.cuda.is_current_stream_capturing():
+                    raise KernelError("a recorded step needs more room for partial sums than the steps before it")
+                self._mid_partial = torch.empty(max(partial_floats.value, 8 << 20), dtype=torch.float32, device=self.device)
+            if self._mid_counters is None or self._mid_counters.numel() < counters.value:
+                if torch.cuda.is_current_stream_capturing():
+                    raise KernelError("a recorded step needs more counters than the steps before it")
+                self._mid_counters = torch.zeros(max(counters.value, 4096), dtype=torch.int32, device=self.device)
+        self._check(self.lib.akv_linear_mid(_ptr(x), _ptr(packed.data), _ptr(out), _code(out), _ptr(self._mid_partial),
+                                            _ptr(self._mid_counters), rows, outs, packed.k, packed.n_tiles,
+                                            packed.k_tiles, 1 if gated else 0, 0, 0, 0, 0, self._stream()),
+                    "mid-size product")
+
+    MEASURED_ROWS = (32, 48, 64, 128, 256, 512)
+
+    def measure_products(self, rows_measured=MEASURED_ROWS, log=None) -> dict:
+        """For every matrix shape prepared so far and a row count of every bucket from 17 to 512 rows: the kernels
+        that can take the product ("own" up to 64 rows, "mid", "library" where there is one), each timed twice on the
+        device; the fastest enters `product_choices`.  Before every timed run reads of 256 MB empty the caches, as the
+        other layers' weights do in a real step, and keep the device busy while the host queues the run, so that
+        the host's launch time is not part of what is measured.  Meant to be called once after loading
+        (`EngineConfig.product_choices = "measure"`); returns the table, which `save_product_choices` writes for
+        later runs.  Every decision is reported through `log` (default: the logger "ampere_kv_engine_amd.kernels")."""
         import logging
         report = log or logging.getLogger("ampere_kv_engine_amd.kernels").info
-        if self.library_products_above is None:
-            return self.product_choices
         if self._spacer is None:
             self._spacer = torch.zeros(64 << 20, dtype=torch.float32, device=self.device)
         for (kind, outs, k), weight in sorted(self._products.items(), key=lambda item: item[0]):
-            for tiles in row_tiles:
-                rows = 16 * tiles
-                if rows <= self.library_products_above or rows > self.OWN_SKINNY_ROWS:
+            for rows in rows_measured:
+                bucket = self._row_bucket(rows)
+                if rows <= 16 or bucket is None:
                     continue
                 x = torch.randn(rows, k, device=self.device).to(torch.bfloat16)
                 out = torch.empty(rows, outs, dtype=torch.bfloat16, device=self.device)
+                row_major = weight.stacked if kind == "gated" else weight.row_major
+                candidates = (["own"] if rows <= self.OWN_SKINNY_ROWS else []) + ["mid"]
+                if row_major is not None and self.library_products_above is not None and rows > self.library_products_above:
+                    candidates.append("library")
                 scratch = torch.empty(rows, 2 * outs, dtype=torch.bfloat16, device=self.device) if kind == "gated" else None
                 run = (lambda: self.gated_linear(x, weight, out, scratch)) if kind == "gated" else (lambda: self.linear(x, weight, out))
                 best = {}
-                for choice in ("own", "library"):
-                    self.product_choices[kind, outs, k, tiles] = choice
+                for choice in candidates:
+                    self.product_choices[kind, outs, k, bucket] = choice
                     run()                                            # (the first call may load code)
                     samples = []
                     for _ in range(2):
@@ -300,10 +347,10 @@ class HipKernels:
                         samples.append((start, end))
                     torch.cuda.synchronize(self.device)
                     best[choice] = min(a.elapsed_time(b) for a, b in samples)
-                choice = "own" if best["own"] <= best["library"] else "library"
-                self.product_choices[kind, outs, k, tiles] = choice
-                report(f"product {kind} {outs}x{k}, {rows} rows: own {best['own'] * 1000:.1f} us, library "
-                       f"{best['library'] * 1000:.1f} us -> {choice}")
+                choice = min(best, key=best.get)
+                self.product_choices[kind, outs, k, bucket] = choice
+                report(f"product {kind} {outs}x{k}, {rows} rows: "
+                       + ", ".join(f"{name} {time * 1000:.1f} us" for name, time in best.items()) + f" -> {choice}")
         return self.product_choices
 
     def save_product_choices(self, path: str) -> None:
@@ -314,7 +361,7 @@ class HipKernels:
 
     @staticmethod
     def load_product_choices(path: str) -> dict:
-        """The table `save_product_choices` wrote: {"linear:6144x4096:2": "own", ...} -> {(kind, outs, k, tiles): choice}."""
+        """The table `save_product_choices` wrote: {"linear:6144x4096:2": "own", ...} -> {(kind, outs, k, bucket): choice}."""
         import json
         with open(path) as handle:
             raw = json.load(handle)
@@ -322,8 +369,8 @@ class HipKernels:
         for name, choice in raw.items():
             kind, shape, tiles = name.split(":")
             outs, k = shape.split("x")
-            if choice not in ("own", "library"):
-                raise ValueError(f"{path}: the choice for {name} is {choice!r}, not 'own' or 'library'")
+            if choice not in ("own", "mid", "library"):
+                raise ValueError(f"{path}: the choice for {name} is {choice!r}, not 'own', 'mid' or 'library'")
             table[kind, int(outs), int(k), int(tiles)] = choice
         return table
 
@@ -333,17 +380,17 @@ class HipKernels:
             self._dense(x, "x", torch.bfloat16, (rows, weight.k))
             self._dense(out, "out", None, (rows, weight.outs))
             self._dense(weight.data, "packed weight", torch.bfloat16)
-
-            def own():
+            route = "own" if rows <= 16 else self._route("linear", weight.outs, weight.k, rows,
+                                                         weight.row_major is not None, out.dtype)
+            if route == "library":
+                torch.mm(x, weight.row_major.t(), out=out)
+            elif route == "mid":
+                self._mid(x, weight, out, rows, weight.outs, False)
+            else:
                 operand, packed_rows = self._operand_rows(x, rows, weight.k)
                 self._check(self.lib.akv_linear_packed(_ptr(operand), _ptr(weight.data), _ptr(out), _code(out), rows,
                                                        weight.outs, weight.k, weight.n_tiles, weight.k_tiles,
                                                        packed_rows, self._stream()), "linear")
-            if self._library_product(rows, weight.row_major, out):
-                self._own_or_library(("linear", weight.outs, weight.k), rows, own,
-                                     lambda: torch.mm(x, weight.row_major.t(), out=out))
-            else:
-                own()
             return
         rows, k = x.shape
         outs = weight.shape[0]
@@ -425,40 +472,34 @@ class HipKernels:
     def gated_scratch(self, weight: GatedWeight, rows: int, dtype: torch.dtype):
         """Shape of the buffer `gated_linear` wants for this many rows (the stacked product of the library path),
         or None."""
-        wanted = (weight.stacked is not None and self.library_products_above is not None
-                  and rows > self.library_products_above and dtype == torch.bfloat16)
+        wanted = (rows > 16 and dtype == torch.bfloat16
+                  and self._route("gated", weight.inter, weight.k, rows, weight.stacked is not None, dtype) == "library")
         return (rows, 2 * weight.inter) if wanted else None
 
     def gated_linear(self, x, weight: GatedWeight, out, scratch=None):
-        """out [rows, inter] = silu(x Wgate^T) * (x Wup^T): one kernel, from float32 accumulators; with many rows the
-        library's stacked product into `scratch`, then the activation kernel."""
+        """out [rows, inter] = silu(x Wgate^T) * (x Wup^T): one kernel, from float32 accumulators; where the library
+        takes the product, its stacked product into `scratch`, then the activation kernel."""
         rows = x.shape[0]
         packed = weight.packed
         self._dense(x, "x", torch.bfloat16, (rows, weight.k))
         self._dense(out, "out", None, (rows, weight.inter))
         self._dense(packed.data, "packed weight", torch.bfloat16)
-        if self._library_product(rows, weight.stacked, out):
+        route = "own" if rows <= 16 else self._route("gated", weight.inter, weight.k, rows, weight.stacked is not None,
+                                                     out.dtype)
+        if route == "library":
             if scratch is None:
-                raise KernelError(f"gated_linear of {rows} rows may take the library path and needs the scratch "
+                raise KernelError(f"gated_linear of {rows} rows takes the library path and needs the scratch "
                                   "buffer that gated_scratch() describes")
             self._dense(scratch, "scratch", torch.bfloat16, (rows, 2 * weight.inter))
-
-            def own():
-                operand, packed_rows = self._operand_rows(x, rows, weight.k)
-                self._check(self.lib.akv_linear_packed_swiglu(_ptr(operand), _ptr(packed.data), _ptr(out), _code(out),
-                                                              rows, weight.inter, weight.k, packed.n_tiles,
-                                                              packed.k_tiles, packed_rows, self._stream()),
-                            "gated_linear")
-
-            def library():
-                torch.mm(x, weight.stacked.t(), out=scratch)
-                self.swiglu(scratch, out)
-            self._own_or_library(("gated", weight.inter, weight.k), rows, own, library)
-            return
-        operand, packed_rows = self._operand_rows(x, rows, weight.k)
-        self._check(self.lib.akv_linear_packed_swiglu(_ptr(operand), _ptr(packed.data), _ptr(out), _code(out), rows,
-                                                      weight.inter, weight.k, packed.n_tiles, packed.k_tiles,
-                                                      packed_rows, self._stream()), "gated_linear")
+            torch.mm(x, weight.stacked.t(), out=scratch)
+            self.swiglu(scratch, out)
+        elif route == "mid":
+            self._mid(x, packed, out, rows, weight.inter, True)
+        else:
+            operand, packed_rows = self._operand_rows(x, rows, weight.k)
+            self._check(self.lib.akv_linear_packed_swiglu(_ptr(operand), _ptr(packed.data), _ptr(out), _code(out), rows,
+                                                          weight.inter, weight.k, packed.n_tiles, packed.k_tiles,
+                                                          packed_rows, self._stream()), "gated_linear")
 
     def swiglu(self, gate_up, out):
         tokens, inter = out.shape

@@ -31,9 +31,15 @@ def hip_own():
 
 @pytest.fixture(scope="module")
 def hip_library():
-    """Every bfloat16 product of more than 16 rows in the BLAS library (the rule without a table of exceptions)."""
+    """Every bfloat16 product of more than 16 rows in the BLAS library (a table of choices that names it for all)."""
     from ampere_kv_engine_amd.kernels.hip import HipKernels
-    return HipKernels("cuda:0")
+
+    class Always(dict):
+        def get(self, key, default=None):
+            return "library"
+    kernels = HipKernels("cuda:0")
+    kernels.product_choices = Always()
+    return kernels
 
 
 @pytest.fixture(params=["own", "library"])
@@ -192,7 +198,8 @@ def test_gated_linear(hip_either, ref, y_dtype, rows, inter, k):
     ref.gated_linear(x, (gate, up), want)
     got = torch.full((rows, inter), float("nan"), dtype=y_dtype, device="cuda")
     shape = hip.gated_scratch(weight, rows, y_dtype)
-    assert (shape is not None) == (hip.library_products_above is not None and rows > 16 and y_dtype == torch.bfloat16)
+    library = hip.library_products_above is not None and rows > 16 and y_dtype == torch.bfloat16
+    assert (shape is not None) == (library and hip._route("gated", inter, k, rows, True, y_dtype) == "library")
     hip.gated_linear(x.cuda(), weight, got, torch.empty(shape, dtype=y_dtype, device="cuda") if shape else None)
     t = dict(rtol=2e-4, atol=2e-5 * k ** 0.5) if y_dtype == torch.float32 else tol(torch.bfloat16)
     torch.testing.assert_close(got.cpu().float(), want.float(), **t)
@@ -265,11 +272,11 @@ def test_gated_linear_after_norm(hip, ref, rows):
     torch.testing.assert_close(new.cpu(), want_stream, rtol=0, atol=0)
 
 
-def test_products_of_17_to_64_rows_follow_a_table_that_is_measured_on_request(hip, ref, tmp_path):
-    """Between 17 and 64 rows a product goes to the library unless the table of choices names the engine's own kernel
-    for its matrix shape and number of row tiles.  Nothing is timed by a product call; `measure_products` fills the
-    table for the shapes prepared so far and reports every decision; the table can be saved and loaded; either choice
-    gives the product."""
+def test_products_of_17_to_512_rows_follow_a_table_that_is_measured_on_request(hip, ref, tmp_path):
+    """Which kernel takes a product of 17..512 rows - the skinny one (up to 64), the mid-size one, the library - is
+    decided by a fixed rule unless the table of choices names the product (matrix shape and row bucket).  Nothing is
+    timed by a product call; `measure_products` fills the table for the shapes prepared so far and reports every
+    decision; the table can be saved and loaded; every choice gives the product."""
     from ampere_kv_engine_amd.kernels.hip import HipKernels
     kernels = HipKernels("cuda:0")
     w = rand(320, 256, dtype=torch.bfloat16, seed=41, scale=0.05)
@@ -278,27 +285,98 @@ def test_products_of_17_to_64_rows_follow_a_table_that_is_measured_on_request(hi
     gated = kernels.prepare_gated_linear(gate.cuda(), up.cuda())
 
     def products():
-        for rows in (8, 20, 31, 64, 65):
+        for rows in (8, 20, 31, 64, 65, 130, 300, 600):
             x = rand(rows, 256, dtype=torch.bfloat16, seed=42)
             want = torch.empty(rows, 320, dtype=torch.bfloat16)
             ref.linear(x, w, want)
-            got = torch.empty(rows, 320, dtype=torch.bfloat16, device="cuda")
+            got = torch.full((rows, 320), float("nan"), dtype=torch.bfloat16, device="cuda")
             kernels.linear(x.cuda(), packed, got)
+            torch.testing.assert_close(got.cpu().float(), want.float(), **tol(torch.bfloat16))
+            want = torch.empty(rows, 64, dtype=torch.bfloat16)
+            ref.gated_linear(x, ref.prepare_gated_linear(gate, up), want)
+            got = torch.full((rows, 64), float("nan"), dtype=torch.bfloat16, device="cuda")
+            shape = kernels.gated_scratch(gated, rows, torch.bfloat16)
+            scratch = torch.empty(shape, dtype=torch.bfloat16, device="cuda") if shape is not None else None
+            kernels.gated_linear(x.cuda(), gated, got, scratch)
             torch.testing.assert_close(got.cpu().float(), want.float(), **tol(torch.bfloat16))
     products()
     assert kernels.product_choices == {}                       # calls decide nothing
     lines = []
     table = kernels.measure_products(log=lines.append)
-    assert set(table) == {(kind, outs, 256, tiles) for kind, outs in (("linear", 320), ("gated", 64)) for tiles in (2, 3, 4)}
-    assert set(table.values()) <= {"own", "library"} and len(lines) == 6 and all("->" in line for line in lines)
+    assert set(table) == {(kind, outs, 256, bucket) for kind, outs in (("linear", 320), ("gated", 64))
+                          for bucket in (2, 3, 4, 8, 16, 32)}
+    assert set(table.values()) <= {"own", "mid", "library"} and len(lines) == 12 and all("->" in line for line in lines)
     products()
-    for forced in ("own", "library"):
+    for forced in ("own", "mid", "library"):
         kernels.product_choices = {key: forced for key in table}
         products()
     path = str(tmp_path / "choices.json")
     kernels.save_product_choices(path)
     assert HipKernels.load_product_choices(path) == kernels.product_choices
     assert HipKernels("cuda:0", product_choices=HipKernels.load_product_choices(path)).product_choices == kernels.product_choices
+
+
+MID_CASES = [  # rows, outs, k: every row-tile count, several blocks of rows, ragged k and outs, long and short k
+    (17, 100, 72), (20, 304, 520), (33, 48, 2048), (50, 4096, 4096), (64, 320, 256), (100, 4096, 4096),
+    (128, 520, 1032), (300, 1000, 2048), (512, 1536, 512), (48, 640, 12288), (5, 64, 32),
+]
+
+
+@pytest.mark.parametrize("rows,outs,k", MID_CASES)
+def test_mid_size_product(hip_own, ref, rows, outs, k):
+    """`akv_linear_mid` alone, with every cut it can be told to make (waves along a band, row tiles per wave, depth of
+    the weight ring, blocks along k) and the cut it chooses itself, into bfloat16 and float32; twice each, since a
+    launch that cuts k over blocks must leave its counters at zero for the next."""
+    import ctypes
+    from ampere_kv_engine_amd.kernels.hip import _ptr
+    lib = hip_own.lib
+    w = rand(outs, k, dtype=torch.bfloat16, seed=81, scale=0.05)
+    x = rand(rows, k, dtype=torch.bfloat16, seed=82)
+    packed = hip_own.prepare_linear(w.cuda())
+    want = x.float() @ w.float().T
+    partial = torch.empty(8 << 20, dtype=torch.float32, device="cuda")
+    counters = torch.zeros(4096, dtype=torch.int32, device="cuda")
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    xd = x.cuda()
+    for along, rt, depth, parts in ((0, 0, 0, 0), (2, 1, 2, 1), (3, 2, 2, 2), (4, 1, 4, 4), (4, 2, 2, 8), (3, 1, 4, 1)):
+        for code, dtype in ((1, torch.bfloat16), (0, torch.float32)):
+            for _ in range(2):
+                got = torch.full((rows, outs), float("nan"), dtype=dtype, device="cuda")
+                status = lib.akv_linear_mid(_ptr(xd), _ptr(packed.data), _ptr(got), code, _ptr(partial), _ptr(counters), rows,
+                                            outs, k, packed.n_tiles, packed.k_tiles, 0, along, rt, depth, parts, stream)
+                assert status == 0, (along, rt, depth, parts, status)
+                limits = tol(dtype) if dtype == torch.bfloat16 else dict(rtol=2e-5, atol=2e-5 * float(want.abs().max()))
+                torch.testing.assert_close(got.cpu().float(), want if dtype == torch.float32 else want.bfloat16().float(), **limits,
+                                           msg=lambda m: f"along {along} rt {rt} depth {depth} parts {parts} {dtype}: {m}")
+            assert int(counters.abs().sum()) == 0
+    # what is cut over blocks is added in the order of the parts, whoever comes last: two launches agree bit for bit
+    first = torch.empty((rows, outs), dtype=torch.float32, device="cuda")
+    again = torch.empty((rows, outs), dtype=torch.float32, device="cuda")
+    for target in (first, again):
+        assert lib.akv_linear_mid(_ptr(xd), _ptr(packed.data), _ptr(target), 0, _ptr(partial), _ptr(counters), rows, outs, k,
+                                  packed.n_tiles, packed.k_tiles, 0, 4, 1, 4, 4, stream) == 0
+    assert torch.equal(first, again)
+
+
+@pytest.mark.parametrize("rows,inter,k", [(40, 208, 264), (64, 512, 2048), (130, 208, 520), (17, 16, 8), (256, 1024, 1024)])
+def test_mid_size_gated_product(hip_own, ref, rows, inter, k):
+    import ctypes
+    from ampere_kv_engine_amd.kernels.hip import _ptr
+    lib = hip_own.lib
+    gate, up = (rand(inter, k, dtype=torch.bfloat16, seed=91 + i, scale=0.05) for i in range(2))
+    x = rand(rows, k, dtype=torch.bfloat16, seed=93)
+    weight = hip_own.prepare_gated_linear(gate.cuda(), up.cuda())
+    want = torch.empty(rows, inter, dtype=torch.bfloat16)
+    ref.gated_linear(x, ref.prepare_gated_linear(gate, up), want)
+    partial = torch.empty(8 << 20, dtype=torch.float32, device="cuda")
+    counters = torch.zeros(4096, dtype=torch.int32, device="cuda")
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for along, parts in ((0, 0), (2, 1), (3, 2), (4, 4)):
+        got = torch.full((rows, inter), float("nan"), dtype=torch.bfloat16, device="cuda")
+        assert lib.akv_linear_mid(_ptr(x.cuda()), _ptr(weight.packed.data), _ptr(got), 1, _ptr(partial), _ptr(counters), rows,
+                                  inter, k, weight.packed.n_tiles, weight.packed.k_tiles, 1, along, 2, 2, parts, stream) == 0
+        torch.testing.assert_close(got.cpu().float(), want.float(), **tol(torch.bfloat16))
+    assert int(counters.abs().sum()) == 0
 
 
 def test_linear_keeps_other_weights_row_major(hip):
