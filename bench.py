@@ -15,10 +15,13 @@ not change the time a step takes).  One JSON line is printed:
             own kernels (by default bfloat16 products of more than 16 rows go to the BLAS library)
 Peaks are MI355X's published ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s.
 
-Two further workloads run through the scheduler and print a line of their own (`--workload`):
-  serving-14b   Qwen3-14B layer sizes: 32 requests, prompt lengths uniform in [128, 4096], 256 tokens each,
-                prompts fed in portions of at most 2,048 tokens beside the decoding requests
-  batch-32b     Qwen3-32B layer sizes: 16 requests with 8,192-token prompts, 128 greedy tokens each
+Further workloads run through the scheduler and print a line of their own (`--workload`):
+  serving-14b      Qwen3-14B layer sizes: 32 requests, prompt lengths uniform in [128, 4096], 256 tokens each,
+                   prompts fed in portions of at most 2,048 tokens beside the decoding requests
+  batch-32b        Qwen3-32B layer sizes: 16 requests with 8,192-token prompts, 128 greedy tokens each
+  offline-512-32   the reference's offline batch (docs/BENCHMARK.md:9-24 there) at Qwen3-8B layer sizes: B = 1 and
+                   B = 4 requests of 512 input tokens, 32 greedy output tokens each, end-of-sequence ignored; one
+                   warm-up, five samples from submission to the last token on the host
 """
 
 from __future__ import annotations
@@ -32,11 +35,11 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-# BASELINE.json configs[2]: Qwen3-8B layer sizes, page size 16, context 8,192, prefill of 2,048 tokens
+# Qwen3-8B layer sizes; the measurement's page size 16, context 8,192, prefill of 2,048 tokens
 QWEN3_8B = dict(architectures=["Qwen3ForCausalLM"], num_hidden_layers=36, hidden_size=4096, num_attention_heads=32,
                 num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=151936, rope_theta=1000000.0,
                 rms_norm_eps=1e-6, tie_word_embeddings=False, hidden_act="silu")
-# BASELINE.json configs[3] and configs[4]: the layer sizes of the two larger dense models
+# the layer sizes of the two larger dense models (Qwen3-14B, Qwen3-32B)
 QWEN3_14B = dict(QWEN3_8B, num_hidden_layers=40, hidden_size=5120, num_attention_heads=40, intermediate_size=17408)
 QWEN3_32B = dict(QWEN3_8B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, intermediate_size=25600)
 PAGE_SIZE, CONTEXT, PREFILL_TOKENS = 16, 8192, 2048
@@ -92,6 +95,54 @@ def scheduler_workload(name: str, layers: int | None, library_above: int | None)
     return 0
 
 
+def spread(values, digits: int = 3) -> dict:
+    """Raw samples, their median and their range."""
+    ordered = sorted(values)
+    middle = ordered[len(ordered) // 2] if len(ordered) % 2 else (ordered[len(ordered) // 2 - 1] + ordered[len(ordered) // 2]) / 2
+    return {"samples": [round(v, digits) for v in values], "median": round(middle, digits),
+            "range": round(ordered[-1] - ordered[0], digits)}
+
+
+def offline_workload(layers: int | None) -> int:
+    """B requests of 512 input tokens, 32 greedy output tokens each, submitted together; a sample runs from the
+    submission to the moment the last token is on the host.  One warm-up, five samples, for B = 1 and B = 4."""
+    import torch
+    from ampere_kv_engine_amd.config import EngineConfig, Qwen3Config
+    from ampere_kv_engine_amd.engine import Engine
+    from ampere_kv_engine_amd.engine.scheduler import Scheduler
+
+    raw = dict(QWEN3_8B, num_hidden_layers=layers or QWEN3_8B["num_hidden_layers"])
+    config = Qwen3Config.from_dict(raw)
+    prompt_tokens, new_tokens, most = 512, 32, 4
+    pages = most * ((prompt_tokens + new_tokens + 2 * PAGE_SIZE) // PAGE_SIZE) + 8
+    engine = Engine.from_random(config, seed=0, engine_config=EngineConfig(
+        dtype="bfloat16", page_size=PAGE_SIZE, num_pages=pages, max_seqs=most, max_batched_tokens=most * prompt_tokens,
+        max_seq_len=prompt_tokens + new_tokens + PAGE_SIZE, device="cuda:0"))
+    generator = torch.Generator().manual_seed(0)
+    record = {"workload": "offline-512-32", "input_tokens": prompt_tokens, "output_tokens": new_tokens,
+              "layers": raw["num_hidden_layers"], "dtype": "bf16", "samples_per_batch": 5,
+              "data": "synthetic: random-init weights, uniform random token ids"}
+    for batch in (1, 4):
+        ids = [torch.randint(0, config.vocab_size, (prompt_tokens,), generator=generator).tolist() for _ in range(batch)]
+        samples = []
+        for run in range(6):                                    # the first run warms up (graphs are recorded in it)
+            scheduler = Scheduler(engine)
+            torch.cuda.synchronize(engine.device)
+            started = time.perf_counter()
+            requests = [scheduler.submit(f"{batch}_{run}_{i}", tokens, max_new_tokens=new_tokens, ignore_eos=True)
+                        for i, tokens in enumerate(ids)]
+            scheduler.run_until_idle()
+            elapsed = (time.perf_counter() - started) * 1e3
+            if run:
+                samples.append(elapsed)
+            assert all(len(r.output_ids) == new_tokens for r in requests)
+            assert engine.cache.num_free_pages == [pages]
+        record[f"b{batch}"] = {"completion_ms": spread(samples),
+                               "output_tok_per_s": round(batch * new_tokens / (spread(samples)["median"] / 1e3), 2)}
+    print(json.dumps(record))
+    return 0
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -106,7 +157,7 @@ def main() -> int:
                         "'32768,512x63' (overrides --batch and --context; no further points, no prefill)")
     parser.add_argument("--no-prefill", action="store_true")
     parser.add_argument("--prefill-only", action="store_true", help="time the prefill alone (for kernel profiles)")
-    parser.add_argument("--workload", choices=["decode", "serving-14b", "batch-32b"], default="decode",
+    parser.add_argument("--workload", choices=["decode", "serving-14b", "batch-32b", "offline-512-32"], default="decode",
                         help="decode: the headline measurement; the others run a set of requests through the scheduler")
     parser.add_argument("--library-above", type=int, default=16,
                         help="bfloat16 products of more rows than this go to the BLAS library; -1: none does")
@@ -116,6 +167,8 @@ def main() -> int:
         print("bench.py measures one GPU: this engine has no multi-GPU path, run it with --gpus 1")
         return 2
 
+    if args.workload == "offline-512-32":
+        return offline_workload(args.layers if args.layers != QWEN3_8B["num_hidden_layers"] else None)
     if args.workload != "decode":
         return scheduler_workload(args.workload, args.layers if args.layers != QWEN3_8B["num_hidden_layers"] else None,
                                   library_above)
@@ -152,8 +205,9 @@ def main() -> int:
     generator = torch.Generator().manual_seed(0)
     sync = lambda: torch.cuda.synchronize(engine.device)
 
-    def decode(batch: int, steps: int, warmup: int) -> float:
-        """Seconds for `steps` decode steps of `batch` requests whose caches hold `context` tokens."""
+    def decode(batch: int, steps: int, warmup: int) -> tuple[float, list[float]]:
+        """Seconds for `steps` decode steps of `batch` requests whose caches hold `context` tokens, and the moments
+        (seconds since the start) at which each step's tokens were on the host."""
         seqs = [engine.open(f"b{batch}_{i}") for i in range(batch)]
         for index, seq in enumerate(seqs):
             engine.cache.reserve(seq, (contexts[index] if contexts is not None else args.context) - 1)
@@ -169,17 +223,26 @@ def main() -> int:
             one_step()
         sync()
         started = time.perf_counter()
+        moments = []
         for _ in range(steps):
-            one_step()
+            one_step()                       # (returns with the chosen tokens on the host: the step is over)
+            moments.append(time.perf_counter() - started)
         sync()
         elapsed = time.perf_counter() - started
         for seq in seqs:
             engine.close(seq)
         assert engine.cache.num_free_pages == [pages]
-        return elapsed
+        return elapsed, moments
 
-    def prefill(repeats: int = 3) -> float:
-        """Median seconds to feed one 2,048-token prompt whole and choose its first token."""
+    def fifths(moments: list[float]) -> dict:
+        """The timed steps as five consecutive samples: milliseconds per step of each fifth."""
+        edges = [round(i * len(moments) / 5) for i in range(6)]
+        samples = [(moments[b - 1] - (moments[a - 1] if a else 0.0)) / (b - a) * 1e3
+                   for a, b in zip(edges, edges[1:]) if b > a]
+        return spread(samples, 4)
+
+    def prefill(repeats: int = 5) -> tuple[float, list[float]]:
+        """Median seconds to feed one 2,048-token prompt whole and choose its first token, and all samples."""
         prompt = torch.randint(0, config.vocab_size, (PREFILL_TOKENS,), generator=generator).tolist()
         samples = []
         for run in range(repeats + 1):
@@ -192,14 +255,14 @@ def main() -> int:
             if run:                          # the first run warms up
                 samples.append(time.perf_counter() - started)
             engine.close(seq)
-        return sorted(samples)[len(samples) // 2]
+        return sorted(samples)[len(samples) // 2], samples
 
     if args.prefill_only:
-        seconds = prefill()
+        seconds, _ = prefill()
         print(json.dumps({"prefill_ms": round(seconds * 1000, 3), "tokens": PREFILL_TOKENS,
                           "tok_per_s": round(PREFILL_TOKENS / seconds, 1), "layers": args.layers}))
         return 0
-    elapsed = decode(args.batch, args.steps, args.warmup)
+    elapsed, moments = decode(args.batch, args.steps, args.warmup)
     ms_per_step = elapsed / args.steps * 1000
     value = args.batch * args.steps / elapsed
     weight_bytes = engine.model.weight_bytes_per_step()
@@ -209,7 +272,7 @@ def main() -> int:
     record = {
         "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2,048 tokens (Qwen3-8B bf16)",
         "value": round(value, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms_per_step, 4), "samples": fifths(moments), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic: random-init weights N(0, 0.02), uniform random token ids, random cache",
         "config": {"model": "Qwen3-8B layer sizes", "global_batch": args.batch, "seq_len": args.context,
                    "parallelism": "single GPU", "layers": args.layers, "layers_of_config": QWEN3_8B["num_hidden_layers"],
@@ -227,20 +290,21 @@ def main() -> int:
         record["points"] = {}
         for batch in points:
             steps = max(8, args.steps // 2) if batch > args.batch else args.steps
-            seconds = decode(batch, steps, max(2, args.warmup // 2))
+            seconds, _ = decode(batch, steps, max(2, args.warmup // 2))
             record["points"][f"decode_b{batch}"] = round(batch * steps / seconds, 2)
     if not args.no_prefill:
-        seconds = prefill()
+        seconds, prefill_samples = prefill()
         layer_params = sum(engine.model.blocks[e.layer].mixer.weight_bytes() + engine.model.blocks[e.layer].feed_forward.weight_bytes()
                            for e in engine.spec.run_order) / 2
         flops = 2 * PREFILL_TOKENS * layer_params                              # the layers' matrix products
         flops += 2 * PREFILL_TOKENS * PREFILL_TOKENS * config.q_size * args.layers   # causal attention (QK^T and PV halves)
         flops += 2 * config.vocab_size * config.hidden_size                     # the head on the one wanted row
         record["prefill"] = {"value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS,
-                             "ms": round(seconds * 1000, 3), "frac": round(flops / seconds / BF16_PEAK_FLOPS, 4)}
+                             "ms": round(seconds * 1000, 3), "frac": round(flops / seconds / BF16_PEAK_FLOPS, 4),
+                             "samples_ms": [round(x * 1000, 3) for x in prefill_samples]}
         if points and engine.kernels.library_products_above is not None:
             kept, engine.kernels.library_products_above = engine.kernels.library_products_above, None
-            record["points"]["prefill_own_products"] = round(PREFILL_TOKENS / prefill(), 1)
+            record["points"]["prefill_own_products"] = round(PREFILL_TOKENS / prefill(3)[0], 1)
             engine.kernels.library_products_above = kept
     print(json.dumps(record))
     return 0

@@ -42,6 +42,25 @@ def test_the_line_of_a_short_run():
     assert prefill["tokens"] == 2048 and prefill["ms"] > 0 and 0 < prefill["frac"] < 1
     assert abs(prefill["value"] - 2048 / (prefill["ms"] / 1e3)) < 1e-2 * prefill["value"]
     assert line["points"]["decode_b1"] > 0
+    # raw samples beside median and range: the timed steps as consecutive fifths, the prefill's five runs
+    samples = line["samples"]
+    assert 1 <= len(samples["samples"]) <= 5 and samples["range"] >= 0 and min(samples["samples"]) <= samples["median"] <= max(samples["samples"])
+    assert len(prefill["samples_ms"]) == 5 and min(prefill["samples_ms"]) <= prefill["ms"] <= max(prefill["samples_ms"])
+
+
+@pytest.mark.gpu
+def test_the_offline_batch_of_the_reference():
+    """`--workload offline-512-32`: B = 1 and B = 4 requests of 512 tokens in, 32 out; five samples each with median,
+    range and output tokens per second."""
+    result = subprocess.run([sys.executable, BENCH, "--workload", "offline-512-32", "--layers", "2"], capture_output=True,
+                            text=True, timeout=600, cwd=ROOT)
+    assert result.returncode == 0, result.stderr[-2000:]
+    line = json.loads(result.stdout.strip().splitlines()[-1])
+    assert line["workload"] == "offline-512-32" and line["input_tokens"] == 512 and line["output_tokens"] == 32
+    for batch in (1, 4):
+        entry = line[f"b{batch}"]
+        assert len(entry["completion_ms"]["samples"]) == 5 and entry["completion_ms"]["median"] > 0
+        assert abs(entry["output_tok_per_s"] - batch * 32 / (entry["completion_ms"]["median"] / 1e3)) < 0.01 * entry["output_tok_per_s"]
 
 
 @pytest.mark.gpu
