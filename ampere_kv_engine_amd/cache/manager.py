@@ -22,7 +22,7 @@ import torch
 
 from ..parts.base import PagedKV, SlotState
 from .pages import BlockTable, PageAllocator, PagePoolExhausted
-from .slots import SlotTable
+from .slots import SlotArrays, SlotTable
 
 
 @dataclass
@@ -60,9 +60,11 @@ class Sequence:
 class CacheManager:
     def __init__(self, needs: dict[int, PagedKV | SlotState | None], *, page_size: int, num_pages: int,
                  max_seqs: int, dtype: torch.dtype = torch.bfloat16, device: str | torch.device = "cpu",
-                 allocate_tensors: bool = True):
-        """`needs[cache_layer]` is what that layer's mixer asked for."""
+                 allocate_tensors: bool = True, max_pages_per_seq: int | None = None):
+        """`needs[cache_layer]` is what that layer's mixer asked for.  `max_pages_per_seq` is the width of the block
+        tables kept on the device (default: the whole pool)."""
         self.page_size, self.num_pages, self.max_seqs = page_size, num_pages, max_seqs
+        self.max_pages_per_seq = max_pages_per_seq if max_pages_per_seq is not None else num_pages
         self.dtype, self.device = dtype, device
         self.slots = SlotTable(max_seqs)
         self.groups: list[PagedGroup] = []
@@ -98,6 +100,9 @@ class CacheManager:
                     self._state_tensors.append((state, need))
             elif need is None:
                 self.layer_cache[layer] = LayerCache()
+        # what every request keeps on the device between steps: its slot's words and its rows of the block tables
+        self.arrays = (SlotArrays(max_seqs, len(self.groups), self.max_pages_per_seq, device)
+                       if allocate_tensors else None)
 
     # ---- sizes --------------------------------------------------------------------------------------
     def pages_for(self, num_tokens: int, group: PagedGroup | None = None, chunk: int | None = None) -> int:
@@ -122,10 +127,15 @@ class CacheManager:
         return [g.allocator.num_free for g in self.groups]
 
     # ---- a request's life ---------------------------------------------------------------------------
-    def open(self, request_id: str) -> Sequence:
+    def open(self, request_id: str, temperature: float = 0.0, seed: int = 0) -> Sequence:
+        """A new request takes a slot.  `temperature` and `seed` are what the sampler will find in the slot."""
         if request_id in self._live:
             raise ValueError(f"request {request_id!r} already holds a sequence")
+        if temperature < 0 or not 0 <= seed < 2 ** 63:
+            raise ValueError("temperature must not be negative and the seed must fit in 63 bits")
         slot = self.slots.take()
+        if self.arrays is not None:
+            self.arrays.take(slot, temperature, seed)
         for state, need in self._state_tensors:     # a reused slot starts as a fresh one
             if need.init is not None:
                 need.init(state[slot])
@@ -165,6 +175,8 @@ class CacheManager:
         for table in seq.tables:
             table.release()
         self.slots.give_back(seq.slot)
+        if self.arrays is not None:
+            self.arrays.give_back(seq.slot)
         seq.closed = True
         self._live.pop(seq.request_id, None)
 

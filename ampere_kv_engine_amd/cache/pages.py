@@ -58,6 +58,13 @@ class BlockTable:
         self._mirror = np.empty(16, dtype=np.int32)   # the same ids as an array, for the step's metadata
         self._length = 0
         self._first_live = 0      # logical index of the first page not yet given back
+        self._changed: list[int] = []   # entries that changed since `take_changes` (what a device copy must be told)
+
+    def take_changes(self) -> list[tuple[int, int]]:
+        """(index, page id or RELEASED) of every entry that was appended or given back since the last call."""
+        changes = [(index, int(self._mirror[index])) for index in self._changed]
+        self._changed.clear()
+        return changes
 
     @property
     def length(self) -> int:
@@ -104,6 +111,7 @@ class BlockTable:
             self._allocator.free(self._pages[index])
             self._pages[index] = RELEASED
             self._mirror[index] = RELEASED
+            self._changed.append(index)
         self._first_live += passed
         if required > len(self._mirror):
             grown = np.empty(max(required, 2 * len(self._mirror)), dtype=np.int32)
@@ -112,6 +120,7 @@ class BlockTable:
         for _ in range(additional):
             page = self._allocator.allocate()
             self._mirror[len(self._pages)] = page
+            self._changed.append(len(self._pages))
             self._pages.append(page)
         self._length = start + num_tokens
         return start
@@ -132,5 +141,6 @@ class BlockTable:
         for page in self._pages[self._first_live:]:
             self._allocator.free(page)
         self._pages.clear()
+        self._changed.clear()
         self._length = 0
         self._first_live = 0

@@ -8,7 +8,9 @@
 extern "C" {
 
 int akv_embed(const int* ids, const void* table, int table_dtype, float* out, int tokens, int hidden, int vocab,
-              hipStream_t stream);
+              const int* seq_of_token, const int* seq_slots, const int* slot_words, hipStream_t stream);
+int akv_step_prologue(int* state, long state_size, const int* patches, const int* count, int capacity,
+                      const int* seq_slots, const int* seq_lens, int seqs, hipStream_t stream);
 int akv_add_rmsnorm(float* stream_buf, const void* delta, const float* weight, float eps, void* out, int dtype,
                     int tokens, int hidden, hipStream_t stream);
 int akv_rmsnorm_rows(const void* x, long token_stride, const float* weight, float eps, void* out, int dtype,
@@ -52,11 +54,14 @@ int akv_linear_mid(const void* x, const void* wp, void* y, int y_dtype, float* p
                    int outs, int k, int n_tiles, int k_tiles, int gated, int along, int rt, int depth, int parts,
                    hipStream_t stream);
 int akv_attention_rows(const void* q, const void* k_pages, const void* v_pages, const int* seq_of_token,
-                       const int* positions, const int* block_table, int table_width, void* out, int dtype,
+                       const int* positions, const int* block_table, const int* table_rows, int table_width, void* out,
+                       int dtype,
                        long tokens, int q_heads, int kv_heads, int dim, int page_size, long num_pages, float scale,
                        int window, hipStream_t stream);
 int akv_decode_plan(const int* seq_lens, int seq_first, int seq_count, int window, int items_wanted, int min_segment,
                     int items_grid, int* plan, hipStream_t stream);
 int akv_sample(const float* logits, const float* temperature, const unsigned long long* seeds,
                const unsigned int* draws, int* out, int rows, int vocab, hipStream_t stream);
+int akv_sample_slots(const float* logits, const int* rows_of, const int* seq_of_token, const int* seq_slots,
+                     int* slot_words, int* out, int rows, int vocab, hipStream_t stream);
 }

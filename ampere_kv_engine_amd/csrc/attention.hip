@@ -26,7 +26,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void attention_rows_kernel(
     const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int* __restrict__ seq_of_token, const int* __restrict__ positions, const int* __restrict__ block_table,
-    int table_width, T* __restrict__ out, long tokens, int q_heads, int kv_heads, int dim, int page_size,
+    const int* __restrict__ table_rows, int table_width, T* __restrict__ out, long tokens, int q_heads, int kv_heads, int dim, int page_size,
     long num_pages, float scale, int window) {
   extern __shared__ unsigned char lds_raw[];
   const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
@@ -41,7 +41,7 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(
   const long n = row / q_heads;
   const int h = static_cast<int>(row % q_heads);
   const int kvh = h / (q_heads / kv_heads);
-  const int r = seq_of_token[n];
+  const int r = table_rows != nullptr ? table_rows[seq_of_token[n]] : seq_of_token[n];   // the table's row of the request
   const int pos = positions[n];
   const int lowest = window > 0 ? max(0, pos - window + 1) : 0;
   for (int i = lane; i < dim; i += kWave) qs[i] = to_float(q[row * dim + i]);
@@ -156,7 +156,8 @@ extern "C" int akv_decode_plan(const int* seq_lens, int seq_first, int seq_count
 }
 
 extern "C" int akv_attention_rows(const void* q, const void* k_pages, const void* v_pages, const int* seq_of_token,
-                                  const int* positions, const int* block_table, int table_width, void* out, int dtype,
+                                  const int* positions, const int* block_table, const int* table_rows, int table_width,
+                                  void* out, int dtype,
                                   long tokens, int q_heads, int kv_heads, int dim, int page_size, long num_pages,
                                   float scale, int window, hipStream_t stream) {
   if (tokens <= 0) return 0;
@@ -166,7 +167,8 @@ extern "C" int akv_attention_rows(const void* q, const void* k_pages, const void
   AKV_DISPATCH(dtype, T,
                attention_rows_kernel<T><<<static_cast<unsigned>((rows + 3) / 4), 256, lds, stream>>>(
                    static_cast<const T*>(q), static_cast<const T*>(k_pages), static_cast<const T*>(v_pages),
-                   seq_of_token, positions, block_table, table_width, static_cast<T*>(out), tokens, q_heads, kv_heads,
+                   seq_of_token, positions, block_table, table_rows, table_width, static_cast<T*>(out), tokens, q_heads,
+                   kv_heads,
                    dim, page_size, num_pages, scale, window));
   return AKV_LAUNCH_STATUS();
 }

@@ -68,7 +68,8 @@ struct Args {
   float* partial;             // SPLIT: [tile][grid.y][split][16 * NQ][PSTRIDE]
   const int* q_start;         // [requests + 1] first token row of each request
   const int* seq_lens;        // [requests] tokens held after this step
-  const int* block_table;     // [requests, table_width]
+  const int* block_table;     // [requests, table_width], or, with `table_rows`, [slots, table_width]
+  const int* table_rows;      // null, or [requests]: the row of the table that holds a request's pages (its slot)
   int table_width;
   int seq_first, seq_count;   // the launch covers requests seq_first .. seq_first + seq_count - 1
   int tiles;                  // tiles over those requests
@@ -339,7 +340,7 @@ __global__ __launch_bounds__(64, (SPLIT && NQ == 1 && D <= 128) ? 2 : 1) void at
     for (int dt = 0; dt < DT; ++dt) o[nq][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
   bool poisoned = false;  // a key inside the range lies in a page that is not the request's
-  const int* table = a.block_table + static_cast<long>(t.request) * a.table_width;
+  const int* table = a.block_table + static_cast<long>(a.table_rows != nullptr ? a.table_rows[t.request] : t.request) * a.table_width;
   const int key_in_step = (r16 >> 2) * 8 + (r16 & 3);  // + j * 4: this lane's key row of tile j
 
   // A page's byte offset is 64-bit (pools of many gigabytes); what is added inside a page fits 32 bits and is
@@ -733,7 +734,7 @@ __global__ __launch_bounds__(64 * kSharedWaves, D <= 128 ? (NQ == 1 ? 3 : 2) : 1
   }
 
   // ---- the block's loads: pieces of 16 bytes, piece p * 256 + tid ------------------------------------------------------
-  const int* table = a.block_table + static_cast<long>(t.request) * a.table_width;
+  const int* table = a.block_table + static_cast<long>(a.table_rows != nullptr ? a.table_rows[t.request] : t.request) * a.table_width;
   const char* k_bytes = reinterpret_cast<const char*>(a.k_pages);
   const char* v_bytes = reinterpret_cast<const char*>(a.v_pages);
   const uint32_t page_bytes = static_cast<uint32_t>(a.kv_heads) * D * 2u << page_shift;
@@ -1222,6 +1223,8 @@ int launch(const Args& a, int tiles, bool shared, hipStream_t stream) {
 // 16 * nq query columns; `tiles` is the number of tiles over those requests (sum of ceil(tokens / tokens_per_tile));
 // with num_splits > 1 `partial` must hold tiles * kv_heads * head_groups * num_splits * 16 * nq * (D + 4) floats.
 // page_size must be a power of two, at least 4.  `single_tokens` says that every request brings exactly one token.
+// `table_rows` (may be null): request r's pages are row table_rows[r] of `block_table` instead of row r - the table
+// then is the engine's persistent one, a row per request slot.
 // `shared`: blocks of four waves that share keys and values through LDS; `tiles` then counts tiles of
 // 4 * tokens_per_tile tokens, num_splits must be 1 and pages hold at least 8 tokens.
 // `plan` (not null: single tokens, at most 64 requests): seg_keys and num_splits are not used; the requests' keys were
@@ -1233,7 +1236,8 @@ int launch(const Args& a, int tiles, bool shared, hipStream_t stream) {
 // itself and writes the new keys and values to the tokens' slots, which the block tables must already name.
 extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
     const void* q, const void* k_pages, const void* v_pages, void* out, float* partial, const int* q_start,
-    const int* seq_lens, const int* block_table, int table_width, int seq_first, int seq_count, int tiles, int nq,
+    const int* seq_lens, const int* block_table, const int* table_rows, int table_width, int seq_first, int seq_count,
+    int tiles, int nq,
     int q_heads, int kv_heads, int heads_per_tile, int head_groups, int tokens_per_tile, int page_size, long num_pages,
     float scale, int window, int seg_keys, int num_splits, int single_tokens, int shared, const void* qkv,
     const float* q_weight, const float* k_weight, float eps, const float* rope_table, int table_positions,
@@ -1256,6 +1260,7 @@ extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
   a.q_start = q_start;
   a.seq_lens = seq_lens;
   a.block_table = block_table;
+  a.table_rows = table_rows;
   a.table_width = table_width;
   a.seq_first = seq_first;
   a.seq_count = seq_count;

@@ -9,12 +9,37 @@ using namespace akv;
 
 namespace {
 
+// ---- per-request state of fixed size: SLOT_WORDS 32-bit words per slot -----------------------------------------
+// word 0 tokens held, 1 the token chosen last (-1: none yet), 2 temperature (float bits), 3 and 4 the seed's low
+// and high half, 5 draws made so far, 6 whether a request holds the slot.
+constexpr int kSlotWords = 8;
+constexpr int kSlotLength = 0, kSlotLastToken = 1;
+
+// What a step changes in the persistent integer state before its first kernel reads it: `count` (offset, value) pairs
+// - block-table entries of pages the step's requests were given or gave back - and the requests' new lengths.
+__global__ void step_prologue_kernel(int* __restrict__ state, long state_size, const int* __restrict__ patches,
+                                     const int* __restrict__ count, int capacity, const int* __restrict__ seq_slots,
+                                     const int* __restrict__ seq_lens, int seqs) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < capacity && i < count[0]) {
+    const long at = patches[2 * i];
+    if (at >= 0 && at < state_size) state[at] = patches[2 * i + 1];   // (never write outside the state)
+  }
+  if (i < seqs) {
+    const long at = static_cast<long>(seq_slots[i]) * kSlotWords + kSlotLength;
+    if (at >= 0 && at < state_size) state[at] = seq_lens[i];
+  }
+}
+
 // ---- embedding: out[n, :] = table[ids[n], :] widened to float32 (no scaling) ------------------------------
+// An id of -1 stands for the token that was chosen last for the row's request (kept in its slot by the sampler).
 template <typename T>
 __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out,
-                             int hidden, int vocab) {
+                             int hidden, int vocab, const int* __restrict__ seq_of_token,
+                             const int* __restrict__ seq_slots, const int* __restrict__ slot_words) {
   const int n = blockIdx.x;
-  const int id = ids[n];
+  int id = ids[n];
+  if (id == -1 && slot_words != nullptr) id = slot_words[seq_slots[seq_of_token[n]] * kSlotWords + kSlotLastToken];
   float* dst = out + static_cast<size_t>(n) * hidden;
   if (id < 0 || id >= vocab) {  // never read outside the table; a poisoned row shows the fault downstream
     for (int d = threadIdx.x; d < hidden; d += blockDim.x) dst[d] = __uint_as_float(0x7fc00000u);
@@ -445,11 +470,28 @@ inline unsigned blocks_for(long items, int per_block) { return static_cast<unsig
 
 extern "C" {
 
+// `seq_of_token`, `seq_slots`, `slot_words` (all three or none): where an id of -1 finds the token chosen last for its
+// request.  Without them -1 is an id outside the table like any other.
 int akv_embed(const int* ids, const void* table, int table_dtype, float* out, int tokens, int hidden, int vocab,
-              hipStream_t stream) {
+              const int* seq_of_token, const int* seq_slots, const int* slot_words, hipStream_t stream) {
   if (tokens <= 0) return 0;
+  if (slot_words != nullptr && (seq_of_token == nullptr || seq_slots == nullptr)) return -2;
   AKV_DISPATCH(table_dtype, T,
-               embed_kernel<T><<<tokens, 256, 0, stream>>>(ids, static_cast<const T*>(table), out, hidden, vocab));
+               embed_kernel<T><<<tokens, 256, 0, stream>>>(ids, static_cast<const T*>(table), out, hidden, vocab,
+                                                           seq_of_token, seq_slots, slot_words));
+  return AKV_LAUNCH_STATUS();
+}
+
+// state[patches[2 i]] = patches[2 i + 1] for i < min(count[0], capacity), and the slots' lengths:
+// state[seq_slots[r] * 8] = seq_lens[r] for r < seqs.  `count` lives on the device, so a recorded step applies
+// however many changes the replayed step brings, up to the capacity it was recorded with.
+int akv_step_prologue(int* state, long state_size, const int* patches, const int* count, int capacity,
+                      const int* seq_slots, const int* seq_lens, int seqs, hipStream_t stream) {
+  const int threads = capacity > seqs ? capacity : seqs;
+  if (threads <= 0) return 0;
+  if (state_size <= 0 || capacity < 0 || seqs < 0) return -2;
+  step_prologue_kernel<<<(threads + 255) / 256, 256, 0, stream>>>(state, state_size, patches, count, capacity, seq_slots,
+                                                                  seq_lens, seqs);
   return AKV_LAUNCH_STATUS();
 }
 

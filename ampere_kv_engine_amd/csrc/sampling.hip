@@ -31,11 +31,19 @@ __device__ __forceinline__ uint32_t philox_first(uint32_t c0, uint32_t c1, uint3
   return c0;
 }
 
+// SLOTS: the sampling state is not handed in row by row but read from (and written to) the slot of the row's request:
+// the row's token row is rows_of[row], its request seq_of_token[...], its slot seq_slots[...]; slot words 2..5 hold
+// temperature, seed and draws made so far, word 1 receives the chosen token and word 5 counts the draw.
+constexpr int kSlotWords = 8;
+
+template <bool SLOTS>
 __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ logits,
                                                       const float* __restrict__ temperature,
                                                       const unsigned long long* __restrict__ seeds,
                                                       const unsigned int* __restrict__ draws, int* __restrict__ out,
-                                                      int vocab) {
+                                                      int vocab, const int* __restrict__ rows_of,
+                                                      const int* __restrict__ seq_of_token,
+                                                      const int* __restrict__ seq_slots, int* __restrict__ slot_words) {
   __shared__ float best_value[16];
   __shared__ int best_index[16];
   __shared__ int any_nan;
@@ -44,10 +52,22 @@ __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ 
   bool saw_nan = false;
   const int row = blockIdx.x;
   const float* x = logits + static_cast<size_t>(row) * vocab;
-  const float t = temperature != nullptr ? temperature[row] : 0.f;
-  const uint32_t k0 = t > 0.f ? static_cast<uint32_t>(seeds[row]) : 0u;
-  const uint32_t k1 = t > 0.f ? static_cast<uint32_t>(seeds[row] >> 32) : 0u;
-  const uint32_t draw = t > 0.f ? draws[row] : 0u;
+  float t;
+  uint32_t k0, k1, draw;
+  int* words = nullptr;
+  if constexpr (SLOTS) {
+    words = slot_words + static_cast<size_t>(seq_slots[seq_of_token[rows_of[row]]]) * kSlotWords;
+    t = __int_as_float(words[2]);
+    k0 = static_cast<uint32_t>(words[3]);
+    k1 = static_cast<uint32_t>(words[4]);
+    draw = static_cast<uint32_t>(words[5]);
+    __syncthreads();   // every thread has read the state before thread 0 writes it below
+  } else {
+    t = temperature != nullptr ? temperature[row] : 0.f;
+    k0 = t > 0.f ? static_cast<uint32_t>(seeds[row]) : 0u;
+    k1 = t > 0.f ? static_cast<uint32_t>(seeds[row] >> 32) : 0u;
+    draw = t > 0.f ? draws[row] : 0u;
+  }
   float value = -INFINITY;
   int index = vocab;  // "none yet"; any real index is lower
   // eight loads of a thread are on their way before the first is looked at; ids still ascend per thread, so the
@@ -85,7 +105,12 @@ __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ 
   if (threadIdx.x == 0) {
     for (int w = 1; w < blockDim.x / kWave; ++w)
       if (best_value[w] > value || (best_value[w] == value && best_index[w] < index)) { value = best_value[w]; index = best_index[w]; }
-    out[row] = (index < vocab && any_nan == 0) ? index : -1;
+    const int token = (index < vocab && any_nan == 0) ? index : -1;
+    out[row] = token;
+    if constexpr (SLOTS) {
+      words[1] = token;
+      words[5] = static_cast<int>(draw + 1u);
+    }
   }
 }
 
@@ -94,6 +119,18 @@ __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ 
 extern "C" int akv_sample(const float* logits, const float* temperature, const unsigned long long* seeds,
                           const unsigned int* draws, int* out, int rows, int vocab, hipStream_t stream) {
   if (rows <= 0) return 0;
-  sample_kernel<<<rows, 1024, 0, stream>>>(logits, temperature, seeds, draws, out, vocab);
+  sample_kernel<false><<<rows, 1024, 0, stream>>>(logits, temperature, seeds, draws, out, vocab, nullptr, nullptr, nullptr,
+                                                  nullptr);
+  return AKV_LAUNCH_STATUS();
+}
+
+// The same choice with every row's temperature, seed and draw count read from the slot of its request, where the
+// chosen token and the new draw count are left too.  rows_of [rows]: the step's token row that logits row i belongs
+// to.  No two rows may belong to one request (they would share a draw count).
+extern "C" int akv_sample_slots(const float* logits, const int* rows_of, const int* seq_of_token, const int* seq_slots,
+                                int* slot_words, int* out, int rows, int vocab, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  sample_kernel<true><<<rows, 1024, 0, stream>>>(logits, nullptr, nullptr, nullptr, out, vocab, rows_of, seq_of_token,
+                                                 seq_slots, slot_words);
   return AKV_LAUNCH_STATUS();
 }

@@ -3,7 +3,10 @@ flattened to `tokens` rows, plus everything kernels need to find each token's re
 
 The reference builds three different inputs for its three forward functions and uploads block tables once
 per layer (ampere_kv/runner.py:205-215, :227-229; ampere_kv/scheduler.py:133-139).  Here one batch layout
-serves every step and all of its integer metadata reaches the device in one copy.
+serves every step and all of its integer metadata reaches the device in one copy.  Block tables are not part of it:
+they live on the device, a row per request slot, and a step brings only the entries that changed - the pages its
+requests were handed or gave back - as (offset, value) pairs that a small kernel applies before anything reads them.
+A decode step of 64 requests with 32,768 tokens each thus uploads some hundreds of integers instead of 130,000.
 """
 
 from __future__ import annotations
@@ -15,6 +18,10 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, Sequence
+
+
+LAST_TOKEN = (-1,)      # as a `StepEntry`'s tokens: the one token that was chosen last for the request (the sampler
+                        # left it in the request's slot on the device; the host need not send it back)
 
 
 @dataclass
@@ -29,10 +36,12 @@ class StepEntry:
 @dataclass
 class PagedMeta:
     """Per cache group: where each new token's key/value goes and where each request's pages are."""
-    block_table: torch.Tensor     # int32 [seqs, width]; RELEASED (-1) or stale entries are never read
+    block_table: torch.Tensor     # int32 [slots, width]: the group's persistent table; RELEASED (-1) or stale entries
+                                  # are never read
     slot_map: torch.Tensor        # int32 [tokens]: page * page_size + offset of the token's own slot
-    width: int
+    width: int                    # entries of a table row
     window: int | None
+    rows: torch.Tensor | None = None   # int32 [seqs]: the table row of each request of the step (its slot); None: row r
 
 
 class Arena:
@@ -107,6 +116,13 @@ class StepContext:
     spare_buffer: torch.Tensor | None = None    # float32 [a few rows, hidden]: where a small step may move it
     stream: torch.Tensor | None = None          # the step's residual sum, wherever it is now
     spare_stream: torch.Tensor | None = None    # the other buffer's rows, or None where the step has too many
+    # the device's persistent integer state (slot words, block tables) and what this step changes in it
+    table_pages: int = 0                        # bound on the pages of the step's longest request (sizes launches)
+    patches: torch.Tensor | None = None         # int32 [2 * patch_room]: (offset into slot_state, value) pairs
+    patch_count: torch.Tensor | None = None     # int32 [1]: how many of them this step brings
+    patch_room: int = 0
+    slot_state: torch.Tensor | None = None      # int32: the whole state
+    slot_words: torch.Tensor | None = None      # int32 [slots, SLOT_WORDS]: its first part
 
 
 class BatchBuilder:
@@ -118,8 +134,11 @@ class BatchBuilder:
         self.device = torch.device(device)
         self.max_tokens, self.max_seqs, self.max_width = max_batched_tokens, max_seqs, max_pages_per_seq
         groups = len(cache.groups)
+        if cache.arrays is not None:        # a request cannot outgrow its row of the device's block table
+            self.max_width = min(self.max_width, cache.arrays.table_width)
+        most_patches = groups * 2 * (self.max_tokens // cache.page_size + 2 * self.max_seqs)
         capacity = (3 * self.max_tokens + 3 * self.max_seqs + 1 + self.max_tokens
-                    + groups * (self.max_tokens + self.max_seqs * self.max_width))
+                    + groups * self.max_tokens + 1 + 2 * most_patches)
         pin = self.device.type == "cuda"
         # Two pinned staging buffers in turn: the copy of one step may still be in flight while the host
         # lays out the next, so a buffer is written again only after the copy that read it has finished.
@@ -129,10 +148,17 @@ class BatchBuilder:
         self._device = torch.empty(capacity, dtype=torch.int32, device=self.device)
         self.arenas = (Arena(self.device), Arena(self.device))
 
+    def patch_capacity(self, counts) -> int:
+        """The most block-table entries a step can change whose requests bring `counts` tokens: per request and group
+        the pages its tokens may open, and as many that a window may close."""
+        page = self.cache.page_size
+        return len(self.cache.groups) * sum(2 * ((count + page - 1) // page + 1) for count in counts)
+
     def build(self, entries: list[StepEntry], width_multiple: int = 1) -> tuple[StepContext, list[int]]:
         """Returns the context and, for every entry in the caller's order, the offset of its first wanted
-        row in the logits the step returns.  The block tables' width is rounded up to `width_multiple` pages:
-        steps of equal shape then lay their metadata out at equal addresses (what a recorded graph needs)."""
+        row in the logits the step returns.  `ctx.table_pages` is the longest request's page count rounded up to
+        `width_multiple` pages: a bound that sizes launches and is the same for all steps under it (what a recorded
+        graph needs)."""
         if not entries:
             raise ValueError("a step needs at least one entry")
         if len(entries) > self.max_seqs:
@@ -162,6 +188,8 @@ class BatchBuilder:
         width = max(max((t.num_pages for t in e.seq.tables), default=1) for e in ordered)
         width = max(width, 1)
         width = min((width + width_multiple - 1) // width_multiple * width_multiple, max(self.max_width, width))
+        arrays = self.cache.arrays
+        patch_room = self.patch_capacity(len(e.tokens) for e in ordered)
         self._turn ^= 1
         if self._copied[self._turn] is not None:
             self._copied[self._turn].synchronize()
@@ -187,8 +215,10 @@ class BatchBuilder:
         group_spans = []
         for g in self.cache.groups:
             slot_map, s_sm = region(n)
-            table, s_bt = region(r * width)
-            group_spans.append((slot_map, s_sm, table.reshape(r, width), s_bt))
+            group_spans.append((slot_map, s_sm))
+        patch_count, s_pc = region(1)
+        patches, s_pa = region(2 * patch_room)
+        changed = 0
 
         row = 0
         first_row_of = [0] * len(entries)
@@ -207,10 +237,19 @@ class BatchBuilder:
             seq_lens[index] = start + count
             seq_slots[index] = e.seq.slot
             first_row_of[order[index]] = row
-            for g, (slot_map, _, table, _) in zip(self.cache.groups, group_spans):
-                pages = e.seq.tables[g.index].page_array
-                table[index, :len(pages)] = pages
-                table[index, len(pages):] = -1
+            for g, (slot_map, _) in zip(self.cache.groups, group_spans):
+                table = e.seq.tables[g.index]
+                pages = table.page_array
+                if arrays is not None:      # what this step changed in the request's row of the device's table
+                    changes = table.take_changes()
+                    if len(changes) > 2 * ((count + page_size - 1) // page_size + 1):
+                        # (tokens were registered outside a step: the row goes to the device as a whole)
+                        arrays.write_row(g.index, e.seq.slot, pages)
+                        changes = ()
+                    for entry, page in changes:
+                        patches[2 * changed] = arrays.table_offset(g.index, e.seq.slot, entry)
+                        patches[2 * changed + 1] = page
+                        changed += 1
                 if count == 1:
                     slot_map[row] = int(pages[start // page_size]) * page_size + start % page_size
                 else:
@@ -226,14 +265,17 @@ class BatchBuilder:
                 logit_rows[want_cursor] = first_row + place
                 want_cursor += 1
         q_start[r] = row
+        assert changed <= patch_room, "a step changed more block-table entries than its requests' tokens allow"
+        patch_count[0] = changed
 
         self._device[:cursor].copy_(host_tensor[:cursor], non_blocking=True)
         if self._copied[self._turn] is not None:
             self._copied[self._turn].record()
         dev = lambda span: self._device[span[0]:span[1]]
-        paged = [PagedMeta(block_table=dev(s_bt).view(r, width), slot_map=dev(s_sm), width=width,
-                           window=g.need.window)
-                 for g, (_, s_sm, _, s_bt) in zip(self.cache.groups, group_spans)]
+        paged = [PagedMeta(block_table=arrays.tables[g.index] if arrays is not None else None, slot_map=dev(s_sm),
+                           width=arrays.table_width if arrays is not None else width, window=g.need.window,
+                           rows=dev(s_ss))
+                 for g, (_, s_sm) in zip(self.cache.groups, group_spans)]
         for arena in self.arenas:
             arena.reset()
         ctx = StepContext(
@@ -243,7 +285,9 @@ class BatchBuilder:
             host_q_start=[int(x) for x in q_start[:r + 1]], host_seq_lens=[int(x) for x in seq_lens[:r]],
             host_seq_slots=[int(x) for x in seq_slots[:r]],
             max_seq_len=int(seq_lens[:r].max()), max_new_tokens=max(len(e.tokens) for e in ordered),
-            arenas=self.arenas,
+            arenas=self.arenas, table_pages=width, patches=dev(s_pa), patch_count=dev(s_pc), patch_room=patch_room,
+            slot_state=arrays.state if arrays is not None else None,
+            slot_words=arrays.words if arrays is not None else None,
         )
         return ctx, first_wanted_of
 

@@ -18,7 +18,7 @@ from ..config.specs import ModelSpec
 from ..parts.base import Runtime
 from ..weights.loader import Checkpoint
 from ..weights.random import RandomSource
-from .batch import BatchBuilder, StepEntry
+from .batch import LAST_TOKEN, BatchBuilder, StepEntry  # noqa: F401
 from .model import Model
 
 _TORCH_DTYPE = {"bfloat16": torch.bfloat16, "float32": torch.float32}
@@ -45,7 +45,8 @@ class Engine:
         self.model = Model(spec, self.runtime)
         self.cache = CacheManager(self.model.cache_needs(), page_size=engine_config.page_size,
                                   num_pages=engine_config.num_pages, max_seqs=engine_config.max_seqs,
-                                  dtype=self.dtype, device=self.device)
+                                  dtype=self.dtype, device=self.device,
+                                  max_pages_per_seq=engine_config.max_pages_per_seq)
         self.builder = BatchBuilder(self.cache, self.device, engine_config.max_batched_tokens,
                                     engine_config.max_seqs, engine_config.max_pages_per_seq)
         self.stream_buffer = torch.empty((engine_config.max_batched_tokens, spec.hidden_size),
@@ -55,6 +56,7 @@ class Engine:
         self.spare_buffer = torch.empty((self.SPARE_STREAM_ROWS, spec.hidden_size), dtype=torch.float32,
                                         device=self.device)
         self.loaded = False
+        self._chooser = None
         self._graphs: dict[tuple, object] = {}               # (tokens per request, wanted rows, table width) -> graph
         self._graph_logits = None                            # [max_seqs, vocab] float32, where recorded steps write
         self._recordable = (engine_config.decode_graphs and self.device.type == "cuda" and all(
@@ -93,8 +95,10 @@ class Engine:
             self.kernels.measure_products()
 
     # ---- requests ---------------------------------------------------------------------------------
-    def open(self, request_id: str) -> Sequence:
-        return self.cache.open(request_id)
+    def open(self, request_id: str, temperature: float = 0.0, seed: int = 0) -> Sequence:
+        """A new request: it takes a slot, whose state on the device starts fresh - nothing held, no token chosen, no
+        draw made - with the request's own temperature and seed for `choose`."""
+        return self.cache.open(request_id, temperature, seed)
 
     def close(self, seq: Sequence) -> None:
         self.cache.close(seq)
@@ -118,14 +122,31 @@ class Engine:
                 return logits if borrow_logits else logits.clone()
         ctx, _ = self.builder.build(entries)
         ctx.stream_buffer, ctx.spare_buffer = self.stream_buffer, self.spare_buffer
+        self._last_step = ctx
         return self.model.forward(ctx, self.cache.layer_cache)
+
+    @torch.no_grad()
+    def choose(self, logits: torch.Tensor) -> list[int]:
+        """The next token for every wanted row of the step just run (`logits` is what that step returned): greedy or
+        drawn, by the temperature, seed and draw count that the row's request keeps in its slot on the device.  The
+        kernel leaves the chosen token and the new draw count in the slot - `StepEntry(seq, LAST_TOKEN)` feeds that
+        token without the host sending it - and nothing is uploaded for the choice; one copy brings the tokens to
+        the host.  `NO_TOKEN` (-1) for a row that holds a NaN or no finite logit.  At most one wanted row per request."""
+        ctx = getattr(self, "_last_step", None)
+        if ctx is None or logits is None or logits.shape[0] != ctx.logit_rows.shape[0]:
+            raise ValueError("choose() takes the logits of the step that was run last")
+        if self._chooser is None:
+            from ..sampling.sampler import SlotSampler
+            self._chooser = SlotSampler(self.kernels, self.device, self.config.max_seqs)
+        return self._chooser.choose(logits, ctx)
 
     def _check_token_ids(self, entries: list[StepEntry]) -> None:
         """Every token id must name a row of the embedding table; one comparison per entry, not one per token."""
         vocab = self.spec.vocab_size
         for e in entries:
             if len(e.tokens) == 1:
-                bad = not 0 <= int(e.tokens[0]) < vocab
+                # (-1 alone: the token chosen last for the request, which its slot on the device holds)
+                bad = not 0 <= int(e.tokens[0]) < vocab and not (int(e.tokens[0]) == -1 and e.seq.length > 0)
             else:
                 ids = np.asarray(e.tokens)
                 if ids.dtype.kind not in "iu":
@@ -145,7 +166,8 @@ class Engine:
 
     def _recordable_shape(self, entries: list[StepEntry]):
         """(tokens per request in the step's order - single tokens first -, wanted rows), or None for a step that
-        is run as it is: nothing wanted, more wanted rows than the shared logits buffer has, or long portions."""
+        is run as it is: nothing wanted, more wanted rows than the shared logits buffer has, or long portions.  (The
+        numbers of tokens also fix how many block-table changes the step may bring at most.)"""
         counts = tuple(sorted((len(e.tokens) for e in entries), key=lambda count: count != 1))
         wanted = sum(len(e.want) for e in entries)
         if wanted == 0 or wanted > self.config.max_seqs:
@@ -165,7 +187,8 @@ class Engine:
         counts, wanted = shape
         ctx, _ = self.builder.build(entries, width_multiple=self.GRAPH_WIDTH_MULTIPLE)
         ctx.stream_buffer, ctx.spare_buffer = self.stream_buffer, self.spare_buffer
-        width = ctx.paged[0].width if ctx.paged else 0
+        self._last_step = ctx
+        width = ctx.table_pages        # the longest request's pages, rounded up: a bound the recording is made for
         key = (counts, wanted, width)
         # sizes of launches come from the bound, not from this step's lengths
         bound = max(width * self.config.page_size, 1)

@@ -7,8 +7,8 @@ import time
 
 import torch
 
-from ..sampling.sampler import NO_TOKEN, Sampler, SamplingParams
-from .batch import StepEntry
+from ..sampling.sampler import NO_TOKEN, SamplingParams
+from .batch import LAST_TOKEN, StepEntry
 
 MAX_NEW_TOKENS = 32  # the reference's default (ampere_kv/runner.py:17); it counts the token the prefill yields
 
@@ -26,10 +26,7 @@ def generate_tokens(engine, input_ids, *, max_new_tokens: int = MAX_NEW_TOKENS, 
         raise ValueError("the prompt is empty")
     if max_new_tokens <= 0:
         raise ValueError("max_new_tokens must be positive")
-    params = SamplingParams(temperature, seed)
-    sampler = getattr(engine, "_sampler", None)
-    if sampler is None:
-        sampler = engine._sampler = Sampler(engine.kernels, engine.device, engine.config.max_seqs)
+    SamplingParams(temperature, seed)       # (checks the two)
     eos = set() if ignore_eos else set(engine.spec.eos_token_ids)
     limit = engine.config.max_batched_tokens
     chunk = min(prefill_chunk_size or limit, limit)
@@ -37,7 +34,7 @@ def generate_tokens(engine, input_ids, *, max_new_tokens: int = MAX_NEW_TOKENS, 
         if engine.device.type == "cuda":
             torch.cuda.synchronize(engine.device)
         started = time.perf_counter()
-    seq = engine.open(request_id)
+    seq = engine.open(request_id, temperature, seed)
     generated: list[int] = []
     try:
         for start in range(0, len(prompt), chunk):
@@ -45,7 +42,7 @@ def generate_tokens(engine, input_ids, *, max_new_tokens: int = MAX_NEW_TOKENS, 
             last = start + chunk >= len(prompt)
             logits = engine.step([StepEntry(seq, portion, [len(portion) - 1] if last else [])], borrow_logits=True)
         while True:
-            token = sampler.sample(logits, [params], [len(generated)])[0]
+            token = engine.choose(logits)[0]
             if token == NO_TOKEN:
                 raise RuntimeError(f"the step gave request {request_id!r} no finite logit after {len(generated)} tokens")
             if timings is not None:
@@ -55,7 +52,7 @@ def generate_tokens(engine, input_ids, *, max_new_tokens: int = MAX_NEW_TOKENS, 
             generated.append(token)
             if token in eos or len(generated) >= max_new_tokens:
                 break
-            logits = engine.step([StepEntry(seq, [token], [0])], borrow_logits=True)
+            logits = engine.step([StepEntry(seq, LAST_TOKEN, [0])], borrow_logits=True)
         final_length = seq.length
     finally:
         engine.close(seq)

@@ -85,7 +85,9 @@ class Model:
         ctx.stream = ctx.stream_buffer[:ctx.num_tokens]
         spare = getattr(ctx, "spare_buffer", None)
         ctx.spare_stream = spare[:ctx.num_tokens] if spare is not None and ctx.num_tokens <= spare.shape[0] else None
-        self.embedding.forward(ctx.token_ids, ctx.stream)
+        if getattr(ctx, "slot_state", None) is not None:
+            k.step_prologue(ctx)        # block-table changes and new lengths reach the device's persistent state
+        self.embedding.forward(ctx.token_ids, ctx.stream, ctx)
         pending = None
         for step_index, entry in enumerate(self.spec.run_order):
             ctx.arena = arenas[step_index & 1]

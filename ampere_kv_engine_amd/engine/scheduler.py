@@ -21,8 +21,8 @@ from __future__ import annotations
 
 import time
 
-from ..sampling.sampler import NO_TOKEN, Sampler, SamplingParams
-from .batch import StepEntry
+from ..sampling.sampler import NO_TOKEN, SamplingParams
+from .batch import LAST_TOKEN, StepEntry
 
 WAITING, PREFILLING, RUNNING, FINISHED = "waiting", "prefilling", "running", "finished"
 STOP_LIMIT, STOP_EOS, STOP_CANCELLED, STOP_EXPIRED = "reached limit", "EOS", "cancelled", "expired"
@@ -80,7 +80,6 @@ class Scheduler:
         self.prefilling: list[Request] = []
         self.running: list[Request] = []
         self.eos_ids = set(engine.spec.eos_token_ids)
-        self.sampler = Sampler(engine.kernels, engine.device, cfg.max_seqs)
         self.rounds = 0
         self.mixed_rounds = 0           # rounds in which decodes and portions shared one step
         self.last_portions: list[int] = []
@@ -181,7 +180,8 @@ class Scheduler:
     def _run(self, decodes: list[Request], portions: list[tuple[Request, int, bool]]) -> None:
         entries, takers = [], []
         for request in decodes:
-            entries.append(StepEntry(request.seq, [request.output_ids[-1]], [0]))
+            # (the token chosen in the round before lies in the request's slot on the device: it is not sent again)
+            entries.append(StepEntry(request.seq, LAST_TOKEN, [0]))
             takers.append(request)
         for request, count, last in portions:
             start = request.prefilled
@@ -191,7 +191,8 @@ class Scheduler:
         logits = self.engine.step(entries, borrow_logits=True)     # sampled from at once, below
         if not takers:
             return
-        tokens = self.sampler.sample(logits, [r.sampling for r in takers], [len(r.output_ids) for r in takers])
+        # every wanted row belongs to another request; temperature, seed and draw count are read from the slots
+        tokens = self.engine.choose(logits)
         for request, token in zip(takers, tokens):
             self._give(request, token)
 
@@ -221,7 +222,7 @@ class Scheduler:
             self.waiting.pop(0)
             for g, b in enumerate(head.budget_pages):
                 self.reserved_pages[g] += b
-            head.seq = self.engine.open(head.request_id)
+            head.seq = self.engine.open(head.request_id, head.sampling.temperature, head.sampling.seed)
             head.status = PREFILLING
             self.prefilling.append(head)
 

@@ -125,7 +125,7 @@ class HipKernels:
                      "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
                      "akv_linear_tiled", "akv_linear_packed", "akv_linear_packed_swiglu", "akv_linear_packed_normed",
                      "akv_pack_rows", "akv_linear_packed_static", "akv_linear_mid", "akv_linear_mid_workspace",
-                     "akv_attention_rows", "akv_decode_plan", "akv_sample"):
+                     "akv_attention_rows", "akv_decode_plan", "akv_sample", "akv_sample_slots", "akv_step_prologue"):
             getattr(self.lib, name).restype = ctypes.c_int
 
     # ---- helpers -----------------------------------------------------------------------------------------
@@ -166,14 +166,38 @@ class HipKernels:
             raise KernelError(f"page_size {page_size} must be positive")
 
     # ---- token-wise --------------------------------------------------------------------------------------
-    def embed(self, ids, table, out):
+    def embed(self, ids, table, out, ctx=None):
+        """out[n] = table[ids[n]].  With the step's context, an id of -1 stands for the token chosen last for the row's
+        request, which the sampler left in the request's slot."""
         tokens = ids.shape[0]
         self._dense(ids, "ids", torch.int32, (tokens,))
         self._dense(table, "table")
         vocab, hidden = table.shape
         self._dense(out, "out", torch.float32, (tokens, hidden))
+        words = getattr(ctx, "slot_words", None) if ctx is not None else None
+        seq_of_token = seq_slots = None
+        if words is not None:
+            seq_of_token, seq_slots = ctx.seq_of_token, ctx.seq_slots
+            self._dense(words, "slot_words", torch.int32)
+            self._dense(seq_of_token, "seq_of_token", torch.int32, (tokens,))
+            self._dense(seq_slots, "seq_slots", torch.int32, (ctx.num_seqs,))
+            if max(ctx.host_seq_slots) >= words.shape[0]:
+                raise KernelError("a request's slot lies outside the slot words")
         self._check(self.lib.akv_embed(_ptr(ids), _ptr(table), _code(table), _ptr(out), tokens, hidden, vocab,
-                                       self._stream()), "embed")
+                                       _ptr(seq_of_token), _ptr(seq_slots), _ptr(words), self._stream()), "embed")
+
+    def step_prologue(self, ctx) -> None:
+        """Applies what the step changes in the device's persistent integer state before anything reads it: the
+        block-table entries of pages its requests were handed or gave back, and the requests' new lengths."""
+        state = ctx.slot_state
+        self._dense(state, "slot_state", torch.int32)
+        self._dense(ctx.patches, "patches", torch.int32, (2 * ctx.patch_room,))
+        self._dense(ctx.patch_count, "patch_count", torch.int32, (1,))
+        self._dense(ctx.seq_slots, "seq_slots", torch.int32, (ctx.num_seqs,))
+        self._dense(ctx.seq_lens, "seq_lens", torch.int32, (ctx.num_seqs,))
+        self._check(self.lib.akv_step_prologue(_ptr(state), ctypes.c_long(state.numel()), _ptr(ctx.patches),
+                                               _ptr(ctx.patch_count), ctx.patch_room, _ptr(ctx.seq_slots),
+                                               _ptr(ctx.seq_lens), ctx.num_seqs, self._stream()), "step_prologue")
 
     def add_rmsnorm(self, stream, delta, weight, eps, out):
         tokens, hidden = stream.shape
@@ -623,7 +647,8 @@ class HipKernels:
         qkv, q_weight, k_weight, eps, table = fresh if fresh is not None else (None, None, None, 0.0, None)
         self._check(self._attention_mfma_entry(head_dim)(
             _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial), _ptr(ctx.q_start), _ptr(ctx.seq_lens),
-            _ptr(meta.block_table), meta.width, seq_first, seq_count, tiles, nq, q_heads, kv_heads, heads_per_tile,
+            _ptr(meta.block_table), _ptr(getattr(meta, "rows", None)), meta.width, seq_first, seq_count, tiles, nq,
+            q_heads, kv_heads, heads_per_tile,
             head_groups, tokens_per_tile, page_size, ctypes.c_long(num_pages), ctypes.c_float(scale),
             int(window) if window is not None else 0, seg_keys, num_splits, 1 if single else 0, 1 if shared else 0,
             _ptr(qkv), _ptr(q_weight), _ptr(k_weight), ctypes.c_float(eps), _ptr(table),
@@ -744,7 +769,14 @@ class HipKernels:
         self._dense(q, "q", None, (tokens, q_heads * head_dim))
         self._dense(out, "out", q.dtype, (tokens, q_heads * head_dim))
         num_pages, page_size = self._pages(k_pages, v_pages, kv_heads, head_dim, q.dtype)
-        self._dense(meta.block_table, "block_table", torch.int32, (ctx.num_seqs, meta.width))
+        rows = getattr(meta, "rows", None)
+        if rows is None:    # a table of the step's own: row r is request r's
+            self._dense(meta.block_table, "block_table", torch.int32, (ctx.num_seqs, meta.width))
+        else:               # the persistent table: request r's pages are row rows[r] (its slot)
+            self._dense(rows, "table rows", torch.int32, (ctx.num_seqs,))
+            self._dense(meta.block_table, "block_table", torch.int32, (meta.block_table.shape[0], meta.width))
+            if max(ctx.host_seq_slots) >= meta.block_table.shape[0] or min(ctx.host_seq_slots) < 0:
+                raise KernelError("a request's slot lies outside the block table")
         if ctx.max_seq_len > meta.width * page_size:
             raise KernelError(f"a request of {ctx.max_seq_len} tokens does not fit a block table of {meta.width} pages")
         if fresh is not None and not self._matrix_core_attention(q.dtype, page_size):
@@ -780,7 +812,7 @@ class HipKernels:
         self._dense(ctx.positions, "positions", torch.int32, (tokens,))
         self._check(self.lib.akv_attention_rows(
             _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(ctx.seq_of_token), _ptr(ctx.positions),
-            _ptr(meta.block_table), meta.width, _ptr(out), _code(q), ctypes.c_long(tokens), q_heads, kv_heads,
+            _ptr(meta.block_table), _ptr(rows), meta.width, _ptr(out), _code(q), ctypes.c_long(tokens), q_heads, kv_heads,
             head_dim, page_size, ctypes.c_long(num_pages), ctypes.c_float(scale),
             int(window) if window is not None else 0, self._stream()), "attention")
 
@@ -795,6 +827,22 @@ class HipKernels:
             self._dense(draws, "draws", torch.int32, (rows,))
         self._check(self.lib.akv_sample(_ptr(logits), _ptr(temperature), _ptr(seeds), _ptr(draws), _ptr(out), rows,
                                         vocab, self._stream()), "sample")
+
+    def sample_slots(self, logits, ctx, out):
+        """The next token of every wanted row of the step `ctx`, chosen with the sampling state that the row's request
+        keeps in its slot (temperature, seed, draws so far); the chosen token and the new draw count are left there."""
+        rows, vocab = logits.shape
+        self._dense(logits, "logits", torch.float32)
+        self._dense(out, "out", torch.int32, (rows,))
+        self._dense(ctx.logit_rows, "logit_rows", torch.int32, (rows,))
+        self._dense(ctx.seq_of_token, "seq_of_token", torch.int32, (ctx.num_tokens,))
+        self._dense(ctx.seq_slots, "seq_slots", torch.int32, (ctx.num_seqs,))
+        self._dense(ctx.slot_words, "slot_words", torch.int32)
+        if max(ctx.host_seq_slots) >= ctx.slot_words.shape[0]:
+            raise KernelError("a request's slot lies outside the slot words")
+        self._check(self.lib.akv_sample_slots(_ptr(logits), _ptr(ctx.logit_rows), _ptr(ctx.seq_of_token),
+                                              _ptr(ctx.seq_slots), _ptr(ctx.slot_words), _ptr(out), rows, vocab,
+                                              self._stream()), "sample_slots")
 
     def argmax(self, logits, out):
         self.sample(logits, None, None, None, out)

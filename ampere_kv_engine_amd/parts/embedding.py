@@ -26,9 +26,10 @@ class Embedding(Part):
     def weight_bytes(self):
         return 0  # a step reads one row per token, not the table
 
-    def forward(self, token_ids: torch.Tensor, stream: torch.Tensor) -> torch.Tensor:
-        """token_ids int32 [tokens] -> stream float32 [tokens, hidden] (the start of the residual sum)."""
-        self.rt.kernels.embed(token_ids, self.weight, stream)
+    def forward(self, token_ids: torch.Tensor, stream: torch.Tensor, ctx=None) -> torch.Tensor:
+        """token_ids int32 [tokens] -> stream float32 [tokens, hidden] (the start of the residual sum).  With the
+        step's context an id of -1 is the token chosen last for the row's request."""
+        self.rt.kernels.embed(token_ids, self.weight, stream, ctx)
         return stream
 
 

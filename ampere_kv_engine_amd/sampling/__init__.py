@@ -1,3 +1,3 @@
-from .sampler import Sampler, SamplingParams
+from .sampler import NO_TOKEN, Sampler, SamplingParams, SlotSampler
 
-__all__ = ["Sampler", "SamplingParams"]
+__all__ = ["NO_TOKEN", "Sampler", "SamplingParams", "SlotSampler"]

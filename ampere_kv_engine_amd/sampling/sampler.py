@@ -4,6 +4,10 @@ The reference samples greedily only (`logits.argmax()`, ampere_kv/runner.py:346;
 Here a request has a temperature: 0 is that same argmax (ties to the lowest id), above 0 a draw from
 softmax(logits / temperature).  Draws are numbered per request and keyed by the request's seed, so what a request
 generates does not depend on which other requests share its steps.
+
+`SlotSampler` is what the engine uses: temperature, seed and draw count live in the request's slot on the device,
+the kernel reads them there and leaves the chosen token and the new count there - nothing is uploaded per step.
+`Sampler` takes the same parameters row by row from the caller (measurements and tests of the kernel alone).
 """
 
 from __future__ import annotations
@@ -65,5 +69,27 @@ class Sampler:
             return out.tolist()
         # into pinned memory, then one wait for the stream: no staging copy on the way
         self._host_out[:rows].copy_(out, non_blocking=True)
+        torch.cuda.current_stream(self.device).synchronize()
+        return self._host_out[:rows].tolist()
+
+
+class SlotSampler:
+    """Chooses from the logits of a step with the sampling state of the requests' slots (see `Engine.choose`)."""
+
+    def __init__(self, kernels, device, max_rows: int):
+        self.kernels, self.device, self.max_rows = kernels, torch.device(device), max_rows
+        pin = self.device.type == "cuda"
+        self._out = torch.empty(max_rows, dtype=torch.int32, device=self.device)
+        self._host_out = torch.empty(max_rows, dtype=torch.int32, pin_memory=pin)
+
+    def choose(self, logits: torch.Tensor, ctx) -> list[int]:
+        rows = logits.shape[0]
+        if rows > self.max_rows:
+            raise ValueError(f"{rows} rows to choose from; the sampler was built for {self.max_rows}")
+        out = self._out[:rows]
+        self.kernels.sample_slots(logits, ctx, out)
+        if self.device.type != "cuda":
+            return out.tolist()
+        self._host_out[:rows].copy_(out, non_blocking=True)      # into pinned memory, then one wait for the stream
         torch.cuda.current_stream(self.device).synchronize()
         return self._host_out[:rows].tolist()

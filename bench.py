@@ -175,8 +175,7 @@ def main() -> int:
 
     import torch
     from ampere_kv_engine_amd.config import EngineConfig, Qwen3Config
-    from ampere_kv_engine_amd.engine import Engine, StepEntry
-    from ampere_kv_engine_amd.sampling import Sampler, SamplingParams
+    from ampere_kv_engine_amd.engine import LAST_TOKEN, Engine, StepEntry
 
     contexts = None
     if args.contexts:
@@ -189,10 +188,10 @@ def main() -> int:
     max_batch = max([args.batch] + points)
     raw = dict(QWEN3_8B, num_hidden_layers=args.layers)
     config = Qwen3Config.from_dict(raw)
-    tokens_per_request = args.context + PRIMING + args.warmup + args.steps + 1
+    tokens_per_request = args.context + PRIMING + args.warmup + args.steps + 2
     pages = max_batch * ((tokens_per_request + PAGE_SIZE - 1) // PAGE_SIZE) + PREFILL_TOKENS // PAGE_SIZE + 2
     if contexts is not None:
-        grown = PRIMING + args.warmup + args.steps + 1
+        grown = PRIMING + args.warmup + args.steps + 2
         pages = sum((length + grown + PAGE_SIZE - 1) // PAGE_SIZE for length in contexts) + PREFILL_TOKENS // PAGE_SIZE + 2
     engine_config = EngineConfig(dtype="bfloat16", page_size=PAGE_SIZE, num_pages=pages, max_seqs=max_batch,
                                  max_batched_tokens=PREFILL_TOKENS,
@@ -201,7 +200,6 @@ def main() -> int:
     engine = Engine.from_random(config, seed=0, engine_config=engine_config)
     for group in engine.cache.groups:       # any finite keys and values: their content does not change the timing
         group.pages.normal_(0.0, 0.5)
-    sampler = Sampler(engine.kernels, engine.device, max_batch)
     generator = torch.Generator().manual_seed(0)
     sync = lambda: torch.cuda.synchronize(engine.device)
 
@@ -211,13 +209,15 @@ def main() -> int:
         seqs = [engine.open(f"b{batch}_{i}") for i in range(batch)]
         for index, seq in enumerate(seqs):
             engine.cache.reserve(seq, (contexts[index] if contexts is not None else args.context) - 1)
-        tokens = torch.randint(0, config.vocab_size, (batch,), generator=generator).tolist()
-        greedy, draws = [SamplingParams() for _ in range(batch)], [0] * batch
+        first = torch.randint(0, config.vocab_size, (batch,), generator=generator).tolist()
+        logits = engine.step([StepEntry(seq, [token], [0]) for seq, token in zip(seqs, first)], borrow_logits=True)
+        engine.choose(logits)
 
         def one_step():
-            nonlocal tokens
-            logits = engine.step([StepEntry(seq, [token], [0]) for seq, token in zip(seqs, tokens)], borrow_logits=True)
-            tokens = sampler.sample(logits, greedy, draws)
+            # every request feeds the token that was chosen for it in the step before (it lies in its slot on the
+            # device) and the sampler chooses the next one from the slot's own state; the tokens come to the host
+            logits = engine.step([StepEntry(seq, LAST_TOKEN, [0]) for seq in seqs], borrow_logits=True)
+            return engine.choose(logits)
 
         for _ in range(PRIMING + warmup):
             one_step()
@@ -250,7 +250,7 @@ def main() -> int:
             sync()
             started = time.perf_counter()
             logits = engine.step([StepEntry(seq, prompt, [PREFILL_TOKENS - 1])])
-            sampler.sample(logits, [SamplingParams()], [0])
+            engine.choose(logits)
             sync()
             if run:                          # the first run warms up
                 samples.append(time.perf_counter() - started)

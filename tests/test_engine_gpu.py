@@ -161,9 +161,10 @@ def test_a_wrong_page_is_seen_in_bfloat16(case, fault):
         if eng is engine:
             table, other = seqs["c"].tables[0], seqs["d"].tables[0]
             own_page, foreign_page = table._pages[1], other._pages[1]
+            device_row = eng.cache.arrays.tables[0][seqs["c"].slot]      # the request's row of the table on the device
+            assert device_row[:table.num_pages].tolist() == list(table.pages)
             if fault == "table entry":
-                table._pages[1] = foreign_page
-                table._mirror[1] = foreign_page
+                device_row[1] = foreign_page
                 restore = own_page
             else:
                 layer = eng.cache.layer_cache[0]
@@ -175,8 +176,7 @@ def test_a_wrong_page_is_seen_in_bfloat16(case, fault):
             rows.append(out.float().cpu().clone())
         logits[name] = torch.stack(rows)                     # [8, 2 requests, vocab]
         if restore is not None:
-            table._pages[1] = restore
-            table._mirror[1] = restore
+            device_row[1] = restore
         for seq in seqs.values():
             eng.close(seq)
     assert engine.cache.num_free_pages == [engine.config.num_pages]

@@ -931,3 +931,117 @@ def test_attention_window_edge(hip, ref, dtype, history):
         torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(dtype))
         seen_value = v_pages[int(table[winner // page]), 0, :, winner % page].float()
         torch.testing.assert_close(got.cpu().float()[0, :dim], seen_value, rtol=0.05, atol=0.05)
+
+
+# ---- the device's persistent per-request state -------------------------------------------------------------------------
+
+def _with_table_rows(ctx, meta, slots: int, seed: int):
+    """The same step with its block table moved into a table of `slots` rows, request r's pages in row rows[r];
+    every other row names no page (a kernel that read one would poison its result)."""
+    generator = torch.Generator().manual_seed(seed)
+    rows = torch.randperm(slots, generator=generator)[:ctx.num_seqs].int()
+    table = torch.full((slots, meta.width), -1, dtype=torch.int32)
+    table[rows.long()] = meta.block_table
+    moved = SimpleNamespace(**vars(meta))
+    moved.block_table, moved.rows = table, rows
+    where = SimpleNamespace(**vars(ctx))
+    where.host_seq_slots, where.seq_slots = rows.tolist(), rows
+    return where, moved
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("portions", [[(64, 1), (17, 1), (0, 1)], [(5, 7), (63, 2), (130, 1), (0, 70)], [(1500, 1), (2, 1), (700, 1)]])
+def test_attention_finds_a_request_s_pages_in_the_row_of_its_slot(hip, ref, dtype, portions):
+    """Block tables that live on the device, a row per request slot: the kernels are told which row is which
+    request's (`meta.rows`) and must give what they give for a table of the step's own."""
+    q_heads, kv_heads, dim, page_size = 8, 2, 64, 16
+    q, k_pages, v_pages, ctx, meta, _, _ = _attention_case(dtype, q_heads, kv_heads, dim, page_size, portions, None, 31)
+    ctx.num_decode_seqs = sum(1 for _, n in portions if n == 1) if all(n == 1 for _, n in portions) else 0
+    want = torch.empty_like(q)
+    ref.attention(q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, dim, dim ** -0.5, None, want)
+    where, moved = _with_table_rows(ctx, meta, slots=len(portions) + 5, seed=3)
+    again = torch.empty_like(q)
+    ref.attention(q, k_pages, v_pages, where, moved, q_heads, kv_heads, dim, dim ** -0.5, None, again)
+    assert torch.equal(again, want)                          # (the double reads the rows too)
+    cctx, cmeta = _to_cuda(where, moved)
+    cctx.seq_slots, cmeta.rows = where.seq_slots.cuda(), moved.rows.cuda()
+    got = torch.full_like(q, float("nan"), device="cuda")
+    hip.attention(q.cuda(), k_pages.cuda(), v_pages.cuda(), cctx, cmeta, q_heads, kv_heads, dim, dim ** -0.5, None, got)
+    assert not torch.isnan(got).any()
+    torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(dtype))
+
+
+def test_step_prologue_applies_a_step_s_changes(hip, ref):
+    """(offset, value) pairs up to the count that lies on the device - never more than the capacity, never outside
+    the state - and the requests' lengths into word 0 of their slots."""
+    slots, width = 6, 10
+    state = torch.arange(slots * 8 + slots * width, dtype=torch.int32) + 1000
+    patches = torch.tensor([50, -1, 61, 7, 48, 3, 10 ** 6, 9, 55, 5, 56, 6], dtype=torch.int32)      # 6 pairs, one outside
+    for count in (0, 4, 6):
+        ctx = SimpleNamespace(slot_state=state.clone(), patches=patches.clone(), patch_count=torch.tensor([count], dtype=torch.int32),
+                              patch_room=5, seq_slots=torch.tensor([4, 1], dtype=torch.int32),
+                              seq_lens=torch.tensor([77, 9], dtype=torch.int32), num_seqs=2)
+        ctx.patches = ctx.patches[:10]
+        want = state.clone()
+        for offset, value in list(zip(patches[0::2].tolist(), patches[1::2].tolist()))[:min(count, 5)]:
+            if 0 <= offset < want.numel():
+                want[offset] = value
+        want[4 * 8], want[1 * 8] = 77, 9
+        on = SimpleNamespace(**{k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in vars(ctx).items()})
+        hip.step_prologue(on)
+        assert torch.equal(on.slot_state.cpu(), want), count
+
+
+def test_sampling_from_the_slots_equals_sampling_with_the_same_state_handed_in(hip, ref):
+    """`sample_slots` reads temperature, seed and draw count from the slot of each row's request, chooses what `sample`
+    chooses for them, and leaves the token and the next draw count in the slot; other slots are not touched."""
+    import struct
+    vocab, slots = 1000, 7
+    logits = torch.randn(3, vocab, generator=torch.Generator().manual_seed(5)) * 3
+    logits[2, 5] = float("nan")
+    words = torch.full((slots, 8), 99, dtype=torch.int32)
+    state = {5: (0.0, 0, 4), 2: (0.8, (1 << 40) + 12345, 7), 0: (1.5, 3, 0)}       # slot -> temperature, seed, draws
+    for slot, (t, seed, draws) in state.items():
+        words[slot] = torch.tensor([11, -1, struct.unpack("<i", struct.pack("<f", t))[0], seed & 0xFFFFFFFF, seed >> 32, draws, 1, 0])
+    # three requests in slots 5, 2, 0; five token rows; the wanted rows are rows 4, 0 and 2
+    ctx = SimpleNamespace(num_tokens=5, num_seqs=3, logit_rows=torch.tensor([4, 0, 2], dtype=torch.int32),
+                          seq_of_token=torch.tensor([1, 1, 2, 2, 0], dtype=torch.int32),
+                          seq_slots=torch.tensor([5, 2, 0], dtype=torch.int32), host_seq_slots=[5, 2, 0], slot_words=words.clone())
+    order = [5, 2, 0]                                                             # the slots of the three logits rows
+    want = torch.empty(3, dtype=torch.int32)
+    ref.sample(logits, torch.tensor([state[s][0] for s in order]), torch.tensor([state[s][1] for s in order]),
+               torch.tensor([state[s][2] for s in order], dtype=torch.int32), want)
+    assert want[2] == -1
+    on = SimpleNamespace(**{k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in vars(ctx).items()})
+    got = torch.empty(3, dtype=torch.int32, device="cuda")
+    hip.sample_slots(logits.cuda(), on, got)
+    assert got.cpu().tolist() == want.tolist()
+    after = on.slot_words.cpu()
+    for row, slot in enumerate(order):
+        assert after[slot, 1] == want[row] and after[slot, 5] == state[slot][2] + 1
+        assert after[slot, 0] == 11 and after[slot, 2:5].tolist() == words[slot, 2:5].tolist()
+    assert torch.equal(after[[1, 3, 4, 6]], words[[1, 3, 4, 6]])
+    double = SimpleNamespace(**vars(ctx))
+    double.slot_words = words.clone()
+    chosen = torch.empty(3, dtype=torch.int32)
+    ref.sample_slots(logits, double, chosen)
+    assert chosen.tolist() == want.tolist() and torch.equal(double.slot_words, after)
+
+
+def test_embed_takes_the_token_chosen_last_from_the_slot(hip, ref):
+    table = torch.randn(50, 24, generator=torch.Generator().manual_seed(1)).bfloat16()
+    words = torch.zeros(4, 8, dtype=torch.int32)
+    words[3, 1], words[1, 1] = 17, 42
+    ctx = SimpleNamespace(num_seqs=2, seq_of_token=torch.tensor([0, 1, 1], dtype=torch.int32),
+                          seq_slots=torch.tensor([3, 1], dtype=torch.int32), host_seq_slots=[3, 1], slot_words=words)
+    ids = torch.tensor([-1, 7, -1], dtype=torch.int32)
+    want = table[[17, 7, 42]].float()
+    out = torch.empty(3, 24)
+    ref.embed(ids, table, out, ctx)
+    assert torch.equal(out, want)
+    on = SimpleNamespace(**{k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in vars(ctx).items()})
+    got = torch.empty(3, 24, device="cuda")
+    hip.embed(ids.cuda(), table.cuda(), got, on)
+    assert torch.equal(got.cpu(), want)
+    hip.embed(ids.cuda(), table.cuda(), got)                                     # without the slots -1 is no token
+    assert torch.isnan(got[0]).all() and torch.equal(got[1].cpu(), want[1])

@@ -102,6 +102,7 @@ def test_attention_mixer_alone(dtype, q_heads, kv_heads, head_dim, window):
     for step in range(2):
         entries = [StepEntry(seqs[i], [0] * (cuts[i][step][1] - cuts[i][step][0]), []) for i in range(2)]
         ctx, _ = builder.build(entries)
+        rt.kernels.step_prologue(ctx)       # (the model's pass does this before its first kernel)
         order = sorted(range(2), key=lambda i: (cuts[i][step][1] - cuts[i][step][0] != 1, i))
         x = torch.cat([xs[i][cuts[i][step][0]:cuts[i][step][1]] for i in order]).cuda()
         y = mixer.forward(x, ctx, cache.layer_cache[0]).cpu().float()
@@ -142,6 +143,7 @@ def test_attention_mixer_through_the_parts_own_entry_points(dtype):
         mixer.load(loader({}, dtype), "L.")
         cache, builder, seqs = step_context(rt, {0: mixer.cache_request()}, [0], page_size)
         ctx, _ = builder.build([StepEntry(seqs[0], [0] * 19, [])])
+        rt.kernels.step_prologue(ctx)
         results.append(mixer.forward(x.cuda(), ctx, cache.layer_cache[0]).cpu().float())
     torch.testing.assert_close(results[0], results[1], **tol(dtype))
 
@@ -154,6 +156,7 @@ def test_swiglu_part(dtype):
     ff.load(loader(weights, dtype), "L.")
     cache, builder, seqs = step_context(rt, {0: None}, [0], 8)
     ctx, _ = builder.build([StepEntry(seqs[0], [0] * 11, [])])
+    rt.kernels.step_prologue(ctx)
     x = torch.randn(11, 72).to(dtype)
     got = ff.forward(x.cuda(), ctx).cpu().float()
     want = P.swiglu_feed_forward(x.float(), weights["L.mlp.gate_proj.weight"], weights["L.mlp.up_proj.weight"],
@@ -176,6 +179,7 @@ def test_block_alone(dtype):
     block.load(loader(weights, dtype), "L.")
     cache, builder, seqs = step_context(rt, {0: mixer.cache_request()}, [0], page_size)
     ctx, _ = builder.build([StepEntry(seqs[0], [0] * 17, [])])
+    rt.kernels.step_prologue(ctx)
     ctx.arena = ctx.arenas[0]
     h0 = torch.randn(17, hidden)
     stream = h0.clone().cuda()
@@ -429,3 +433,27 @@ def test_recorded_decode_steps_equal_eager_ones(dtype, model_folders):
     for name in list(last):
         close(name)
     assert recorded.cache.num_free_pages == eager.cache.num_free_pages == [96]
+
+
+def test_a_slot_that_is_used_again_starts_clean_on_the_device(model_folders):
+    """The per-request state on the device (slot words, row of the block table) of a slot that another request used:
+    the next request finds it fresh, draws what it draws in an engine of its own, and nothing is uploaded for a
+    choice (the sampler reads the slot)."""
+    raw, _, page = TINY["B"]
+    config = lambda seqs: EngineConfig(dtype="bfloat16", page_size=page, num_pages=32, max_seqs=seqs, max_batched_tokens=64,
+                                       max_seq_len=256, device="cuda:0")
+    prompt = random_ids(raw["vocab_size"], 11, seed=21)
+    alone = generate_tokens(Engine.from_folder(model_folders["B"], config(4)), prompt, max_new_tokens=6, ignore_eos=True,
+                            temperature=0.9, seed=77)
+    engine = Engine.from_folder(model_folders["B"], config(1))
+    generate_tokens(engine, random_ids(raw["vocab_size"], 20, seed=22), max_new_tokens=9, ignore_eos=True,
+                    temperature=1.3, seed=5)
+    words, table = engine.cache.arrays.words, engine.cache.arrays.tables[0]
+    assert words[0].tolist()[:2] == [28, words[0, 1].item()] and int(words[0, 5]) == 9 and int(words[0, 6]) == 0
+    seq = engine.open("next", 0.9, 77)
+    torch.cuda.synchronize()
+    assert seq.slot == 0 and words[0].tolist()[:2] == [0, -1] and int(words[0, 5]) == 0 and int(words[0, 6]) == 1
+    assert int((table[0] >= 0).sum()) == 0
+    engine.close(seq)
+    assert generate_tokens(engine, prompt, max_new_tokens=6, ignore_eos=True, temperature=0.9, seed=77) == alone
+    assert len(set(alone)) > 1

@@ -219,3 +219,29 @@ def test_a_request_without_finite_logits_is_retired_with_an_error(model_folders)
     done, _ = drive(scheduler)
     assert good in done and good.stop_reason == STOP_LIMIT and len(good.output_ids) == 6
     assert engine.cache.num_free_pages == [32] and engine.cache.slots.num_free == 4
+
+
+def test_a_slot_that_is_used_again_starts_clean(model_folders):
+    """What a request keeps on the device - tokens held, the token chosen last, temperature, seed, draws made, its row
+    of the block table - starts fresh when another request takes the slot: the second request draws what it draws
+    in an engine of its own, whatever its predecessor did there."""
+    from ampere_kv_engine_amd.cache.slots import (NO_TOKEN, WORD_DRAWS, WORD_LAST_TOKEN, WORD_LENGTH, WORD_SEED_LOW,
+                                                    WORD_TAKEN)
+    raw, _, page = TINY["B"]
+    prompt = random_ids(raw["vocab_size"], 11, seed=21)
+    alone = alone_tokens = generate_tokens(make_engine(model_folders["B"], page, 32), prompt, max_new_tokens=6,
+                                           ignore_eos=True, temperature=0.9, seed=77)
+    engine = make_engine(model_folders["B"], page, 32, max_seqs=1)
+    generate_tokens(engine, random_ids(raw["vocab_size"], 20, seed=22), max_new_tokens=9, ignore_eos=True,
+                    temperature=1.3, seed=5)
+    words, table = engine.cache.arrays.words, engine.cache.arrays.tables[0]
+    assert int(words[0, WORD_TAKEN]) == 0 and int(words[0, WORD_DRAWS]) == 9 and int(words[0, WORD_LENGTH]) == 28
+    assert int((table[0] >= 0).sum()) == 4                      # the predecessor's pages are still named in the row
+    seq = engine.open("next", 0.9, 77)
+    assert seq.slot == 0
+    assert [int(words[0, w]) for w in (WORD_LENGTH, WORD_LAST_TOKEN, WORD_DRAWS, WORD_TAKEN, WORD_SEED_LOW)] == [0, NO_TOKEN, 0, 1, 77]
+    assert int((table[0] >= 0).sum()) == 0
+    engine.close(seq)
+    again = generate_tokens(engine, prompt, max_new_tokens=6, ignore_eos=True, temperature=0.9, seed=77)
+    assert again == alone and len(set(alone_tokens)) > 1
+    assert int(words[0, WORD_DRAWS]) == 6 and int(words[0, WORD_LAST_TOKEN]) == again[-1]

@@ -26,8 +26,22 @@ class TorchKernels:
             raise ValueError("q_heads must be a multiple of kv_heads")
 
     # ---- token-wise ------------------------------------------------------------------------------------
-    def embed(self, ids, table, out):
-        out.copy_(table[ids.long()].float())
+    def embed(self, ids, table, out, ctx=None):
+        """An id of -1 stands for the token chosen last for the row's request (word 1 of its slot)."""
+        ids = ids.long().clone()
+        words = getattr(ctx, "slot_words", None) if ctx is not None else None
+        if words is not None:
+            last = words[ctx.seq_slots.long()[ctx.seq_of_token.long()], 1].long()
+            ids = torch.where(ids == -1, last, ids)
+        out.copy_(table[ids].float())
+
+    def step_prologue(self, ctx):
+        """state[offset] = value for the step's (offset, value) pairs; word 0 of every request's slot = its length."""
+        count = int(ctx.patch_count[0])
+        assert count <= ctx.patch_room
+        pairs = ctx.patches[:2 * count].view(count, 2).long()
+        ctx.slot_state[pairs[:, 0]] = pairs[:, 1].int()
+        ctx.slot_words[ctx.seq_slots.long(), 0] = ctx.seq_lens
 
     def add_rmsnorm(self, stream, delta, weight, eps, out):
         if delta is not None:
@@ -127,6 +141,8 @@ class TorchKernels:
         page_size = k_pages.shape[2]
         group = q_heads // kv_heads
         table = meta.block_table.cpu()
+        if getattr(meta, "rows", None) is not None:          # the persistent table: a row per slot
+            table = table[meta.rows.cpu().long()]
         for r in range(ctx.num_seqs):
             first, last = ctx.host_q_start[r], ctx.host_q_start[r + 1]
             length = ctx.host_seq_lens[r]
@@ -170,6 +186,21 @@ class TorchKernels:
 
     def argmax(self, logits, out):
         self.sample(logits, None, None, None, out)
+
+    def sample_slots(self, logits, ctx, out):
+        """`sample` with every row's temperature (word 2, float bits), seed (words 3 and 4) and draw count (word 5)
+        read from its request's slot; the chosen token goes to word 1 and the draw count rises by one."""
+        words = ctx.slot_words
+        slots = ctx.seq_slots.long()[ctx.seq_of_token.long()[ctx.logit_rows.long()]]
+        assert len(set(slots.tolist())) == len(slots), "two wanted rows of one request"
+        state = words[slots].cpu()
+        temperature = state[:, 2].contiguous().view(torch.float32)
+        seeds = (state[:, 3].long() & 0xFFFFFFFF) | ((state[:, 4].long() & 0xFFFFFFFF) << 32)
+        chosen = torch.empty(len(slots), dtype=torch.int32)
+        self.sample(logits.cpu(), temperature, seeds, state[:, 5], chosen)
+        out.copy_(chosen)
+        words[slots, 1] = chosen.to(words.device)
+        words[slots, 5] += 1
 
 
 def philox_first(c0, c1, k0, k1):
