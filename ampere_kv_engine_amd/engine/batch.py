@@ -31,6 +31,10 @@ class StepEntry:
     seq: Sequence
     tokens: Seq[int]
     want: Seq[int] = ()
+    # further integers per token for parts that need more than a position (the axes of a multi-axis position encoding,
+    # a segment id): name -> [len(tokens)][width].  Every entry of a step carries the same names and widths; the parts
+    # find them on the device as `ctx.extra[name]`, int32 [tokens, width].
+    extra: dict | None = None
 
 
 @dataclass
@@ -123,11 +127,14 @@ class StepContext:
     patch_room: int = 0
     slot_state: torch.Tensor | None = None      # int32: the whole state
     slot_words: torch.Tensor | None = None      # int32 [slots, SLOT_WORDS]: its first part
+    extra: dict = field(default_factory=dict)   # name -> int32 [tokens, width]: what the entries brought per token
 
 
 class BatchBuilder:
     """Turns entries into a `StepContext`: registers the new tokens with the cache manager (which hands out
     pages), lays the tokens out with single-token requests first, and uploads the metadata in one copy."""
+
+    EXTRA_WORDS_PER_TOKEN = 8       # room for the entries' further integers per token, all names together
 
     def __init__(self, cache: CacheManager, device, max_batched_tokens: int, max_seqs: int, max_pages_per_seq: int):
         self.cache = cache
@@ -138,7 +145,7 @@ class BatchBuilder:
             self.max_width = min(self.max_width, cache.arrays.table_width)
         most_patches = groups * 2 * (self.max_tokens // cache.page_size + 2 * self.max_seqs)
         capacity = (3 * self.max_tokens + 3 * self.max_seqs + 1 + self.max_tokens
-                    + groups * self.max_tokens + 1 + 2 * most_patches)
+                    + groups * self.max_tokens + 1 + 2 * most_patches + self.EXTRA_WORDS_PER_TOKEN * self.max_tokens)
         pin = self.device.type == "cuda"
         # Two pinned staging buffers in turn: the copy of one step may still be in flight while the host
         # lays out the next, so a buffer is written again only after the copy that read it has finished.
@@ -219,6 +226,7 @@ class BatchBuilder:
         patch_count, s_pc = region(1)
         patches, s_pa = region(2 * patch_room)
         changed = 0
+        extra_spans = self._extra_regions(ordered, n, region)
 
         row = 0
         first_row_of = [0] * len(entries)
@@ -233,6 +241,8 @@ class BatchBuilder:
                 token_ids[row:row + count] = np.asarray(e.tokens, dtype=np.int64)
                 positions[row:row + count] = np.arange(start, start + count)
                 seq_of_token[row:row + count] = index
+            for name, (view, _, width_of) in extra_spans.items():
+                view.reshape(n, width_of)[row:row + count] = np.asarray(e.extra[name], dtype=np.int64).reshape(count, width_of)
             q_start[index] = row
             seq_lens[index] = start + count
             seq_slots[index] = e.seq.slot
@@ -288,8 +298,32 @@ class BatchBuilder:
             arenas=self.arenas, table_pages=width, patches=dev(s_pa), patch_count=dev(s_pc), patch_room=patch_room,
             slot_state=arrays.state if arrays is not None else None,
             slot_words=arrays.words if arrays is not None else None,
+            extra={name: dev(span).view(n, width_of) for name, (_, span, width_of) in extra_spans.items()},
         )
         return ctx, first_wanted_of
+
+    def _extra_regions(self, ordered: list[StepEntry], n: int, region) -> dict:
+        """Room in the step's upload for the further per-token integers the entries bring: name -> (host view, span,
+        width).  All entries must agree on names and widths."""
+        first = ordered[0].extra or {}
+        widths = {}
+        for name, rows in first.items():
+            array = np.asarray(rows)
+            if array.ndim != 2 or array.shape[0] != len(ordered[0].tokens) or array.dtype.kind not in "iu":
+                raise ValueError(f"extra {name!r} must hold one row of integers per token")
+            widths[name] = int(array.shape[1])
+        for e in ordered[1:]:
+            other = e.extra or {}
+            if set(other) != set(widths) or any(np.asarray(other[name]).shape != (len(e.tokens), w) for name, w in widths.items()):
+                raise ValueError("every entry of a step must bring the same further integers per token (names and widths)")
+        if sum(widths.values()) > self.EXTRA_WORDS_PER_TOKEN:
+            raise ValueError(f"{sum(widths.values())} further integers per token; the step's upload has room for "
+                             f"{self.EXTRA_WORDS_PER_TOKEN}")
+        spans = {}
+        for name in sorted(widths):
+            view, span = region(n * widths[name])
+            spans[name] = (view, span, widths[name])
+        return spans
 
     def _check_pages(self, ordered: list[StepEntry]) -> None:
         """Plays the step's registrations through in the order they will be made (a request first gives back the

@@ -170,7 +170,7 @@ class Engine:
         numbers of tokens also fix how many block-table changes the step may bring at most.)"""
         counts = tuple(sorted((len(e.tokens) for e in entries), key=lambda count: count != 1))
         wanted = sum(len(e.want) for e in entries)
-        if wanted == 0 or wanted > self.config.max_seqs:
+        if wanted == 0 or wanted > self.config.max_seqs or any(e.extra for e in entries):
             return None
         if counts[-1] != 1 and sum(counts) > self.RECORD_MAX_TOKENS:
             return None

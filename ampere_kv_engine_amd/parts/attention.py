@@ -113,8 +113,12 @@ class Attention(Part):
         else:
             k.copy_heads(q_in, q3)
             k.copy_heads(k_in, k3)
-        self.position.apply(q3, ctx.positions)
-        self.position.apply(k3, ctx.positions)
+        if getattr(self.position, "wants_context", False):     # an encoding of more than the position: it reads the step
+            self.position.apply(q3, ctx.positions, ctx)
+            self.position.apply(k3, ctx.positions, ctx)
+        else:
+            self.position.apply(q3, ctx.positions)
+            self.position.apply(k3, ctx.positions)
         if writes_cache:
             k.kv_write(k3, v_in, meta.slot_map, cache.k, cache.v)
 

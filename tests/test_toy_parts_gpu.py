@@ -312,3 +312,99 @@ def test_a_routed_feed_forward_and_another_position_encoding(tmp_path):
         parts.append(engine.step([StepEntry(seq, ids[lo:hi], list(range(hi - lo)))]).cpu())
     engine.close(seq)
     torch.testing.assert_close(torch.cat(parts), want, rtol=1e-4, atol=1e-5)
+
+
+class TwoAxisRotary(Part):
+    """A position encoding of two axes (a row and a column per token, as for patches of a picture): the first half of
+    a head's rotation pairs turns with the row, the second half with the column.  The axes are not the token's
+    position in its request: the entries bring them as further integers per token (`extra["axes"]`, [tokens, 2])."""
+    wants_context = True
+
+    def __init__(self, spec, runtime):
+        self.head_dim, self.theta = int(spec["head_dim"]), float(spec["theta"])
+        quarter = self.head_dim // 4
+        self.inv_freq = 1.0 / (self.theta ** (torch.arange(0, quarter, dtype=torch.float32) / quarter))
+        self.table = None
+
+    def apply(self, x, positions, ctx):
+        axes = ctx.extra["axes"].to(x.device).float()                         # [tokens, 2]
+        angles = torch.cat((axes[:, :1] * self.inv_freq.to(x.device)[None, :], axes[:, 1:] * self.inv_freq.to(x.device)[None, :]), dim=1)
+        cos, sin = angles.cos()[:, None, :], angles.sin()[:, None, :]          # [tokens, 1, d/2]
+        half = self.head_dim // 2
+        lo, hi = x[..., :half].float(), x[..., half:].float()
+        x.copy_(torch.cat((lo * cos - hi * sin, hi * cos + lo * sin), dim=-1).to(x.dtype))
+        return x
+
+
+@dataclass(frozen=True)
+class TwoAxisConfig(ToyConfig):
+    architecture = "ToyTwoAxisForCausalLM"
+
+    def to_model_spec(self):
+        h = self.hidden_size
+        norm = part("rmsnorm", size=h, eps=self.eps)
+        block = part("prenorm", hidden_size=h, norm=norm)
+        attention = part("attention", hidden_size=h, q_heads=2, kv_heads=1, head_dim=16, window=None, qk_norm=None,
+                         position=part("two_axis_rotary", head_dim=16, theta=1e3), scale=0.25, name="self_attn")
+        dense = part("swiglu", hidden_size=h, intermediate_size=40, name="mlp")
+        return ModelSpec(self.architecture, self.vocab_size, h,
+                         part("embedding", vocab_size=self.vocab_size, hidden_size=h, name="model.embed_tokens.weight"),
+                         (LayerSpec(block, attention, dense, "model.layers.0."),), (RunEntry(0, 0),),
+                         part("rmsnorm", size=h, eps=self.eps, name="model.norm.weight"),
+                         part("linear_head", vocab_size=self.vocab_size, hidden_size=h, name="lm_head.weight", tied_to=None))
+
+
+def test_a_position_encoding_of_two_axes_reads_further_integers_of_the_step(tmp_path):
+    """Positions need not be one integer per token: an entry may bring further integers per token, the step carries
+    them to the device beside its other metadata, and a position part that asks for the step's context reads them.
+    Whole and in portions, two requests in one step, against a plain computation."""
+    from safetensors.torch import load_file
+    register_part("position", "two_axis_rotary", TwoAxisRotary, replace=True)
+    register_architecture(TwoAxisConfig.architecture, TwoAxisConfig, replace=True)
+    config = TwoAxisConfig(vocab_size=61, hidden_size=32, decay=0.0, eps=1e-5)
+    folder = write_random_model(str(tmp_path / "two_axes"), config, seed=13)
+    engine = Engine.from_folder(folder, EngineConfig(dtype="float32", page_size=8, num_pages=16, max_seqs=2,
+                                                     max_batched_tokens=64, max_seq_len=64, device="cuda:0"))
+    w = {k: v.float() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+
+    def plain(ids, axes):
+        n, p = len(ids), "model.layers.0."
+        h = w["model.embed_tokens.weight"][torch.tensor(ids)]
+        inv = 1.0 / (1e3 ** (torch.arange(0, 4, dtype=torch.float32) / 4))
+        a = torch.tensor(axes).float()
+        angles = torch.cat((a[:, :1] * inv[None], a[:, 1:] * inv[None]), dim=1)
+        cos, sin = angles.cos()[:, None, :], angles.sin()[:, None, :]
+        rotate = lambda x: torch.cat((x[..., :8] * cos - x[..., 8:] * sin, x[..., 8:] * cos + x[..., :8] * sin), dim=-1)
+        x = P.rms_norm(h, w[p + "input_layernorm.weight"], config.eps)
+        q = rotate((x @ w[p + "self_attn.q_proj.weight"].T).reshape(n, 2, 16))
+        k = rotate((x @ w[p + "self_attn.k_proj.weight"].T).reshape(n, 1, 16))
+        v = (x @ w[p + "self_attn.v_proj.weight"].T).reshape(n, 1, 16)
+        h = h + P.causal_attention(q, k, v).reshape(n, 32) @ w[p + "self_attn.o_proj.weight"].T
+        x = P.rms_norm(h, w[p + "post_attention_layernorm.weight"], config.eps)
+        h = h + P.swiglu_feed_forward(x, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+        return P.rms_norm(h, w["model.norm.weight"], config.eps) @ w["lm_head.weight"].T
+
+    requests = {}
+    for name, count, seed in (("a", 19, 14), ("b", 7, 15)):
+        ids = random_ids(61, count, seed=seed)
+        axes = [[t // 5, (3 * t) % 5] for t in range(count)]             # rows and columns of a grid, not 0, 1, 2, ...
+        requests[name] = (ids, axes, plain(ids, axes))
+    seqs = {name: engine.open(name) for name in requests}
+    got = {name: [] for name in requests}
+    for cuts in ({"a": (0, 9), "b": (0, 2)}, {"a": (9, 11), "b": (2, 7)}, {"a": (11, 19)}):
+        entries = [StepEntry(seqs[name], requests[name][0][lo:hi], list(range(hi - lo)), extra={"axes": requests[name][1][lo:hi]})
+                   for name, (lo, hi) in cuts.items()]
+        logits = engine.step(entries).cpu()
+        row = 0
+        for name, (lo, hi) in cuts.items():
+            got[name].append(logits[row:row + hi - lo])
+            row += hi - lo
+    for name, seq in seqs.items():
+        engine.close(seq)
+        torch.testing.assert_close(torch.cat(got[name]), requests[name][2], rtol=1e-4, atol=1e-5)
+    with pytest.raises(ValueError, match="same further integers"):
+        a, b = engine.open("a"), engine.open("b")
+        try:
+            engine.step([StepEntry(a, [1, 2], [], extra={"axes": [[0, 0], [0, 1]]}), StepEntry(b, [3], [])])
+        finally:
+            engine.close(a), engine.close(b)
