@@ -48,6 +48,11 @@ int akv_pack_rows(const void* x, void* xp, int rows, int k, hipStream_t stream);
 // threads) race; calls that follow each other on a stream do not.
 int akv_linear_packed_static(const void* x, const void* wp, void* y, int y_dtype, int rows, int outs, int k,
                              int n_tiles, int k_tiles, hipStream_t stream);
+int akv_linear_adds(const void* x, const void* wp, float* stream_out, float* sums_out, int rows, int outs, int k,
+                    int n_tiles, int k_tiles, hipStream_t stream);
+int akv_linear_scaled(const float* stream_in, const float* sums, int sum_tiles, const float* gain, float eps,
+                      const void* wp, void* y, int rows, int outs, int k, int n_tiles, int k_tiles, int gated,
+                      hipStream_t stream);
 int akv_linear_mid_workspace(int rows, int n_tiles, int k_tiles, int gated, int along, int rt, int depth, int parts,
                              long* partial_floats, long* counters);
 int akv_linear_mid(const void* x, const void* wp, void* y, int y_dtype, float* partial, unsigned* counters, int rows,

@@ -19,7 +19,7 @@ import time
 from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCES = ("elementwise.hip", "gemm.hip", "gemm_mfma.hip", "gemm_mid.hip", "attention.hip", "sampling.hip")
+SOURCES = ("elementwise.hip", "gemm.hip", "gemm_mfma.hip", "gemm_mid.hip", "gemm_decode.hip", "attention.hip", "sampling.hip")
 HEADERS = ("common.h", "mfma_tiles.h", "api.h")
 LIBRARY = "libakv_kernels.so"
 ATTENTION_SOURCE = "attention_mfma.hip"        # compiled once per head size, into its own small library

@@ -1,0 +1,332 @@
+// bfloat16 products of up to 16 rows (decode steps) that take the residual sum and the norm between two products
+// into the products themselves, so that a layer of a decode step launches no kernel for either:
+//
+//   ADDS    a branch's last product (o, down) does not store its result: it rounds it to bfloat16, adds it to the
+//           float32 residual sum in place, and leaves the sums of squares of the new residual rows, one partial sum per
+//           (row tile of 16 outputs, row) - every output is owned by one lane, so no value depends on an order;
+//   SCALED  the product that reads the norm of the residual sum (q/k/v, gate and up) does not read normed rows: every
+//           block norms the rows for itself into LDS while its first weights are on their way.  The rows' sums of
+//           squares are not formed again: a wave adds the partial sums in a fixed order (the same in every block) and
+//           forms rsqrt(mean + eps); then every thread norms pieces of 8 values as the norm kernel does - scaled,
+//           rounded, times the weight, rounded - and puts them where the matrix cores' operand wants them.
+//
+// Otherwise this is the skinny kernel of gemm_mfma.hip for one tile of rows: a wave owns RT row tiles of the packed
+// weight and a part of k, streams its tiles once (two groups of registers in turn, loads marked as read-once), the
+// parts of k are summed through LDS in a fixed order.  GATED as there (a pair of gate and up tiles, RT = 2).
+// The results equal those of the separate kernels up to the order in which a row's squares are added.
+
+#include <mutex>
+
+#include "common.h"
+#include "mfma_tiles.h"
+#include "api.h"
+
+using namespace akv;
+
+namespace {
+
+struct DecodeArgs {
+  const bf16_t* x;          // not SCALED: [rows, k]
+  const float* stream;      // SCALED: [rows, k], the residual sum
+  const float* sums;        // SCALED: [sum_tiles][16] partial sums of squares of the residual rows
+  const float* gain;        // SCALED: [k], the norm's weight
+  const uintx4* wp;         // the packed weight
+  bf16_t* y;                // not ADDS: [rows, outs]
+  float* stream_out;        // ADDS: [rows, outs], updated in place
+  float* sums_out;          // ADDS: [n_tiles][16]
+  float eps;
+  int sum_tiles, rows, outs, k, k_tiles, n_tiles, k_split, red_floats;
+};
+
+constexpr int kGroup = 4;   // k-tiles per group of loads; two groups are in flight
+constexpr size_t kMaxLds = 160 * 1024;   // a compute unit's LDS: the most a block can have
+
+template <int RT, bool GATED, bool SCALED, bool ADDS>
+__global__ __launch_bounds__(768) void linear_decode_kernel(const DecodeArgs a) {
+  static_assert(!(GATED && ADDS) && (!GATED || RT == 2), "the gated pair is a wave's two row tiles");
+  constexpr int U = kGroup;
+  extern __shared__ float red[];   // [wave][RT][4][64] for the sum over the parts of k - SCALED: before that, the rows' scales and the normed rows
+  const int lane = threadIdx.x & 63, waves = blockDim.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r = lane & 15, g = lane >> 4;
+  const int row_tile = (blockIdx.x * (waves / a.k_split) + wave / a.k_split) * RT;
+  const int part = wave % a.k_split;
+  const int per_part = (a.k_tiles + a.k_split - 1) / a.k_split;
+  const int kt0 = part * per_part, kt1 = min(a.k_tiles, kt0 + per_part);
+  const bool works = row_tile < a.n_tiles && kt0 < kt1;
+  const bool ragged = (a.k & 31) != 0;
+  const uintx4 zero = {0u, 0u, 0u, 0u};
+  floatx4 acc[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) acc[rt] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  // Weights: every load is issued whatever the sizes are - a tile beyond the wave's part or the matrix reads the last
+  // valid one again and is not used - so that the loop's loads sit behind no branch and the compiler can wait for
+  // exactly the group it needs while the next is in flight.
+  const int last_tile = max(kt1 - 1, 0);
+  const uintx4* w_lane = a.wp + lane;
+  uintx4 w0[RT][U], w1[RT][U];
+  auto fetch_weights = [&](int kt, uintx4 (&w)[RT][U]) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+        w[rt][u] = load_once(w_lane + tile_index<GATED>(min(row_tile + rt, a.n_tiles - 1), min(kt + u, last_tile), a.k_tiles) * 64);
+  };
+  // SCALED: the rows as the operand wants them, [k tile][k chunk of 8][row] x 16 bytes: lane (r, g) reads chunk g, row r
+  constexpr int kScaleFloats = 12 * 16 + 16;   // SCALED: every wave's share of the rows' sums of squares, then the scales
+  uintx4* rows_lds = reinterpret_cast<uintx4*>(red + (SCALED ? kScaleFloats : 0));
+  fetch_weights(kt0, w0);   // on their way while the rows are normed
+  if constexpr (SCALED) {
+    // The rows' sums of squares: sum_tiles x 16 partial sums.  The waves share the tiles; a lane adds up quads of
+    // rows (lane % 4 fixes which four), the lanes of a wave are folded in a fixed order, then the waves' shares - the
+    // same order in every block.
+    float* shares = red;
+    float* scales = red + 12 * 16;
+    {
+      const int quads = a.sum_tiles * 4, per_wave = ((quads + waves - 1) / waves + 63) / 64 * 64;
+      const int q0 = wave * per_wave, q1 = min(quads, q0 + per_wave);
+      float4 part = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll 4
+      for (int q = q0 + lane; q < q1; q += 64) {
+        const float4 v = reinterpret_cast<const float4*>(a.sums)[q];
+        part.x += v.x, part.y += v.y, part.z += v.z, part.w += v.w;
+      }
+#pragma unroll
+      for (int step = 4; step < 64; step <<= 1) {
+        part.x += __shfl_xor(part.x, step, kWave);
+        part.y += __shfl_xor(part.y, step, kWave);
+        part.z += __shfl_xor(part.z, step, kWave);
+        part.w += __shfl_xor(part.w, step, kWave);
+      }
+      if (lane < 4) *reinterpret_cast<float4*>(shares + wave * 16 + lane * 4) = part;
+    }
+    __syncthreads();
+    if (threadIdx.x < 16) {
+      float total = 0.f;
+      for (int w = 0; w < waves; ++w) total += shares[w * 16 + threadIdx.x];
+      scales[threadIdx.x] = static_cast<int>(threadIdx.x) < a.rows ? rsqrtf(total / static_cast<float>(a.k) + a.eps) : 0.f;
+    }
+    __syncthreads();
+    auto normed = [&](float4 lo, float4 hi, float4 g0, float4 g1, float scale) {
+      const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      const float gains[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
+      uintx4 packed;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        packed[j] = bf16_bits(rounded<bf16_t>(v[2 * j] * scale) * gains[2 * j]) |
+                    (static_cast<uint32_t>(bf16_bits(rounded<bf16_t>(v[2 * j + 1] * scale) * gains[2 * j + 1])) << 16);
+      return packed;
+    };
+    const int pieces_per_row = a.k >> 3, pieces = a.rows * pieces_per_row;
+    for (int p = threadIdx.x; p < pieces; p += blockDim.x) {
+      const int row = p / pieces_per_row, piece = p - row * pieces_per_row;
+      const float* from = a.stream + static_cast<size_t>(row) * a.k + piece * 8;
+      rows_lds[piece * a.rows + row] =   // piece = k tile * 4 + chunk
+          normed(*reinterpret_cast<const float4*>(from), *reinterpret_cast<const float4*>(from + 4),
+                 *reinterpret_cast<const float4*>(a.gain + piece * 8), *reinterpret_cast<const float4*>(a.gain + piece * 8 + 4), scales[row]);
+    }
+    __syncthreads();
+  }
+
+  // the operand of the rows: lane (r, g) brings row r, 8 values at k = g * 8 of the k-tile.  Rows beyond `rows` read
+  // the last row again (their results are never stored); the chunks of a ragged last k-tile beyond k count as zero.
+  const int row_read = min(r, a.rows - 1);
+  const bool lane_outside = ragged && (a.k_tiles - 1) * 32 + g * 8 >= a.k;
+  uintx4 x0[U], x1[U];
+  auto fetch_rows = [&](int kt, uintx4 (&x)[U]) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int tile = min(kt + u, last_tile);
+      const int chunk = (lane_outside && tile == a.k_tiles - 1) ? 0 : g;
+      if constexpr (SCALED) x[u] = rows_lds[(tile * 4 + chunk) * a.rows + row_read];
+      else x[u] = *reinterpret_cast<const uintx4*>(a.x + static_cast<size_t>(row_read) * a.k + tile * 32 + chunk * 8);
+    }
+  };
+  auto multiply = [&](int kt, const uintx4 (&w)[RT][U], const uintx4 (&x)[U]) {
+    if (kt + U <= kt1 && !(ragged && kt + U == a.k_tiles)) {
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) acc[rt] = mfma16(w[rt][u], x[u], acc[rt]);
+    } else {   // the group at the end of the part: tiles beyond it are left out, the ragged last one loses its lanes
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (kt + u < kt1) {
+          const bool drop = lane_outside && kt + u == a.k_tiles - 1;
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) acc[rt] = mfma16(w[rt][u], drop ? zero : x[u], acc[rt]);
+        }
+    }
+  };
+  if (works) {
+    fetch_rows(kt0, x0);
+    int kt = kt0;
+    if (kt < kt1) {
+      for (; kt + 2 * U < kt1; kt += 2 * U) {   // both groups asked for here hold tiles of the part
+        fetch_weights(kt + U, w1);
+        fetch_rows(kt + U, x1);
+        multiply(kt, w0, x0);
+        fetch_weights(kt + 2 * U, w0);
+        fetch_rows(kt + 2 * U, x0);
+        multiply(kt + U, w1, x1);
+      }
+      if (kt + U < kt1) {
+        fetch_weights(kt + U, w1);
+        fetch_rows(kt + U, x1);
+        multiply(kt, w0, x0);
+        multiply(kt + U, w1, x1);
+      } else {
+        multiply(kt, w0, x0);
+      }
+    }
+  }
+
+  if (a.k_split > 1) {   // part 0 + part 1 + ...: every wave leaves its sums in LDS, the wave of part 0 adds them up
+    constexpr int kSet = RT * 4 * 64;
+    if constexpr (SCALED) __syncthreads();   // the rows have been read: their memory takes the sums
+    float* mine = red + static_cast<size_t>(wave) * kSet;
+    if (part != 0) {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mine[(rt * 4 + i) * 64 + lane] = acc[rt][i];
+    }
+    __syncthreads();
+    if (part != 0) return;
+    for (int other = 1; other < a.k_split; ++other) {
+      const float* theirs = mine + static_cast<size_t>(other) * kSet;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[rt][i] += theirs[(rt * 4 + i) * 64 + lane];
+    }
+  }
+  if (row_tile >= a.n_tiles) return;
+  if constexpr (ADDS) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const int tile = row_tile + rt;
+      if (tile >= a.n_tiles) break;
+      const int feature = tile * 16 + g * 4;
+      float squares = 0.f;
+      if (r < a.rows) {
+        float* at = a.stream_out + static_cast<size_t>(r) * a.outs + feature;
+        if (feature + 3 < a.outs && (a.outs & 3) == 0) {
+          float4 s = *reinterpret_cast<float4*>(at);
+          s.x += rounded<bf16_t>(acc[rt][0]);
+          s.y += rounded<bf16_t>(acc[rt][1]);
+          s.z += rounded<bf16_t>(acc[rt][2]);
+          s.w += rounded<bf16_t>(acc[rt][3]);
+          *reinterpret_cast<float4*>(at) = s;
+          squares = s.x * s.x + s.y * s.y + s.z * s.z + s.w * s.w;
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (feature + i < a.outs) {
+              const float s = at[i] + rounded<bf16_t>(acc[rt][i]);
+              at[i] = s;
+              squares += s * s;
+            }
+        }
+      }
+      squares += __shfl_xor(squares, 16, kWave);
+      squares += __shfl_xor(squares, 32, kWave);
+      if (g == 0) a.sums_out[tile * 16 + r] = squares;
+    }
+  } else if constexpr (GATED) {
+    store_tile<bf16_t>(a.y, silu_times(acc[0], acc[1]), r, (row_tile >> 1) * 16 + g * 4, a.rows, a.outs);
+  } else {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+      if (row_tile + rt < a.n_tiles) store_tile<bf16_t>(a.y, acc[rt], r, (row_tile + rt) * 16 + g * 4, a.rows, a.outs);
+  }
+}
+
+template <int RT, bool GATED, bool SCALED, bool ADDS>
+int launch_decode(DecodeArgs a, hipStream_t stream) {
+  // as many waves as the skinny kernel takes: k is split over the waves of a block while the row tiles are few
+  const int wave_rows = (a.n_tiles + RT - 1) / RT;
+  int k_split = 1;
+  while (k_split < 8) {
+    const int waves_now = wave_rows * k_split, part_after = a.k_tiles / (k_split * 2);
+    if (!((waves_now < 1536 && part_after >= 4) || (waves_now < 2048 && part_after >= 4 * kGroup))) break;
+    k_split *= 2;
+  }
+  // Waves per block: k_split * m for m wave-rows.  All blocks are resident at once and the compute units share the
+  // memory system evenly, so the product is over when the unit with the most blocks is: m is chosen so that the blocks
+  // spread evenly over the units (768 wave-rows: 3 per block make 256 blocks, one a unit) - and where that ties, a
+  // SCALED product takes the larger blocks (every block norms the rows for itself), the others the smaller.
+  constexpr int kUnits = 256, kMostWaves = 12;
+  int m = 1, best = 0;
+  for (int tried = 1; tried * k_split <= kMostWaves; ++tried) {
+    const int blocks_tried = (wave_rows + tried - 1) / tried;
+    const int longest = (blocks_tried + kUnits - 1) / kUnits * tried;   // wave-rows on the busiest unit
+    if (best == 0 || longest < best || (SCALED && longest == best)) best = longest, m = tried;
+  }
+  if (!SCALED && k_split < 4 && m * k_split < 4) m = (4 + k_split - 1) / k_split;   // blocks of at least 4 waves
+  const int waves = k_split * m;
+  const int rows_per_block = m;
+  const int blocks = (wave_rows + rows_per_block - 1) / rows_per_block;
+  a.k_split = k_split;
+  a.red_floats = k_split > 1 ? waves * RT * 4 * 64 : 0;
+  const size_t lds = max(static_cast<size_t>(a.red_floats) * 4, SCALED ? (12 * 16 + 16) * 4 + static_cast<size_t>(a.rows) * a.k * 2 : 0);
+  if (lds > kMaxLds) return -2;
+  if (lds > 64 * 1024) {   // more than a block may have without asking: asked once per kernel and device
+    static std::mutex guard;
+    static bool asked[64] = {};
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return -2;
+    std::lock_guard<std::mutex> lock(guard);
+    if (!asked[device]) {
+      const hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_decode_kernel<RT, GATED, SCALED, ADDS>),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLds));
+      if (status != hipSuccess) return static_cast<int>(status);
+      asked[device] = true;
+    }
+  }
+  linear_decode_kernel<RT, GATED, SCALED, ADDS><<<blocks, waves * 64, lds, stream>>>(a);
+  return AKV_LAUNCH_STATUS();
+}
+
+}  // namespace
+
+// stream_out [rows, outs] += bfloat16(x W^T) in place (float32); sums_out [n_tiles][16] receives, for every row tile of
+// 16 outputs and every row, the sum of squares of the new values (rows beyond `rows`: 0).  rows <= 16, k % 8 == 0.
+extern "C" int akv_linear_adds(const void* x, const void* wp, float* stream_out, float* sums_out, int rows, int outs,
+                               int k, int n_tiles, int k_tiles, hipStream_t stream) {
+  if (rows <= 0 || outs <= 0) return 0;
+  if (rows > 16 || (k & 7) != 0 || n_tiles * 16 < outs || (n_tiles - 1) * 16 >= outs || k_tiles * 32 < k) return -2;
+  DecodeArgs a{};
+  a.x = static_cast<const bf16_t*>(x);
+  a.wp = static_cast<const uintx4*>(wp);
+  a.stream_out = stream_out;
+  a.sums_out = sums_out;
+  a.rows = rows, a.outs = outs, a.k = k, a.k_tiles = k_tiles, a.n_tiles = n_tiles;
+  return launch_decode<1, false, false, true>(a, stream);
+}
+
+// y [rows, outs] = norm(stream) W^T (gated: y [rows, inter] = silu(. Wgate^T) * (. Wup^T), wp as for
+// akv_linear_packed_swiglu), where norm(stream) is what akv_add_rmsnorm gives for the float32 rows `stream` [rows, k]
+// and the weight `gain` [k] - with the rows' sums of squares not formed here but taken from `sums`
+// [sum_tiles][16] (what akv_linear_adds left: sum_tiles = ceil(k / 16)).  rows <= 16, k % 8 == 0, and the normed rows
+// (rows * k bfloat16) fit into a compute unit's LDS (160 KB) beside 832 bytes; -2 otherwise.
+extern "C" int akv_linear_scaled(const float* stream_in, const float* sums, int sum_tiles, const float* gain, float eps,
+                                 const void* wp, void* y, int rows, int outs, int k, int n_tiles, int k_tiles, int gated,
+                                 hipStream_t stream) {
+  if (rows <= 0 || outs <= 0) return 0;
+  if (rows > 16 || (k & 7) != 0 || k_tiles * 32 < k || sum_tiles != (k + 15) / 16) return -2;
+  if (gated ? ((outs & 15) != 0 || n_tiles * 8 != outs) : n_tiles * 16 < outs) return -2;
+  DecodeArgs a{};
+  a.stream = stream_in;
+  a.sums = sums;
+  a.sum_tiles = sum_tiles;
+  a.gain = gain;
+  a.eps = eps;
+  a.wp = static_cast<const uintx4*>(wp);
+  a.y = static_cast<bf16_t*>(y);
+  a.rows = rows, a.outs = outs, a.k = k, a.k_tiles = k_tiles, a.n_tiles = n_tiles;
+  if (gated) return launch_decode<2, true, true, false>(a, stream);
+  if (rows >= 4 && n_tiles >= 384 && n_tiles < 2048) return launch_decode<2, false, true, false>(a, stream);
+  return launch_decode<1, false, true, false>(a, stream);
+}

@@ -87,7 +87,7 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
 #pragma unroll
       for (int u = 0; u < U; ++u)
         early[rt][u] = (works && kt0 + u < kt1 && row_tile + rt < n_tiles)
-                           ? load_once(wp + (static_cast<size_t>(row_tile + rt) * k_tiles + kt0 + u) * 64 + lane) : none;
+                           ? load_once(wp + tile_index<GATED>(row_tile + rt, kt0 + u, k_tiles) * 64 + lane) : none;
     uint16_t* rows_lds = reinterpret_cast<uint16_t*>(red + norm.red_floats);
     // the waves share the rows: waves / rows of them take a row, each its own stride of the row's pieces of 8
     const int waves_per_row = max(1, waves / rows);
@@ -146,8 +146,11 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
   }
   if (works) {
     // Addresses: a scalar base per wave plus a 32-bit lane offset, so that a load is one instruction.
-    const size_t w_tile_row = static_cast<size_t>(k_tiles) * 1024;  // bytes of one row tile
-    const char* w_wave = reinterpret_cast<const char*>(wp) + static_cast<size_t>(row_tile) * w_tile_row;
+    // bytes from the wave's first row tile to its rt-th, and from a k-tile to the next (a gated pair lies side by side)
+    const size_t w_tile_bytes = static_cast<size_t>(k_tiles) * 1024;
+    auto w_of = [&](int rt) { return GATED ? (rt >> 1) * 2 * w_tile_bytes + (rt & 1) * 1024 : rt * w_tile_bytes; };
+    constexpr uint32_t kStep = GATED ? 2048u : 1024u;
+    const char* w_wave = reinterpret_cast<const char*>(wp) + tile_index<GATED>(row_tile, 0, k_tiles) * 1024;
     const uint32_t w_lane = lane * 16u;
     const char* x_bytes = reinterpret_cast<const char*>(x);
     const uint32_t x_step = x_packed ? 1024u : 64u;  // bytes from a k-tile's operand to the next
@@ -168,21 +171,21 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
     // which leaves the caches to the activations that every wave reads.
     uintx4 a0[RT][U], a1[RT][U], b0[MT][U], b1[MT][U];
     auto fetch = [&](int kt, uintx4 (&a)[RT][U], uintx4 (&b)[MT][U]) {
-      const char* w_at = w_wave + static_cast<size_t>(kt) * 1024;
+      const char* w_at = w_wave + static_cast<size_t>(kt) * kStep;
       const char* x_at = x_bytes + static_cast<size_t>(kt) * x_step;
       if (kt + U <= kt1 && row_tile + RT <= n_tiles) {  // the whole group exists: no test per load
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
           for (int u = 0; u < U; ++u)
-            a[rt][u] = load_once(reinterpret_cast<const uintx4*>(w_at + rt * w_tile_row + w_lane + u * 1024u));
+            a[rt][u] = load_once(reinterpret_cast<const uintx4*>(w_at + w_of(rt) + w_lane + u * kStep));
       } else {
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
           for (int u = 0; u < U; ++u)
             a[rt][u] = (kt + u < kt1 && row_tile + rt < n_tiles)
-                           ? load_once(reinterpret_cast<const uintx4*>(w_at + rt * w_tile_row + w_lane + u * 1024u)) : zero;
+                           ? load_once(reinterpret_cast<const uintx4*>(w_at + w_of(rt) + w_lane + u * kStep)) : zero;
       }
       if constexpr (NORMED) {  // the rows lie in LDS, normed: lane (r, g) reads row r, 16 bytes at k = g * 8 of the k-tile
         const char* rows_lds = reinterpret_cast<const char*>(red + norm.red_floats);
@@ -445,11 +448,10 @@ __global__ __launch_bounds__(256, 2) void linear_wide_kernel(const bf16_t* __res
     w_row[n] = tile0 + n < n_tiles;
     w_at[n] = lane * 16u;
   }
-  const size_t w_tile_row = static_cast<size_t>(k_tiles) * 1024;  // bytes of one row tile
   auto weights = [&](int kt, uintx4 (&a)[4]) {
 #pragma unroll
     for (int n = 0; n < 4; ++n) {
-      const char* at = w_bytes + (static_cast<size_t>(tile0 + n) * w_tile_row + static_cast<size_t>(kt) * 1024);
+      const char* at = w_bytes + tile_index<GATED>(tile0 + n, kt, k_tiles) * 1024;
       a[n] = (w_row[n] && kt < k_tiles) ? *reinterpret_cast<const uintx4*>(at + w_at[n]) : zero;
     }
   };

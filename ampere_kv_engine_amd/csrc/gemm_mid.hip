@@ -114,13 +114,13 @@ __global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_ker
 
   auto fetch_weights = [&](int stage, uintx4 (&a)[RT][S]) {
     const int kt = mine0 + stage * S;
-    const uintx4* at = wp + (static_cast<size_t>(tile0) * k_tiles + kt) * 64 + lane;
+    const uintx4* at = wp + lane;
     if (kt + S <= mine1 && tile0 + RT <= n_tiles) {   // the whole group exists: no test per load
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int u = 0; u < S; ++u) {
-          const uintx4* from = at + (static_cast<size_t>(rt) * k_tiles + u) * 64;
+          const uintx4* from = at + tile_index<GATED>(tile0 + rt, kt + u, k_tiles) * 64;
           a[rt][u] = shared_weights ? *from : load_once(from);
         }
     } else {
@@ -128,7 +128,7 @@ __global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_ker
       for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int u = 0; u < S; ++u) {
-          const uintx4* from = at + (static_cast<size_t>(rt) * k_tiles + u) * 64;
+          const uintx4* from = at + tile_index<GATED>(tile0 + rt, kt + u, k_tiles) * 64;
           a[rt][u] = (kt + u < mine1 && tile0 + rt < n_tiles) ? (shared_weights ? *from : load_once(from)) : zero;
         }
     }

@@ -18,6 +18,17 @@ __device__ __forceinline__ floatx4 mfma16(uintx4 a, uintx4 b, floatx4 c) {
 // A 16-byte read of data that is used once: it does not displace what others re-read from the caches.
 __device__ __forceinline__ uintx4 load_once(const uintx4* p) { return __builtin_nontemporal_load(p); }
 
+// Where tile (row_tile, kt) of a packed matrix lies, counted in tiles of 1 KB.  Plain: [row tile][k tile].  PAIRED (the
+// gated feed-forward's matrix, whose row tiles come in pairs of gate and up rows that one wave always owns together):
+// [pair][k tile][2] - the pair's two tiles of a k-tile lie side by side, so the wave streams ONE contiguous run of
+// memory along k instead of two runs a whole row tile apart (measured at 2 x 12,288 x 4,096: 39 -> 34 us for the
+// bare reads of a decode step's product).
+template <bool PAIRED>
+__host__ __device__ __forceinline__ size_t tile_index(int row_tile, int kt, int k_tiles) {
+  return PAIRED ? (static_cast<size_t>(row_tile >> 1) * k_tiles + kt) * 2 + (row_tile & 1)
+                : static_cast<size_t>(row_tile) * k_tiles + kt;
+}
+
 template <typename TY> __device__ __forceinline__ void store4(TY* p, floatx4 v);
 template <> __device__ __forceinline__ void store4<float>(float* p, floatx4 v) {
   *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);

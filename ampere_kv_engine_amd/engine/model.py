@@ -11,6 +11,7 @@ import torch
 
 from ..config.specs import ModelSpec
 from ..parts.base import PagedKV, Runtime, SlotState, build_part
+from ..parts.norm import StreamSums
 from ..weights.spec import TensorSpec
 
 
@@ -89,11 +90,18 @@ class Model:
             k.step_prologue(ctx)        # block-table changes and new lengths reach the device's persistent state
         self.embedding.forward(ctx.token_ids, ctx.stream, ctx)
         pending = None
-        for step_index, entry in enumerate(self.spec.run_order):
+        order = self.spec.run_order
+        for step_index, entry in enumerate(order):
             ctx.arena = arenas[step_index & 1]
             ctx.arena.reset()
+            # a block's last branch may add its output to the residual sum itself and hand on the rows' sums of squares
+            # instead, if whoever reads `pending` next knows what to make of that: the next block, or the end below
+            following = self.blocks[order[step_index + 1].layer] if step_index + 1 < len(order) else None
+            ctx.fold_into_stream = following is None or getattr(following, "takes_stream_sums", False)
             pending = self.blocks[entry.layer].forward(ctx.stream, pending, ctx, layer_cache[entry.cache_layer],
                                                        entry.writes_cache)
+        if isinstance(pending, StreamSums):      # the last branch's output is in the residual sum already
+            pending = None
         stream = ctx.stream
         wanted = ctx.logit_rows.shape[0]
         if wanted == 0:

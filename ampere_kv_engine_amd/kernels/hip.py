@@ -26,11 +26,13 @@ class KernelError(RuntimeError):
 
 class PackedWeight:
     """A bfloat16 matrix [outs, k] re-laid for the matrix cores: tiles of 16 rows x 32 k, 1 KB each, stored
-    [row tile][k tile][lane][8] with lane = (k chunk of 8) * 16 + row; rows and k beyond the matrix are zero."""
+    [row tile][k tile][lane][8] with lane = (k chunk of 8) * 16 + row; rows and k beyond the matrix are zero.
+    `paired` (an even number of row tiles): [pair of row tiles][k tile][2][lane][8] - the two tiles of a pair lie side
+    by side at every k-tile, for kernels in which one wave always owns both and so streams one run of memory."""
 
-    def __init__(self, matrix: torch.Tensor, keep_row_major: bool = False):
+    def __init__(self, matrix: torch.Tensor, keep_row_major: bool = False, paired: bool = False):
         outs, k = matrix.shape
-        self.outs, self.k = outs, k
+        self.outs, self.k, self.paired = outs, k, paired
         self.row_major = matrix if keep_row_major else None   # what a library product reads
         self.n_tiles, self.k_tiles = (outs + 15) // 16, (k + 31) // 32
         padded = matrix
@@ -39,17 +41,26 @@ class PackedWeight:
             padded[:outs, :k] = matrix
         self.data = (padded.view(self.n_tiles, 16, self.k_tiles, 4, 8).permute(0, 2, 3, 1, 4).contiguous()
                      .view(self.n_tiles, self.k_tiles, 512))
+        if paired:
+            if self.n_tiles % 2:
+                raise KernelError("a paired packing takes an even number of row tiles")
+            self.data = (self.data.view(self.n_tiles // 2, 2, self.k_tiles, 512).permute(0, 2, 1, 3).contiguous()
+                         .view(self.n_tiles, self.k_tiles, 512))     # (the shape no longer says where a tile lies)
         self.dtype, self.device, self.shape = matrix.dtype, matrix.device, (outs, k)
 
     def unpack(self) -> torch.Tensor:
         """The matrix back in row-major order (for checks)."""
-        full = self.data.view(self.n_tiles, self.k_tiles, 4, 16, 8).permute(0, 3, 1, 2, 4)
+        data = self.data
+        if self.paired:
+            data = data.view(self.n_tiles // 2, self.k_tiles, 2, 512).permute(0, 2, 1, 3).reshape(self.n_tiles, self.k_tiles, 512)
+        full = data.view(self.n_tiles, self.k_tiles, 4, 16, 8).permute(0, 3, 1, 2, 4)
         return full.reshape(self.n_tiles * 16, self.k_tiles * 32)[:self.outs, :self.k].contiguous()
 
 
 class GatedWeight:
     """Gate and up matrices [inter, k] of a gated feed-forward as ONE packed matrix whose row tiles alternate:
-    tile 2t holds gate rows 16t .. 16t + 15, tile 2t + 1 the up rows of the same features."""
+    tile 2t holds gate rows 16t .. 16t + 15, tile 2t + 1 the up rows of the same features; the packing is `paired`,
+    so the wave that owns both reads them as one run."""
 
     def __init__(self, gate: torch.Tensor, up: torch.Tensor, keep_row_major: bool = False):
         inter, k = gate.shape
@@ -57,7 +68,7 @@ class GatedWeight:
         # what a library product reads: gate rows, then up rows
         self.stacked = torch.cat((gate, up), dim=0).contiguous() if keep_row_major else None
         paired = torch.stack((gate.view(inter // 16, 16, k), up.view(inter // 16, 16, k)), dim=1).reshape(2 * inter, k)
-        self.packed = PackedWeight(paired)
+        self.packed = PackedWeight(paired, paired=True)
 
     def unpack(self) -> tuple[torch.Tensor, torch.Tensor]:
         paired = self.packed.unpack().view(self.inter // 16, 2, 16, self.k)
@@ -125,6 +136,7 @@ class HipKernels:
                      "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
                      "akv_linear_tiled", "akv_linear_packed", "akv_linear_packed_swiglu", "akv_linear_packed_normed",
                      "akv_pack_rows", "akv_linear_packed_static", "akv_linear_mid", "akv_linear_mid_workspace",
+                     "akv_linear_adds", "akv_linear_scaled",
                      "akv_attention_rows", "akv_decode_plan", "akv_sample", "akv_sample_slots", "akv_step_prologue"):
             getattr(self.lib, name).restype = ctypes.c_int
 
@@ -423,6 +435,58 @@ class HipKernels:
         self._dense(out, "out", None, (rows, outs))
         self._check(self.lib.akv_linear_tiled(_ptr(x), _code(x), _ptr(weight), _code(weight), _ptr(out), _code(out),
                                               rows, outs, k, self._stream()), "linear")
+
+    # ---- decode steps: the residual sum and the norm inside the products -----------------------------------------
+    FOLD_NORM_ROWS = 8              # steps of up to this many rows fold the residual sum and the norm into products
+                                    # (the kernels take 16; measured at 1 and 8 rows, where it is no loss)
+    FOLD_NORM_BYTES = 160 * 1024 - 832   # ... while the normed rows fit into a compute unit's LDS beside the scales
+    fold_norms = True
+
+    def folds_norm(self, rows: int, hidden: int, dtype) -> bool:
+        """Whether a step of `rows` rows may let a branch's last product add itself to the residual sum
+        (`linear_adds`) and the next product norm its rows itself from the sums left there (`linear_scaled`)."""
+        return (self.fold_norms and 0 < rows <= self.FOLD_NORM_ROWS and dtype == torch.bfloat16 and hidden % 8 == 0
+                and rows * hidden * 2 <= self.FOLD_NORM_BYTES)
+
+    def adds_to_stream(self, rows: int, weight, dtype) -> bool:
+        return isinstance(weight, PackedWeight) and self.folds_norm(rows, weight.outs, dtype)
+
+    def norms_rows_in_product(self, rows: int, weight, dtype) -> bool:
+        packed = weight.packed if isinstance(weight, GatedWeight) else weight
+        return isinstance(packed, PackedWeight) and self.folds_norm(rows, packed.k, dtype)
+
+    def linear_adds(self, x, weight: PackedWeight, stream, sums) -> None:
+        """stream [rows, outs] (float32) += bfloat16(x W^T), in place; sums [ceil(outs / 16), 16] (float32) receives
+        per tile of 16 outputs and row the sum of squares of the new values."""
+        rows = x.shape[0]
+        if not isinstance(weight, PackedWeight) or rows > 16:
+            raise KernelError("the product that adds to the residual sum takes a packed matrix and up to 16 rows")
+        self._dense(x, "x", torch.bfloat16, (rows, weight.k))
+        self._dense(stream, "stream", torch.float32, (rows, weight.outs))
+        self._dense(sums, "sums", torch.float32, ((weight.outs + 15) // 16, 16))
+        self._dense(weight.data, "packed weight", torch.bfloat16)
+        self._check(self.lib.akv_linear_adds(_ptr(x), _ptr(weight.data), _ptr(stream), _ptr(sums), rows, weight.outs,
+                                             weight.k, weight.n_tiles, weight.k_tiles, self._stream()), "linear_adds")
+
+    def linear_scaled(self, stream, sums, norm_weight, eps, weight, out) -> None:
+        """out = norm(stream) W^T (a `GatedWeight`: silu(. Wgate^T) * (. Wup^T)) with the norm of `add_rmsnorm`
+        (scaled, rounded, times the weight, rounded) applied to the float32 rows as they become operands; the rows'
+        sums of squares are not formed but added up from `sums`, as `linear_adds` left them."""
+        gated = isinstance(weight, GatedWeight)
+        packed = weight.packed if gated else weight
+        rows, k = stream.shape
+        if not isinstance(packed, PackedWeight) or rows > 16 or k != packed.k:
+            raise KernelError("the product that norms its rows takes a packed matrix of the rows' width and up to 16 rows")
+        self._dense(stream, "stream", torch.float32, (rows, k))
+        self._dense(sums, "sums", torch.float32, ((k + 15) // 16, 16))
+        self._dense(norm_weight, "norm weight", torch.float32, (k,))
+        outs = weight.inter if gated else packed.outs
+        self._dense(out, "out", torch.bfloat16, (rows, outs))
+        self._dense(packed.data, "packed weight", torch.bfloat16)
+        self._check(self.lib.akv_linear_scaled(_ptr(stream), _ptr(sums), (k + 15) // 16, _ptr(norm_weight),
+                                               ctypes.c_float(eps), _ptr(packed.data), _ptr(out), rows, outs, k,
+                                               packed.n_tiles, packed.k_tiles, 1 if gated else 0, self._stream()),
+                    "linear_scaled")
 
     STATIC_ROWS_ELEMENTS = 64 * 32768   # bfloat16 elements of the library's static device memory for repacked rows
 

@@ -94,6 +94,10 @@ class Attention(Part):
             self._encode_with_parts(qkv, q, ctx, meta, cache, writes_cache)
             k.attention(q, cache.k, cache.v, ctx, meta, self.q_heads, self.kv_heads, self.head_dim,
                         self.scale, self.window, merged)
+        if getattr(ctx, "fold_into_stream", False):     # the output product adds itself to the residual sum
+            sums = self.out.add_to_stream(merged, ctx)
+            if sums is not None:
+                return sums
         out = ctx.arena.take((tokens, self.hidden), self.rt.dtype)
         return self.out.forward(merged, out)
 

@@ -1,15 +1,19 @@
 """Arrangement of a layer's parts.  `prenorm` (ampere_kv/runner.py:117-121, :165-179):
     h1 = h + mixer(norm_a(h));  h2 = h1 + feed_forward(norm_b(h1))
 The residual sum `stream` is float32.  A branch's output is not added by itself: it is handed on as
-`pending` and added inside the next norm's kernel, which reads the stream anyway."""
+`pending` and added inside the next norm's kernel, which reads the stream anyway.  In steps of few rows a branch
+may instead add its output to the stream inside its last product and hand on the rows' sums of squares
+(`StreamSums`); the next norm then happens inside the product that reads it, and the layer launches no norm kernel."""
 
 from __future__ import annotations
 
 from .base import Part, build_part, register_part
+from .norm import StreamSums
 
 
 class PreNormBlock(Part):
     graph_safe = True
+    takes_stream_sums = True        # `pending` may be a `StreamSums`: the stream then already holds the branch's output
 
     def __init__(self, spec, runtime, mixer, feed_forward):
         self.rt = runtime
@@ -38,19 +42,33 @@ class PreNormBlock(Part):
     def forward(self, stream, pending, ctx, cache, writes_cache=True):
         """stream [tokens, hidden] float32 (updated in place); pending: the previous branch's output, not
         yet added, or None.  Returns this block's own pending output."""
-        normed, unnormed = self._normed(self.mixer_norm, self.mixer, stream, pending, ctx)
+        folds = getattr(self.rt.kernels, "folds_norm", None)
+        fold = folds is not None and folds(stream.shape[0], self.hidden, self.rt.dtype)
+        later = ctx.fold_into_stream if hasattr(ctx, "fold_into_stream") else False   # whoever comes next takes sums
+        normed, unnormed = self._normed(self.mixer_norm, self.mixer, stream, pending, ctx, fold)
+        ctx.fold_into_stream = fold         # the mixer's output meets this block's own second norm
         mixed = self.mixer.forward(normed, ctx, cache, writes_cache)
         stream = self._after(unnormed, stream, ctx)
-        normed, unnormed = self._normed(self.feed_forward_norm, self.feed_forward, stream, mixed, ctx)
+        normed, unnormed = self._normed(self.feed_forward_norm, self.feed_forward, stream, mixed, ctx, fold)
+        ctx.fold_into_stream = fold and later
         out = self.feed_forward.forward(normed, ctx)
+        ctx.fold_into_stream = later
         self._after(unnormed, stream, ctx)
         return out
 
-    def _normed(self, norm, reader, stream, delta, ctx):
+    def _normed(self, norm, reader, stream, delta, ctx, fold=False):
         """norm(stream + delta) for `reader`: computed now - or, in steps of few rows (the context then has a spare
         buffer for the residual sum), handed on unnormed to a reader that can take that, whose first product may
         norm the rows itself: one launch less."""
-        spare = getattr(ctx, "spare_stream", None)
+        if isinstance(delta, StreamSums):    # the stream holds the branch's output already; its sums of squares are known
+            if getattr(reader, "takes_pending_norm", False) and hasattr(norm, "scaled"):
+                unnormed = norm.scaled(stream, delta, ctx.arena)
+                return unnormed, unnormed
+            normed = ctx.arena.take((stream.shape[0], self.hidden), self.rt.dtype)
+            norm.forward_residual(stream, None, normed)
+            return normed, None
+        # (while branches add themselves to the stream it stays in its buffer: a branch finds it through the context)
+        spare = None if fold else getattr(ctx, "spare_stream", None)
         if spare is not None and getattr(reader, "takes_pending_norm", False) and hasattr(norm, "pending"):
             unnormed = norm.pending(stream, delta, spare, ctx.arena)
             return unnormed, unnormed

@@ -59,6 +59,10 @@ class SwiGLU(Part):
             gate_up = ctx.arena.take((tokens, 2 * self.inter), self.rt.dtype)
             self.gate_up.forward(x, gate_up)
             self.rt.kernels.swiglu(gate_up, act)
+        if getattr(ctx, "fold_into_stream", False):     # the down product adds itself to the residual sum
+            sums = self.down.add_to_stream(act, ctx)
+            if sums is not None:
+                return sums
         out = ctx.arena.take((tokens, self.hidden), self.rt.dtype)
         return self.down.forward(act, out)
 

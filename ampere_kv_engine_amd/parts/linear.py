@@ -48,6 +48,20 @@ class Linear(Part):
     def weight_bytes(self):
         return self._bytes
 
+    def add_to_stream(self, x: torch.Tensor, ctx):
+        """stream += x W^T (rounded to the activation dtype first, as a stored result would be), where the kernel set
+        has a product that does that for a step of this size: returns the `StreamSums` the product left, or None -
+        then the caller computes `forward` and hands its output on as before."""
+        kernels = self.rt.kernels
+        can = getattr(kernels, "adds_to_stream", None)
+        stream = getattr(ctx, "stream", None)
+        if can is None or stream is None or not can(x.shape[0], self.weight, self.rt.dtype) or stream.shape[1] != self.total_out:
+            return None
+        from .norm import StreamSums
+        sums = ctx.arena.take(((self.total_out + 15) // 16, 16), torch.float32)
+        kernels.linear_adds(x, self.weight, stream, sums)
+        return StreamSums(sums)
+
     def forward(self, x, out: torch.Tensor) -> torch.Tensor:
         """x: [rows, in] in the activation dtype, or rows that are still to be normed (`PendingNorm`)."""
         if hasattr(x, "product"):

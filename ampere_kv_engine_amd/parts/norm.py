@@ -42,6 +42,53 @@ class RMSNorm(Part):
         """`forward_residual` not yet computed: for a consumer whose first product can compute it itself."""
         return PendingNorm(self, stream, delta, stream_out, arena)
 
+    def scaled(self, stream: torch.Tensor, sums: "StreamSums", arena) -> "ScaledNorm":
+        """The norm of a residual sum whose rows' sums of squares are already known (`StreamSums`): for a consumer
+        whose first product can norm its rows itself from them."""
+        return ScaledNorm(self, stream, sums, arena)
+
+
+class StreamSums:
+    """What a branch hands on instead of its output when its last product has already added that output to the
+    residual sum (`Linear.add_to_stream`): the partial sums of squares of the new residual rows, float32
+    `[ceil(width / 16), 16]`, from which the next norm's scale follows without a pass over the rows."""
+
+    def __init__(self, sums: torch.Tensor):
+        self.sums = sums
+
+
+class ScaledNorm:
+    """norm(stream) for a stream whose sums of squares are at hand, before anybody has computed it.  Like
+    `PendingNorm` it is read exactly once, through a `Linear` or the gated product: where the kernel set's product
+    norms its rows itself (`linear_scaled`) it does; otherwise the rows are normed by the norm's own kernel."""
+
+    moved = False               # the residual sum stays where it is
+
+    def __init__(self, norm: RMSNorm, stream, sums: StreamSums, arena):
+        self.norm, self.stream, self.sums, self.arena = norm, stream, sums, arena
+        self.shape = (stream.shape[0], norm.size)
+        self.dtype = norm.rt.dtype
+        self._used = False
+
+    def _once(self):
+        if self._used:
+            raise RuntimeError("rows that were handed on unnormed can be read once")
+        self._used = True
+
+    def product(self, weight, out: torch.Tensor) -> bool:
+        kernels = self.norm.rt.kernels
+        can = getattr(kernels, "norms_rows_in_product", None)
+        if can is None or not can(self.shape[0], weight, out.dtype):
+            return False
+        self._once()
+        kernels.linear_scaled(self.stream, self.sums.sums, self.norm.weight, self.norm.eps, weight, out)
+        return True
+
+    def rows(self) -> torch.Tensor:
+        self._once()
+        out = self.arena.take(self.shape, self.dtype)
+        return self.norm.forward_residual(self.stream, None, out)
+
 
 class PendingNorm:
     """The rows norm(stream + delta) before anybody has computed them.  A part that `takes_pending_norm` reads them

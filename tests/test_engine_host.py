@@ -20,3 +20,33 @@ def engine(case):
 @pytest.mark.parametrize("cutting", [n[5:] for n in dir(cases) if n.startswith("case_")])
 def test_cutting(engine, case, cutting):
     getattr(cases, "case_" + cutting)(engine, case)
+
+
+def test_branches_that_add_themselves_to_the_residual_sum_give_the_same_bits(case):
+    """In steps of few rows a branch's last product may add its output to the residual sum itself and the next product
+    norm its rows from the sums of squares left there (what the HIP kernel set does in decode steps).  With a double
+    that offers the same two products, the parts take that path - and the logits are bit for bit those of the
+    ordinary path: the arithmetic is the same, only the kernels' borders have moved."""
+    import schedules
+    calls = {"adds": 0, "scaled": 0}
+
+    class Counting(TorchKernels):
+        def linear_adds(self, *args):
+            calls["adds"] += 1
+            return super().linear_adds(*args)
+
+        def linear_scaled(self, *args):
+            calls["scaled"] += 1
+            return super().linear_scaled(*args)
+
+    ordinary = cases.make_engine(case, "bfloat16", "cpu", kernels=TorchKernels())
+    folding = cases.make_engine(case, "bfloat16", "cpu", kernels=Counting(fold_rows=16))
+    schedule = schedules.mixed(case["requests"], cases.PROMPTS, case["page_size"], folding.config.num_pages, seed=5)
+    want, _ = schedules.run(ordinary, case["requests"], schedule)
+    got, _ = schedules.run(folding, case["requests"], schedule)
+    layers = case["raw"]["num_hidden_layers"]
+    small_steps = sum(1 for entries, _ in schedule if sum(count for _, count in entries) <= 16)
+    assert calls["adds"] == 2 * layers * small_steps              # both branches of every layer
+    assert calls["scaled"] == (2 * layers - 1) * small_steps      # every norm but the first, which meets no sums yet
+    for name in want:
+        assert (got[name] == want[name]).all(), name

@@ -56,6 +56,19 @@ def tol(dtype):
     return dict(rtol=2e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=1.6e-2, atol=1e-3)
 
 
+def assert_close_but_for_flipped_roundings(got, want):
+    """A product whose rows were normed with the squares added in another order: a normed value on a rounding
+    boundary now and then falls to the other side (one bfloat16 step of a value of size ~1 to 4), which moves a whole
+    output row by that step times a weight.  So: nearly all outputs within the usual limit, none further off than a
+    small part of the largest output."""
+    got, want = got.float().cpu(), want.float().cpu()
+    t = tol(torch.bfloat16)
+    outside = (got - want).abs() > t["atol"] + t["rtol"] * want.abs()
+    assert outside.float().mean() < 1e-3, f"{int(outside.sum())} of {outside.numel()} outside the usual limit"
+    beyond = ((got - want).abs() - t["rtol"] * want.abs()).clamp(min=0).max()
+    assert beyond <= 2.0 ** -9 * want.abs().max(), "an output is off by more than a flipped rounding explains"
+
+
 def attention_tol(dtype):
     """bfloat16: the reference's own bound for its paged attention against float32 attention
     (ampere_kv/scheduler.py:410, ampere_kv/paged_decode.py:62-81: rtol 0.01, atol 0.002); softmax weights enter the
@@ -270,6 +283,98 @@ def test_gated_linear_after_norm(hip, ref, rows):
         del hip.NORM_IN_PRODUCT_ROWS
     torch.testing.assert_close(got.cpu().float(), want.float(), **tol(torch.bfloat16))
     torch.testing.assert_close(new.cpu(), want_stream, rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("rows", [1, 3, 8, 16])
+@pytest.mark.parametrize("outs,k", [(320, 256), (4096, 4096), (520, 48), (4096, 12288), (1000, 1032), (5120, 3416)])
+def test_a_product_adds_itself_to_the_residual_sum_and_leaves_its_rows_sums_of_squares(hip, ref, rows, outs, k, monkeypatch):
+    """`linear_adds` against the product followed by the sum: the new residual rows are the same bits (the product is
+    rounded to bfloat16 before it is added, as a stored one would be), and the partial sums add up to the rows' sums of
+    squares.  Widths that are no multiple of 16 or 32, a k that is cut over the waves of a block, and one that is not."""
+    monkeypatch.setattr(hip, "fold_norms", True)
+    monkeypatch.setattr(hip, "FOLD_NORM_ROWS", 16)       # what the kernels take; the engine folds steps of fewer rows
+    stream = rand(rows, outs, seed=71, scale=2.0)
+    x = rand(rows, k, dtype=torch.bfloat16, seed=72)
+    w = rand(outs, k, dtype=torch.bfloat16, seed=73, scale=0.05)
+    y = torch.empty(rows, outs, dtype=torch.bfloat16)
+    ref.linear(x, w, y)
+    packed = hip.prepare_linear(w.cuda())
+    # (the engine folds only where the next product can hold the normed rows in LDS; the kernel takes any 16 rows)
+    assert hip.adds_to_stream(rows, packed, torch.bfloat16) == (rows * outs * 2 <= hip.FOLD_NORM_BYTES)
+    assert not hip.adds_to_stream(17, packed, torch.bfloat16)
+    got = stream.cuda()
+    tiles = (outs + 15) // 16
+    sums = torch.full((tiles, 16), float("nan"), device="cuda")
+    hip.linear_adds(x.cuda(), packed, got, sums)
+    mine = torch.empty(rows, outs, dtype=torch.bfloat16, device="cuda")
+    hip.linear(x.cuda(), packed, mine)          # the same tiles, maybe another cut of k: a last bit here and there
+    apart = (got.cpu() - (stream + mine.cpu().float())).abs()
+    assert (apart > 0).float().mean() < 0.01 and apart.max() <= 2.0 ** -7 * mine.float().abs().max().item()
+    torch.testing.assert_close(got.cpu(), stream + y.float(), rtol=0, atol=2.0 ** -7 * y.float().abs().max().item())
+    sums = sums.cpu()
+    assert torch.isfinite(sums).all() and (sums[:, rows:] == 0).all()
+    padded = torch.zeros(rows, tiles * 16)
+    padded[:, :outs] = got.cpu()
+    want_sums = padded.double().pow(2).reshape(rows, tiles, 16).sum(-1).T
+    torch.testing.assert_close(sums[:, :rows].double(), want_sums, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("rows,outs,k", [(1, 320, 256), (16, 320, 256), (2, 6144, 4096), (8, 6144, 4096), (5, 48, 520),
+                                         (16, 48, 520), (6, 4096, 5120), (1, 1000, 1032), (13, 1000, 1032),
+                                         (11, 256, 96), (10, 400, 96), (16, 12288, 4096), (3, 512, 10240), (7, 512, 10240)])
+def test_a_product_norms_its_rows_from_the_sums_of_squares_it_is_given(hip, ref, rows, outs, k, monkeypatch):
+    """`linear_scaled` against the norm kernel followed by the product.  The sums it is given are those of another
+    product's `linear_adds`, so the pair is what a layer runs; the residual rows are left as they are."""
+    monkeypatch.setattr(hip, "fold_norms", True)
+    monkeypatch.setattr(hip, "FOLD_NORM_ROWS", 16)       # what the kernels take; the engine folds steps of fewer rows
+    stream = rand(rows, k, seed=74, scale=2.0)
+    x = rand(rows, 64, dtype=torch.bfloat16, seed=75)
+    before = rand(k, 64, dtype=torch.bfloat16, seed=76, scale=0.2)
+    gain = 1 + rand(k, seed=77, scale=0.1)
+    w = rand(outs, k, dtype=torch.bfloat16, seed=78, scale=0.05)
+    residual = stream.cuda()
+    sums = torch.full(((k + 15) // 16, 16), float("nan"), device="cuda")
+    hip.linear_adds(x.cuda(), hip.prepare_linear(before.cuda()), residual, sums)
+    rows_now = residual.cpu()
+    normed, want = torch.empty(rows, k, dtype=torch.bfloat16), torch.empty(rows, outs, dtype=torch.bfloat16)
+    ref.add_rmsnorm(rows_now.clone(), None, gain, 1e-5, normed)
+    ref.linear(normed, w, want)
+    packed = hip.prepare_linear(w.cuda())
+    assert hip.norms_rows_in_product(rows, packed, torch.bfloat16)
+    assert not hip.norms_rows_in_product(hip.FOLD_NORM_BYTES // (2 * k) + 1, packed, torch.bfloat16)     # the rows must fit into LDS
+    got = torch.full((rows, outs), float("nan"), dtype=torch.bfloat16, device="cuda")
+    hip.linear_scaled(residual, sums, gain.cuda(), 1e-5, packed, got)
+    assert_close_but_for_flipped_roundings(got, want)
+    torch.testing.assert_close(residual.cpu(), rows_now, rtol=0, atol=0)
+    # against this kernel set's own norm and product the difference is a last bit of a normed value here and there
+    mine_normed = torch.empty(rows, k, dtype=torch.bfloat16, device="cuda")
+    hip.add_rmsnorm(residual.clone(), None, gain.cuda(), 1e-5, mine_normed)
+    mine = torch.empty(rows, outs, dtype=torch.bfloat16, device="cuda")
+    hip.linear(mine_normed, packed, mine)
+    assert (got.float() - mine.float()).abs().max() <= 0.02 * mine.float().abs().max()
+    assert (got != mine).float().mean() < 0.05
+
+
+@pytest.mark.parametrize("rows,inter,k", [(1, 208, 264), (16, 208, 264), (7, 12288, 4096), (8, 1008, 520), (16, 1008, 520)])
+def test_a_gated_product_norms_its_rows_from_the_sums_of_squares(hip, ref, rows, inter, k, monkeypatch):
+    monkeypatch.setattr(hip, "fold_norms", True)
+    monkeypatch.setattr(hip, "FOLD_NORM_ROWS", 16)       # what the kernels take; the engine folds steps of fewer rows
+    inter = (inter + 15) // 16 * 16
+    residual = rand(rows, k, seed=79, scale=2.0).cuda()
+    gain = 1 + rand(k, seed=80, scale=0.1)
+    gate, up = (rand(inter, k, dtype=torch.bfloat16, seed=81 + i, scale=0.05) for i in range(2))
+    padded = torch.zeros(rows, (k + 15) // 16 * 16)
+    padded[:, :k] = residual.cpu()
+    sums = torch.zeros((k + 15) // 16, 16)
+    sums[:, :rows] = padded.pow(2).reshape(rows, -1, 16).sum(-1).T
+    normed, want = torch.empty(rows, k, dtype=torch.bfloat16), torch.empty(rows, inter, dtype=torch.bfloat16)
+    ref.add_rmsnorm(residual.cpu().clone(), None, gain, 1e-6, normed)
+    ref.gated_linear(normed, ref.prepare_gated_linear(gate, up), want)
+    weight = hip.prepare_gated_linear(gate.cuda(), up.cuda())
+    assert hip.norms_rows_in_product(rows, weight, torch.bfloat16)
+    got = torch.full((rows, inter), float("nan"), dtype=torch.bfloat16, device="cuda")
+    hip.linear_scaled(residual, sums.cuda(), gain.cuda(), 1e-6, weight, got)
+    assert_close_but_for_flipped_roundings(got, want)
 
 
 def test_products_of_17_to_512_rows_follow_a_table_that_is_measured_on_request(hip, ref, tmp_path):

@@ -21,6 +21,11 @@ def _round(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
 class TorchKernels:
     name = "torch-double"
 
+    def __init__(self, fold_rows: int = 0):
+        """`fold_rows`: steps of up to this many rows let a branch's last product add itself to the residual sum and
+        the next product norm its rows itself, as the HIP kernel set does in decode steps (0: never)."""
+        self.fold_rows = fold_rows
+
     def check_attention_sizes(self, q_heads, kv_heads, head_dim, page_size):
         if q_heads % kv_heads:
             raise ValueError("q_heads must be a multiple of kv_heads")
@@ -74,6 +79,36 @@ class TorchKernels:
 
     def prepare_gated_linear(self, gate, up):
         return (gate, up)
+
+    # ---- the residual sum and the norm inside the products (decode steps) -------------------------------
+    def folds_norm(self, rows, hidden, dtype):
+        return 0 < rows <= self.fold_rows and dtype == torch.bfloat16
+
+    def adds_to_stream(self, rows, weight, dtype):
+        return isinstance(weight, torch.Tensor) and self.folds_norm(rows, weight.shape[0], dtype)
+
+    def norms_rows_in_product(self, rows, weight, dtype):
+        matrix = weight[0] if isinstance(weight, tuple) else weight
+        return isinstance(matrix, torch.Tensor) and self.folds_norm(rows, matrix.shape[1], dtype)
+
+    def linear_adds(self, x, weight, stream, sums):
+        y = torch.empty(x.shape[0], weight.shape[0], dtype=x.dtype)
+        self.linear(x, weight, y)
+        stream += y.float()
+        rows, outs = stream.shape
+        padded = torch.zeros(rows, sums.shape[0] * 16)
+        padded[:, :outs] = stream
+        sums.zero_()
+        sums[:, :rows] = (padded * padded).view(rows, -1, 16).sum(-1).T
+
+    def linear_scaled(self, stream, sums, norm_weight, eps, weight, out):
+        rows, k = stream.shape
+        scale = torch.rsqrt(sums.sum(0)[:rows, None] / k + eps)
+        normed = _round(_round(stream * scale, out.dtype).float() * norm_weight, out.dtype)
+        if isinstance(weight, tuple):
+            self.gated_linear(normed, weight, out)
+        else:
+            self.linear(normed, weight, out)
 
     def gated_scratch(self, weight, rows, dtype):
         return None
