@@ -20,6 +20,9 @@ int akv_copy_rows(const void* x, long token_stride, void* out, int dtype, long t
 int akv_gather_rows(const float* stream_buf, const void* pending, int dtype, const int* rows, float* out, int wanted,
                     int hidden, int tokens, hipStream_t stream);
 int akv_swiglu(const void* gate_up, void* out, int dtype, long tokens, int inter, hipStream_t stream);
+// Reads `bytes` (a multiple of 16) once, as the decode products read their weights, and leaves the xor of the words a
+// block read in out[block]: a measure of what memory gives to a kernel that does nothing else.
+int akv_read_probe(const void* data, long bytes, unsigned int* out, int blocks, hipStream_t stream);
 int akv_rope_table(const float* inv_freq, float* table, int positions, int half, hipStream_t stream);
 int akv_rope(void* x, int dtype, const int* positions, const float* table, long tokens, int heads, int dim,
              int table_positions, hipStream_t stream);

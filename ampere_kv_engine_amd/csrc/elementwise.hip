@@ -466,6 +466,35 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
 
 inline unsigned blocks_for(long items, int per_block) { return static_cast<unsigned>((items + per_block - 1) / per_block); }
 
+// What a kernel that only reads can draw from memory: every wave walks its own contiguous span in pieces of 1 KB, eight
+// loads in flight, marked as read-once - the access pattern of the decode products' weights without any of their work.
+// The words are folded with xor, a word per block, so that the reads cannot be dropped and a test can check them.
+typedef unsigned int probe_uintx4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void read_probe_kernel(const probe_uintx4* __restrict__ data, long pieces, unsigned int* out) {
+  constexpr int U = 8;
+  __shared__ unsigned int folded[4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const long waves = static_cast<long>(gridDim.x) * 4, tiles = pieces / 64;   // a tile: 64 pieces of 16 bytes
+  const long mine = static_cast<long>(blockIdx.x) * 4 + wave;
+  const long t0 = tiles * mine / waves, t1 = tiles * (mine + 1) / waves;
+  unsigned int word = 0;
+  for (long t = t0; t < t1; t += U) {
+    probe_uintx4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(data + min(t + u, t1 - 1) * 64 + lane);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (t + u < t1) word ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+  }
+  if (mine == waves - 1)   // the pieces beyond the last whole tile
+    for (long p = tiles * 64 + lane; p < pieces; p += 64) word ^= data[p].x ^ data[p].y ^ data[p].z ^ data[p].w;
+#pragma unroll
+  for (int offset = 32; offset > 0; offset >>= 1) word ^= __shfl_xor(word, offset, kWave);
+  if (lane == 0) folded[wave] = word;
+  __syncthreads();
+  if (threadIdx.x == 0) out[blockIdx.x] = folded[0] ^ folded[1] ^ folded[2] ^ folded[3];
+}
+
 }  // namespace
 
 extern "C" {
@@ -537,6 +566,12 @@ int akv_gather_rows(const float* stream_buf, const void* pending, int dtype, con
   AKV_DISPATCH(dtype, T,
                gather_rows_kernel<T><<<wanted, 256, 0, stream>>>(stream_buf, static_cast<const T*>(pending), rows, out,
                                                                  hidden, tokens));
+  return AKV_LAUNCH_STATUS();
+}
+
+int akv_read_probe(const void* data, long bytes, unsigned int* out, int blocks, hipStream_t stream) {
+  if (bytes <= 0 || (bytes & 15) != 0 || blocks <= 0) return -2;
+  read_probe_kernel<<<blocks, 256, 0, stream>>>(static_cast<const probe_uintx4*>(data), bytes / 16, out);
   return AKV_LAUNCH_STATUS();
 }
 

@@ -136,7 +136,7 @@ class HipKernels:
                      "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
                      "akv_linear_tiled", "akv_linear_packed", "akv_linear_packed_swiglu", "akv_linear_packed_normed",
                      "akv_pack_rows", "akv_linear_packed_static", "akv_linear_mid", "akv_linear_mid_workspace",
-                     "akv_linear_adds", "akv_linear_scaled",
+                     "akv_linear_adds", "akv_linear_scaled", "akv_read_probe",
                      "akv_attention_rows", "akv_decode_plan", "akv_sample", "akv_sample_slots", "akv_step_prologue"):
             getattr(self.lib, name).restype = ctypes.c_int
 
@@ -263,6 +263,21 @@ class HipKernels:
             code = _code(pending)
         self._check(self.lib.akv_gather_rows(_ptr(stream), _ptr(pending), code, _ptr(rows), _ptr(out), wanted, hidden,
                                              tokens, self._stream()), "gather_rows")
+
+    def read_probe(self, data: torch.Tensor, out: torch.Tensor | None = None, blocks: int | None = None) -> torch.Tensor:
+        """Reads `data` once the way the decode products read their weights (a contiguous span per wave, loads marked
+        as read-once) and returns the xor of its 32-bit words per block, int32 [blocks]: timed over memory that no cache
+        holds, it says what a kernel that only reads can draw - the ceiling the products are measured against."""
+        self._dense(data, "data", None)
+        size = data.numel() * data.element_size()
+        if size % 16:
+            raise KernelError("the read probe takes a multiple of 16 bytes")
+        blocks = blocks or 4 * self.compute_units
+        if out is None:
+            out = torch.empty(blocks, dtype=torch.int32, device=self.device)
+        self._dense(out, "out", torch.int32, (blocks,))
+        self._check(self.lib.akv_read_probe(_ptr(data), ctypes.c_long(size), _ptr(out), blocks, self._stream()), "read_probe")
+        return out
 
     def prepare_linear(self, matrix: torch.Tensor):
         """bfloat16 matrices whose k is a multiple of 8 are packed for the MFMA kernels; others stay row-major and

@@ -12,7 +12,8 @@ not change the time a step takes).  One JSON line is printed:
   prefill   one request's 2,048-token prompt fed whole: tokens/s, ms, and flops / time / bf16 MFMA peak
   roofline  bytes a decode step has to read (every weight once + the live requests' cache) / its time / HBM peak
   points    decoded tokens per second at batch 1 and 64; prefill tokens per second with every product in the engine's
-            own kernels (by default bfloat16 products of more than 16 rows go to the BLAS library)
+            own kernels (by default bfloat16 products of more than 16 rows go to the BLAS library); hbm_read_gbs,
+            what a kernel that only reads draws from this device's memory (the ceiling to hold `roofline` against)
 Peaks are MI355X's published ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s.
 
 Further workloads run through the scheduler and print a line of their own (`--workload`):
@@ -306,8 +307,32 @@ def main() -> int:
             kept, engine.kernels.library_products_above = engine.kernels.library_products_above, None
             record["points"]["prefill_own_products"] = round(PREFILL_TOKENS / prefill(3)[0], 1)
             engine.kernels.library_products_above = kept
+    if points:
+        record["points"]["hbm_read_gbs"] = measured_read_rate(engine.kernels, engine.device)
     print(json.dumps(record))
     return 0
+
+
+def measured_read_rate(kernels, device, gib: int = 8, part_mib: int = 1024) -> float:
+    """GB/s that a kernel which only reads draws from memory on this device: parts of a buffer larger than
+    every cache, one after the other, the median over the parts (1 GiB each of 8 GiB).  What the decode step could reach at most if it
+    were nothing but its reads; the step's own rate (`roofline.achieved`) is to be held against this, not only
+    against the data sheet's peak."""
+    import torch
+    buffer = torch.empty(gib << 30, dtype=torch.uint8, device=device)
+    buffer.zero_()
+    out = torch.empty(4 * kernels.compute_units, dtype=torch.int32, device=device)
+    parts = [buffer[i * (part_mib << 20):(i + 1) * (part_mib << 20)] for i in range((gib << 10) // part_mib)]
+    kernels.read_probe(parts[0], out)
+    rates = []
+    for part in parts[1:]:
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        kernels.read_probe(part, out)
+        stop.record()
+        torch.cuda.synchronize(device)
+        rates.append(part.numel() / (start.elapsed_time(stop) * 1e-3) / 1e9)
+    return round(sorted(rates)[len(rates) // 2], 1)
 
 
 if __name__ == "__main__":

@@ -1150,3 +1150,17 @@ def test_embed_takes_the_token_chosen_last_from_the_slot(hip, ref):
     assert torch.equal(got.cpu(), want)
     hip.embed(ids.cuda(), table.cuda(), got)                                     # without the slots -1 is no token
     assert torch.isnan(got[0]).all() and torch.equal(got[1].cpu(), want[1])
+
+
+@pytest.mark.parametrize("words,blocks", [(4 * 64 * 1000, 64), (4 * 977, 7), (4 * 64 * 3 + 4 * 5, 1024), (4, 3)])
+def test_read_probe_reads_every_word_once(hip, words, blocks):
+    """The kernel that measures what memory gives: the xor over its per-block results is the xor of all words, whatever
+    the split into blocks and waves (spans that are no whole tiles, more waves than tiles)."""
+    data = torch.randint(-2 ** 31, 2 ** 31 - 1, (words,), dtype=torch.int32, generator=torch.Generator().manual_seed(3))
+    want = 0
+    for word in data.tolist():
+        want ^= word & 0xffffffff
+    got = 0
+    for word in hip.read_probe(data.cuda(), blocks=blocks).cpu().tolist():
+        got ^= word & 0xffffffff
+    assert got == want
