@@ -1,0 +1,107 @@
+"""What the matrix products of a decode step cost beside a bare read of the same bytes.
+
+    python -m ampere_kv_engine_amd.bench_products --rows 1 8
+    python -m ampere_kv_engine_amd.bench_products --rows 8 --hidden 5120 --intermediate 17408 --q-heads 40
+
+For the four products of a layer (q/k/v, o, gate-up, down) at Qwen3-8B sizes, or the sizes given: the time of the
+product as a decode step runs it (the plain kernel, and the one that takes the residual sum or the norm into itself),
+and the time `read_probe` takes to read as many bytes and nothing else.  Every timed call reads a matrix that no
+cache holds: the program keeps several copies of each matrix, more bytes together than the device's caches, and
+goes round them.  Before each timed call the device is kept busy with reads, so that the host has queued the call
+before the device reaches it and no launch time of the host is measured.  One JSON line per product and row count;
+times in microseconds, the median of --repeats calls.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import statistics
+
+import torch
+
+from .kernels.hip import HipKernels
+
+CACHE_BYTES = 768 << 20         # copies of a matrix hold at least this much together (the device caches 256 MB)
+
+
+def main(argv=None) -> int:
+    parser = argparse.ArgumentParser(description=__doc__.split("\n")[0])
+    parser.add_argument("--rows", type=int, nargs="+", default=[1, 8], help="rows of the step (1..16)")
+    parser.add_argument("--hidden", type=int, default=4096)
+    parser.add_argument("--intermediate", type=int, default=12288)
+    parser.add_argument("--q-heads", type=int, default=32)
+    parser.add_argument("--kv-heads", type=int, default=8)
+    parser.add_argument("--head-dim", type=int, default=128)
+    parser.add_argument("--repeats", type=int, default=15)
+    args = parser.parse_args(argv)
+    if any(not 1 <= rows <= 16 for rows in args.rows):
+        parser.error("--rows: decode steps of 1 to 16 rows")
+    device = torch.device("cuda:0")
+    kernels = HipKernels(device, library_products_above=None)
+    generator = torch.Generator(device=device).manual_seed(0)
+    hidden, inter, q_size = args.hidden, args.intermediate, args.q_heads * args.head_dim
+    qkv_outs = q_size + 2 * args.kv_heads * args.head_dim
+    spacer = torch.zeros(64 << 20, dtype=torch.float32, device=device)
+
+    def matrix(outs, k):
+        return (torch.randn(outs, k, device=device, generator=generator) * 0.02).to(torch.bfloat16)
+
+    def timed(calls):
+        """Median time of the calls, each on its own matrix, each behind a quarter of a millisecond of other reads."""
+        times = []
+        for call in calls:
+            for _ in range(4):
+                spacer.sum()
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            call()
+            stop.record()
+            times.append((start, stop))
+        torch.cuda.synchronize(device)
+        return round(statistics.median(a.elapsed_time(b) for a, b in times) * 1e3, 1)
+
+    products = (("q/k/v", qkv_outs, hidden, "scaled"), ("o", hidden, q_size, "adds"),
+                ("gate-up", inter, hidden, "gated"), ("down", hidden, inter, "adds"))
+    for name, outs, k, kind in products:
+        size = outs * k * 2 * (2 if kind == "gated" else 1)
+        copies = max(2, -(-CACHE_BYTES // size))
+        if kind == "gated":
+            weights = [kernels.prepare_gated_linear(matrix(outs, k), matrix(outs, k)) for _ in range(copies)]
+            data = [w.packed.data for w in weights]
+        else:
+            weights = [kernels.prepare_linear(matrix(outs, k)) for _ in range(copies)]
+            data = [w.data for w in weights]
+        probe_out = torch.empty(4 * kernels.compute_units, dtype=torch.int32, device=device)
+        for rows in args.rows:
+            x = (torch.randn(rows, k, device=device, generator=generator)).to(torch.bfloat16)
+            out = torch.empty(rows, outs, dtype=torch.bfloat16, device=device)
+            record = {"product": name, "outs": outs, "k": k, "rows": rows, "megabytes": round(size / 1e6, 1)}
+            turn = lambda i: i % copies
+            record["read_only_us"] = timed([(lambda i=i: kernels.read_probe(data[turn(i)], probe_out)) for i in range(args.repeats)])
+            if kind == "gated":
+                record["plain_us"] = timed([(lambda i=i: kernels.gated_linear(x, weights[turn(i)], out)) for i in range(args.repeats)])
+            else:
+                record["plain_us"] = timed([(lambda i=i: kernels.linear(x, weights[turn(i)], out)) for i in range(args.repeats)])
+            if kind == "adds":      # the product adds itself to the residual sum and leaves the rows' sums of squares
+                stream = torch.randn(rows, outs, device=device, generator=generator)
+                sums = torch.empty((outs + 15) // 16, 16, dtype=torch.float32, device=device)
+                record["adds_to_stream_us"] = timed([(lambda i=i: kernels.linear_adds(x, weights[turn(i)], stream, sums))
+                                                     for i in range(args.repeats)])
+            elif rows * k * 2 <= kernels.FOLD_NORM_BYTES:   # the product norms the residual rows itself
+                stream = torch.randn(rows, k, device=device, generator=generator)
+                sums = torch.zeros((k + 15) // 16, 16, dtype=torch.float32, device=device)
+                sums[:, :rows] = (stream * stream).view(rows, -1, 16).sum(-1).T if k % 16 == 0 else 1.0
+                gain = torch.ones(k, device=device)
+                normed = torch.empty(rows, k, dtype=torch.bfloat16, device=device)
+                record["norm_kernel_us"] = timed([(lambda: kernels.add_rmsnorm(stream, None, gain, 1e-6, normed))
+                                                  for _ in range(args.repeats)])
+                record["norms_its_rows_us"] = timed([(lambda i=i: kernels.linear_scaled(stream, sums, gain, 1e-6, weights[turn(i)], out))
+                                                     for i in range(args.repeats)])
+            print(json.dumps(record), flush=True)
+        del weights, data
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())

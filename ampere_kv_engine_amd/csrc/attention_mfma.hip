@@ -637,8 +637,8 @@ __global__ __launch_bounds__(64, (SPLIT && NQ == 1 && D <= 128) ? 2 : 1) void at
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
         uintx2 packed;
-        packed.x = bf16_bits(o[nq][dt][0] * inv) | (static_cast<uint32_t>(bf16_bits(o[nq][dt][1] * inv)) << 16);
-        packed.y = bf16_bits(o[nq][dt][2] * inv) | (static_cast<uint32_t>(bf16_bits(o[nq][dt][3] * inv)) << 16);
+        packed.x = bf16_pair(o[nq][dt][0] * inv, o[nq][dt][1] * inv);
+        packed.y = bf16_pair(o[nq][dt][2] * inv, o[nq][dt][3] * inv);
         *reinterpret_cast<uintx2*>(a.out + col_at[nq] + dt * 16 + g * 4) = packed;
       }
     }
@@ -1081,8 +1081,8 @@ __global__ __launch_bounds__(64 * kSharedWaves, D <= 128 ? (NQ == 1 ? 3 : 2) : 1
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       uintx2 packed;
-      packed.x = bf16_bits(o[nq][dt][0] * inv) | (static_cast<uint32_t>(bf16_bits(o[nq][dt][1] * inv)) << 16);
-      packed.y = bf16_bits(o[nq][dt][2] * inv) | (static_cast<uint32_t>(bf16_bits(o[nq][dt][3] * inv)) << 16);
+      packed.x = bf16_pair(o[nq][dt][0] * inv, o[nq][dt][1] * inv);
+      packed.y = bf16_pair(o[nq][dt][2] * inv, o[nq][dt][3] * inv);
       *reinterpret_cast<uintx2*>(a.out + col_at[nq] + dt * 16 + g * 4) = packed;
     }
   }

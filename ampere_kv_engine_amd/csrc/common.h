@@ -17,11 +17,16 @@ struct bf16_t {
 __device__ __forceinline__ float to_float(float x) { return x; }
 __device__ __forceinline__ float to_float(bf16_t x) { return __uint_as_float(static_cast<uint32_t>(x.bits) << 16); }
 
-__device__ __forceinline__ uint16_t bf16_bits(float x) {
-  uint32_t u = __float_as_uint(x);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);  // quiet NaN
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return static_cast<uint16_t>(u >> 16);
+// (gfx950 converts in hardware - v_cvt_pk_bf16_f32, two values an instruction - which the compiler emits for a cast to
+// its own bfloat type; in software the same rounding is seven instructions a value.)
+__device__ __forceinline__ uint16_t bf16_bits(float x) { return __builtin_bit_cast(uint16_t, static_cast<__bf16>(x)); }
+
+// Two values rounded and packed as they lie in memory: `low` in the lower half.
+__device__ __forceinline__ uint32_t bf16_pair(float low, float high) {
+  typedef __attribute__((ext_vector_type(2))) float float_pair;
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16_pair_t;
+  const float_pair both = {low, high};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(both, bf16_pair_t));
 }
 
 template <typename T> __device__ __forceinline__ T from_float(float x);

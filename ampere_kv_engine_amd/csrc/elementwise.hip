@@ -65,8 +65,8 @@ template <typename T> __device__ __forceinline__ void store4(T* p, float4 v);
 template <> __device__ __forceinline__ void store4<float>(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
 template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float4 v) {
   uint2 packed;
-  packed.x = bf16_bits(v.x) | (static_cast<uint32_t>(bf16_bits(v.y)) << 16);
-  packed.y = bf16_bits(v.z) | (static_cast<uint32_t>(bf16_bits(v.w)) << 16);
+  packed.x = bf16_pair(v.x, v.y);
+  packed.y = bf16_pair(v.z, v.w);
   *reinterpret_cast<uint2*>(p) = packed;
 }
 
@@ -282,10 +282,10 @@ template <> __device__ __forceinline__ void store8<float>(float* p, const float 
 }
 template <> __device__ __forceinline__ void store8<bf16_t>(bf16_t* p, const float (&v)[8]) {
   uint4 u;
-  u.x = bf16_bits(v[0]) | (static_cast<uint32_t>(bf16_bits(v[1])) << 16);
-  u.y = bf16_bits(v[2]) | (static_cast<uint32_t>(bf16_bits(v[3])) << 16);
-  u.z = bf16_bits(v[4]) | (static_cast<uint32_t>(bf16_bits(v[5])) << 16);
-  u.w = bf16_bits(v[6]) | (static_cast<uint32_t>(bf16_bits(v[7])) << 16);
+  u.x = bf16_pair(v[0], v[1]);
+  u.y = bf16_pair(v[2], v[3]);
+  u.z = bf16_pair(v[4], v[5]);
+  u.w = bf16_pair(v[6], v[7]);
   *reinterpret_cast<uint4*>(p) = u;
 }
 

@@ -137,8 +137,7 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
         uintx4 packed;
 #pragma unroll
         for (int w = 0; w < 4; ++w)
-          packed[w] = bf16_bits(rounded<bf16_t>(v[2 * w] * scale) * gain[2 * w]) |
-                      (static_cast<uint32_t>(bf16_bits(rounded<bf16_t>(v[2 * w + 1] * scale) * gain[2 * w + 1])) << 16);
+          packed[w] = bf16_pair(rounded<bf16_t>(v[2 * w] * scale) * gain[2 * w], rounded<bf16_t>(v[2 * w + 1] * scale) * gain[2 * w + 1]);
         *reinterpret_cast<uintx4*>(rows_lds + static_cast<size_t>(row) * k + i) = packed;
       }
     }

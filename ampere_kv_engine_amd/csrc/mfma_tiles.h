@@ -35,8 +35,8 @@ template <> __device__ __forceinline__ void store4<float>(float* p, floatx4 v) {
 }
 template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, floatx4 v) {
   uint2 packed;
-  packed.x = bf16_bits(v[0]) | (static_cast<uint32_t>(bf16_bits(v[1])) << 16);
-  packed.y = bf16_bits(v[2]) | (static_cast<uint32_t>(bf16_bits(v[3])) << 16);
+  packed.x = bf16_pair(v[0], v[1]);
+  packed.y = bf16_pair(v[2], v[3]);
   *reinterpret_cast<uint2*>(p) = packed;
 }
 
