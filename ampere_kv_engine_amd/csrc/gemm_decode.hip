@@ -341,6 +341,10 @@ extern "C" int akv_linear_scaled(const float* stream_in, const float* sums, int 
   a.y = static_cast<bf16_t*>(y);
   a.rows = rows, a.outs = outs, a.k = k, a.k_tiles = k_tiles, a.n_tiles = n_tiles;
   if (gated) return launch_decode<2, true, true, false>(a, stream);
-  if (rows >= 4 && n_tiles >= 384 && n_tiles < 2048) return launch_decode<2, false, true, false>(a, stream);
+  // The rows come from LDS, so two row tiles per wave save no loads of activations; they are two runs of memory per
+  // wave where one is faster (q/k/v at 4 rows: 19.4 -> 16.3 us, at 8: 20.3 -> 19.4).  They pay where the normed rows fill
+  // so much LDS that a compute unit holds one block and the larger blocks keep more of it busy (16 rows: 28.8 -> 23.0).
+  if (static_cast<size_t>(rows) * k * 2 > 80 * 1024 && n_tiles >= 384 && n_tiles < 2048)
+    return launch_decode<2, false, true, false>(a, stream);
   return launch_decode<1, false, true, false>(a, stream);
 }
