@@ -37,8 +37,11 @@ def plan_memory(spec: ModelSpec, engine_config: EngineConfig, memory_bytes: int)
     model = Model(spec, dry_runtime())
     tensors = [t for t in model.tensors() if not t.optional]
     weight_bytes = sum(_count(t.shape) for t in tensors) * element
-    matrices = sum(_count(t.shape) for t in tensors if t.role == MATRIX)
+    # (what a part keeps twice it says itself: a part with storage of its own is counted once)
+    matrices = sum(_count(t.shape) for t in tensors if t.library_copy)
     second = matrices * element if engine_config.dtype == "bfloat16" and engine_config.library_products_above is not None else 0
+    if engine_config.dtype == "bfloat16" and spec.head.get("tied_to") is not None:
+        second += spec.vocab_size * spec.hidden_size * element      # a tied head: the table's packing beside the table
     cache = CacheManager(model.cache_needs(), page_size=engine_config.page_size, num_pages=1,
                          max_seqs=engine_config.max_seqs, allocate_tensors=False)
     page_bytes = sum(g.bytes_per_token(element) for g in cache.groups) * engine_config.page_size

@@ -47,7 +47,7 @@ class LinearHead(Part):
     def tensors(self, prefix=""):
         if self.tied_to is not None:
             return []
-        return [TensorSpec(self.name, (self.vocab, self.hidden), MATRIX)]
+        return self.linear.tensors("")
 
     def load(self, fetch, prefix="", tied_weight=None):
         if self.tied_to is not None:

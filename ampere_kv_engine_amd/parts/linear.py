@@ -25,7 +25,7 @@ class Linear(Part):
         return sum(self.out_features)
 
     def tensors(self, prefix: str):
-        return [TensorSpec(prefix + name, (out, self.in_features), self.role)
+        return [TensorSpec(prefix + name, (out, self.in_features), self.role, library_copy=True)
                 for name, out in zip(self.names, self.out_features)]
 
     def load(self, fetch, prefix: str):

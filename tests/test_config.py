@@ -107,3 +107,24 @@ def test_plan_memory_counts_weights_copies_and_pages():
     assert full.weight_bytes == 2 * plan.weight_bytes and full.second_copy_bytes == 0 and full.page_bytes == 2 * plan.page_bytes
     with pytest.raises(ValueError, match="not a page"):
         plan_memory(spec, config, plan.weight_bytes + plan.second_copy_bytes + plan.fixed_bytes + plan.page_bytes)
+
+
+def test_plan_memory_counts_a_second_copy_only_where_a_part_keeps_one():
+    """The row-major copy for the BLAS library is `Linear`'s doing: it marks its tensors (`TensorSpec.library_copy`).
+    A part with storage of its own - the toy routed feed-forward of the GPU tests, whose experts' matrices are plain
+    `TensorSpec`s - is counted once."""
+    import test_toy_parts_gpu as toy
+    from ampere_kv_engine_amd.config import EngineConfig
+    from ampere_kv_engine_amd.engine import plan_memory
+    from ampere_kv_engine_amd.parts import register_part
+    register_part("feed_forward", "routed", toy.RoutedFeedForward, replace=True)
+    register_part("position", "adjacent_pair_rotary", toy.AdjacentPairRotary, replace=True)
+    spec = toy.RoutedConfig(vocab_size=97, hidden_size=32, decay=0.0, eps=1e-5).to_model_spec()
+    config = EngineConfig(dtype="bfloat16", page_size=8, num_pages=1, max_seqs=2, max_batched_tokens=16, max_seq_len=64)
+    plan = plan_memory(spec, config, 1 << 30)
+    attention = 3 * 2 * 16 * 32 + 32 * 2 * 16                       # q/k/v and o of one layer
+    dense = 3 * 40 * 32
+    experts = 3 * 32 + 3 * (2 * 24 * 32 + 32 * 24)                   # router and three experts
+    head = 97 * 32
+    assert plan.second_copy_bytes == 2 * (2 * attention + dense + head)
+    assert plan.weight_bytes >= 2 * (2 * attention + dense + experts + 2 * head)
