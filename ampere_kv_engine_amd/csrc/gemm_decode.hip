@@ -257,28 +257,49 @@ __global__ __launch_bounds__(768) void linear_decode_kernel(const DecodeArgs a) 
   }
 }
 
-template <int RT, bool GATED, bool SCALED, bool ADDS>
-int launch_decode(DecodeArgs a, hipStream_t stream) {
+struct DecodePlan {
+  int k_split, m;     // parts of k over the waves of a block; wave-rows per block
+  double work;        // bytes' worth of work on the busiest compute unit
+};
+
+// How a product is cut into blocks.  `rt`: row tiles per wave; `normed_rows`: rows that every block norms for itself
+// (a SCALED product), else 0.
+DecodePlan plan_decode(int rt, int n_tiles, int k_tiles, int k, int normed_rows) {
   // as many waves as the skinny kernel takes: k is split over the waves of a block while the row tiles are few
-  const int wave_rows = (a.n_tiles + RT - 1) / RT;
+  const int wave_rows = (n_tiles + rt - 1) / rt;
   int k_split = 1;
   while (k_split < 8) {
-    const int waves_now = wave_rows * k_split, part_after = a.k_tiles / (k_split * 2);
+    const int waves_now = wave_rows * k_split, part_after = k_tiles / (k_split * 2);
     if (!((waves_now < 1536 && part_after >= 4) || (waves_now < 2048 && part_after >= 4 * kGroup))) break;
     k_split *= 2;
   }
-  // Waves per block: k_split * m for m wave-rows.  All blocks are resident at once and the compute units share the
-  // memory system evenly, so the product is over when the unit with the most blocks is: m is chosen so that the blocks
-  // spread evenly over the units (768 wave-rows: 3 per block make 256 blocks, one a unit) - and where that ties, a
-  // SCALED product takes the larger blocks (every block norms the rows for itself), the others the smaller.
+  // Waves per block: k_split * m for m wave-rows.  The compute units share the memory system evenly, so the product
+  // is over when the unit with the most bytes is: m is chosen for the least work on the busiest unit - its blocks'
+  // wave-rows (768 wave-rows: 3 per block make 256 blocks, one a unit; 384 blocks would leave half the units with
+  // two) and, where blocks norm rows, those rows (counted at 1.5 times their bytes: measured, norming 64 KB of rows
+  // costs a block what streaming 90 KB of weights does).  A unit holds as many blocks at once as its 160 KB of LDS and
+  // its 32 waves allow; blocks beyond that wait for a further round.
   constexpr int kUnits = 256, kMostWaves = 12;
-  int m = 1, best = 0;
+  const size_t rows_bytes = normed_rows ? static_cast<size_t>(normed_rows) * k * 2 + (12 * 16 + 16) * 4 : 0;
+  const double row_bytes = static_cast<double>(rt) * k_tiles * 1024, norm_bytes = 1.5 * normed_rows * k * 2;
+  DecodePlan plan{k_split, 1, 0.0};
   for (int tried = 1; tried * k_split <= kMostWaves; ++tried) {
-    const int blocks_tried = (wave_rows + tried - 1) / tried;
-    const int longest = (blocks_tried + kUnits - 1) / kUnits * tried;   // wave-rows on the busiest unit
-    if (best == 0 || longest < best || (SCALED && longest == best)) best = longest, m = tried;
+    const int blocks_tried = (wave_rows + tried - 1) / tried, waves_tried = tried * k_split;
+    const size_t lds_tried = max(rows_bytes, k_split > 1 ? static_cast<size_t>(waves_tried) * rt * 1024 : 0);
+    const int at_once = max(1, min(static_cast<int>(lds_tried ? kMaxLds / lds_tried : 32), 32 / waves_tried));
+    int on_busiest = (blocks_tried + kUnits - 1) / kUnits;               // blocks of the unit with the most
+    if (on_busiest > at_once) on_busiest = (on_busiest + at_once - 1) / at_once * at_once;   // whole rounds
+    const double work = on_busiest * (tried * row_bytes + norm_bytes);
+    if (plan.work == 0.0 || work < plan.work) plan.work = work, plan.m = tried;
   }
-  if (!SCALED && k_split < 4 && m * k_split < 4) m = (4 + k_split - 1) / k_split;   // blocks of at least 4 waves
+  if (!normed_rows && k_split < 4 && plan.m * k_split < 4) plan.m = (4 + k_split - 1) / k_split;   // blocks of at least 4 waves
+  return plan;
+}
+
+template <int RT, bool GATED, bool SCALED, bool ADDS>
+int launch_decode(DecodeArgs a, hipStream_t stream) {
+  const DecodePlan plan = plan_decode(RT, a.n_tiles, a.k_tiles, a.k, SCALED ? a.rows : 0);
+  const int wave_rows = (a.n_tiles + RT - 1) / RT, k_split = plan.k_split, m = plan.m;
   const int waves = k_split * m;
   const int rows_per_block = m;
   const int blocks = (wave_rows + rows_per_block - 1) / rows_per_block;
@@ -342,9 +363,10 @@ extern "C" int akv_linear_scaled(const float* stream_in, const float* sums, int 
   a.rows = rows, a.outs = outs, a.k = k, a.k_tiles = k_tiles, a.n_tiles = n_tiles;
   if (gated) return launch_decode<2, true, true, false>(a, stream);
   // The rows come from LDS, so two row tiles per wave save no loads of activations; they are two runs of memory per
-  // wave where one is faster (q/k/v at 4 rows: 19.4 -> 16.3 us, at 8: 20.3 -> 19.4).  They pay where the normed rows fill
-  // so much LDS that a compute unit holds one block and the larger blocks keep more of it busy (16 rows: 28.8 -> 23.0).
-  if (static_cast<size_t>(rows) * k * 2 > 80 * 1024 && n_tiles >= 384 && n_tiles < 2048)
+  // wave where one is faster (q/k/v at 4 rows: 19.4 -> 16.3 us, at 8: 20.3 -> 19.4; counted as 1.3 times the bytes, which puts the rule where the measurements are).
+  // They pay where the normed rows fill so much LDS that a compute unit holds one block, and the blocks of one row tile
+  // per wave would need a second round (16 rows of 4,096: 28.8 -> 23.0 us).
+  if (n_tiles >= 2 && plan_decode(2, n_tiles, k_tiles, k, rows).work * 1.3 < plan_decode(1, n_tiles, k_tiles, k, rows).work)
     return launch_decode<2, false, true, false>(a, stream);
   return launch_decode<1, false, true, false>(a, stream);
 }
