@@ -51,25 +51,10 @@ int akv_pack_rows(const void* x, void* xp, int rows, int k, hipStream_t stream);
 // threads) race; calls that follow each other on a stream do not.
 int akv_linear_packed_static(const void* x, const void* wp, void* y, int y_dtype, int rows, int outs, int k,
                              int n_tiles, int k_tiles, hipStream_t stream);
-int akv_linear_adds(const void* x, const void* wp, float* stream_out, float* sums_out, int rows, int outs, int k,
-                    int n_tiles, int k_tiles, hipStream_t stream);
+int akv_linear_decode_plan(int rt, int n_tiles, int k_tiles, int k, int normed_rows, int may_straddle, int* out);
+int akv_linear_adds(const void* x, const void* wp, float* stream_out, float* sums_out, float* pieces,
+                    unsigned int* arrivals, int rows, int outs, int k, int n_tiles, int k_tiles, hipStream_t stream);
 int akv_linear_scaled(const float* stream_in, const float* sums, int sum_tiles, const float* gain, float eps,
-                      const void* wp, void* y, int rows, int outs, int k, int n_tiles, int k_tiles, int gated,
-                      hipStream_t stream);
-int akv_linear_mid_workspace(int rows, int n_tiles, int k_tiles, int gated, int along, int rt, int depth, int parts,
-                             long* partial_floats, long* counters);
-int akv_linear_mid(const void* x, const void* wp, void* y, int y_dtype, float* partial, unsigned* counters, int rows,
-                   int outs, int k, int n_tiles, int k_tiles, int gated, int along, int rt, int depth, int parts,
-                   hipStream_t stream);
-int akv_attention_rows(const void* q, const void* k_pages, const void* v_pages, const int* seq_of_token,
-                       const int* positions, const int* block_table, const int* table_rows, int table_width, void* out,
-                       int dtype,
-                       long tokens, int q_heads, int kv_heads, int dim, int page_size, long num_pages, float scale,
-                       int window, hipStream_t stream);
-int akv_decode_plan(const int* seq_lens, int seq_first, int seq_count, int window, int items_wanted, int min_segment,
-                    int items_grid, int* plan, hipStream_t stream);
-int akv_sample(const float* logits, const float* temperature, const unsigned long long* seeds,
-               const unsigned int* draws, int* out, int rows, int vocab, hipStream_t stream);
-int akv_sample_slots(const float* logits, const int* rows_of, const int* seq_of_token, const int* seq_slots,
-                     int* slot_words, int* out, int rows, int vocab, hipStream_t stream);
+                      const void* wp, void* y, float* pieces, unsigned int* arrivals, int rows, int outs, int k,
+                      int n_tiles, int k_tiles, int gated, hipStream_t stream);
 }

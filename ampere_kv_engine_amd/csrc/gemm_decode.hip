@@ -36,6 +36,8 @@ struct DecodeArgs {
   float* sums_out;          // ADDS: [n_tiles][16]
   float eps;
   int sum_tiles, rows, outs, k, k_tiles, n_tiles, k_split, red_floats;
+  float* pieces;            // [wave-row][2][RT][4][64]: the sums of a wave-row whose parts of k lie in two blocks
+  unsigned int* arrivals;   // [wave-row], zero between launches: how many of the two have left their sums
 };
 
 constexpr int kGroup = 4;   // k-tiles per group of loads; two groups are in flight
@@ -49,8 +51,11 @@ __global__ __launch_bounds__(768) void linear_decode_kernel(const DecodeArgs a) 
   const int lane = threadIdx.x & 63, waves = blockDim.x >> 6;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, g = lane >> 4;
-  const int row_tile = (blockIdx.x * (waves / a.k_split) + wave / a.k_split) * RT;
-  const int part = wave % a.k_split;
+  // The product's work is cut into units - (wave-row of RT row tiles, part of k) - numbered wave-row by wave-row; a
+  // block's waves take consecutive units, whole wave-rows or not.
+  const int first_unit = blockIdx.x * waves, unit = first_unit + wave;
+  const int wave_row = unit / a.k_split, part = unit % a.k_split;
+  const int row_tile = wave_row * RT;
   const int per_part = (a.k_tiles + a.k_split - 1) / a.k_split;
   const int kt0 = part * per_part, kt1 = min(a.k_tiles, kt0 + per_part);
   const bool works = row_tile < a.n_tiles && kt0 < kt1;
@@ -76,7 +81,8 @@ __global__ __launch_bounds__(768) void linear_decode_kernel(const DecodeArgs a) 
   // SCALED: the rows as the operand wants them, [k tile][k chunk of 8][row] x 16 bytes: lane (r, g) reads chunk g, row r
   constexpr int kScaleFloats = 12 * 16 + 16;   // SCALED: every wave's share of the rows' sums of squares, then the scales
   uintx4* rows_lds = reinterpret_cast<uintx4*>(red + (SCALED ? kScaleFloats : 0));
-  fetch_weights(kt0, w0);   // on their way while the rows are normed
+  fetch_weights(kt0, w0);       // two groups on their way while the rows are normed
+  fetch_weights(kt0 + U, w1);
   if constexpr (SCALED) {
     // (Asking for what the norm needs BEFORE the first weights - a wave's loads come back in the order in which they
     // were asked for - was measured and is no gain: 15.0 -> 16.0 us at one row, 23.1 -> 22.8 at eight, q/k/v.)
@@ -175,45 +181,72 @@ __global__ __launch_bounds__(768) void linear_decode_kernel(const DecodeArgs a) 
   };
   if (works) {
     fetch_rows(kt0, x0);
+    fetch_rows(kt0 + U, x1);
     int kt = kt0;
-    if (kt < kt1) {
-      for (; kt + 2 * U < kt1; kt += 2 * U) {   // both groups asked for here hold tiles of the part
-        fetch_weights(kt + U, w1);
-        fetch_rows(kt + U, x1);
-        multiply(kt, w0, x0);
-        fetch_weights(kt + 2 * U, w0);
-        fetch_rows(kt + 2 * U, x0);
-        multiply(kt + U, w1, x1);
-      }
-      if (kt + U < kt1) {
-        fetch_weights(kt + U, w1);
-        fetch_rows(kt + U, x1);
-        multiply(kt, w0, x0);
-        multiply(kt + U, w1, x1);
-      } else {
-        multiply(kt, w0, x0);
+    for (; kt + 2 * U < kt1; kt += 2 * U) {   // two groups are in flight; the one after them holds tiles of the part
+      multiply(kt, w0, x0);
+      fetch_weights(kt + 2 * U, w0);
+      fetch_rows(kt + 2 * U, x0);
+      multiply(kt + U, w1, x1);
+      if (kt + 3 * U < kt1) {
+        fetch_weights(kt + 3 * U, w1);
+        fetch_rows(kt + 3 * U, x1);
       }
     }
+    multiply(kt, w0, x0);
+    if (kt + U < kt1) multiply(kt + U, w1, x1);
   }
 
-  if (a.k_split > 1) {   // part 0 + part 1 + ...: every wave leaves its sums in LDS, the wave of part 0 adds them up
+  if (a.k_split > 1) {
+    // The parts of k are added up in their order.  The units of this wave's wave-row that the block holds are
+    // [lo, hi): every wave leaves its sums in LDS, the wave of unit lo adds them up.  Where the block holds the whole
+    // wave-row that is the result.  Otherwise the wave-row's other parts lie in the neighbouring block (never in
+    // more than two: a block has at least k_split waves): both leave their sums in `pieces` with device-scope
+    // stores - acknowledged when the wave's counters are back at zero - and tick `arrivals`; the second to arrive
+    // adds piece 0 + piece 1 (the same bits whichever it is), sets the counter back and goes on to the store.
+    // Nobody waits for anybody.
     constexpr int kSet = RT * 4 * 64;
     if constexpr (SCALED) __syncthreads();   // the rows have been read: their memory takes the sums
+    const int row_first = wave_row * a.k_split;
+    const int lo = max(first_unit, row_first), hi = min(first_unit + waves, row_first + a.k_split);
     float* mine = red + static_cast<size_t>(wave) * kSet;
-    if (part != 0) {
+    if (unit != lo) {
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) mine[(rt * 4 + i) * 64 + lane] = acc[rt][i];
     }
     __syncthreads();
-    if (part != 0) return;
-    for (int other = 1; other < a.k_split; ++other) {
+    if (unit != lo) return;
+    for (int other = 1; other < hi - lo; ++other) {
       const float* theirs = mine + static_cast<size_t>(other) * kSet;
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[rt][i] += theirs[(rt * 4 + i) * 64 + lane];
+    }
+    if (hi - lo < a.k_split && row_tile < a.n_tiles) {
+      const int piece = lo == row_first ? 0 : 1;
+      float* ours = a.pieces + (static_cast<size_t>(wave_row) * 2 + piece) * kSet;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          __hip_atomic_store(ours + (rt * 4 + i) * 64 + lane, acc[rt][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __builtin_amdgcn_s_waitcnt(0);   // every counter at zero: the stores above have arrived
+      unsigned int before = 0;
+      if (lane == 0) before = __hip_atomic_fetch_add(a.arrivals + wave_row, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      before = __shfl(before, 0, kWave);
+      if (before == 0u) return;        // the other block will finish this wave-row
+      if (lane == 0) __hip_atomic_store(a.arrivals + wave_row, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
+      const float* theirs = a.pieces + (static_cast<size_t>(wave_row) * 2 + (1 - piece)) * kSet;
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float other = __hip_atomic_load(theirs + (rt * 4 + i) * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          acc[rt][i] = piece == 0 ? acc[rt][i] + other : other + acc[rt][i];
+        }
     }
   }
   if (row_tile >= a.n_tiles) return;
@@ -258,13 +291,14 @@ __global__ __launch_bounds__(768) void linear_decode_kernel(const DecodeArgs a) 
 }
 
 struct DecodePlan {
-  int k_split, m;     // parts of k over the waves of a block; wave-rows per block
-  double work;        // bytes' worth of work on the busiest compute unit
+  int k_split, waves, blocks;   // parts of k; waves (units) per block; blocks
+  bool straddles;               // wave-rows may have their parts of k in two blocks
+  double work;                  // bytes' worth of work on the busiest compute unit
 };
 
 // How a product is cut into blocks.  `rt`: row tiles per wave; `normed_rows`: rows that every block norms for itself
-// (a SCALED product), else 0.
-DecodePlan plan_decode(int rt, int n_tiles, int k_tiles, int k, int normed_rows) {
+// (a SCALED product), else 0; `may_straddle`: the caller brought memory for wave-rows whose parts lie in two blocks.
+DecodePlan plan_decode(int rt, int n_tiles, int k_tiles, int k, int normed_rows, bool may_straddle) {
   // as many waves as the skinny kernel takes: k is split over the waves of a block while the row tiles are few
   const int wave_rows = (n_tiles + rt - 1) / rt;
   int k_split = 1;
@@ -273,36 +307,44 @@ DecodePlan plan_decode(int rt, int n_tiles, int k_tiles, int k, int normed_rows)
     if (!((waves_now < 1536 && part_after >= 4) || (waves_now < 2048 && part_after >= 4 * kGroup))) break;
     k_split *= 2;
   }
-  // Waves per block: k_split * m for m wave-rows.  The compute units share the memory system evenly, so the product
-  // is over when the unit with the most bytes is: m is chosen for the least work on the busiest unit - its blocks'
-  // wave-rows (768 wave-rows: 3 per block make 256 blocks, one a unit; 384 blocks would leave half the units with
-  // two) and, where blocks norm rows, those rows (counted at 1.5 times their bytes: measured, norming 64 KB of rows
-  // costs a block what streaming 90 KB of weights does).  A unit holds as many blocks at once as its 160 KB of LDS and
-  // its 32 waves allow; blocks beyond that wait for a further round.
+  // Waves per block.  The compute units share the memory system evenly, so the product is over when the unit with
+  // the most bytes is: the number of waves a block gets is chosen for the least work on the busiest unit - its blocks'
+  // units (768 wave-rows of 4 parts: 12 waves a block make 256 blocks, one a unit; 8 waves, 384 blocks, would leave
+  // half the units with two) and, where blocks norm rows, those rows (counted at 1.5 times their bytes: measured,
+  // norming 64 KB of rows costs a block what streaming 90 KB of weights does).  A unit holds as many blocks at once as
+  // its 160 KB of LDS and its 32 waves allow; blocks beyond that wait for a further round.  Blocks need not hold
+  // whole wave-rows: 320 wave-rows of 8 parts are 256 blocks of 10 waves, one and a quarter wave-rows each - the price
+  // is the exchange of one wave-row's sums between two blocks, counted as 96 KB (measured: q/k/v of 6,144 x 4,096 gains
+  // nothing from it, o of 5,120 x 8,192 goes from 26 to 20 us, down of 5,120 x 25,600 from 62 to 48).
   constexpr int kUnits = 256, kMostWaves = 12;
   const size_t rows_bytes = normed_rows ? static_cast<size_t>(normed_rows) * k * 2 + (12 * 16 + 16) * 4 : 0;
-  const double row_bytes = static_cast<double>(rt) * k_tiles * 1024, norm_bytes = 1.5 * normed_rows * k * 2;
-  DecodePlan plan{k_split, 1, 0.0};
-  for (int tried = 1; tried * k_split <= kMostWaves; ++tried) {
-    const int blocks_tried = (wave_rows + tried - 1) / tried, waves_tried = tried * k_split;
-    const size_t lds_tried = max(rows_bytes, k_split > 1 ? static_cast<size_t>(waves_tried) * rt * 1024 : 0);
-    const int at_once = max(1, min(static_cast<int>(lds_tried ? kMaxLds / lds_tried : 32), 32 / waves_tried));
-    int on_busiest = (blocks_tried + kUnits - 1) / kUnits;               // blocks of the unit with the most
+  const double unit_bytes = static_cast<double>(rt) * ((k_tiles + k_split - 1) / k_split) * 1024;
+  const double norm_bytes = 1.5 * normed_rows * k * 2, exchange_bytes = 96.0 * 1024;
+  const int units = wave_rows * k_split;
+  DecodePlan plan{k_split, k_split, 0, false, 0.0};
+  for (int waves = k_split; waves <= kMostWaves; ++waves) {
+    const bool whole = waves % k_split == 0;
+    if (!whole && (!may_straddle || k_split == 1)) continue;
+    const int blocks = whole ? (wave_rows + waves / k_split - 1) / (waves / k_split) : (units + waves - 1) / waves;
+    const size_t lds = max(rows_bytes, k_split > 1 ? static_cast<size_t>(waves) * rt * 1024 : 0);
+    const int at_once = max(1, min(static_cast<int>(lds ? kMaxLds / lds : 32), 32 / waves));
+    int on_busiest = (blocks + kUnits - 1) / kUnits;                     // blocks of the unit with the most
     if (on_busiest > at_once) on_busiest = (on_busiest + at_once - 1) / at_once * at_once;   // whole rounds
-    const double work = on_busiest * (tried * row_bytes + norm_bytes);
-    if (plan.work == 0.0 || work < plan.work) plan.work = work, plan.m = tried;
+    const double work = on_busiest * (waves * unit_bytes + norm_bytes) + (whole ? 0.0 : exchange_bytes);
+    if (plan.work == 0.0 || work < plan.work) plan = DecodePlan{k_split, waves, blocks, !whole, work};
   }
-  if (!normed_rows && k_split < 4 && plan.m * k_split < 4) plan.m = (4 + k_split - 1) / k_split;   // blocks of at least 4 waves
+  if (!normed_rows && plan.waves < 4) {   // blocks of at least 4 waves
+    plan.waves = 4;
+    plan.blocks = (wave_rows + 4 / k_split - 1) / (4 / k_split);
+    plan.straddles = false;
+  }
   return plan;
 }
 
 template <int RT, bool GATED, bool SCALED, bool ADDS>
 int launch_decode(DecodeArgs a, hipStream_t stream) {
-  const DecodePlan plan = plan_decode(RT, a.n_tiles, a.k_tiles, a.k, SCALED ? a.rows : 0);
-  const int wave_rows = (a.n_tiles + RT - 1) / RT, k_split = plan.k_split, m = plan.m;
-  const int waves = k_split * m;
-  const int rows_per_block = m;
-  const int blocks = (wave_rows + rows_per_block - 1) / rows_per_block;
+  const DecodePlan plan = plan_decode(RT, a.n_tiles, a.k_tiles, a.k, SCALED ? a.rows : 0, a.pieces != nullptr);
+  const int k_split = plan.k_split, waves = plan.waves, blocks = plan.blocks;
   a.k_split = k_split;
   a.red_floats = k_split > 1 ? waves * RT * 4 * 64 : 0;
   const size_t lds = max(static_cast<size_t>(a.red_floats) * 4, SCALED ? (12 * 16 + 16) * 4 + static_cast<size_t>(a.rows) * a.k * 2 : 0);
@@ -328,8 +370,20 @@ int launch_decode(DecodeArgs a, hipStream_t stream) {
 
 // stream_out [rows, outs] += bfloat16(x W^T) in place (float32); sums_out [n_tiles][16] receives, for every row tile of
 // 16 outputs and every row, the sum of squares of the new values (rows beyond `rows`: 0).  rows <= 16, k % 8 == 0.
-extern "C" int akv_linear_adds(const void* x, const void* wp, float* stream_out, float* sums_out, int rows, int outs,
-                               int k, int n_tiles, int k_tiles, hipStream_t stream) {
+// `pieces` (n_tiles * 512 floats) and `arrivals` (n_tiles words, zero; left zero) may be null: with them the product
+// may be cut into blocks that do not hold whole row tiles' parts of k (see plan_decode).  Launches that share them
+// follow each other on one stream.
+// What plan_decode makes of a product (for tests and measurements): out[0..3] = parts of k, waves per block, blocks,
+// whether row tiles may have their parts of k in two blocks.
+extern "C" int akv_linear_decode_plan(int rt, int n_tiles, int k_tiles, int k, int normed_rows, int may_straddle, int* out) {
+  const DecodePlan plan = plan_decode(rt, n_tiles, k_tiles, k, normed_rows, may_straddle != 0);
+  out[0] = plan.k_split, out[1] = plan.waves, out[2] = plan.blocks, out[3] = plan.straddles ? 1 : 0;
+  return 0;
+}
+
+extern "C" int akv_linear_adds(const void* x, const void* wp, float* stream_out, float* sums_out, float* pieces,
+                               unsigned int* arrivals, int rows, int outs, int k, int n_tiles, int k_tiles,
+                               hipStream_t stream) {
   if (rows <= 0 || outs <= 0) return 0;
   if (rows > 16 || (k & 7) != 0 || n_tiles * 16 < outs || (n_tiles - 1) * 16 >= outs || k_tiles * 32 < k) return -2;
   DecodeArgs a{};
@@ -337,6 +391,7 @@ extern "C" int akv_linear_adds(const void* x, const void* wp, float* stream_out,
   a.wp = static_cast<const uintx4*>(wp);
   a.stream_out = stream_out;
   a.sums_out = sums_out;
+  if (pieces != nullptr && arrivals != nullptr) a.pieces = pieces, a.arrivals = arrivals;
   a.rows = rows, a.outs = outs, a.k = k, a.k_tiles = k_tiles, a.n_tiles = n_tiles;
   return launch_decode<1, false, false, true>(a, stream);
 }
@@ -345,10 +400,11 @@ extern "C" int akv_linear_adds(const void* x, const void* wp, float* stream_out,
 // akv_linear_packed_swiglu), where norm(stream) is what akv_add_rmsnorm gives for the float32 rows `stream` [rows, k]
 // and the weight `gain` [k] - with the rows' sums of squares not formed here but taken from `sums`
 // [sum_tiles][16] (what akv_linear_adds left: sum_tiles = ceil(k / 16)).  rows <= 16, k % 8 == 0, and the normed rows
-// (rows * k bfloat16) fit into a compute unit's LDS (160 KB) beside 832 bytes; -2 otherwise.
+// (rows * k bfloat16) fit into a compute unit's LDS (160 KB) beside 832 bytes; -2 otherwise.  `pieces`, `arrivals`: as
+// for akv_linear_adds.
 extern "C" int akv_linear_scaled(const float* stream_in, const float* sums, int sum_tiles, const float* gain, float eps,
-                                 const void* wp, void* y, int rows, int outs, int k, int n_tiles, int k_tiles, int gated,
-                                 hipStream_t stream) {
+                                 const void* wp, void* y, float* pieces, unsigned int* arrivals, int rows, int outs,
+                                 int k, int n_tiles, int k_tiles, int gated, hipStream_t stream) {
   if (rows <= 0 || outs <= 0) return 0;
   if (rows > 16 || (k & 7) != 0 || k_tiles * 32 < k || sum_tiles != (k + 15) / 16) return -2;
   if (gated ? ((outs & 15) != 0 || n_tiles * 8 != outs) : n_tiles * 16 < outs) return -2;
@@ -360,13 +416,15 @@ extern "C" int akv_linear_scaled(const float* stream_in, const float* sums, int 
   a.eps = eps;
   a.wp = static_cast<const uintx4*>(wp);
   a.y = static_cast<bf16_t*>(y);
+  if (pieces != nullptr && arrivals != nullptr) a.pieces = pieces, a.arrivals = arrivals;
+  const bool may = a.pieces != nullptr;
   a.rows = rows, a.outs = outs, a.k = k, a.k_tiles = k_tiles, a.n_tiles = n_tiles;
   if (gated) return launch_decode<2, true, true, false>(a, stream);
   // The rows come from LDS, so two row tiles per wave save no loads of activations; they are two runs of memory per
   // wave where one is faster (q/k/v at 4 rows: 19.4 -> 16.3 us, at 8: 20.3 -> 19.4; counted as 1.3 times the bytes, which puts the rule where the measurements are).
   // They pay where the normed rows fill so much LDS that a compute unit holds one block, and the blocks of one row tile
   // per wave would need a second round (16 rows of 4,096: 28.8 -> 23.0 us).
-  if (n_tiles >= 2 && plan_decode(2, n_tiles, k_tiles, k, rows).work * 1.3 < plan_decode(1, n_tiles, k_tiles, k, rows).work)
+  if (n_tiles >= 2 && plan_decode(2, n_tiles, k_tiles, k, rows, may).work * 1.3 < plan_decode(1, n_tiles, k_tiles, k, rows, may).work)
     return launch_decode<2, false, true, false>(a, stream);
   return launch_decode<1, false, true, false>(a, stream);
 }

@@ -120,6 +120,7 @@ class HipKernels:
             raise KernelError(f"the kernel library {path} could not be loaded: {error}") from error
         self.library_path = path
         self._attention_entry = {}      # head size -> entry point of that head size's attention library
+        self._exchange_tiles, self._exchange_pieces, self._exchange_arrivals = 0, None, None
         self.decode_wave_target = 2048  # decode attention cuts the keys until about this many waves are at work,
         self.decode_min_segment = 128   # but into segments no shorter than this many keys (measured: 64 and 256 are slower)
         self.decode_max_splits = 128    # and no more than this many (four waves of the merge share them)
@@ -136,7 +137,7 @@ class HipKernels:
                      "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
                      "akv_linear_tiled", "akv_linear_packed", "akv_linear_packed_swiglu", "akv_linear_packed_normed",
                      "akv_pack_rows", "akv_linear_packed_static", "akv_linear_mid", "akv_linear_mid_workspace",
-                     "akv_linear_adds", "akv_linear_scaled", "akv_read_probe",
+                     "akv_linear_adds", "akv_linear_scaled", "akv_linear_decode_plan", "akv_read_probe",
                      "akv_attention_rows", "akv_decode_plan", "akv_sample", "akv_sample_slots", "akv_step_prologue"):
             getattr(self.lib, name).restype = ctypes.c_int
 
@@ -285,6 +286,7 @@ class HipKernels:
         if matrix.dtype == torch.bfloat16 and matrix.shape[1] % 8 == 0:
             weight = PackedWeight(matrix, keep_row_major=self.library_products_above is not None)
             self._products.setdefault(("linear", weight.outs, weight.k), weight)
+            self._reserve_exchange(weight.n_tiles)
             return weight
         return matrix
 
@@ -463,6 +465,31 @@ class HipKernels:
         return (self.fold_norms and 0 < rows <= self.FOLD_NORM_ROWS and dtype == torch.bfloat16 and hidden % 8 == 0
                 and rows * hidden * 2 <= self.FOLD_NORM_BYTES)
 
+    def _reserve_exchange(self, n_tiles: int) -> None:
+        """Called when a matrix is prepared: the memory through which two blocks of a decode product exchange the sums
+        of a row tile whose parts of k they share (512 floats and a counter per row tile; the counters are zero between
+        launches).  One pair of buffers for all products - they follow each other on the stream."""
+        if self._exchange_tiles < n_tiles:
+            self._exchange_tiles = max(n_tiles, 4096)
+            self._exchange_pieces = torch.empty(self._exchange_tiles * 512, dtype=torch.float32, device=self.device)
+            self._exchange_arrivals = torch.zeros(self._exchange_tiles, dtype=torch.int32, device=self.device)
+
+    def _exchange(self, n_tiles: int):
+        """The exchange buffers if they serve a matrix of `n_tiles` row tiles (they do for every prepared matrix; they
+        are never replaced inside a step, whose recording may hold their addresses) - else the product keeps whole
+        row tiles in a block."""
+        if self._exchange_tiles < n_tiles:
+            return None, None
+        return self._exchange_pieces, self._exchange_arrivals
+
+    def decode_plan(self, weight, row_tiles_per_wave: int = 1, normed_rows: int = 0) -> dict:
+        """How `linear_adds` / `linear_scaled` cut a product over this matrix into blocks (for tests and measurements)."""
+        packed = weight.packed if isinstance(weight, GatedWeight) else weight
+        out = (ctypes.c_int * 4)()
+        may = 1 if self._exchange(packed.n_tiles)[0] is not None else 0
+        self.lib.akv_linear_decode_plan(row_tiles_per_wave, packed.n_tiles, packed.k_tiles, packed.k, normed_rows, may, out)
+        return dict(k_split=out[0], waves=out[1], blocks=out[2], straddles=bool(out[3]))
+
     def adds_to_stream(self, rows: int, weight, dtype) -> bool:
         return isinstance(weight, PackedWeight) and self.folds_norm(rows, weight.outs, dtype)
 
@@ -480,8 +507,10 @@ class HipKernels:
         self._dense(stream, "stream", torch.float32, (rows, weight.outs))
         self._dense(sums, "sums", torch.float32, ((weight.outs + 15) // 16, 16))
         self._dense(weight.data, "packed weight", torch.bfloat16)
-        self._check(self.lib.akv_linear_adds(_ptr(x), _ptr(weight.data), _ptr(stream), _ptr(sums), rows, weight.outs,
-                                             weight.k, weight.n_tiles, weight.k_tiles, self._stream()), "linear_adds")
+        pieces, arrivals = self._exchange(weight.n_tiles)
+        self._check(self.lib.akv_linear_adds(_ptr(x), _ptr(weight.data), _ptr(stream), _ptr(sums), _ptr(pieces),
+                                             _ptr(arrivals), rows, weight.outs, weight.k, weight.n_tiles,
+                                             weight.k_tiles, self._stream()), "linear_adds")
 
     def linear_scaled(self, stream, sums, norm_weight, eps, weight, out) -> None:
         """out = norm(stream) W^T (a `GatedWeight`: silu(. Wgate^T) * (. Wup^T)) with the norm of `add_rmsnorm`
@@ -498,10 +527,11 @@ class HipKernels:
         outs = weight.inter if gated else packed.outs
         self._dense(out, "out", torch.bfloat16, (rows, outs))
         self._dense(packed.data, "packed weight", torch.bfloat16)
+        pieces, arrivals = self._exchange(packed.n_tiles)
         self._check(self.lib.akv_linear_scaled(_ptr(stream), _ptr(sums), (k + 15) // 16, _ptr(norm_weight),
-                                               ctypes.c_float(eps), _ptr(packed.data), _ptr(out), rows, outs, k,
-                                               packed.n_tiles, packed.k_tiles, 1 if gated else 0, self._stream()),
-                    "linear_scaled")
+                                               ctypes.c_float(eps), _ptr(packed.data), _ptr(out), _ptr(pieces),
+                                               _ptr(arrivals), rows, outs, k, packed.n_tiles, packed.k_tiles,
+                                               1 if gated else 0, self._stream()), "linear_scaled")
 
     STATIC_ROWS_ELEMENTS = 64 * 32768   # bfloat16 elements of the library's static device memory for repacked rows
 
@@ -569,6 +599,7 @@ class HipKernels:
                 and gate.shape[1] % 8 == 0 and gate.shape[0] % 16 == 0):
             weight = GatedWeight(gate, up, keep_row_major=self.library_products_above is not None)
             self._products.setdefault(("gated", weight.inter, weight.k), weight)
+            self._reserve_exchange(weight.packed.n_tiles)
             return weight
         return None
 

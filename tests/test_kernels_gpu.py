@@ -377,6 +377,59 @@ def test_a_gated_product_norms_its_rows_from_the_sums_of_squares(hip, ref, rows,
     assert_close_but_for_flipped_roundings(got, want)
 
 
+@pytest.mark.parametrize("rows", [1, 8])
+@pytest.mark.parametrize("outs,k", [(5120, 8192), (5120, 5120), (5136, 8200), (5120, 17416)])
+def test_row_tiles_whose_parts_of_k_lie_in_two_blocks(hip, ref, rows, outs, k, monkeypatch):
+    """The decode products cut their work into equal blocks even where that splits a row tile's parts of k between two
+    blocks (320 row tiles on 256 compute units); the two exchange their sums through memory and the later one finishes
+    the tile.  Against the same products made to keep whole row tiles in a block (no exchange memory): equal up to the
+    order of the sum; twice in a row, since the counters must be back at zero; and against the double."""
+    monkeypatch.setattr(hip, "fold_norms", True)
+    monkeypatch.setattr(hip, "FOLD_NORM_ROWS", 16)
+    x = rand(rows, k, dtype=torch.bfloat16, seed=91)
+    w = rand(outs, k, dtype=torch.bfloat16, seed=92, scale=0.05)
+    packed = hip.prepare_linear(w.cuda())
+    plan = hip.decode_plan(packed)
+    assert plan["straddles"] and plan["blocks"] <= 256 and plan["waves"] % plan["k_split"] != 0, plan
+    stream = rand(rows, outs, seed=93, scale=2.0)
+    want = torch.empty(rows, outs, dtype=torch.bfloat16)
+    ref.linear(x, w, want)
+    tiles = (outs + 15) // 16
+
+    def adds():
+        got, sums = stream.cuda(), torch.full((tiles, 16), float("nan"), device="cuda")
+        hip.linear_adds(x.cuda(), packed, got, sums)
+        return got.cpu(), sums.cpu()
+
+    first, second = adds(), adds()
+    assert torch.equal(first[0], second[0]) and torch.equal(first[1], second[1])
+    assert int(hip._exchange_arrivals.abs().sum()) == 0
+    with monkeypatch.context() as patch:
+        patch.setattr(hip, "_exchange", lambda n_tiles: (None, None))
+        whole = adds()
+    apart = (first[0] - whole[0]).abs()
+    assert (apart > 0).float().mean() < 0.01 and apart.max() <= 2.0 ** -7 * want.float().abs().max().item()
+    torch.testing.assert_close(first[0], stream + want.float(), rtol=0, atol=2.0 ** -7 * want.float().abs().max().item())
+    torch.testing.assert_close(first[1].sum(0)[:rows].double(), first[0].double().pow(2).sum(-1), rtol=1e-5, atol=1e-6)
+    # the product that norms its rows, over the same matrix read the other way round (k of the norm = outs here)
+    if rows * outs * 2 <= hip.FOLD_NORM_BYTES and outs % 8 == 0:
+        back = hip.prepare_linear(rand(5120, outs, dtype=torch.bfloat16, seed=94, scale=0.05).cuda())
+        gain = 1 + rand(outs, seed=95, scale=0.1)
+        residual, sums = first[0].cuda(), first[1].cuda()
+
+        def scaled():
+            got = torch.full((rows, 5120), float("nan"), dtype=torch.bfloat16, device="cuda")
+            hip.linear_scaled(residual, sums, gain.cuda(), 1e-6, back, got)
+            return got.cpu()
+
+        got = scaled()
+        assert torch.equal(got, scaled()) and int(hip._exchange_arrivals.abs().sum()) == 0
+        normed, want_back = torch.empty(rows, outs, dtype=torch.bfloat16), torch.empty(rows, 5120, dtype=torch.bfloat16)
+        ref.add_rmsnorm(first[0].clone(), None, gain, 1e-6, normed)
+        ref.linear(normed, back.unpack().cpu(), want_back)
+        assert_close_but_for_flipped_roundings(got, want_back)
+
+
 def test_products_of_17_to_512_rows_follow_a_table_that_is_measured_on_request(hip, ref, tmp_path):
     """Which kernel takes a product of 17..512 rows - the skinny one (up to 64), the mid-size one, the library - is
     decided by a fixed rule unless the table of choices names the product (matrix shape and row bucket).  Nothing is
