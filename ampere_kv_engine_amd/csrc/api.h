@@ -53,8 +53,9 @@ int akv_linear_packed_static(const void* x, const void* wp, void* y, int y_dtype
                              int n_tiles, int k_tiles, hipStream_t stream);
 int akv_linear_decode_plan(int rt, int n_tiles, int k_tiles, int k, int normed_rows, int may_straddle, int* out);
 int akv_linear_adds(const void* x, const void* wp, float* stream_out, float* sums_out, float* pieces,
-                    unsigned int* arrivals, int rows, int outs, int k, int n_tiles, int k_tiles, hipStream_t stream);
+                    unsigned int* arrivals, int exchange_tiles, int rows, int outs, int k, int n_tiles, int k_tiles,
+                    hipStream_t stream);
 int akv_linear_scaled(const float* stream_in, const float* sums, int sum_tiles, const float* gain, float eps,
-                      const void* wp, void* y, float* pieces, unsigned int* arrivals, int rows, int outs, int k,
-                      int n_tiles, int k_tiles, int gated, hipStream_t stream);
+                      const void* wp, void* y, float* pieces, unsigned int* arrivals, int exchange_tiles, int rows,
+                      int outs, int k, int n_tiles, int k_tiles, int gated, hipStream_t stream);
 }

@@ -370,7 +370,8 @@ int launch_decode(DecodeArgs a, hipStream_t stream) {
 
 // stream_out [rows, outs] += bfloat16(x W^T) in place (float32); sums_out [n_tiles][16] receives, for every row tile of
 // 16 outputs and every row, the sum of squares of the new values (rows beyond `rows`: 0).  rows <= 16, k % 8 == 0.
-// `pieces` (n_tiles * 512 floats) and `arrivals` (n_tiles words, zero; left zero) may be null: with them the product
+// `pieces` (exchange_tiles * 512 floats) and `arrivals` (exchange_tiles words, zero; left zero) may be null, or hold
+// fewer than n_tiles row tiles' worth, and are then not used: with them the product
 // may be cut into blocks that do not hold whole row tiles' parts of k (see plan_decode).  Launches that share them
 // follow each other on one stream.
 // What plan_decode makes of a product (for tests and measurements): out[0..3] = parts of k, waves per block, blocks,
@@ -382,8 +383,8 @@ extern "C" int akv_linear_decode_plan(int rt, int n_tiles, int k_tiles, int k, i
 }
 
 extern "C" int akv_linear_adds(const void* x, const void* wp, float* stream_out, float* sums_out, float* pieces,
-                               unsigned int* arrivals, int rows, int outs, int k, int n_tiles, int k_tiles,
-                               hipStream_t stream) {
+                               unsigned int* arrivals, int exchange_tiles, int rows, int outs, int k, int n_tiles,
+                               int k_tiles, hipStream_t stream) {
   if (rows <= 0 || outs <= 0) return 0;
   if (rows > 16 || (k & 7) != 0 || n_tiles * 16 < outs || (n_tiles - 1) * 16 >= outs || k_tiles * 32 < k) return -2;
   DecodeArgs a{};
@@ -391,7 +392,7 @@ extern "C" int akv_linear_adds(const void* x, const void* wp, float* stream_out,
   a.wp = static_cast<const uintx4*>(wp);
   a.stream_out = stream_out;
   a.sums_out = sums_out;
-  if (pieces != nullptr && arrivals != nullptr) a.pieces = pieces, a.arrivals = arrivals;
+  if (pieces != nullptr && arrivals != nullptr && exchange_tiles >= n_tiles) a.pieces = pieces, a.arrivals = arrivals;
   a.rows = rows, a.outs = outs, a.k = k, a.k_tiles = k_tiles, a.n_tiles = n_tiles;
   return launch_decode<1, false, false, true>(a, stream);
 }
@@ -403,8 +404,8 @@ extern "C" int akv_linear_adds(const void* x, const void* wp, float* stream_out,
 // (rows * k bfloat16) fit into a compute unit's LDS (160 KB) beside 832 bytes; -2 otherwise.  `pieces`, `arrivals`: as
 // for akv_linear_adds.
 extern "C" int akv_linear_scaled(const float* stream_in, const float* sums, int sum_tiles, const float* gain, float eps,
-                                 const void* wp, void* y, float* pieces, unsigned int* arrivals, int rows, int outs,
-                                 int k, int n_tiles, int k_tiles, int gated, hipStream_t stream) {
+                                 const void* wp, void* y, float* pieces, unsigned int* arrivals, int exchange_tiles,
+                                 int rows, int outs, int k, int n_tiles, int k_tiles, int gated, hipStream_t stream) {
   if (rows <= 0 || outs <= 0) return 0;
   if (rows > 16 || (k & 7) != 0 || k_tiles * 32 < k || sum_tiles != (k + 15) / 16) return -2;
   if (gated ? ((outs & 15) != 0 || n_tiles * 8 != outs) : n_tiles * 16 < outs) return -2;
@@ -416,7 +417,7 @@ extern "C" int akv_linear_scaled(const float* stream_in, const float* sums, int 
   a.eps = eps;
   a.wp = static_cast<const uintx4*>(wp);
   a.y = static_cast<bf16_t*>(y);
-  if (pieces != nullptr && arrivals != nullptr) a.pieces = pieces, a.arrivals = arrivals;
+  if (pieces != nullptr && arrivals != nullptr && exchange_tiles >= n_tiles) a.pieces = pieces, a.arrivals = arrivals;
   const bool may = a.pieces != nullptr;
   a.rows = rows, a.outs = outs, a.k = k, a.k_tiles = k_tiles, a.n_tiles = n_tiles;
   if (gated) return launch_decode<2, true, true, false>(a, stream);

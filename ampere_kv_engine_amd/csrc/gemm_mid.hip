@@ -286,11 +286,14 @@ MidPlan plan_mid(int rows, int n_tiles, int k_tiles, bool gated, int along, int 
         if (parts == 0 && p.partial_floats > kMostPartialFloats) continue;
         const long blocks = static_cast<long>(p.bands) * p.parts * m_blocks;
         const long rounds = (blocks + kComputeUnits - 1) / kComputeUnits;
-        // tiles the busiest compute unit streams (+ a little per block, and what the exchange of partial sums moves:
-        // 4 bytes x parts per result against 1 KB per tile); of equal cuts the one with more waves along the band
-        // wins (they share the activations), then the one with fewer parts
-        double cost = static_cast<double>(rounds) * (static_cast<double>(a) * r * p.part_tiles + 8.0);
-        if (p.parts > 1) cost += static_cast<double>(a) * r * mt * p.parts / 8.0;
+        // What the busiest compute unit moves, counted in weight tiles (1 KB from memory, about 50 ns at the rate a
+        // unit gets when all read): its blocks' weight tiles; the activation tiles they stage through LDS, which come
+        // from the caches and cost two thirds of a weight tile each (fitted: the down product of 4,096 x 12,288 at 64
+        // rows takes 45.7 us with 768 activation tiles a block, 33.2 with 384); a little per block; and the exchange
+        // of partial sums (fitted on the same product: 9 us for 8 parts of 8 row tiles x 4 tiles of rows).  Of equal
+        // cuts the one with more waves along the band wins, then the one with fewer parts.
+        double cost = static_cast<double>(rounds) * (static_cast<double>(a) * r * p.part_tiles + 0.68 * mt * p.part_tiles + 8.0);
+        if (p.parts > 1) cost += static_cast<double>(a) * r * mt * p.parts / 1.6;
         cost += 0.01 * (4 - a) + 0.001 * p.parts;
         if (best_cost < 0.0 || cost < best_cost) best = p, best_cost = cost;
       }
@@ -353,9 +356,11 @@ extern "C" int akv_linear_mid_workspace(int rows, int n_tiles, int k_tiles, int 
 // x [rows, k] bfloat16 row-major, 1 <= rows; wp the packed weight; y [rows, outs] (gated: [rows, inter], wp as for
 // akv_linear_packed_swiglu).  `along` (waves along a band: 2..4), `rt` (row tiles per wave, 1 or 2), `depth` (register
 // sets of the weight ring: 2, or 4 with rt = 1) and `parts` (blocks along k, a power of two) may be 0: chosen here.
-extern "C" int akv_linear_mid(const void* x, const void* wp, void* y, int y_dtype, float* partial, unsigned* counters,
-                              int rows, int outs, int k, int n_tiles, int k_tiles, int gated, int along, int rt,
-                              int depth, int parts, hipStream_t stream) {
+// `partial_floats` and `counter_words` say how much `partial` and `counters` hold: a cut that needs more
+// (akv_linear_mid_workspace tells) is refused with -3 and nothing is launched.
+extern "C" int akv_linear_mid(const void* x, const void* wp, void* y, int y_dtype, float* partial, long partial_floats,
+                              unsigned* counters, long counter_words, int rows, int outs, int k, int n_tiles,
+                              int k_tiles, int gated, int along, int rt, int depth, int parts, hipStream_t stream) {
   if (rows <= 0 || outs <= 0) return 0;
   if ((k & 7) != 0 || k_tiles * 32 < k) return -2;
   if (gated ? ((outs & 15) != 0 || n_tiles * 8 != outs) : n_tiles * 16 < outs) return -2;
@@ -363,6 +368,7 @@ extern "C" int akv_linear_mid(const void* x, const void* wp, void* y, int y_dtyp
   const MidPlan p = plan_mid(rows, n_tiles, k_tiles, gated != 0, along, rt, depth, parts);
   if (p.along == 0) return -2;
   if (p.parts > 1 && (partial == nullptr || counters == nullptr)) return -2;
+  if (p.parts > 1 && (static_cast<long>(p.partial_floats) > partial_floats || static_cast<long>(p.counters) > counter_words)) return -3;
   if (gated) {
     if (y_dtype == kF32) return dispatch_mid<true, float>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, stream);
     if (y_dtype == kBF16) return dispatch_mid<true, bf16_t>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, stream);

@@ -353,8 +353,10 @@ class HipKernels:
                 if torch.cuda.is_current_stream_capturing():
                     raise KernelError("a recorded step needs more counters than the steps before it")
                 self._mid_counters = torch.zeros(max(counters.value, 4096), dtype=torch.int32, device=self.device)
+        held = lambda buffer: ctypes.c_long(buffer.numel() if buffer is not None else 0)
         self._check(self.lib.akv_linear_mid(_ptr(x), _ptr(packed.data), _ptr(out), _code(out), _ptr(self._mid_partial),
-                                            _ptr(self._mid_counters), rows, outs, packed.k, packed.n_tiles,
+                                            held(self._mid_partial), _ptr(self._mid_counters), held(self._mid_counters),
+                                            rows, outs, packed.k, packed.n_tiles,
                                             packed.k_tiles, 1 if gated else 0, 0, 0, 0, 0, self._stream()),
                     "mid-size product")
 
@@ -509,7 +511,8 @@ class HipKernels:
         self._dense(weight.data, "packed weight", torch.bfloat16)
         pieces, arrivals = self._exchange(weight.n_tiles)
         self._check(self.lib.akv_linear_adds(_ptr(x), _ptr(weight.data), _ptr(stream), _ptr(sums), _ptr(pieces),
-                                             _ptr(arrivals), rows, weight.outs, weight.k, weight.n_tiles,
+                                             _ptr(arrivals), self._exchange_tiles if pieces is not None else 0,
+                                             rows, weight.outs, weight.k, weight.n_tiles,
                                              weight.k_tiles, self._stream()), "linear_adds")
 
     def linear_scaled(self, stream, sums, norm_weight, eps, weight, out) -> None:
@@ -530,7 +533,8 @@ class HipKernels:
         pieces, arrivals = self._exchange(packed.n_tiles)
         self._check(self.lib.akv_linear_scaled(_ptr(stream), _ptr(sums), (k + 15) // 16, _ptr(norm_weight),
                                                ctypes.c_float(eps), _ptr(packed.data), _ptr(out), _ptr(pieces),
-                                               _ptr(arrivals), rows, outs, k, packed.n_tiles, packed.k_tiles,
+                                               _ptr(arrivals), self._exchange_tiles if pieces is not None else 0,
+                                               rows, outs, k, packed.n_tiles, packed.k_tiles,
                                                1 if gated else 0, self._stream()), "linear_scaled")
 
     STATIC_ROWS_ELEMENTS = 64 * 32768   # bfloat16 elements of the library's static device memory for repacked rows

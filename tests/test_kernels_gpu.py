@@ -500,7 +500,7 @@ def test_mid_size_product(hip_own, ref, rows, outs, k):
         for code, dtype in ((1, torch.bfloat16), (0, torch.float32)):
             for _ in range(2):
                 got = torch.full((rows, outs), float("nan"), dtype=dtype, device="cuda")
-                status = lib.akv_linear_mid(_ptr(xd), _ptr(packed.data), _ptr(got), code, _ptr(partial), _ptr(counters), rows,
+                status = lib.akv_linear_mid(_ptr(xd), _ptr(packed.data), _ptr(got), code, _ptr(partial), ctypes.c_long(partial.numel()), _ptr(counters), ctypes.c_long(counters.numel()), rows,
                                             outs, k, packed.n_tiles, packed.k_tiles, 0, along, rt, depth, parts, stream)
                 assert status == 0, (along, rt, depth, parts, status)
                 limits = tol(dtype) if dtype == torch.bfloat16 else dict(rtol=2e-5, atol=2e-5 * float(want.abs().max()))
@@ -511,9 +511,15 @@ def test_mid_size_product(hip_own, ref, rows, outs, k):
     first = torch.empty((rows, outs), dtype=torch.float32, device="cuda")
     again = torch.empty((rows, outs), dtype=torch.float32, device="cuda")
     for target in (first, again):
-        assert lib.akv_linear_mid(_ptr(xd), _ptr(packed.data), _ptr(target), 0, _ptr(partial), _ptr(counters), rows, outs, k,
+        assert lib.akv_linear_mid(_ptr(xd), _ptr(packed.data), _ptr(target), 0, _ptr(partial), ctypes.c_long(partial.numel()), _ptr(counters), ctypes.c_long(counters.numel()), rows, outs, k,
                                   packed.n_tiles, packed.k_tiles, 0, 4, 1, 4, 4, stream) == 0
     assert torch.equal(first, again)
+    # a workspace that is too small for the cut is refused before anything is launched
+    need, words = ctypes.c_long(0), ctypes.c_long(0)
+    lib.akv_linear_mid_workspace(rows, packed.n_tiles, packed.k_tiles, 0, 4, 1, 4, 4, ctypes.byref(need), ctypes.byref(words))
+    assert lib.akv_linear_mid(_ptr(xd), _ptr(packed.data), _ptr(first), 0, _ptr(partial), ctypes.c_long(16), _ptr(counters),
+                              ctypes.c_long(counters.numel()), rows, outs, k, packed.n_tiles, packed.k_tiles, 0, 4, 1, 4, 4,
+                              stream) == (-3 if need.value > 16 else 0)
 
 
 @pytest.mark.parametrize("rows,inter,k", [(40, 208, 264), (64, 512, 2048), (130, 208, 520), (17, 16, 8), (256, 1024, 1024)])
@@ -531,7 +537,7 @@ def test_mid_size_gated_product(hip_own, ref, rows, inter, k):
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     for along, parts in ((0, 0), (2, 1), (3, 2), (4, 4)):
         got = torch.full((rows, inter), float("nan"), dtype=torch.bfloat16, device="cuda")
-        assert lib.akv_linear_mid(_ptr(x.cuda()), _ptr(weight.packed.data), _ptr(got), 1, _ptr(partial), _ptr(counters), rows,
+        assert lib.akv_linear_mid(_ptr(x.cuda()), _ptr(weight.packed.data), _ptr(got), 1, _ptr(partial), ctypes.c_long(partial.numel()), _ptr(counters), ctypes.c_long(counters.numel()), rows,
                                   inter, k, weight.packed.n_tiles, weight.packed.k_tiles, 1, along, 2, 2, parts, stream) == 0
         torch.testing.assert_close(got.cpu().float(), want.float(), **tol(torch.bfloat16))
     assert int(counters.abs().sum()) == 0
