@@ -6,14 +6,18 @@
 //           (row tile of 16 outputs, row) - every output is owned by one lane, so no value depends on an order;
 //   SCALED  the product that reads the norm of the residual sum (q/k/v, gate and up) does not read normed rows: every
 //           block norms the rows for itself into LDS while its first weights are on their way.  The rows' sums of
-//           squares are not formed again: a wave adds the partial sums in a fixed order (the same in every block) and
-//           forms rsqrt(mean + eps); then every thread norms pieces of 8 values as the norm kernel does - scaled,
-//           rounded, times the weight, rounded - and puts them where the matrix cores' operand wants them.
+//           squares are not formed again: the block's waves add the partial sums in a fixed order and form
+//           rsqrt(mean + eps); then every thread norms pieces of 8 values as the norm kernel does - scaled, rounded,
+//           times the weight, rounded - and puts them where the matrix cores' operand wants them.
 //
 // Otherwise this is the skinny kernel of gemm_mfma.hip for one tile of rows: a wave owns RT row tiles of the packed
 // weight and a part of k, streams its tiles once (two groups of registers in turn, loads marked as read-once), the
 // parts of k are summed through LDS in a fixed order.  GATED as there (a pair of gate and up tiles, RT = 2).
-// The results equal those of the separate kernels up to the order in which a row's squares are added.
+// The work is numbered in units - (RT row tiles, part of k) - and a block takes as many consecutive units as gives
+// every compute unit the same share (plan_decode); where that leaves a row tile's parts in two neighbouring blocks,
+// the later of the two finishes the tile from sums that both leave in memory.
+// The results equal those of the separate kernels up to the order in which a row's squares, and the parts of k, are
+// added.
 
 #include <mutex>
 
