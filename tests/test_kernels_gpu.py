@@ -430,6 +430,49 @@ def test_row_tiles_whose_parts_of_k_lie_in_two_blocks(hip, ref, rows, outs, k, m
         assert_close_but_for_flipped_roundings(got, want_back)
 
 
+def test_decode_products_at_random_sizes(hip, ref, monkeypatch):
+    """The products that add themselves to the residual sum and norm their rows, at sixty random sizes - outputs and k
+    that are no multiples of the tiles, every number of rows, small matrices (one block) and large ones (blocks that
+    share row tiles) - against the double's product, sum and norm."""
+    monkeypatch.setattr(hip, "fold_norms", True)
+    monkeypatch.setattr(hip, "FOLD_NORM_ROWS", 16)
+    generator = torch.Generator().manual_seed(2024)
+    pick = lambda low, high: int(torch.randint(low, high + 1, (1,), generator=generator))
+    for case in range(60):
+        large = case % 6 == 0
+        rows = pick(1, 16)
+        outs = pick(4800, 7200) if large else pick(1, 700)
+        k = 8 * (pick(500, 1100) if large else pick(1, 300))
+        hidden = 8 * pick(2, 300)                      # width of the residual rows that the second product norms
+        x = rand(rows, k, dtype=torch.bfloat16, seed=1000 + case)
+        w = rand(hidden, k, dtype=torch.bfloat16, seed=2000 + case, scale=0.05)
+        stream = rand(rows, hidden, seed=3000 + case, scale=2.0)
+        what = f"case {case}: rows {rows}, {hidden} x {k}, then {outs} x {hidden}"
+        y = torch.empty(rows, hidden, dtype=torch.bfloat16)
+        ref.linear(x, w, y)
+        residual = stream.cuda()
+        tiles = (hidden + 15) // 16
+        sums = torch.full((tiles, 16), float("nan"), device="cuda")
+        hip.linear_adds(x.cuda(), hip.prepare_linear(w.cuda()), residual, sums)
+        scale = y.float().abs().max().item()
+        torch.testing.assert_close(residual.cpu(), stream + y.float(), rtol=0, atol=2.0 ** -7 * scale, msg=lambda m: f"{what}: {m}")
+        torch.testing.assert_close(sums.cpu().sum(0)[:rows].double(), residual.cpu().double().pow(2).sum(-1), rtol=1e-5, atol=1e-6,
+                                   msg=lambda m: f"{what}: {m}")
+        assert (sums.cpu()[:, rows:] == 0).all(), what
+        if rows * hidden * 2 > hip.FOLD_NORM_BYTES:
+            continue
+        gain = 1 + rand(hidden, seed=4000 + case, scale=0.1)
+        second = rand(outs, hidden, dtype=torch.bfloat16, seed=5000 + case, scale=0.05)
+        normed, want = torch.empty(rows, hidden, dtype=torch.bfloat16), torch.empty(rows, outs, dtype=torch.bfloat16)
+        ref.add_rmsnorm(residual.cpu().clone(), None, gain, 1e-6, normed)
+        ref.linear(normed, second, want)
+        got = torch.full((rows, outs), float("nan"), dtype=torch.bfloat16, device="cuda")
+        hip.linear_scaled(residual, sums, gain.cuda(), 1e-6, hip.prepare_linear(second.cuda()), got)
+        assert torch.isfinite(got.float()).all(), what
+        assert_close_but_for_flipped_roundings(got, want)
+    assert int(hip._exchange_arrivals.abs().sum()) == 0
+
+
 def test_products_of_17_to_512_rows_follow_a_table_that_is_measured_on_request(hip, ref, tmp_path):
     """Which kernel takes a product of 17..512 rows - the skinny one (up to 64), the mid-size one, the library - is
     decided by a fixed rule unless the table of choices names the product (matrix shape and row bucket).  Nothing is
