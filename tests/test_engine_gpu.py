@@ -35,6 +35,16 @@ def test_cutting(engine, case, cutting):
     getattr(cases, "case_" + cutting)(engine, case)
 
 
+@pytest.mark.parametrize("cutting", ["last_32_one_by_one", "mixed_with_pages_used_again"])
+def test_cutting_with_the_norm_kernels_of_their_own(case, cutting):
+    """By default decode steps of bfloat16 run without norm kernels inside the layers (the products add themselves to
+    the residual sum and norm their rows).  With that switched off the layers go through `add_rmsnorm` - and, for a step
+    of one row, through the product that norms its one row, sums of squares included: the same limits hold."""
+    engine = cases.make_engine(case, "bfloat16", "cuda:0")
+    engine.kernels.fold_norms = False
+    getattr(cases, "case_" + cutting)(engine, case)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_program(case, dtype, tmp_path):
     """bin/trace_run as a user runs it: JSON steps on stdin, <step>.f32 files out, `done <step>` lines - fed all four
