@@ -289,10 +289,12 @@ MidPlan plan_mid(int rows, int n_tiles, int k_tiles, bool gated, int along, int 
         // What the busiest compute unit moves, counted in weight tiles (1 KB from memory, about 50 ns at the rate a
         // unit gets when all read): its blocks' weight tiles; the activation tiles they stage through LDS, which come
         // from the caches and cost two thirds of a weight tile each (fitted: the down product of 4,096 x 12,288 at 64
-        // rows takes 45.7 us with 768 activation tiles a block, 33.2 with 384); a little per block; and the exchange
-        // of partial sums (fitted on the same product: 9 us for 8 parts of 8 row tiles x 4 tiles of rows).  Of equal
-        // cuts the one with more waves along the band wins, then the one with fewer parts.
-        double cost = static_cast<double>(rounds) * (static_cast<double>(a) * r * p.part_tiles + 0.68 * mt * p.part_tiles + 8.0);
+        // rows takes 45.7 us with 768 activation tiles a block, 33.2 with 384); what a block costs before and after
+        // its stream, about 1.2 us (the down product of 5,120 x 17,408 at 32 rows: 57 us as 1,280 blocks of 34 k tiles,
+        // 42 us as 216 blocks of 136); and the exchange of partial sums (fitted on the first product: 9 us for 8 parts
+        // of 8 row tiles x 4 tiles of rows).  Of equal cuts the one with more waves along the band wins, then the one
+        // with fewer parts.
+        double cost = static_cast<double>(rounds) * (static_cast<double>(a) * r * p.part_tiles + 0.68 * mt * p.part_tiles + 24.0);
         if (p.parts > 1) cost += static_cast<double>(a) * r * mt * p.parts / 1.6;
         cost += 0.01 * (4 - a) + 0.001 * p.parts;
         if (best_cost < 0.0 || cost < best_cost) best = p, best_cost = cost;
