@@ -135,6 +135,17 @@ def case_mixed_with_pages_used_again(engine, case):
     assert any(pages[a] & pages[b] for i, a in enumerate(names) for b in names[i + 1:]), "no page was used again"
 
 
+def case_mixed_in_other_orders(engine, case):
+    """The mixed schedule again with the requests arriving in other orders and cut by other draws."""
+    import random
+    for seed in (21, 22):
+        names = list(case["requests"])
+        random.Random(seed).shuffle(names)
+        requests = {name: case["requests"][name] for name in names}
+        sub = dict(case, requests=requests, expected={name: case["expected"][name] for name in names})
+        check(engine, sub, schedules.mixed(requests, PROMPTS, case["page_size"], engine.config.num_pages, seed=seed))
+
+
 def case_first_tokens_and_one_token_prompt(engine, case):
     requests = {"x": case["requests"]["a"][:1], "y": case["requests"]["c"][:3]}
     sub = dict(case, requests=requests, expected={k: case["expected"][n][:len(v)] for (k, v), n in zip(requests.items(), "ac")})
