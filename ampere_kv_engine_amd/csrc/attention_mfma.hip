@@ -1120,6 +1120,19 @@ __global__ __launch_bounds__(64 * kMergeWaves) void attention_merge_kernel(const
     src = a.partial + ((static_cast<long>(a.plan[4 + 2 * blockIdx.x]) * gridDim.y + blockIdx.y) * (16 * NQ) + c) * PSTRIDE;
     split_stride *= gridDim.y;
   }
+  // this wave's segments: z = wave + kMergeWaves * i.  Eight segments' loads go out together; the first eight are
+  // asked for before the maxima - they do not depend on them, and the kernel is a chain of trips to memory.
+  const int mine = (splits - wave + kMergeWaves - 1) / kMergeWaves;
+  auto fetch8 = [&](int i0, int ii0, int count, float (&v)[8][PER]) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float* p = src + (wave + static_cast<long>(kMergeWaves) * (i0 + min(ii0 + j, count - 1))) * split_stride;
+#pragma unroll
+      for (int e = 0; e < PER; ++e) v[j][e] = lane + e * 64 < D ? p[lane + e * 64] : 0.f;
+    }
+  };
+  float ahead[8][PER] = {};
+  if (mine > 0) fetch8(0, 0, min(64, mine), ahead);
   // every wave finds the maximum over all segments (a lane per segment)
   float top = -INFINITY;
   bool poisoned = false;
@@ -1131,8 +1144,6 @@ __global__ __launch_bounds__(64 * kMergeWaves) void attention_merge_kernel(const
   }
   top = wave_max(top);
   poisoned = __any(poisoned);
-  // this wave's segments: z = wave + kMergeWaves * i
-  const int mine = (splits - wave + kMergeWaves - 1) / kMergeWaves;
   float denom = 0.f, acc[PER];
 #pragma unroll
   for (int i = 0; i < PER; ++i) acc[i] = 0.f;
@@ -1146,13 +1157,15 @@ __global__ __launch_bounds__(64 * kMergeWaves) void attention_merge_kernel(const
       denom += w * src[z * split_stride + D + 1];
     }
     const int count = min(64, mine - i0);
-    for (int ii0 = 0; ii0 < count; ii0 += 8) {  // ascending segments; eight segments' loads go out together
+    for (int ii0 = 0; ii0 < count; ii0 += 8) {  // ascending segments
       float v[8][PER];
+      if (i0 == 0 && ii0 == 0) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float* p = src + (wave + static_cast<long>(kMergeWaves) * (i0 + min(ii0 + j, count - 1))) * split_stride;
+        for (int j = 0; j < 8; ++j)
 #pragma unroll
-        for (int e = 0; e < PER; ++e) v[j][e] = lane + e * 64 < D ? p[lane + e * 64] : 0.f;
+          for (int e = 0; e < PER; ++e) v[j][e] = ahead[j][e];
+      } else {
+        fetch8(i0, ii0, count, v);
       }
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
