@@ -2,6 +2,8 @@
 // cache write, the fused q/k-norm + rotation + cache write, SwiGLU, row gather.
 // Statistics, angles and the residual sum are float32 whatever the activation type T is.
 
+#include <type_traits>
+
 #include "common.h"
 #include "api.h"
 
@@ -174,10 +176,34 @@ __global__ void gather_rows_kernel(const float* __restrict__ stream, const T* __
 }
 
 // ---- SwiGLU: out[n, i] = silu(gate_up[n, i]) * gate_up[n, inter + i] ----------------------------------------
-// A thread handles 4 consecutive outputs (16-byte accesses for float32, 8-byte for bfloat16) when `inter` allows.
+// A thread handles 8 consecutive bfloat16 outputs or 4 float32 ones (16-byte accesses) when `inter` allows.
+template <typename T> long swiglu_threads(long tokens, int inter) {
+  if (std::is_same<T, bf16_t>::value && (inter & 7) == 0) return tokens * (inter / 8);
+  return (inter & 3) == 0 ? tokens * (inter / 4) : tokens * inter;
+}
 template <typename T>
 __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, long tokens, int inter) {
   const long index = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if constexpr (std::is_same<T, bf16_t>::value) {
+    if ((inter & 7) == 0) {   // 16-byte accesses; the stacked product is read once and never again
+      const int octets = inter / 8;
+      if (index >= tokens * octets) return;
+      const long n = index / octets;
+      const int i = static_cast<int>(index % octets) * 8;
+      typedef __attribute__((ext_vector_type(4))) unsigned int words4;
+      const words4 gw = __builtin_nontemporal_load(reinterpret_cast<const words4*>(gate_up + n * 2 * inter + i));
+      const words4 uw = __builtin_nontemporal_load(reinterpret_cast<const words4*>(gate_up + n * 2 * inter + inter + i));
+      words4 pw;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
+        const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
+        pw[j] = bf16_pair(g0 / (1.f + expf(-g0)) * u0, g1 / (1.f + expf(-g1)) * u1);
+      }
+      *reinterpret_cast<words4*>(out + n * inter + i) = pw;
+      return;
+    }
+  }
   if ((inter & 3) == 0) {
     const int quads = inter / 4;
     if (index >= tokens * quads) return;
@@ -578,7 +604,7 @@ int akv_read_probe(const void* data, long bytes, unsigned int* out, int blocks, 
 int akv_swiglu(const void* gate_up, void* out, int dtype, long tokens, int inter, hipStream_t stream) {
   if (tokens <= 0) return 0;
   AKV_DISPATCH(dtype, T,
-               swiglu_kernel<T><<<blocks_for((inter & 3) == 0 ? tokens * (inter / 4) : tokens * inter, 256), 256, 0, stream>>>(
+               swiglu_kernel<T><<<blocks_for(swiglu_threads<T>(tokens, inter), 256), 256, 0, stream>>>(
                    static_cast<const T*>(gate_up), static_cast<T*>(out), tokens, inter));
   return AKV_LAUNCH_STATUS();
 }
