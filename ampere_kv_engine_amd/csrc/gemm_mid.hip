@@ -7,8 +7,9 @@
 //   * a block owns a band of A * RT row tiles of the packed weight (see gemm_mfma.hip for the packing); 2 A of its
 //     waves multiply, A along the band x 2 along k (each half of the block's k);
 //   * per stage of S k-tiles the block's activations [16 * MT rows][S * 32 k] of either k half go through LDS,
-//     double-buffered, one barrier per stage, already in the lane order of the matrix-core operand (a tile of 16 rows
-//     x 32 k is 1 KB that lane l reads at l * 16: no bank conflicts).  Four further waves do nothing but fetch them,
+//     double-buffered, one barrier per stage, as tiles of the matrix-core operand (16 rows x 32 k, 1 KB; the places
+//     of a tile's 64 pieces are permuted so that neither readers nor writers meet in a bank).  Four further waves do
+//     nothing but fetch them, whole cache lines of a few rows per load,
 //     two stages ahead: a wave's loads come back in the order they were issued, so a multiplying wave that fetched
 //     activations between its weight loads would have to wait for ALL weights it has asked for before it could use
 //     the activations - which brings the weights' distance down to one stage (measured: 1.6 us per stage, whatever
@@ -37,6 +38,11 @@ constexpr int kFetchers = 4;
 constexpr int kComputeUnits = 256;
 
 template <int MT> constexpr int kStage = MT <= 4 ? 4 : 2;     // k-tiles per stage and k half
+
+// Where the 16 bytes of operand lane (r, g) lie inside the 1 KB tile of the stage's k-tile u.  A multiplying wave reads a
+// tile's 64 places at once, a fetching wave writes, per load, the places of a few rows r and all (u, g): with the
+// row's lowest bits turned by (u, g) both spread evenly over the memory's banks.
+__device__ __forceinline__ int slot_of(int u, int g, int r) { return g * 16 + (r ^ ((u * 4 + g) & 7)); }
 
 template <int A, int MT, int RT, int G, bool GATED, typename TY>
 __global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_kernel(const bf16_t* __restrict__ x, const uintx4* __restrict__ wp,
@@ -69,19 +75,34 @@ __global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_ker
   const uintx4 zero = {0u, 0u, 0u, 0u};
 
   if (wave >= kMultipliers) {
-    // ---- a fetching wave: activation tile i = (k half, k-tile of the stage, row tile); this wave brings
-    //      i = f, f + 4, ... of every stage, two stages ahead of the multiplying waves
+    // ---- a fetching wave.  A load brings 1 KB of the stage's activations as they lie in memory: 16 / S rows, of each
+    //      the S * 32 consecutive k of one k half (whole cache lines; lane (r, g) of the operand asking for its own
+    //      16 bytes would touch 16 rows a load and keep the cache's tag lookup busier than the weights do).  A stage
+    //      has kTiles such loads; this wave brings i = f, f + 4, ... of every stage, two stages ahead of the
+    //      multiplying waves, and files each 16-byte piece at its place of the operand tile (see `slot_of`).
     const int f = wave - kMultipliers;
+    constexpr int kRowsPerLoad = 16 / S;
+    const int row_in_load = lane / (4 * S), piece = lane % (4 * S);   // piece = k-tile of the stage * 4 + chunk of 8
     uintx4 fetched[2][kLoads];
     auto fetch_rows = [&](int stage, uintx4 (&into)[kLoads]) {
 #pragma unroll
       for (int j = 0; j < kLoads; ++j) {
         const int i = f + kFetchers * j;
-        const int h = i / (S * MT), u = (i / MT) % S, mt = i % MT;
-        const int kt = kb0 + h * per_half + stage * S + u;
-        const int row = row0 + mt * 16 + r, col = kt * 32 + g * 8;
+        const int h = i / (S * MT), group = i % (S * MT);
+        const int kt = kb0 + h * per_half + stage * S + piece / 4;
+        const int row = row0 + group * kRowsPerLoad + row_in_load, col = kt * 32 + (piece % 4) * 8;
         const bool there = kt < min(kb1, kb0 + (h + 1) * per_half) && row < rows && col < k;
         into[j] = there ? *reinterpret_cast<const uintx4*>(x + static_cast<size_t>(row) * k + col) : zero;
+      }
+    };
+    auto file_rows = [&](int buffer, const uintx4 (&from)[kLoads]) {
+#pragma unroll
+      for (int j = 0; j < kLoads; ++j) {
+        const int i = f + kFetchers * j;
+        const int h = i / (S * MT), group = i % (S * MT);
+        const int row = group * kRowsPerLoad + row_in_load;          // of the block's MT * 16
+        const int u = piece / 4, g = piece % 4;
+        staged[(buffer * kTiles + (h * S + u) * MT + row / 16) * 64 + slot_of(u, g, row % 16)] = from[j];
       }
     };
     fetch_rows(0, fetched[0]);
@@ -91,8 +112,7 @@ __global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_ker
       for (int d = 0; d < 2; ++d) {
         const int stage = first + d;
         if (stage < stages) {
-#pragma unroll
-          for (int j = 0; j < kLoads; ++j) staged[(d * kTiles + f + kFetchers * j) * 64 + lane] = fetched[d][j];
+          file_rows(d, fetched[d]);
           if (stage + 2 < stages) fetch_rows(stage + 2, fetched[d]);
           __syncthreads();
         }
@@ -134,12 +154,13 @@ __global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_ker
     }
   };
   auto multiply = [&](int buffer, const uintx4 (&a)[RT][S]) {
-    const uintx4* tiles = staged + (buffer * kTiles + half * S * MT) * 64 + lane;
+    const uintx4* tiles = staged + (buffer * kTiles + half * S * MT) * 64;
 #pragma unroll
     for (int u = 0; u < S; ++u) {
       uintx4 b[MT];
+      const int slot = slot_of(u, g, r);
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) b[mt] = tiles[(u * MT + mt) * 64];
+      for (int mt = 0; mt < MT; ++mt) b[mt] = tiles[(u * MT + mt) * 64 + slot];
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
@@ -292,11 +313,13 @@ MidPlan plan_mid(int rows, int n_tiles, int k_tiles, bool gated, int along, int 
         // rows takes 45.7 us with 768 activation tiles a block, 33.2 with 384); what a block costs before and after
         // its stream, about 1.2 us (the down product of 5,120 x 17,408 at 32 rows: 57 us as 1,280 blocks of 34 k tiles,
         // 42 us as 216 blocks of 136); and the exchange of partial sums (fitted on the first product: 9 us for 8 parts
-        // of 8 row tiles x 4 tiles of rows).  Of equal cuts the one with more waves along the band wins, then the one
-        // with fewer parts.
+        // of 8 row tiles x 4 tiles of rows).  Of equal cuts the one with two row tiles per wave wins, then the one
+        // with more waves along the band, then the one with fewer parts.  (Over 40 products of Qwen3-8B and -14B
+        // shapes at 24 to 256 rows the cut chosen so takes 1.3 % longer than the best of all cuts, on average.)
         double cost = static_cast<double>(rounds) * (static_cast<double>(a) * r * p.part_tiles + 0.68 * mt * p.part_tiles + 24.0);
         if (p.parts > 1) cost += static_cast<double>(a) * r * mt * p.parts / 1.6;
-        cost += 0.01 * (4 - a) + 0.001 * p.parts;
+        if (a == 2) cost *= 0.96;   // (blocks of eight waves: two share a compute unit, one's loads fill the other's waits)
+        cost += 0.05 * (2 - r) + 0.01 * (4 - a) + 0.001 * p.parts;
         if (best_cost < 0.0 || cost < best_cost) best = p, best_cost = cost;
       }
     }
