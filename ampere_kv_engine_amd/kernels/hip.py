@@ -319,9 +319,11 @@ class HipKernels:
         """Which kernel takes a bfloat16 product of more than 16 rows: "own" (the skinny kernel up to 64 rows, the
         wide one above), "mid" (17..512 rows: the block's waves share the activations through LDS) or "library".
         The table of choices decides where it names the product; otherwise a fixed rule, from measurements at
-        Qwen3-8B shapes: the library where there is one, except for the gated product up to 64 rows and products
-        with a long k (k >= 2 outs) up to 128 rows, which the mid-size kernel streams a fifth to two fifths faster;
-        without the library, the skinny kernel up to 64 rows, the mid-size one up to 512, the wide one beyond."""
+        Qwen3-8B and Qwen3-14B shapes (cold weights, 24 to 256 rows): the library where there is one, except for
+        the gated product up to 64 rows (the mid-size kernel is 8-28 % faster), products with a long k (k >= 2 outs)
+        up to 256 rows (10 % to three times) and products with outs <= k up to 128 rows (from 3 % slower to 19 %
+        faster); the stacked q/k/v product is a tie up to 128 rows and stays with the library.  Without the library:
+        the skinny kernel up to 64 rows, the mid-size one up to 512, the wide one beyond."""
         library = (has_row_major and self.library_products_above is not None and rows > self.library_products_above
                    and out_dtype == torch.bfloat16)
         bucket = self._row_bucket(rows)
@@ -336,7 +338,9 @@ class HipKernels:
             return "own" if rows <= self.OWN_SKINNY_ROWS else "mid"
         if kind == "gated":
             return "mid" if rows <= 64 else "library"
-        return "mid" if (k >= 2 * outs and rows <= 128) else "library"
+        if k >= 2 * outs:
+            return "mid" if rows <= 256 else "library"
+        return "mid" if (outs <= k and rows <= 128) else "library"
 
     def _mid(self, x, packed: PackedWeight, out, rows: int, outs: int, gated: bool) -> None:
         """The mid-size product (`csrc/gemm_mid.hip`).  Where it cuts k over blocks it needs room for partial sums
