@@ -764,7 +764,7 @@ class HipKernels:
                 partial = take(tiles * kv_heads * head_groups * num_splits * 16 * nq * (head_dim + 4))
             most_splits = num_splits
         # The merge of the segments: a block of four waves per column - or, where the requests have few segments and
-        # the launch would be a thousand blocks and more, a wave per column (what such a launch costs is its blocks:
+        # the launch would be two thousand blocks and more, a wave per column (what such a launch costs is its blocks:
         # 64 requests of 8,192 keys, four segments each: 9.0 -> 7.7 us per layer).
         columns = heads_per_tile * (1 if single else tokens_per_tile)
         merge_alone = (most_splits <= self.MERGE_ALONE_SPLITS
@@ -782,7 +782,7 @@ class HipKernels:
 
     PLAN_ENTRIES = 132          # ints of a plan before its items (4 per item)
     MERGE_ALONE_SPLITS = 16     # the merge gives a column to one wave where no request has more segments than this
-    MERGE_ALONE_BLOCKS = 1024   # ... and a block per column would make this many blocks or more
+    MERGE_ALONE_BLOCKS = 2048   # ... and a block per column would make this many blocks or more (at 1,280: 5.6 -> 7.4 us)
 
     def _decode_plan(self, ctx, seq_first, seq_count, window, head_blocks):
         """The cut of the keys of requests seq_first .. + seq_count - 1 (single tokens) into (request, segment) items:
