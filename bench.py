@@ -11,7 +11,8 @@ not change the time a step takes).  One JSON line is printed:
   value     decoded tokens per second at the default batch
   prefill   one request's 2,048-token prompt fed whole: tokens/s, ms, and flops / time / bf16 MFMA peak
   roofline  bytes a decode step has to read (every weight once + the live requests' cache) / its time / HBM peak
-  points    decoded tokens per second at batch 1 and 64; prefill tokens per second with every product in the engine's
+  points    decoded tokens per second at batch 1 and 64; milliseconds of a step that feeds 120 tokens of a prompt beside
+            the batch's decoding requests; prefill tokens per second with every product in the engine's
             own kernels (by default bfloat16 products of more than 16 rows go to the BLAS library); hbm_read_gbs,
             what a kernel that only reads draws from this device's memory (the ceiling to hold `roofline` against)
 Peaks are MI355X's published ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s.
@@ -194,7 +195,7 @@ def main() -> int:
     if contexts is not None:
         grown = PRIMING + args.warmup + args.steps + 2
         pages = sum((length + grown + PAGE_SIZE - 1) // PAGE_SIZE for length in contexts) + PREFILL_TOKENS // PAGE_SIZE + 2
-    engine_config = EngineConfig(dtype="bfloat16", page_size=PAGE_SIZE, num_pages=pages, max_seqs=max_batch,
+    engine_config = EngineConfig(dtype="bfloat16", page_size=PAGE_SIZE, num_pages=pages, max_seqs=max_batch + 1,
                                  max_batched_tokens=PREFILL_TOKENS,
                                  max_seq_len=max(tokens_per_request, PREFILL_TOKENS) + PAGE_SIZE,
                                  device="cuda:0", library_products_above=library_above)
@@ -258,6 +259,33 @@ def main() -> int:
             engine.close(seq)
         return sorted(samples)[len(samples) // 2], samples
 
+    def mixed_step(portion: int = 120, steps: int = 8) -> float:
+        """Milliseconds of a step that feeds `portion` tokens of a prompt beside one token each of `args.batch`
+        decoding requests (what a scheduler's round looks like while a prompt arrives in portions)."""
+        seqs = [engine.open(f"mixed{i}") for i in range(args.batch)]
+        for seq in seqs:
+            engine.cache.reserve(seq, args.context - 1)
+        first = torch.randint(0, config.vocab_size, (args.batch,), generator=generator).tolist()
+        engine.choose(engine.step([StepEntry(seq, [token], [0]) for seq, token in zip(seqs, first)], borrow_logits=True))
+        arriving = engine.open("mixed_prompt")
+        tokens = torch.randint(0, config.vocab_size, (portion,), generator=generator).tolist()
+
+        def one_step():
+            entries = [StepEntry(seq, LAST_TOKEN, [0]) for seq in seqs] + [StepEntry(arriving, tokens, [])]
+            return engine.choose(engine.step(entries, borrow_logits=True))
+
+        for _ in range(3):                   # the first runs eagerly, the second is recorded, the third replays
+            one_step()
+        sync()
+        started = time.perf_counter()
+        for _ in range(steps):
+            one_step()
+        sync()
+        elapsed = time.perf_counter() - started
+        for seq in seqs + [arriving]:
+            engine.close(seq)
+        return elapsed / steps * 1000
+
     if args.prefill_only:
         seconds, _ = prefill()
         print(json.dumps({"prefill_ms": round(seconds * 1000, 3), "tokens": PREFILL_TOKENS,
@@ -308,6 +336,8 @@ def main() -> int:
             record["points"]["prefill_own_products"] = round(PREFILL_TOKENS / prefill(3)[0], 1)
             engine.kernels.library_products_above = kept
     if points:
+        if (3 + 8) * 120 + PAGE_SIZE <= PREFILL_TOKENS and contexts is None:
+            record["points"]["mixed_step_120_beside_batch_ms"] = round(mixed_step(), 3)
         record["points"]["hbm_read_gbs"] = measured_read_rate(engine.kernels, engine.device)
     print(json.dumps(record))
     return 0

@@ -41,7 +41,7 @@ def test_the_line_of_a_short_run():
     prefill = line["prefill"]
     assert prefill["tokens"] == 2048 and prefill["ms"] > 0 and 0 < prefill["frac"] < 1
     assert abs(prefill["value"] - 2048 / (prefill["ms"] / 1e3)) < 1e-2 * prefill["value"]
-    assert line["points"]["decode_b1"] > 0
+    assert line["points"]["decode_b1"] > 0 and line["points"]["mixed_step_120_beside_batch_ms"] > 0
     # what a kernel that only reads draws from memory: below the data sheet's peak, above the decode step's own rate
     assert roofline["achieved"] < line["points"]["hbm_read_gbs"] < roofline["peak"]
     # raw samples beside median and range: the timed steps as consecutive fifths, the prefill's five runs
