@@ -602,12 +602,13 @@ def test_linear_rows_do_not_depend_on_the_batch(hip):
         assert torch.equal(alone[0], whole[row])
 
 
+@pytest.mark.parametrize("inter", [200, 204, 203, 4096])     # widths in steps of 8, of 4 and of 1
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_swiglu(hip, ref, dtype):
-    gate_up = rand(6, 2 * 200, dtype=dtype, seed=15, scale=2.0)
-    want = torch.empty(6, 200, dtype=dtype)
+def test_swiglu(hip, ref, dtype, inter):
+    gate_up = rand(37, 2 * inter, dtype=dtype, seed=15, scale=2.0)
+    want = torch.empty(37, inter, dtype=dtype)
     ref.swiglu(gate_up, want)
-    got = torch.empty(6, 200, dtype=dtype, device="cuda")
+    got = torch.full((37, inter), float("nan"), dtype=dtype, device="cuda")
     hip.swiglu(gate_up.cuda(), got)
     torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dtype))
 
