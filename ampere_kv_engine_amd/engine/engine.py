@@ -140,6 +140,18 @@ class Engine:
             self._chooser = SlotSampler(self.kernels, self.device, self.config.max_seqs)
         return self._chooser.choose(logits, ctx)
 
+    def choose_later(self, logits: torch.Tensor):
+        """`choose` without the wait: the tokens are chosen on the device (the next step may feed them as
+        `LAST_TOKEN` at once) and come to the host meanwhile; the returned object's `tokens()` waits for them.  A
+        caller that launches the next step before it asks hides its own work behind the device's."""
+        ctx = getattr(self, "_last_step", None)
+        if ctx is None or logits is None or logits.shape[0] != ctx.logit_rows.shape[0]:
+            raise ValueError("choose_later() takes the logits of the step that was run last")
+        if self._chooser is None:
+            from ..sampling.sampler import SlotSampler
+            self._chooser = SlotSampler(self.kernels, self.device, self.config.max_seqs)
+        return self._chooser.choose_later(logits, ctx)
+
     def _check_token_ids(self, entries: list[StepEntry]) -> None:
         """Every token id must name a row of the embedding table; one comparison per entry, not one per token."""
         vocab = self.spec.vocab_size

@@ -12,6 +12,13 @@ Where the reference has one prefill slot, decode groups of `max_batch` and an op
 is ONE step: every running request's next token first, then portions of admitted prompts, first come first
 served, until `max_batched_tokens` is spent.  With `mixed=False` the decodes and the portions run as two steps.
 
+With `overlap_decoding` a round of decoding requests alone does not wait for its tokens: they are chosen on the
+device, where the next round finds them in the requests' slots, and come to the host while that next round runs -
+the host launches it first and reads them then.  What the host learns a round late (an EOS) costs the request one
+token of work that is thrown away; what it knows beforehand (the limit of new tokens) costs nothing.  Anything else
+to do - a request waiting, a prompt to feed, a cancellation, a deadline - ends the overlap: the tokens are read, and
+the round is an ordinary one.
+
 When pages run out: by construction they cannot after admission.  A request whose budget does not fit the free
 budget waits at the head of the queue (and holds back those behind it); one whose budget exceeds the whole pool is
 refused at `submit`.
@@ -55,15 +62,20 @@ class Request:
 
 class Scheduler:
     def __init__(self, engine, *, max_batch: int | None = None, prefill_chunk_size: int = 0,
-                 max_batched_tokens: int | None = None, mixed: bool = True, clock=time.monotonic, on_token=None):
+                 max_batched_tokens: int | None = None, mixed: bool = True, clock=time.monotonic, on_token=None,
+                 overlap_decoding: bool = False):
         """`on_token(request, token)`, if given, is called whenever a request has been given a token (right after the
-        round's one synchronisation): measurements hang their clocks there; the scheduler itself keeps no history."""
+        round's one synchronisation): measurements hang their clocks there; the scheduler itself keeps no history.
+        `overlap_decoding`: rounds of decoding requests alone hand their tokens over while the next round runs."""
         cfg = engine.config
         self.engine = engine
         self.max_batch = cfg.max_seqs if max_batch is None else max_batch
         self.prefill_chunk_size = prefill_chunk_size
         self.max_batched_tokens = cfg.max_batched_tokens if max_batched_tokens is None else max_batched_tokens
         self.mixed = mixed
+        self.overlap_decoding = overlap_decoding
+        self._late = None               # (requests, their tokens on the way) of an overlapped round
+        self.overlapped_rounds = 0
         self.clock = clock
         self.on_token = on_token
         if self.max_batch < 1 or self.max_batch > cfg.max_seqs:
@@ -137,7 +149,11 @@ class Scheduler:
         """One round.  Returns the requests that finished in it (stopped at its start or ended normally) and the
         sizes of the decode batches it ran."""
         self.rounds += 1
-        finished = self._stop_round(self.clock())
+        now = self.clock()
+        if self.overlap_decoding and self._only_decoding(now):
+            return self._overlapped_round()
+        finished = self._collect()          # tokens of an overlapped round that are still on their way
+        finished += self._stop_round(now)
         self._admit()
         decodes = list(self.running)
         budget_left = self.max_batched_tokens - len(decodes)
@@ -176,6 +192,47 @@ class Scheduler:
                 request.status = RUNNING
                 self.running.append(request)
         return finished, sizes
+
+    # ---- overlapped decoding -------------------------------------------------------------------------------
+    def _only_decoding(self, now: float) -> bool:
+        """Nothing to do this round but to decode: nobody waits, no prompt is being fed, nobody was cancelled or has
+        run out of time."""
+        if self.waiting or self.prefilling or not self.running:
+            return False
+        return not any(r.stop_reason or (r.deadline is not None and r.deadline <= now) for r in self.running)
+
+    def _overlapped_round(self) -> tuple[list[Request], list[int]]:
+        late = self._late
+        on_their_way = set(id(r) for r in late[0]) if late is not None else ()
+        # who decodes: everybody whom the token on its way cannot be the last for, as far as the host can tell
+        decodes = [r for r in self.running
+                   if len(r.output_ids) + (1 if id(r) in on_their_way else 0) < r.max_new_tokens]
+        launched = None
+        if decodes:
+            logits = self.engine.step([StepEntry(r.seq, LAST_TOKEN, [0]) for r in decodes], borrow_logits=True)
+            launched = (decodes, self.engine.choose_later(logits))
+            self.overlapped_rounds += 1
+        finished = self._collect()          # the round before this one: its tokens have had this launch's time to arrive
+        self._late = launched
+        return finished, [len(decodes)] if decodes else []
+
+    def _collect(self) -> list[Request]:
+        """Reads the tokens of the overlapped round that is on its way, if there is one, gives them out and retires
+        who ends with them.  A request that has ended meanwhile (an EOS a round earlier, a cancellation) gets nothing:
+        the token was work for nothing."""
+        late, self._late = self._late, None
+        if late is None:
+            return []
+        requests, tokens = late
+        for request, token in zip(requests, tokens.tokens()):
+            if request.status == RUNNING and not request.stop_reason:
+                self._give(request, token)
+        finished = []
+        for request in [r for r in self.running if r.stop_reason and r.stop_reason not in (STOP_CANCELLED, STOP_EXPIRED)]:
+            self.running.remove(request)
+            self._retire(request)
+            finished.append(request)
+        return finished
 
     def _run(self, decodes: list[Request], portions: list[tuple[Request, int, bool]]) -> None:
         entries, takers = [], []

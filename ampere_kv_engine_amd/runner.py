@@ -11,7 +11,7 @@ value load - here the matrix-core kernels, and the default).  The reference read
 takes token ids in and gives token ids out, so the prompt is a line of integers on standard input (or `--prompt-ids`,
 or a seeded random prompt with `--prompt-len`); `--prompts-file` holds one such line per request and sends them all
 through the scheduler.  The engine's own sizes are options too: `--page-size`, `--num-pages` or `--kv-gb`,
-`--max-seqs`, `--max-batched-tokens`, `--prefill-chunk`.
+`--max-seqs`, `--max-batched-tokens`, `--prefill-chunk`, `--overlap-decoding`.
 
   generate    token ids, stop reason and count for every request
   benchmark   timed generation of one request: time to first token, time per output token, tokens per second
@@ -82,6 +82,8 @@ def build_parser() -> argparse.ArgumentParser:
                         "as many as it holds, up to 64)")
     parser.add_argument("--max-batched-tokens", type=int, help="most tokens one step carries (default: up to 8,192)")
     parser.add_argument("--prefill-chunk", type=int, default=0, help="feed prompts in portions of this many tokens")
+    parser.add_argument("--overlap-decoding", action="store_true",
+                        help="with --prompts-file: rounds of decoding requests alone read their tokens while the next round runs")
     parser.add_argument("--product-choices", default="fixed", help="'fixed', 'measure' (time own and library products "
                         "of 17..64 rows once at load) or the file of a saved table")
     parser.add_argument("--device", default="cuda:0")
@@ -236,7 +238,7 @@ def generate_many(engine: Engine, prompts: list[list[int]], args) -> list:
     """Every prompt of the file as a request of its own through the scheduler: admitted while slots and pages last,
     prompts fed in portions beside the requests that already decode."""
     from .engine.scheduler import Scheduler
-    scheduler = Scheduler(engine, prefill_chunk_size=args.prefill_chunk)
+    scheduler = Scheduler(engine, prefill_chunk_size=args.prefill_chunk, overlap_decoding=args.overlap_decoding)
     requests = [scheduler.submit(f"prompt{i}", prompt, args.max_new_tokens, ignore_eos=args.ignore_eos,
                                  temperature=args.temperature, seed=args.sample_seed + i)
                 for i, prompt in enumerate(prompts)]

@@ -80,16 +80,48 @@ class SlotSampler:
         self.kernels, self.device, self.max_rows = kernels, torch.device(device), max_rows
         pin = self.device.type == "cuda"
         self._out = torch.empty(max_rows, dtype=torch.int32, device=self.device)
-        self._host_out = torch.empty(max_rows, dtype=torch.int32, pin_memory=pin)
 
     def choose(self, logits: torch.Tensor, ctx) -> list[int]:
+        return self.choose_later(logits, ctx).tokens()
+
+    LATER = 3       # choices that may be on their way to the host at the same time
+
+    def choose_later(self, logits: torch.Tensor, ctx) -> "LaterTokens":
+        """The choice is made on the device now (the slots have their tokens as soon as the kernel has run, for the
+        next step to feed); the tokens are on their way to the host and are waited for only when `tokens()` is asked
+        - so the host may launch the next step first.  At most `LATER` such choices may be outstanding."""
         rows = logits.shape[0]
         if rows > self.max_rows:
             raise ValueError(f"{rows} rows to choose from; the sampler was built for {self.max_rows}")
         out = self._out[:rows]
         self.kernels.sample_slots(logits, ctx, out)
         if self.device.type != "cuda":
-            return out.tolist()
-        self._host_out[:rows].copy_(out, non_blocking=True)      # into pinned memory, then one wait for the stream
-        torch.cuda.current_stream(self.device).synchronize()
-        return self._host_out[:rows].tolist()
+            return LaterTokens(out.tolist(), None, None)
+        if not hasattr(self, "_later"):
+            self._later = [(torch.empty(self.max_rows, dtype=torch.int32, pin_memory=True), torch.cuda.Event())
+                           for _ in range(self.LATER)]
+            self._turn, self._waiting = 0, [None] * self.LATER
+        self._turn = (self._turn + 1) % self.LATER
+        if self._waiting[self._turn] is not None and not self._waiting[self._turn].read:
+            raise RuntimeError(f"more than {self.LATER} choices whose tokens nobody has asked for")
+        host, arrived = self._later[self._turn]
+        host[:rows].copy_(out, non_blocking=True)                # into pinned memory; the event tells when it is there
+        arrived.record(torch.cuda.current_stream(self.device))
+        later = LaterTokens(None, host[:rows], arrived)
+        self._waiting[self._turn] = later
+        return later
+
+
+class LaterTokens:
+    """The tokens of one `choose_later`: `tokens()` waits until they are on the host (once) and returns them."""
+
+    def __init__(self, tokens, host, arrived):
+        self._tokens, self._host, self._arrived = tokens, host, arrived
+        self.read = tokens is not None
+
+    def tokens(self) -> list[int]:
+        if self._tokens is None:
+            self._arrived.synchronize()
+            self._tokens = self._host.tolist()
+            self.read = True
+        return self._tokens

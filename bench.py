@@ -5,9 +5,9 @@
 A "step" is one decode step of the whole batch: every live request feeds its last token through the engine's
 step function and the sampler chooses the next one (greedy), exactly as generation does.  Three untimed steps come
 before the W warm-up steps (the engine runs a batch shape once as it is, records it, then replays the recording), so
-the K timed steps are replays whatever W is.  The requests' caches
-are brought to the context length beforehand (pages filled with random keys and values: what they hold does
-not change the time a step takes).  One JSON line is printed:
+the K timed steps are replays whatever W is.  A step's tokens are read by the host while the next step runs (the
+scheduler's overlapped decoding).  The requests' caches are brought to the context length beforehand (pages filled
+with random keys and values: what they hold does not change the time a step takes).  One JSON line is printed:
   value     decoded tokens per second at the default batch
   prefill   one request's 2,048-token prompt fed whole: tokens/s, ms, and flops / time / bf16 MFMA peak
   roofline  bytes a decode step has to read (every weight once + the live requests' cache) / its time / HBM peak
@@ -73,7 +73,7 @@ def scheduler_workload(name: str, layers: int | None, library_above: int | None)
         library_products_above=library_above))
     samples = []
     for run in range(3):                                    # the first run warms up (graphs are recorded in it)
-        scheduler = Scheduler(engine, prefill_chunk_size=PREFILL_TOKENS)
+        scheduler = Scheduler(engine, prefill_chunk_size=PREFILL_TOKENS, overlap_decoding=True)
         ids = [torch.randint(0, config.vocab_size, (p,), generator=generator).tolist() for p in prompts]
         torch.cuda.synchronize(engine.device)
         started = time.perf_counter()
@@ -128,7 +128,7 @@ def offline_workload(layers: int | None) -> int:
         ids = [torch.randint(0, config.vocab_size, (prompt_tokens,), generator=generator).tolist() for _ in range(batch)]
         samples = []
         for run in range(6):                                    # the first run warms up (graphs are recorded in it)
-            scheduler = Scheduler(engine)
+            scheduler = Scheduler(engine, overlap_decoding=True)
             torch.cuda.synchronize(engine.device)
             started = time.perf_counter()
             requests = [scheduler.submit(f"{batch}_{run}_{i}", tokens, max_new_tokens=new_tokens, ignore_eos=True)
@@ -215,22 +215,32 @@ def main() -> int:
         logits = engine.step([StepEntry(seq, [token], [0]) for seq, token in zip(seqs, first)], borrow_logits=True)
         engine.choose(logits)
 
-        def one_step():
+        def one_step(before=None):
             # every request feeds the token that was chosen for it in the step before (it lies in its slot on the
             # device) and the sampler chooses the next one from the slot's own state; the tokens come to the host
+            # while the next step runs: the host launches that first and reads them then, as the scheduler's
+            # overlapped decoding does
             logits = engine.step([StepEntry(seq, LAST_TOKEN, [0]) for seq in seqs], borrow_logits=True)
-            return engine.choose(logits)
+            later = engine.choose_later(logits)
+            if before is not None:
+                before.tokens()
+            return later
 
+        on_its_way = None
         for _ in range(PRIMING + warmup):
-            one_step()
+            on_its_way = one_step(on_its_way)
+        on_its_way.tokens()
         sync()
         started = time.perf_counter()
         moments = []
+        on_its_way = None
         for _ in range(steps):
-            one_step()                       # (returns with the chosen tokens on the host: the step is over)
+            on_its_way = one_step(on_its_way)    # (returns with the tokens of the step before on the host)
             moments.append(time.perf_counter() - started)
+        on_its_way.tokens()                      # the last step's tokens: every timed step is over
         sync()
         elapsed = time.perf_counter() - started
+        moments = moments[1:] + [elapsed]        # when each step's tokens were on the host
         for seq in seqs:
             engine.close(seq)
         assert engine.cache.num_free_pages == [pages]

@@ -245,3 +245,68 @@ def test_a_slot_that_is_used_again_starts_clean(model_folders):
     again = generate_tokens(engine, prompt, max_new_tokens=6, ignore_eos=True, temperature=0.9, seed=77)
     assert again == alone and len(set(alone_tokens)) > 1
     assert int(words[0, WORD_DRAWS]) == 6 and int(words[0, WORD_LAST_TOKEN]) == again[-1]
+
+
+def test_overlapped_decoding_chooses_the_same_tokens_and_gives_everything_back(model_folders):
+    """Rounds of decoding requests alone launch the next round before they read their tokens.  The outputs are those
+    of ordinary rounds - stops by the limit and by EOS, temperature sampling, a request that arrives later and one
+    that is cancelled in between included -, requests finish one call later at most, and pages, slots and budgets
+    come back."""
+    raw, _, page = TINY["B"]
+    folder = model_folders["B"]
+    prompts = [random_ids(raw["vocab_size"], n, seed=60 + i) for i, n in enumerate((3, 12, 30, 7, 19))]
+    limits = (9, 14, 6, 11, 8)
+
+    def run(overlap):
+        engine = make_engine(folder, page, num_pages=40, max_tokens=40)
+        # a token that the second request reaches on its way stands for EOS: found in a run without stops
+        probe = alone(folder, page, prompts[1], limits[1], temperature=0.5, seed=71)
+        engine.spec = type(engine.spec)(**{**engine.spec.__dict__, "eos_token_ids": (probe[5],)})
+        scheduler = Scheduler(engine, prefill_chunk_size=16, overlap_decoding=overlap)
+        requests = [scheduler.submit(f"r{i}", p, n, ignore_eos=(i != 1), temperature=0.5 if i % 2 else 0.0, seed=70 + i)
+                    for i, (p, n) in enumerate(zip(prompts[:3], limits[:3]))]
+        finished, calls = [], 0
+        while not scheduler.idle:
+            calls += 1
+            if calls == 6:      # another request arrives while the others decode; overlap ends for its prompt
+                requests.append(scheduler.submit("r3", prompts[3], limits[3], ignore_eos=True, temperature=0.5, seed=73))
+            if calls == 9:
+                requests.append(scheduler.submit("r4", prompts[4], limits[4], ignore_eos=True))
+            if calls == 12:
+                scheduler.cancel(requests[4])
+            done, _ = scheduler.step()
+            finished += done
+            assert calls < 200
+        assert scheduler.reserved_pages == [0] and engine.cache.num_free_pages == [40]
+        assert engine.cache.slots.num_free == 4 and all(r.status == FINISHED for r in requests)
+        assert {r.request_id for r in finished} == {f"r{i}" for i in range(5)}
+        return requests, scheduler, calls
+
+    plain_requests, plain_scheduler, plain_calls = run(False)
+    late_requests, late_scheduler, late_calls = run(True)
+    assert plain_scheduler.overlapped_rounds == 0 and late_scheduler.overlapped_rounds > 5
+    for a, b in zip(plain_requests, late_requests):
+        if a.stop_reason == STOP_CANCELLED:         # how far a cancelled request got depends on the round it was cancelled in
+            shorter, longer = sorted((a.output_ids, b.output_ids), key=len)
+            assert b.stop_reason == STOP_CANCELLED and longer[:len(shorter)] == shorter
+            continue
+        assert a.output_ids == b.output_ids and a.stop_reason == b.stop_reason, a.request_id
+    assert plain_requests[1].stop_reason == STOP_EOS and len(plain_requests[1].output_ids) == 6
+    assert late_calls <= plain_calls + 4            # a round late here and there, no more
+
+
+def test_overlapped_rounds_hand_tokens_over_a_round_late(model_folders):
+    raw, _, page = TINY["A"]
+    engine = make_engine(model_folders["A"], page, num_pages=16)
+    scheduler = Scheduler(engine, overlap_decoding=True)
+    prompt = random_ids(raw["vocab_size"], 9, seed=66)
+    request = scheduler.submit("r", prompt, 5, ignore_eos=True)
+    lengths = []
+    while not scheduler.idle:
+        scheduler.step()
+        lengths.append(len(request.output_ids))
+    # the prompt's round gives the first token; the first overlapped round launches and has nothing to read yet; from
+    # then on a token a call, and the last call only reads (the limit was known: no step was launched for nothing)
+    assert lengths == [1, 1, 2, 3, 4, 5]
+    assert request.output_ids == alone(model_folders["A"], page, prompt, 5)
+    assert request.cached_tokens == len(prompt) + 4 and scheduler.overlapped_rounds == 4
