@@ -158,7 +158,7 @@ def neighbours_do_not_matter(engine: Engine, prompts: list[list[int]], tokens: i
             "requests_checked": checked, "tokens_each": tokens}
 
 
-def measure_decode(engine: Engine, history: int, steps: int, repeats: int, batches, emit) -> None:
+def measure_decode(engine: Engine, history: int, steps: int, repeats: int, batches, emit, overlap: bool = False) -> None:
     vocab = engine.spec.vocab_size
     for batch in batches:
         prompts = random_prompts(vocab, batch, history, seed=batch)
@@ -166,7 +166,7 @@ def measure_decode(engine: Engine, history: int, steps: int, repeats: int, batch
             emit(neighbours_do_not_matter(engine, prompts))
         medians, spreads, rates = [], [], []
         for repeat in range(repeats + 1):              # the first repeat warms up (graphs are recorded in it)
-            load = Load.decoding(engine, prompts, steps + 1)
+            load = Load.decoding(engine, prompts, steps + 2, overlap_decoding=overlap)
             walls = []
             for _ in range(steps):
                 started = time.perf_counter()
@@ -179,7 +179,7 @@ def measure_decode(engine: Engine, history: int, steps: int, repeats: int, batch
                 medians.append(statistics.median(walls))
                 spreads.append(max(walls) - min(walls))
                 rates.append(batch * len(walls) / (sum(walls) / 1e3))
-        emit({"experiment": "decode", "batch": batch, "history": history, "rounds": steps,
+        emit({"experiment": "decode", "batch": batch, "history": history, "rounds": steps, "overlapped": overlap,
               "round_ms": summary(medians), "range_inside_a_repeat_ms": summary(spreads),
               "tokens_per_s": summary(rates)})
 
@@ -314,6 +314,8 @@ def main(argv=None) -> int:
     parser.add_argument("--chunks", type=int, nargs="+", default=(0, 128), help="portion sizes (0: as far as the step's budget allows)")
     parser.add_argument("--pending-history", type=int, nargs="+", default=(0, 512),
                         help="calibrate: tokens of the pending prompt fed before the measured round (0: its first portion)")
+    parser.add_argument("--overlap-decoding", action="store_true",
+                        help="decode: rounds read their tokens while the next round runs (Scheduler(overlap_decoding=True))")
     parser.add_argument("--mixed", action="store_true",
                         help="insert: also measure a scheduler that runs a round's decode tokens and its portion apart")
     parser.add_argument("--model", help="folder with config.json and model.safetensors (default: random weights, "
@@ -346,7 +348,7 @@ def main(argv=None) -> int:
           "device": torch.cuda.get_device_properties(engine.device).name, "times": "host wall clock, milliseconds"})
     unique = lambda values: tuple(dict.fromkeys(values))
     if args.only in (None, "decode"):
-        measure_decode(engine, args.history, args.steps, args.repeats, unique(args.batches), emit)
+        measure_decode(engine, args.history, args.steps, args.repeats, unique(args.batches), emit, args.overlap_decoding)
     if args.only in (None, "insert"):
         measure_insert(engine, args.history, args.steps, args.insert_at, unique(args.insert_history), args.repeats,
                        unique(args.chunks), args.mixed, emit)
