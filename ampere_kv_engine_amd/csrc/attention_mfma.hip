@@ -97,7 +97,6 @@ struct Args {
   // first; `items_grid` is a bound the host knows.
   const int* plan;
   int items_grid;
-  int merge_alone;            // the merge gives a wave a column and a block four of them (few segments, many columns)
   int units;                  // compute units of the device (block order of the shared kernel)
   // FRESH launches (single tokens whose projections have not been normed, rotated or written to the cache yet):
   const bf16_t* qkv;          // [tokens, (q_heads + 2 * kv_heads) * D]: query, key and value heads of a token in a row
@@ -1107,27 +1106,21 @@ __global__ __launch_bounds__(64 * kSharedWaves, D <= 128 ? (NQ == 1 ? 3 : 2) : 1
 }
 
 // Merge of the segments' partial results: out = sum_z 2^(m_z - M) O_z / sum_z 2^(m_z - M) l_z, M = max_z m_z
-// (csrc/paged_decode.cu:528-544 of the reference has the same rule in base e).  A lane owns dims lane, lane + 64, ...
-// The segments are summed in kMergeWaves shares - share w holds the segments w, w + kMergeWaves, ... in ascending
-// order - and the shares are added in their order: the order of the whole sum is fixed.
-// TEAM = kMergeWaves: one block per (tile, head group, column), a wave per share.  TEAM = 1 (few segments, many
-// columns: what the launch costs is its number of blocks): a block takes kMergeWaves columns, and the wave of a column
-// sums all its shares, one after the other - the same bits.
+// (csrc/paged_decode.cu:528-544 of the reference has the same rule in base e).  One block of kMergeWaves waves per
+// (tile, head group, column); a lane owns dims lane, lane + 64, ...; wave w sums the segments w, w + kMergeWaves, ...
+// in ascending order, and the waves' sums are added in the order of the waves: the order of the whole sum is fixed.
 constexpr int kMergeWaves = 4;
 
-template <int NQ, int TEAM>
+template <int NQ>
 __global__ __launch_bounds__(64 * kMergeWaves) void attention_merge_kernel(const Args a) {
-  static_assert(TEAM == 1 || TEAM == kMergeWaves, "a wave alone, or all waves of the block");
   constexpr int PER = (D + 63) / 64;
-  constexpr int SHARES = kMergeWaves / TEAM;   // shares this wave sums
   __shared__ float sums[kMergeWaves][PER * 64 + 1];  // per wave: the weighted sum per dim, then the denominator
   const Tile t = find_tile(a, blockIdx.x, a.tokens_per_tile);
   if (!t.found) return;
   const int kvh = blockIdx.y / a.head_groups, hg = blockIdx.y % a.head_groups;
-  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int c = TEAM == 1 ? static_cast<int>(blockIdx.z) * kMergeWaves + wave : static_cast<int>(blockIdx.z);
+  const int c = blockIdx.z, lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int token = c / a.heads_per_tile, head_in_group = hg * a.heads_per_tile + c % a.heads_per_tile;
-  if (c >= 16 * NQ || token >= t.tokens || head_in_group >= a.group) return;   // (TEAM = 1: nobody waits for this wave)
+  if (token >= t.tokens || head_in_group >= a.group) return;
   // the request's partial results: `splits` tiles, `split_stride` floats apart
   const float* src = a.partial + (((static_cast<long>(blockIdx.x) * gridDim.y + blockIdx.y) * a.num_splits) * (16 * NQ) + c) * PSTRIDE;
   long split_stride = static_cast<long>(16 * NQ) * PSTRIDE;
@@ -1137,24 +1130,19 @@ __global__ __launch_bounds__(64 * kMergeWaves) void attention_merge_kernel(const
     src = a.partial + ((static_cast<long>(a.plan[4 + 2 * blockIdx.x]) * gridDim.y + blockIdx.y) * (16 * NQ) + c) * PSTRIDE;
     split_stride *= gridDim.y;
   }
-  // Share `share` holds the segments z = share + kMergeWaves * i.  Eight segments' loads go out together; every
-  // share's first eight are asked for before the maxima - they do not depend on them, and the kernel is a chain of
-  // trips to memory.
-  auto fetch8 = [&](int share, int i0, int ii0, int count, float (&v)[8][PER]) {
+  // this wave's segments: z = wave + kMergeWaves * i.  Eight segments' loads go out together; the first eight are
+  // asked for before the maxima - they do not depend on them, and the kernel is a chain of trips to memory.
+  const int mine = (splits - wave + kMergeWaves - 1) / kMergeWaves;
+  auto fetch8 = [&](int i0, int ii0, int count, float (&v)[8][PER]) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const float* p = src + (share + static_cast<long>(kMergeWaves) * (i0 + min(ii0 + j, count - 1))) * split_stride;
+      const float* p = src + (wave + static_cast<long>(kMergeWaves) * (i0 + min(ii0 + j, count - 1))) * split_stride;
 #pragma unroll
       for (int e = 0; e < PER; ++e) v[j][e] = lane + e * 64 < D ? p[lane + e * 64] : 0.f;
     }
   };
-  float ahead[SHARES][8][PER] = {};
-#pragma unroll
-  for (int sh = 0; sh < SHARES; ++sh) {
-    const int share = TEAM == 1 ? sh : wave;
-    const int mine = (splits - share + kMergeWaves - 1) / kMergeWaves;
-    if (mine > 0) fetch8(share, 0, 0, min(64, mine), ahead[sh]);
-  }
+  float ahead[8][PER] = {};
+  if (mine > 0) fetch8(0, 0, min(64, mine), ahead);
   // every wave finds the maximum over all segments (a lane per segment)
   float top = -INFINITY;
   bool poisoned = false;
@@ -1166,72 +1154,56 @@ __global__ __launch_bounds__(64 * kMergeWaves) void attention_merge_kernel(const
   }
   top = wave_max(top);
   poisoned = __any(poisoned);
-  float denom[SHARES], acc[SHARES][PER];
+  float denom = 0.f, acc[PER];
 #pragma unroll
-  for (int sh = 0; sh < SHARES; ++sh) {
-    const int share = TEAM == 1 ? sh : wave;
-    const int mine = (splits - share + kMergeWaves - 1) / kMergeWaves;
-    float part = 0.f;
+  for (int i = 0; i < PER; ++i) acc[i] = 0.f;
+  for (int i0 = 0; i0 < mine; i0 += 64) {
+    const int i = i0 + lane;
+    float w = 0.f;
+    if (i < mine) {
+      const long z = wave + static_cast<long>(kMergeWaves) * i;
+      const float mz = src[z * split_stride + D];
+      w = (mz == -INFINITY || mz != mz) ? 0.f : __builtin_amdgcn_exp2f(mz - top);
+      denom += w * src[z * split_stride + D + 1];
+    }
+    const int count = min(64, mine - i0);
+    for (int ii0 = 0; ii0 < count; ii0 += 8) {  // ascending segments
+      float v[8][PER];
+      if (i0 == 0 && ii0 == 0) {
 #pragma unroll
-    for (int e = 0; e < PER; ++e) acc[sh][e] = 0.f;
-    for (int i0 = 0; i0 < mine; i0 += 64) {
-      const int i = i0 + lane;
-      float w = 0.f;
-      if (i < mine) {
-        const long z = share + static_cast<long>(kMergeWaves) * i;
-        const float mz = src[z * split_stride + D];
-        w = (mz == -INFINITY || mz != mz) ? 0.f : __builtin_amdgcn_exp2f(mz - top);
-        part += w * src[z * split_stride + D + 1];
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+          for (int e = 0; e < PER; ++e) v[j][e] = ahead[j][e];
+      } else {
+        fetch8(i0, ii0, count, v);
       }
-      const int count = min(64, mine - i0);
-      for (int ii0 = 0; ii0 < count; ii0 += 8) {  // ascending segments
-        float v[8][PER];
-        if (i0 == 0 && ii0 == 0) {
 #pragma unroll
-          for (int j = 0; j < 8; ++j)
+      for (int j = 0; j < 8; ++j) {
+        const float wz = ii0 + j < count ? __shfl(w, ii0 + j, 64) : 0.f;
 #pragma unroll
-            for (int e = 0; e < PER; ++e) v[j][e] = ahead[sh][j][e];
-        } else {
-          fetch8(share, i0, ii0, count, v);
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const float wz = ii0 + j < count ? __shfl(w, ii0 + j, 64) : 0.f;
-#pragma unroll
-          for (int e = 0; e < PER; ++e) acc[sh][e] = fmaf(wz, v[j][e], acc[sh][e]);
-        }
+        for (int e = 0; e < PER; ++e) acc[e] = fmaf(wz, v[j][e], acc[e]);
       }
     }
-    denom[sh] = wave_sum(part);
   }
-  // the shares in their order
-  float total = 0.f, out[PER];
+  denom = wave_sum(denom);
 #pragma unroll
-  for (int e = 0; e < PER; ++e) out[e] = 0.f;
-  if constexpr (TEAM > 1) {
+  for (int e = 0; e < PER; ++e) sums[wave][e * 64 + lane] = acc[e];
+  if (lane == 0) sums[wave][PER * 64] = denom;
+  __syncthreads();
+  if (wave != 0) return;
+  float total = 0.f;
 #pragma unroll
-    for (int e = 0; e < PER; ++e) sums[wave][e * 64 + lane] = acc[0][e];
-    if (lane == 0) sums[wave][PER * 64] = denom[0];
-    __syncthreads();
-    if (wave != 0) return;
-    for (int w = 0; w < kMergeWaves; ++w) {
-      total += sums[w][PER * 64];
+  for (int e = 0; e < PER; ++e) acc[e] = 0.f;
+  for (int w = 0; w < kMergeWaves; ++w) {
+    total += sums[w][PER * 64];
 #pragma unroll
-      for (int e = 0; e < PER; ++e) out[e] += sums[w][e * 64 + lane];
-    }
-  } else {
-#pragma unroll
-    for (int sh = 0; sh < SHARES; ++sh) {
-      total += denom[sh];
-#pragma unroll
-      for (int e = 0; e < PER; ++e) out[e] += acc[sh][e];
-    }
+    for (int e = 0; e < PER; ++e) acc[e] += sums[w][e * 64 + lane];
   }
   bf16_t* dst = a.out + (static_cast<long>(t.first_row + token) * a.q_heads + kvh * a.group + head_in_group) * D;
   const float inv = poisoned ? __uint_as_float(0x7fc00000u) : 1.f / total;
 #pragma unroll
   for (int e = 0; e < PER; ++e)
-    if (lane + e * 64 < D) dst[lane + e * 64] = from_float<bf16_t>(out[e] * inv);
+    if (lane + e * 64 < D) dst[lane + e * 64] = from_float<bf16_t>(acc[e] * inv);
 }
 
 template <int NQ>
@@ -1248,12 +1220,8 @@ int launch(const Args& a, int tiles, bool shared, hipStream_t stream) {
   const bool items = a.plan != nullptr;  // single tokens whose keys were cut on the device: always with the merge
   if (items) grid = dim3(a.kv_heads * a.head_groups, a.items_grid, 1);
   const int columns = a.heads_per_tile * (a.single_tokens ? 1 : a.tokens_per_tile);   // that can be a (token, head) pair
-  const dim3 merge_grid(items ? a.seq_count : tiles, a.kv_heads * a.head_groups,
-                        a.merge_alone ? (columns + kMergeWaves - 1) / kMergeWaves : columns);
-  auto merge = [&]() {
-    if (a.merge_alone) attention_merge_kernel<NQ, 1><<<merge_grid, 64 * kMergeWaves, 0, stream>>>(a);
-    else attention_merge_kernel<NQ, kMergeWaves><<<merge_grid, 64 * kMergeWaves, 0, stream>>>(a);  // a block per column that can be a (token, head) pair
-  };
+  const dim3 merge_grid(items ? a.seq_count : tiles, a.kv_heads * a.head_groups, columns);
+  auto merge = [&]() { attention_merge_kernel<NQ><<<merge_grid, 64 * kMergeWaves, 0, stream>>>(a); };
   if (a.num_splits == 1 && a.qkv == nullptr && !items) grid.x = (tiles + 1) / 2;  // a block takes a late tile and an early one
   // single tokens cut into segments: a key is read by one block per group of query heads - by one block where the
   // heads of a kv head fit one tile
@@ -1303,8 +1271,6 @@ int launch(const Args& a, int tiles, bool shared, hipStream_t stream) {
 // [tokens, (q_heads + 2 * kv_heads) * D]; `q` is not read, the kernel norms (q_weight, k_weight, eps; both weights
 // null: no norm) and rotates (rope_table [table_positions, D / 2, 2], null: no rotation) queries and the new keys
 // itself and writes the new keys and values to the tokens' slots, which the block tables must already name.
-// `merge_alone`: the merge of segments gives every column to one wave (blocks of four columns) instead of a block -
-// for launches with few segments per request and many columns; the results' bits are the same either way.
 extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
     const void* q, const void* k_pages, const void* v_pages, void* out, float* partial, const int* q_start,
     const int* seq_lens, const int* block_table, const int* table_rows, int table_width, int seq_first, int seq_count,
@@ -1312,7 +1278,7 @@ extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
     int q_heads, int kv_heads, int heads_per_tile, int head_groups, int tokens_per_tile, int page_size, long num_pages,
     float scale, int window, int seg_keys, int num_splits, int single_tokens, int shared, const void* qkv,
     const float* q_weight, const float* k_weight, float eps, const float* rope_table, int table_positions,
-    const int* plan, int items_grid, int merge_alone, hipStream_t stream) {
+    const int* plan, int items_grid, hipStream_t stream) {
   if (tiles <= 0 || seq_count <= 0) return 0;
   int page_shift = 0;
   while ((1 << page_shift) < page_size) ++page_shift;
@@ -1351,7 +1317,6 @@ extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
   a.num_splits = num_splits;
   a.plan = plan;
   a.items_grid = items_grid;
-  a.merge_alone = merge_alone != 0;
   a.units = 1;
   a.qkv = static_cast<const bf16_t*>(qkv);
   a.q_weight = q_weight;

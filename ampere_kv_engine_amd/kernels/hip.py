@@ -742,7 +742,7 @@ class HipKernels:
         per_tile = tokens_per_tile * (4 if shared else 1)
         tiles = sum((starts[r + 1] - starts[r] + per_tile - 1) // per_tile
                     for r in range(seq_first, seq_first + seq_count))
-        num_splits, seg_keys, partial, plan, items_grid, most_splits = 1, 0, None, None, 0, 1
+        num_splits, seg_keys, partial, plan, items_grid = 1, 0, None, None, 0
         arena = getattr(ctx, "arena", None)
         take = lambda count: (arena.take((count,), torch.float32) if arena is not None
                               else torch.empty(count, dtype=torch.float32, device=self.device))
@@ -750,7 +750,7 @@ class HipKernels:
                 and max(ctx.host_seq_lens[seq_first:seq_first + seq_count]) > self.decode_min_segment):
             # single tokens: their keys are cut on the device, from the lengths there (requests of 128 keys or
             # fewer are not cut: then the kernel without merge)
-            plan, items_grid, most_splits = self._decode_plan(ctx, seq_first, seq_count, window, kv_heads * head_groups)
+            plan, items_grid = self._decode_plan(ctx, seq_first, seq_count, window, kv_heads * head_groups)
             partial = take(items_grid * kv_heads * head_groups * 16 * nq * (head_dim + 4))
         elif split:
             longest = max(ctx.host_seq_lens[seq_first:seq_first + seq_count])
@@ -762,13 +762,6 @@ class HipKernels:
             num_splits = (longest + seg_keys - 1) // seg_keys
             if num_splits > 1:
                 partial = take(tiles * kv_heads * head_groups * num_splits * 16 * nq * (head_dim + 4))
-            most_splits = num_splits
-        # The merge of the segments: a block of four waves per column - or, where the requests have few segments and
-        # the launch would be two thousand blocks and more, a wave per column (what such a launch costs is its blocks:
-        # 64 requests of 8,192 keys, four segments each: 9.0 -> 7.7 us per layer).
-        columns = heads_per_tile * (1 if single else tokens_per_tile)
-        merge_alone = (most_splits <= self.MERGE_ALONE_SPLITS
-                       and (seq_count if plan is not None else tiles) * kv_heads * head_groups * columns >= self.MERGE_ALONE_BLOCKS)
         qkv, q_weight, k_weight, eps, table = fresh if fresh is not None else (None, None, None, 0.0, None)
         self._check(self._attention_mfma_entry(head_dim)(
             _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(partial), _ptr(ctx.q_start), _ptr(ctx.seq_lens),
@@ -777,20 +770,17 @@ class HipKernels:
             head_groups, tokens_per_tile, page_size, ctypes.c_long(num_pages), ctypes.c_float(scale),
             int(window) if window is not None else 0, seg_keys, num_splits, 1 if single else 0, 1 if shared else 0,
             _ptr(qkv), _ptr(q_weight), _ptr(k_weight), ctypes.c_float(eps), _ptr(table),
-            table.shape[0] if table is not None else 0, _ptr(plan), items_grid, 1 if merge_alone else 0, self._stream()),
+            table.shape[0] if table is not None else 0, _ptr(plan), items_grid, self._stream()),
             "attention")
 
     PLAN_ENTRIES = 132          # ints of a plan before its items (4 per item)
-    MERGE_ALONE_SPLITS = 16     # the merge gives a column to one wave where no request has more segments than this
-    MERGE_ALONE_BLOCKS = 2048   # ... and a block per column would make this many blocks or more (at 1,280: 5.6 -> 7.4 us)
 
     def _decode_plan(self, ctx, seq_first, seq_count, window, head_blocks):
         """The cut of the keys of requests seq_first .. + seq_count - 1 (single tokens) into (request, segment) items:
         segments of one size for all requests - about `decode_wave_target` waves in all, no segment shorter than
         `decode_min_segment` unless it is a request's only one - worked out by a one-wave kernel from the lengths on
         the device.  The cut depends on the lengths alone, so the layers of a step share one plan: it is remembered on
-        the step's context.  Returns the plan, the bound on the number of items that sizes grids and buffers, and the
-        most segments any request has (the device's rule applied to the lengths the host knows)."""
+        the step's context.  Returns the plan and the bound on the number of items that sizes grids and buffers."""
         items = max(1, self.decode_wave_target // head_blocks)
         key = (seq_first, seq_count, int(window) if window is not None else 0, items, self.decode_min_segment)
         plans = getattr(ctx, "decode_plans", None)
@@ -822,12 +812,7 @@ class HipKernels:
         self._dense(ctx.seq_lens, "seq_lens", torch.int32, (ctx.num_seqs,))
         self._check(self.lib.akv_decode_plan(_ptr(ctx.seq_lens), seq_first, seq_count, key[2], items, smallest,
                                              items_grid, _ptr(plan), self._stream()), "decode_plan")
-        spans = []
-        for length in ctx.host_seq_lens[seq_first:seq_first + seq_count]:
-            first = (max(0, length - key[2]) if key[2] > 0 else 0) // 32 * 32
-            spans.append(max(length - first, 0))
-        size = max(smallest, (-(-sum(spans) // items) + 31) // 32 * 32)
-        plans[key] = (plan, items_grid, max(-(-span // size) for span in spans))
+        plans[key] = (plan, items_grid)
         return plans[key]
 
     def _few_portion_blocks(self, ctx, first, q_heads, kv_heads) -> bool:

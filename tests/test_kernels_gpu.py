@@ -850,7 +850,7 @@ def test_decode_plan(hip, lengths, window):
     ctx = SimpleNamespace(seq_lens=seq_lens, num_seqs=len(lengths) + 2, host_seq_lens=[7, 7] + lengths)
     hip.decode_wave_target, kept = items_wanted * 4, hip.decode_wave_target
     try:
-        plan, grid, most = hip._decode_plan(ctx, first_request, len(lengths), window, 4)
+        plan, grid = hip._decode_plan(ctx, first_request, len(lengths), window, 4)
     finally:
         hip.decode_wave_target = kept
     plan = plan.cpu().tolist()
@@ -862,7 +862,7 @@ def test_decode_plan(hip, lengths, window):
         spans.append(pos - first + 1)
     size = max(smallest, (-(-sum(spans) // items_wanted) + 31) // 32 * 32)
     counts = [-(-span // size) for span in spans]
-    assert plan[0] == sum(counts) <= grid and plan[1] == size and most == max(counts)
+    assert plan[0] == sum(counts) <= grid and plan[1] == size
     item = 0
     for r, (length, first, count) in enumerate(zip(lengths, firsts, counts)):
         assert plan[4 + 2 * r:6 + 2 * r] == [item, count]
@@ -886,34 +886,6 @@ def test_attention_of_many_single_tokens_of_very_different_lengths(hip, ref):
     hip.attention(q.cuda(), k_pages.cuda(), v_pages.cuda(), cctx, cmeta, 8, 2, 128, 128 ** -0.5, None, got)
     torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(torch.bfloat16))
     assert len(cctx.decode_plans) == 2
-
-
-def test_the_merge_gives_the_same_bits_with_a_wave_or_a_block_per_column(hip, ref):
-    """The merge of the segments' results sums them in four shares whichever way it is launched - a block per column,
-    a wave per share; or a wave per column, which sums its shares one after the other: 50 requests with 1 to 9
-    segments each, both ways, bit for bit, and against the plain attention."""
-    histories = [150 + 137 * i for i in range(50)]
-    portions = [(h, 1) for h in histories]
-    q, k_pages, v_pages, ctx, meta, _, _ = _attention_case(torch.bfloat16, 8, 2, 128, 16, portions, None, 41)
-    ctx.num_decode_seqs = len(portions)
-    want = torch.empty_like(q)
-    ref.attention(q, k_pages, v_pages, ctx, meta, 8, 2, 128, 128 ** -0.5, None, want)
-    results = []
-    kept = hip.MERGE_ALONE_BLOCKS, hip.MERGE_ALONE_SPLITS, hip.decode_wave_target
-    try:
-        hip.decode_wave_target = 256            # segments of about 800 keys
-        for blocks in (1, 1 << 30):             # a wave per column; a block per column
-            hip.MERGE_ALONE_BLOCKS, hip.MERGE_ALONE_SPLITS = blocks, 16
-            cctx, cmeta = _to_cuda(ctx, meta)
-            got = torch.full_like(q, float("nan"), device="cuda")
-            hip.attention(q.cuda(), k_pages.cuda(), v_pages.cuda(), cctx, cmeta, 8, 2, 128, 128 ** -0.5, None, got)
-            (_, _, most), = cctx.decode_plans.values()
-            assert 4 < most <= 16, most
-            results.append(got.cpu())
-    finally:
-        hip.MERGE_ALONE_BLOCKS, hip.MERGE_ALONE_SPLITS, hip.decode_wave_target = kept
-    assert torch.equal(results[0], results[1])
-    torch.testing.assert_close(results[0].float(), want.float(), **attention_tol(torch.bfloat16))
 
 
 def test_short_portion_after_a_long_history_has_its_keys_cut(hip, ref):
