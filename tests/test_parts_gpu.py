@@ -457,3 +457,37 @@ def test_a_slot_that_is_used_again_starts_clean_on_the_device(model_folders):
     engine.close(seq)
     assert generate_tokens(engine, prompt, max_new_tokens=6, ignore_eos=True, temperature=0.9, seed=77) == alone
     assert len(set(alone)) > 1
+
+
+def test_tokens_read_a_step_late_are_the_tokens_read_at_once(model_folders):
+    """`choose_later` leaves the chosen token in the request's slot for the next step; the host may read it after it
+    has launched that step.  Two requests, greedy and drawn, decoded with the read one step behind give what
+    `generate_tokens` gives; a fourth choice that nobody has read is refused."""
+    from ampere_kv_engine_amd.engine import LAST_TOKEN
+    raw, _, page = TINY["A"]
+    config = EngineConfig(dtype="bfloat16", page_size=page, num_pages=32, max_seqs=2, max_batched_tokens=64,
+                          max_seq_len=256, device="cuda:0")
+    engine = Engine.from_folder(model_folders["A"], config)
+    prompts = [random_ids(raw["vocab_size"], n, seed=60 + n) for n in (13, 7)]
+    draws = [(0.0, 0), (0.8, 9)]
+    want = [generate_tokens(engine, p, max_new_tokens=8, ignore_eos=True, temperature=t, seed=s)
+            for p, (t, s) in zip(prompts, draws)]
+    seqs = [engine.open(f"r{i}", t, s) for i, (t, s) in enumerate(draws)]
+    logits = engine.step([StepEntry(q, p, [len(p) - 1]) for q, p in zip(seqs, prompts)], borrow_logits=True)
+    got, before = [[], []], engine.choose_later(logits)
+    for _ in range(7):
+        logits = engine.step([StepEntry(q, LAST_TOKEN, [0]) for q in seqs], borrow_logits=True)
+        later = engine.choose_later(logits)
+        for mine, token in zip(got, before.tokens()):
+            mine.append(token)
+        before = later
+    for mine, token in zip(got, before.tokens()):
+        mine.append(token)
+    assert got == want
+    unread = [engine.choose_later(logits) for _ in range(3)]
+    with pytest.raises(RuntimeError, match="nobody has asked for"):
+        engine.choose_later(logits)
+    for later in unread:
+        later.tokens()
+    for q in seqs:
+        engine.close(q)
