@@ -319,11 +319,15 @@ class HipKernels:
         """Which kernel takes a bfloat16 product of more than 16 rows: "own" (the skinny kernel up to 64 rows, the
         wide one above), "mid" (17..512 rows: the block's waves share the activations through LDS) or "library".
         The table of choices decides where it names the product; otherwise a fixed rule, from measurements at
-        Qwen3-8B and Qwen3-14B shapes (cold weights, 24 to 256 rows): the library where there is one, except for
-        the gated product up to 64 rows (the mid-size kernel is 8-28 % faster), products with a long k (k >= 2 outs)
-        up to 256 rows (10 % to three times) and products with outs <= k up to 128 rows (from 3 % slower to 19 %
-        faster); the stacked q/k/v product is a tie up to 128 rows and stays with the library.  Without the library:
-        the skinny kernel up to 64 rows, the mid-size one up to 512, the wide one beyond."""
+        Qwen3-8B, -14B and -32B shapes (cold weights, 24 to 256 rows; `bench_products --rows ...` repeats them):
+        the library where there is one, except for the gated product up to 64 rows (the mid-size kernel is 8-28 %
+        faster; from 96 rows on the library is, by up to 40 %), plain products with outs <= k up to 128 rows (from
+        3 % slower to three times faster; the stacked q/k/v product, outs > k, is a tie there and stays with the
+        library) and every plain product from 129 to 256 rows (the library's times jump with the row count there -
+        q/k/v of 7,168 x 5,120: 36 / 50 / 63 us at 128 / 192 / 256 rows, the mid-size kernel 36 / 41 / 42; over
+        three model sizes the mid-size kernel is 10-35 % faster at 192 and 256 rows, except for the 4,096 x 4,096 product at 224
+        and 256 rows, which the library does in 25 us instead of 30).  Without the library: the skinny kernel up to
+        64 rows, the mid-size one up to 512, the wide one beyond."""
         library = (has_row_major and self.library_products_above is not None and rows > self.library_products_above
                    and out_dtype == torch.bfloat16)
         bucket = self._row_bucket(rows)
@@ -338,9 +342,9 @@ class HipKernels:
             return "own" if rows <= self.OWN_SKINNY_ROWS else "mid"
         if kind == "gated":
             return "mid" if rows <= 64 else "library"
-        if k >= 2 * outs:
-            return "mid" if rows <= 256 else "library"
-        return "mid" if (outs <= k and rows <= 128) else "library"
+        if rows > 256:
+            return "library"
+        return "mid" if (rows > 128 or outs <= k) else "library"
 
     def _mid(self, x, packed: PackedWeight, out, rows: int, outs: int, gated: bool) -> None:
         """The mid-size product (`csrc/gemm_mid.hip`).  Where it cuts k over blocks it needs room for partial sums

@@ -77,3 +77,23 @@ def test_a_batch_of_different_context_lengths():
     assert config["global_batch"] == 4 and config["seq_len"] == 700 and config["contexts"] == "700,40x3"
     assert len(config) <= 20 and "prefill" not in line and "points" not in line
     assert abs(line["value"] - 4 / (line["ms_per_step"] / 1e3)) < 1e-2 * line["value"]
+
+
+@pytest.mark.gpu
+def test_the_products_beside_a_bare_read():
+    """`python -m ampere_kv_engine_amd.bench_products` at small sizes: a line per product and row count; up to 16 rows
+    the decode kernels, above that the routed kernel and every kernel that can take the product."""
+    result = subprocess.run([sys.executable, "-m", "ampere_kv_engine_amd.bench_products", "--rows", "8", "40", "--hidden",
+                             "256", "--intermediate", "512", "--q-heads", "4", "--kv-heads", "2", "--head-dim", "64",
+                             "--repeats", "3", "--cache-megabytes", "1"], capture_output=True, text=True, timeout=600,
+                            cwd=ROOT, env=dict(os.environ, PYTHONPATH=ROOT))
+    assert result.returncode == 0, result.stderr[-2000:]
+    records = [json.loads(line) for line in result.stdout.splitlines()]
+    assert [(r["product"], r["rows"]) for r in records] == [(p, n) for p in ("q/k/v", "o", "gate-up", "down") for n in (8, 40)]
+    for record in records:
+        assert record["read_only_us"] > 0
+        if record["rows"] == 8:
+            assert record["plain_us"] > 0
+        else:
+            assert record["routed_to"] in ("mid", "library", "own")
+            assert all(record[key] > 0 for key in ("routed_us", "mid_us", "library_us", "own_us"))
