@@ -73,24 +73,48 @@ __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ 
   // eight loads of a thread are on their way before the first is looked at; ids still ascend per thread, so the
   // first maximum stays
   constexpr int kAhead = 8;
-  for (int i0 = threadIdx.x; i0 < vocab; i0 += kAhead * blockDim.x) {
-    float fetched[kAhead];
-#pragma unroll
-    for (int u = 0; u < kAhead; ++u) {
-      const int i = i0 + u * blockDim.x;
-      fetched[u] = i < vocab ? x[i] : -INFINITY;
+  auto look_at = [&](int i, float score) {
+    saw_nan |= score != score;
+    if (t > 0.f && i < vocab) {
+      const uint32_t bits = philox_first(static_cast<uint32_t>(i), draw, k0, k1);
+      const float u01 = (static_cast<float>(bits >> 8) + 0.5f) * 0x1p-24f;
+      score = score / t - logf(-logf(u01));
     }
+    if (i < vocab && score > value) { value = score; index = i; }
+  };
+  if ((vocab & 3) == 0 && (reinterpret_cast<uintptr_t>(logits) & 15) == 0) {
+    // rows of whole 16-byte pieces: a thread takes four consecutive ids a load (a row of 151,936 logits is 19 trips
+    // to memory with single loads, 5 with these)
+    const int pieces = vocab / 4;
+    for (int p0 = threadIdx.x; p0 < pieces; p0 += kAhead * blockDim.x) {
+      float4 fetched[kAhead];
 #pragma unroll
-    for (int u = 0; u < kAhead; ++u) {
-      const int i = i0 + u * blockDim.x;
-      float score = fetched[u];
-      saw_nan |= score != score;
-      if (t > 0.f && i < vocab) {
-        const uint32_t bits = philox_first(static_cast<uint32_t>(i), draw, k0, k1);
-        const float u01 = (static_cast<float>(bits >> 8) + 0.5f) * 0x1p-24f;
-        score = score / t - logf(-logf(u01));
+      for (int u = 0; u < kAhead; ++u) {
+        const int p = p0 + u * blockDim.x;
+        fetched[u] = p < pieces ? *reinterpret_cast<const float4*>(x + 4 * static_cast<size_t>(p))
+                                : float4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
       }
-      if (i < vocab && score > value) { value = score; index = i; }
+#pragma unroll
+      for (int u = 0; u < kAhead; ++u) {
+        const int i = 4 * (p0 + u * blockDim.x);
+        if (i < vocab) {
+          look_at(i, fetched[u].x);
+          look_at(i + 1, fetched[u].y);
+          look_at(i + 2, fetched[u].z);
+          look_at(i + 3, fetched[u].w);
+        }
+      }
+    }
+  } else {
+    for (int i0 = threadIdx.x; i0 < vocab; i0 += kAhead * blockDim.x) {
+      float fetched[kAhead];
+#pragma unroll
+      for (int u = 0; u < kAhead; ++u) {
+        const int i = i0 + u * blockDim.x;
+        fetched[u] = i < vocab ? x[i] : -INFINITY;
+      }
+#pragma unroll
+      for (int u = 0; u < kAhead; ++u) look_at(i0 + u * blockDim.x, fetched[u]);
     }
   }
   for (int offset = kWave / 2; offset > 0; offset >>= 1) {

@@ -1064,9 +1064,9 @@ def test_attention_finds_a_far_key(hip, ref, dtype):
         torch.testing.assert_close(picked[3], values[r][at, 1].float(), rtol=0.05, atol=0.05)
 
 
-def test_sample(hip):
+@pytest.mark.parametrize("vocab", [1531, 1532, 40004])     # single loads; 16-byte loads; more than one round of them
+def test_sample(hip, vocab):
     import numpy as np
-    vocab = 1531
     logits = rand(6, vocab, seed=24, scale=2.0)
     logits[1, 100] = logits[1, 900] = 50.0                                  # a tie: the lowest id wins
     logits[5] = logits[2]
