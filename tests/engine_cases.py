@@ -71,11 +71,11 @@ def make_case(name, model_folders):
     return dict(name=name, folder=folder, page_size=page_size, requests=requests, expected=expected, raw=raw)
 
 
-def make_engine(case, dtype, device, kernels=None, **engine_options):
+def make_engine(case, dtype, device, kernels=None, num_pages=None, **engine_options):
     from ampere_kv_engine_amd.config import EngineConfig
     from ampere_kv_engine_amd.engine import Engine
     page = case["page_size"]
-    config = EngineConfig(dtype=dtype, page_size=page, num_pages=POOL_TOKENS // page, max_seqs=4,
+    config = EngineConfig(dtype=dtype, page_size=page, num_pages=num_pages or POOL_TOKENS // page, max_seqs=4,
                           max_batched_tokens=256, max_seq_len=512, device=device, **engine_options)
     return Engine.from_folder(case["folder"], config, kernels=kernels)
 
@@ -106,9 +106,11 @@ _DOUBLES = {}
 def double_engine(case, dtype="bfloat16"):
     """The engine of `case` with the torch double of the kernel set, on the CPU (kept between tests)."""
     from torch_kernels import TorchKernels
-    key = (case["name"], case["folder"], dtype)
+    key = (case["name"], case["folder"], dtype, case["page_size"])
     if key not in _DOUBLES:
-        _DOUBLES[key] = make_engine(case, dtype, "cpu", kernels=TorchKernels())
+        # (at least a page for every request that can be live)
+        _DOUBLES[key] = make_engine(case, dtype, "cpu", kernels=TorchKernels(),
+                                    num_pages=max(POOL_TOKENS // case["page_size"], 4))
     return _DOUBLES[key]
 
 

@@ -46,6 +46,17 @@ def test_cutting_with_the_norm_kernels_of_their_own(case, cutting):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cutting", ["last_32_one_by_one", "portions_down_to_two_tokens", "mixed_with_pages_used_again"])
+def test_cutting_with_one_page_a_request(case, dtype, cutting):
+    """Pages as large as a request - what `--cache contiguous` of the command line makes of the pool: a request's keys
+    and values lie in one run of memory each, the block table has one entry.  Three such pages serve the six
+    requests, so every page is used again."""
+    one_page = dict(case, page_size=256)
+    engine = cases.make_engine(one_page, dtype, "cuda:0", num_pages=3)
+    getattr(cases, "case_" + cutting)(engine, one_page)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_program(case, dtype, tmp_path):
     """bin/trace_run as a user runs it: JSON steps on stdin, <step>.f32 files out, `done <step>` lines - fed all four
     cuttings of the same requests one after the other in one trace (whole; last 32 one by one; portions down to two

@@ -22,6 +22,14 @@ def test_cutting(engine, case, cutting):
     getattr(cases, "case_" + cutting)(engine, case)
 
 
+def test_mixed_cutting_with_one_page_a_request(case):
+    """Pages as large as a request (the command line's `--cache contiguous`): block tables of one entry, three pages
+    for six requests."""
+    one_page = dict(case, page_size=256)
+    engine = cases.make_engine(one_page, "float32", "cpu", kernels=TorchKernels(), num_pages=3)
+    cases.case_mixed_with_pages_used_again(engine, one_page)
+
+
 def test_branches_that_add_themselves_to_the_residual_sum_give_the_same_bits(case):
     """In steps of few rows a branch's last product may add its output to the residual sum itself and the next product
     norm its rows from the sums of squares left there (what the HIP kernel set does in decode steps).  With a double

@@ -264,7 +264,13 @@ def test_command_line(model_folders):
     result = run("--random-config", config_file, "--weights-seed", "3", "--mode", "generate", "--max-new-tokens", "4",
                  "--ignore-eos", "--prompt-len", "9")
     assert result.returncode == 0 and "generated_token_ids" in result.stdout, result.stderr[-2000:]
-    result = run("--model", model_folders["A"], "--mode", "generate", "--cache", "contiguous", "--prompt-ids", "1")
+    # every request's keys and values in one run of memory: a page as large as the request
+    for dtype in ("float32", "bfloat16"):
+        result = run("--model", model_folders["A"], "--mode", "generate", "--cache", "contiguous", "--dtype", dtype,
+                     "--max-new-tokens", "6", "--ignore-eos", "--prompt-ids", ",".join(map(str, prompt)))
+        assert result.returncode == 0 and f"generated_token_ids = {want}" in result.stdout, result.stderr[-2000:]
+        assert "cache=contiguous" in result.stderr + result.stdout
+    result = run("--model", model_folders["A"], "--mode", "generate", "--cache", "ring", "--prompt-ids", "1")
     assert result.returncode != 0
 
 
@@ -283,7 +289,7 @@ def test_command_line_with_several_prompts_and_the_engines_own_sizes(model_folde
                                         "--max-new-tokens", "5", "--ignore-eos", "--page-size", "8", *args],
                                        env=env, capture_output=True, text=True, timeout=300)
     for sizes in (("--max-seqs", "2", "--num-pages", "12", "--max-batched-tokens", "16", "--prefill-chunk", "7"),
-                  ("--kv-gb", "0.001"), ()):
+                  ("--kv-gb", "0.001"), (), ("--cache", "contiguous", "--max-seqs", "3")):
         result = run(*sizes)
         assert result.returncode == 0, result.stdout[-1500:] + result.stderr[-1500:]
         records = [json.loads(line) for line in result.stdout.splitlines() if line.startswith("{")]
