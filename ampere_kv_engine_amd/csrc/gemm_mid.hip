@@ -288,8 +288,11 @@ constexpr size_t kMostPartialFloats = 8u << 20;   // 32 MB: more than that is no
 MidPlan plan_mid(int rows, int n_tiles, int k_tiles, bool gated, int along, int rt, int depth, int parts) {
   MidPlan best{};
   double best_cost = -1.0;
-  const int mt = rows > 64 ? 8 : (rows + 15) / 16 < 2 ? 2 : (rows + 15) / 16;
-  const int m_blocks = (rows + mt * 16 - 1) / (mt * 16);
+  // tiles of 16 rows: up to eight a block, dealt evenly to the blocks (132 rows are two blocks of five tiles, not
+  // one of eight and one that multiplies zeros)
+  const int row_tiles = (rows + 15) / 16;
+  const int m_blocks = (row_tiles + 7) / 8;
+  const int mt = row_tiles < 2 ? 2 : (row_tiles + m_blocks - 1) / m_blocks;
   for (int a = 2; a <= 4; ++a) {
     if (along != 0 && a != along) continue;
     for (int r = 1; r <= 2; ++r) {
@@ -352,7 +355,8 @@ int dispatch_mid(const MidPlan& p, const void* x, const void* wp, void* y, float
   if (p.along == A_ && p.mt == MT_ && p.rt == RT_ && p.depth == G_) \
     return launch_mid<A_, MT_, RT_, G_, GATED, TY>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, stream)
 #define AKV_MID_ROWS(A_, RT_, G_) \
-  AKV_MID(A_, 2, RT_, G_); AKV_MID(A_, 3, RT_, G_); AKV_MID(A_, 4, RT_, G_); AKV_MID(A_, 8, RT_, G_)
+  AKV_MID(A_, 2, RT_, G_); AKV_MID(A_, 3, RT_, G_); AKV_MID(A_, 4, RT_, G_); AKV_MID(A_, 5, RT_, G_); \
+  AKV_MID(A_, 6, RT_, G_); AKV_MID(A_, 7, RT_, G_); AKV_MID(A_, 8, RT_, G_)
 #define AKV_MID_ALONG(RT_, G_) AKV_MID_ROWS(2, RT_, G_); AKV_MID_ROWS(3, RT_, G_); AKV_MID_ROWS(4, RT_, G_)
   AKV_MID_ALONG(2, 2);
   if constexpr (!GATED) {

@@ -321,12 +321,11 @@ class HipKernels:
         The table of choices decides where it names the product; otherwise a fixed rule, from measurements at
         Qwen3-8B, -14B and -32B shapes (cold weights, 24 to 256 rows; `bench_products --rows ...` repeats them):
         the library where there is one, except for the gated product up to 64 rows (the mid-size kernel is 8-28 %
-        faster; from 96 rows on the library is, by up to 40 %), plain products with outs <= k up to 128 rows (from
-        3 % slower to three times faster; the stacked q/k/v product, outs > k, is a tie there and stays with the
-        library) and every plain product from 129 to 256 rows (the library's times jump with the row count there -
-        q/k/v of 7,168 x 5,120: 36 / 50 / 63 us at 128 / 192 / 256 rows, the mid-size kernel 36 / 41 / 42; over
-        three model sizes the mid-size kernel is 10-35 % faster at 192 and 256 rows, except for the 4,096 x 4,096 product at 224
-        and 256 rows, which the library does in 25 us instead of 30).  Without the library: the skinny kernel up to
+        faster; beyond, the library is as fast at Qwen3-8B shapes and 2-15 % faster at the larger ones), plain
+        products with outs <= k up to 64 rows (the stacked q/k/v product, outs > k, is 2-6 % faster in the library
+        there) and every plain product from 65 to 256 rows (from 4 % slower to three times faster; the library's
+        times jump with the row count - q/k/v of 7,168 x 5,120: 36 / 50 / 63 us at 128 / 192 / 256 rows, the
+        mid-size kernel 36 / 41 / 42).  Without the library: the skinny kernel up to
         64 rows, the mid-size one up to 512, the wide one beyond."""
         library = (has_row_major and self.library_products_above is not None and rows > self.library_products_above
                    and out_dtype == torch.bfloat16)
@@ -344,7 +343,7 @@ class HipKernels:
             return "mid" if rows <= 64 else "library"
         if rows > 256:
             return "library"
-        return "mid" if (rows > 128 or outs <= k) else "library"
+        return "mid" if (rows > 64 or outs <= k) else "library"
 
     def _mid(self, x, packed: PackedWeight, out, rows: int, outs: int, gated: bool) -> None:
         """The mid-size product (`csrc/gemm_mid.hip`).  Where it cuts k over blocks it needs room for partial sums

@@ -520,6 +520,7 @@ def test_products_of_17_to_512_rows_follow_a_table_that_is_measured_on_request(h
 MID_CASES = [  # rows, outs, k: every row-tile count, several blocks of rows, ragged k and outs, long and short k
     (17, 100, 72), (20, 304, 520), (33, 48, 2048), (50, 4096, 4096), (64, 320, 256), (100, 4096, 4096),
     (128, 520, 1032), (300, 1000, 2048), (512, 1536, 512), (48, 640, 12288), (5, 64, 32),
+    (70, 264, 1032), (90, 4096, 512), (132, 520, 2048), (200, 304, 4096),      # five to seven tiles of rows a block
 ]
 
 
@@ -565,7 +566,8 @@ def test_mid_size_product(hip_own, ref, rows, outs, k):
                               stream) == (-3 if need.value > 16 else 0)
 
 
-@pytest.mark.parametrize("rows,inter,k", [(40, 208, 264), (64, 512, 2048), (130, 208, 520), (17, 16, 8), (256, 1024, 1024)])
+@pytest.mark.parametrize("rows,inter,k", [(40, 208, 264), (64, 512, 2048), (130, 208, 520), (17, 16, 8), (256, 1024, 1024),
+                                          (96, 512, 1032), (110, 208, 2048)])
 def test_mid_size_gated_product(hip_own, ref, rows, inter, k):
     import ctypes
     from ampere_kv_engine_amd.kernels.hip import _ptr
