@@ -128,7 +128,7 @@ class Scheduler:
 
     @property
     def idle(self) -> bool:
-        return not (self.waiting or self.prefilling or self.running)
+        return not (self.waiting or self.prefilling or self.running or self._late is not None)
 
     # ---- budgets ----------------------------------------------------------------------------------------------
     def _budget(self, prompt: int, max_new: int) -> list[int]:

@@ -84,12 +84,13 @@ class SlotSampler:
     def choose(self, logits: torch.Tensor, ctx) -> list[int]:
         return self.choose_later(logits, ctx).tokens()
 
-    LATER = 3       # choices that may be on their way to the host at the same time
+    LATER = 3       # choices that may be on their way to the host at the same time without anybody waiting
 
     def choose_later(self, logits: torch.Tensor, ctx) -> "LaterTokens":
         """The choice is made on the device now (the slots have their tokens as soon as the kernel has run, for the
         next step to feed); the tokens are on their way to the host and are waited for only when `tokens()` is asked
-        - so the host may launch the next step first.  At most `LATER` such choices may be outstanding."""
+        - so the host may launch the next step first.  `LATER` such choices have host memory of their own; a
+        choice whose memory comes round again before anybody has asked for its tokens is read first (that waits)."""
         rows = logits.shape[0]
         if rows > self.max_rows:
             raise ValueError(f"{rows} rows to choose from; the sampler was built for {self.max_rows}")
@@ -102,8 +103,8 @@ class SlotSampler:
                            for _ in range(self.LATER)]
             self._turn, self._waiting = 0, [None] * self.LATER
         self._turn = (self._turn + 1) % self.LATER
-        if self._waiting[self._turn] is not None and not self._waiting[self._turn].read:
-            raise RuntimeError(f"more than {self.LATER} choices whose tokens nobody has asked for")
+        if self._waiting[self._turn] is not None:
+            self._waiting[self._turn].tokens()                   # (keeps them; its memory is about to be written again)
         host, arrived = self._later[self._turn]
         host[:rows].copy_(out, non_blocking=True)                # into pinned memory; the event tells when it is there
         arrived.record(torch.cuda.current_stream(self.device))

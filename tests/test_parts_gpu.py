@@ -468,7 +468,7 @@ def test_a_slot_that_is_used_again_starts_clean_on_the_device(model_folders):
 def test_tokens_read_a_step_late_are_the_tokens_read_at_once(model_folders):
     """`choose_later` leaves the chosen token in the request's slot for the next step; the host may read it after it
     has launched that step.  Two requests, greedy and drawn, decoded with the read one step behind give what
-    `generate_tokens` gives; a fourth choice that nobody has read is refused."""
+    `generate_tokens` gives; choices that nobody reads for several steps keep their tokens."""
     from ampere_kv_engine_amd.engine import LAST_TOKEN
     raw, _, page = TINY["A"]
     config = EngineConfig(dtype="bfloat16", page_size=page, num_pages=32, max_seqs=2, max_batched_tokens=64,
@@ -490,10 +490,15 @@ def test_tokens_read_a_step_late_are_the_tokens_read_at_once(model_folders):
     for mine, token in zip(got, before.tokens()):
         mine.append(token)
     assert got == want
-    unread = [engine.choose_later(logits) for _ in range(3)]
-    with pytest.raises(RuntimeError, match="nobody has asked for"):
-        engine.choose_later(logits)
-    for later in unread:
-        later.tokens()
+    # choices that nobody reads do not get lost when their host memory comes round again: five in a row, read afterwards
+    for q in seqs:
+        engine.close(q)
+    seqs = [engine.open(f"again{i}", t, s) for i, (t, s) in enumerate(draws)]
+    logits = engine.step([StepEntry(q, p, [len(p) - 1]) for q, p in zip(seqs, prompts)], borrow_logits=True)
+    unread = [engine.choose_later(logits)]
+    for _ in range(4):
+        logits = engine.step([StepEntry(q, LAST_TOKEN, [0]) for q in seqs], borrow_logits=True)
+        unread.append(engine.choose_later(logits))
+    assert [[later.tokens()[i] for later in unread] for i in range(2)] == [w[:5] for w in want]
     for q in seqs:
         engine.close(q)

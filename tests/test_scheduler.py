@@ -310,3 +310,25 @@ def test_overlapped_rounds_hand_tokens_over_a_round_late(model_folders):
     assert lengths == [1, 1, 2, 3, 4, 5]
     assert request.output_ids == alone(model_folders["A"], page, prompt, 5)
     assert request.cached_tokens == len(prompt) + 4 and scheduler.overlapped_rounds == 4
+
+
+def test_a_round_launched_for_nothing_is_read_before_the_scheduler_is_idle(model_folders):
+    """An end-of-sequence token is learnt a round late: the next round is already on its way then.  The scheduler is
+    idle only when those tokens have been read too - nothing of the finished request stays outstanding in the
+    engine - and the request has what it would have without the overlap."""
+    raw, _, page = TINY["A"]
+    prompt = random_ids(raw["vocab_size"], 9, seed=66)
+    free_run = alone(model_folders["A"], page, prompt, 6)
+    outputs = {}
+    for overlap in (False, True):
+        engine = make_engine(model_folders["A"], page, num_pages=16)
+        engine.spec = type(engine.spec)(**{**engine.spec.__dict__, "eos_token_ids": (free_run[2],)})
+        scheduler = Scheduler(engine, overlap_decoding=overlap)
+        request = scheduler.submit("r", prompt, 6)
+        scheduler.run_until_idle()
+        assert scheduler._late is None and scheduler.idle
+        assert request.stop_reason == STOP_EOS and engine.cache.num_free_pages == [16]
+        outputs[overlap] = request.output_ids
+        # the engine is as good as new for whoever comes next
+        assert generate_tokens(engine, prompt, max_new_tokens=4, ignore_eos=True) == free_run[:4]
+    assert outputs[True] == outputs[False] == free_run[:free_run.index(free_run[2]) + 1]
