@@ -106,6 +106,7 @@ class HipKernels:
         self._packed_rows = None               # where activations are repacked for the engine's own product
         self._mid_partial = None               # the mid-size product's partial sums, where it cuts k over blocks
         self._mid_counters = None              # and its arrival counters (zero between launches)
+        self._outgrown = []                    # workspaces that were replaced by larger ones: recorded steps may name them
         self.device = torch.device(device)
         if self.device.type == "cuda" and self.device.index is None:
             self.device = torch.device("cuda", 0)
@@ -355,11 +356,13 @@ class HipKernels:
             if self._mid_partial is None or self._mid_partial.numel() < partial_floats.value:
                 if torch.cuda.is_current_stream_capturing():
                     raise KernelError("a recorded step needs more room for partial sums than the steps before it")
+                self._outgrown.append(self._mid_partial)      # (a recorded step may still point at it)
                 self._mid_partial = torch.empty(max(partial_floats.value, 8 << 20), dtype=torch.float32, device=self.device)
             if self._mid_counters is None or self._mid_counters.numel() < counters.value:
                 if torch.cuda.is_current_stream_capturing():
                     raise KernelError("a recorded step needs more counters than the steps before it")
-                self._mid_counters = torch.zeros(max(counters.value, 4096), dtype=torch.int32, device=self.device)
+                self._outgrown.append(self._mid_counters)
+                self._mid_counters = torch.zeros(max(counters.value, 1 << 16), dtype=torch.int32, device=self.device)
         held = lambda buffer: ctypes.c_long(buffer.numel() if buffer is not None else 0)
         self._check(self.lib.akv_linear_mid(_ptr(x), _ptr(packed.data), _ptr(out), _code(out), _ptr(self._mid_partial),
                                             held(self._mid_partial), _ptr(self._mid_counters), held(self._mid_counters),
@@ -480,6 +483,7 @@ class HipKernels:
         launches).  One pair of buffers for all products - they follow each other on the stream."""
         if self._exchange_tiles < n_tiles:
             self._exchange_tiles = max(n_tiles, 4096)
+            self._outgrown += [self._exchange_pieces, self._exchange_arrivals]
             self._exchange_pieces = torch.empty(self._exchange_tiles * 512, dtype=torch.float32, device=self.device)
             self._exchange_arrivals = torch.zeros(self._exchange_tiles, dtype=torch.int32, device=self.device)
 
@@ -809,6 +813,7 @@ class HipKernels:
         if self._plan_buffers[index] is None or self._plan_buffers[index].numel() < need:
             if torch.cuda.is_current_stream_capturing() and self._plan_buffers[index] is not None:
                 raise KernelError("a recorded step needs a larger plan of its keys than the steps before it")
+            self._outgrown.append(self._plan_buffers[index])       # (a recorded step may still point at it)
             self._plan_buffers[index] = torch.empty(max(need, self.PLAN_ENTRIES + 4 * 4096), dtype=torch.int32,
                                                     device=self.device)
         plan = self._plan_buffers[index]
