@@ -72,7 +72,7 @@ def scheduler_workload(name: str, layers: int | None, library_above: int | None)
         max_batched_tokens=PREFILL_TOKENS + len(prompts), max_seq_len=longest + PAGE_SIZE, device="cuda:0",
         library_products_above=library_above))
     samples = []
-    for run in range(3):                                    # the first run warms up (graphs are recorded in it)
+    for run in range(4):                                    # the first run warms up (graphs are recorded in it)
         scheduler = Scheduler(engine, prefill_chunk_size=PREFILL_TOKENS, overlap_decoding=True)
         ids = [torch.randint(0, config.vocab_size, (p,), generator=generator).tolist() for p in prompts]
         torch.cuda.synchronize(engine.device)
