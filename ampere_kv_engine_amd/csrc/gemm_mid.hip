@@ -327,9 +327,10 @@ MidPlan plan_mid(int rows, int n_tiles, int k_tiles, bool gated, int along, int 
       }
     }
   }
-  if (depth == 0) depth = best.rt == 2 ? 2 : 4;
-  if (best.rt == 2 && depth > 2) depth = 2;   // (two row tiles and a deeper ring do not fit the registers)
-  best.depth = depth;
+  // two row tiles a wave: a ring of two register sets (a deeper one does not fit the registers); one row tile: of four
+  // (measured: never slower than two).  `depth` can only ask for what the row tiles allow.
+  if (depth != 0 && depth != (best.rt == 2 ? 2 : 4)) return MidPlan{};
+  best.depth = best.rt == 2 ? 2 : 4;
   return best;
 }
 
@@ -360,7 +361,6 @@ int dispatch_mid(const MidPlan& p, const void* x, const void* wp, void* y, float
 #define AKV_MID_ALONG(RT_, G_) AKV_MID_ROWS(2, RT_, G_); AKV_MID_ROWS(3, RT_, G_); AKV_MID_ROWS(4, RT_, G_)
   AKV_MID_ALONG(2, 2);
   if constexpr (!GATED) {
-    AKV_MID_ALONG(1, 2);
     AKV_MID_ALONG(1, 4);
   }
 #undef AKV_MID_ALONG
@@ -383,8 +383,8 @@ extern "C" int akv_linear_mid_workspace(int rows, int n_tiles, int k_tiles, int 
 }
 
 // x [rows, k] bfloat16 row-major, 1 <= rows; wp the packed weight; y [rows, outs] (gated: [rows, inter], wp as for
-// akv_linear_packed_swiglu).  `along` (waves along a band: 2..4), `rt` (row tiles per wave, 1 or 2), `depth` (register
-// sets of the weight ring: 2, or 4 with rt = 1) and `parts` (blocks along k, a power of two) may be 0: chosen here.
+// akv_linear_packed_swiglu).  `along` (waves along a band: 2..4), `rt` (row tiles per wave, 1 or 2), `depth`
+// (register sets of the weight ring: 2 with rt = 2, 4 with rt = 1) and `parts` (blocks along k, a power of two) may be 0: chosen here.
 // `partial_floats` and `counter_words` say how much `partial` and `counters` hold: a cut that needs more
 // (akv_linear_mid_workspace tells) is refused with -3 and nothing is launched.
 extern "C" int akv_linear_mid(const void* x, const void* wp, void* y, int y_dtype, float* partial, long partial_floats,

@@ -540,7 +540,7 @@ def test_mid_size_product(hip_own, ref, rows, outs, k):
     counters = torch.zeros(4096, dtype=torch.int32, device="cuda")
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     xd = x.cuda()
-    for along, rt, depth, parts in ((0, 0, 0, 0), (2, 1, 2, 1), (3, 2, 2, 2), (4, 1, 4, 4), (4, 2, 2, 8), (3, 1, 4, 1)):
+    for along, rt, depth, parts in ((0, 0, 0, 0), (2, 1, 4, 1), (3, 2, 2, 2), (4, 1, 4, 4), (4, 2, 2, 8), (3, 1, 0, 1), (2, 2, 0, 2)):
         for code, dtype in ((1, torch.bfloat16), (0, torch.float32)):
             for _ in range(2):
                 got = torch.full((rows, outs), float("nan"), dtype=dtype, device="cuda")
@@ -558,6 +558,9 @@ def test_mid_size_product(hip_own, ref, rows, outs, k):
         assert lib.akv_linear_mid(_ptr(xd), _ptr(packed.data), _ptr(target), 0, _ptr(partial), ctypes.c_long(partial.numel()), _ptr(counters), ctypes.c_long(counters.numel()), rows, outs, k,
                                   packed.n_tiles, packed.k_tiles, 0, 4, 1, 4, 4, stream) == 0
     assert torch.equal(first, again)
+    # a ring depth that the row tiles per wave do not allow is refused
+    assert lib.akv_linear_mid(_ptr(xd), _ptr(packed.data), _ptr(first), 0, _ptr(partial), ctypes.c_long(partial.numel()), _ptr(counters),
+                              ctypes.c_long(counters.numel()), rows, outs, k, packed.n_tiles, packed.k_tiles, 0, 2, 2, 4, 1, stream) == -2
     # a workspace that is too small for the cut is refused before anything is launched
     need, words = ctypes.c_long(0), ctypes.c_long(0)
     lib.akv_linear_mid_workspace(rows, packed.n_tiles, packed.k_tiles, 0, 4, 1, 4, 4, ctypes.byref(need), ctypes.byref(words))
