@@ -19,7 +19,7 @@ Peaks are MI355X's published ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s.
 
 Further workloads run through the scheduler and print a line of their own (`--workload`):
   serving-14b      Qwen3-14B layer sizes: 32 requests, prompt lengths uniform in [128, 4096], 256 tokens each,
-                   prompts fed in portions of at most 2,048 tokens beside the decoding requests
+                   prompts fed in portions beside the decoding requests, at most 2,048 tokens a round
   batch-32b        Qwen3-32B layer sizes: 16 requests with 8,192-token prompts, 128 greedy tokens each
   offline-512-32   the reference's offline batch (docs/BENCHMARK.md:9-24 there) at Qwen3-8B layer sizes: B = 1 and
                    B = 4 requests of 512 input tokens, 32 greedy output tokens each, end-of-sequence ignored; one
@@ -69,8 +69,9 @@ def scheduler_workload(name: str, layers: int | None, library_above: int | None)
     pages = sum((p + new_tokens + 2 * PAGE_SIZE) // PAGE_SIZE for p in prompts) + 8
     engine = Engine.from_random(config, seed=0, engine_config=EngineConfig(
         dtype="bfloat16", page_size=PAGE_SIZE, num_pages=pages, max_seqs=len(prompts),
-        max_batched_tokens=PREFILL_TOKENS + len(prompts), max_seq_len=longest + PAGE_SIZE, device="cuda:0",
-        library_products_above=library_above))
+        max_batched_tokens=PREFILL_TOKENS, max_seq_len=longest + PAGE_SIZE, device="cuda:0",
+        library_products_above=library_above))     # (a round's rows, decoding requests included: the library's products
+                                                  # take 2,048 rows in whole tiles, 2,080 in one row of tiles more)
     samples = []
     for run in range(4):                                    # the first run warms up (graphs are recorded in it)
         scheduler = Scheduler(engine, prefill_chunk_size=PREFILL_TOKENS, overlap_decoding=True)
