@@ -106,11 +106,10 @@ _DOUBLES = {}
 def double_engine(case, dtype="bfloat16"):
     """The engine of `case` with the torch double of the kernel set, on the CPU (kept between tests)."""
     from torch_kernels import TorchKernels
-    key = (case["name"], case["folder"], dtype, case["page_size"])
+    pages = max(POOL_TOKENS // case["page_size"], 4, case.get("pool_pages", 0))    # (room for every schedule of the case)
+    key = (case["name"], case["folder"], dtype, case["page_size"], pages)
     if key not in _DOUBLES:
-        # (at least a page for every request that can be live)
-        _DOUBLES[key] = make_engine(case, dtype, "cpu", kernels=TorchKernels(),
-                                    num_pages=max(POOL_TOKENS // case["page_size"], 4))
+        _DOUBLES[key] = make_engine(case, dtype, "cpu", kernels=TorchKernels(), num_pages=pages)
     return _DOUBLES[key]
 
 

@@ -57,6 +57,25 @@ def test_cutting_with_one_page_a_request(case, dtype, cutting):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_mixed_cuttings_with_other_pages_pools_and_orders(case, dtype):
+    """The same requests in random orders, with random prompt lengths, two to four of them live, on pools of other page
+    sizes (4 to 64 tokens) and sizes than the model's own test pool."""
+    import random
+    for trial in range(3):
+        rng = random.Random(7 * trial + len(case["name"]) + ord(case["name"][0]))
+        page = rng.choice([4, 8, 32, 64])
+        num_pages = max(rng.choice([320, 384, 512]) // page, 3)
+        names = list(case["requests"])
+        rng.shuffle(names)
+        requests = {name: case["requests"][name] for name in names}
+        sub = dict(case, page_size=page, pool_pages=num_pages, requests=requests,
+                   expected={name: case["expected"][name] for name in names})
+        prompts = {name: rng.randint(1, len(requests[name])) for name in names}
+        engine = cases.make_engine(sub, dtype, "cuda:0", num_pages=num_pages)
+        cases.check(engine, sub, schedules.mixed(requests, prompts, page, num_pages, seed=trial, max_live=rng.choice([2, 3, 4])))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_program(case, dtype, tmp_path):
     """bin/trace_run as a user runs it: JSON steps on stdin, <step>.f32 files out, `done <step>` lines - fed all four
     cuttings of the same requests one after the other in one trace (whole; last 32 one by one; portions down to two
