@@ -159,6 +159,9 @@ def main() -> int:
     parser.add_argument("--contexts", default="", help="requests of different context lengths in one batch, e.g. "
                         "'32768,512x63' (overrides --batch and --context; no further points, no prefill)")
     parser.add_argument("--no-prefill", action="store_true")
+    parser.add_argument("--no-graphs", action="store_true",
+                        help="every step is launched kernel by kernel instead of replayed from a recording (for counter "
+                             "collection; the host's launches then show in the time)")
     parser.add_argument("--prefill-only", action="store_true", help="time the prefill alone (for kernel profiles)")
     parser.add_argument("--workload", choices=["decode", "serving-14b", "batch-32b", "offline-512-32"], default="decode",
                         help="decode: the headline measurement; the others run a set of requests through the scheduler")
@@ -199,7 +202,8 @@ def main() -> int:
     engine_config = EngineConfig(dtype="bfloat16", page_size=PAGE_SIZE, num_pages=pages, max_seqs=max_batch + 1,
                                  max_batched_tokens=PREFILL_TOKENS,
                                  max_seq_len=max(tokens_per_request, PREFILL_TOKENS) + PAGE_SIZE,
-                                 device="cuda:0", library_products_above=library_above)
+                                 device="cuda:0", library_products_above=library_above,
+                                 decode_graphs=not args.no_graphs)
     engine = Engine.from_random(config, seed=0, engine_config=engine_config)
     for group in engine.cache.groups:       # any finite keys and values: their content does not change the timing
         group.pages.normal_(0.0, 0.5)
