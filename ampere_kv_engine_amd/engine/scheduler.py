@@ -16,8 +16,8 @@ With `overlap_decoding` a round of decoding requests alone does not wait for its
 device, where the next round finds them in the requests' slots, and come to the host while that next round runs -
 the host launches it first and reads them then.  What the host learns a round late (an EOS) costs the request one
 token of work that is thrown away; what it knows beforehand (the limit of new tokens) costs nothing.  Anything else
-to do - a request waiting, a prompt to feed, a cancellation, a deadline - ends the overlap: the tokens are read, and
-the round is an ordinary one.
+to do - a request that can be admitted, a prompt to feed, a cancellation, a deadline - ends the overlap: the tokens
+are read, and the round is an ordinary one.  A queue whose head cannot be admitted yet ends nothing.
 
 When pages run out: by construction they cannot after admission.  A request whose budget does not fit the free
 budget waits at the head of the queue (and holds back those behind it); one whose budget exceeds the whole pool is
@@ -195,11 +195,21 @@ class Scheduler:
 
     # ---- overlapped decoding -------------------------------------------------------------------------------
     def _only_decoding(self, now: float) -> bool:
-        """Nothing to do this round but to decode: nobody waits, no prompt is being fed, nobody was cancelled or has
-        run out of time."""
-        if self.waiting or self.prefilling or not self.running:
+        """Nothing to do this round but to decode: no prompt is being fed, nobody was cancelled or has run out of
+        time, and nobody waits who could be admitted - a queue whose head does not fit (every slot taken, or its page
+        budget larger than what is free) changes nothing about the round, and that is the steady state of a busy
+        server.  When a request retires the head may fit: the next round is then an ordinary one."""
+        if self.prefilling or not self.running or self._head_fits():
             return False
-        return not any(r.stop_reason or (r.deadline is not None and r.deadline <= now) for r in self.running)
+        return not any(r.stop_reason or (r.deadline is not None and r.deadline <= now)
+                       for queue in (self.running, self.waiting) for r in queue)
+
+    def _head_fits(self) -> bool:
+        """Whether the request at the head of the queue could be admitted now."""
+        if not self.waiting or len(self.prefilling) + len(self.running) >= self.max_batch:
+            return False
+        head = self.waiting[0]
+        return not any(r + b > p for r, b, p in zip(self.reserved_pages, head.budget_pages, self.pool_pages))
 
     def _overlapped_round(self) -> tuple[list[Request], list[int]]:
         late = self._late
@@ -272,11 +282,8 @@ class Scheduler:
 
     def _admit(self) -> None:
         """First come, first served; the head waits (and holds the others back) until its budget fits."""
-        while self.waiting and len(self.prefilling) + len(self.running) < self.max_batch:
-            head = self.waiting[0]
-            if any(r + b > p for r, b, p in zip(self.reserved_pages, head.budget_pages, self.pool_pages)):
-                return
-            self.waiting.pop(0)
+        while self._head_fits():
+            head = self.waiting.pop(0)
             for g, b in enumerate(head.budget_pages):
                 self.reserved_pages[g] += b
             head.seq = self.engine.open(head.request_id, head.sampling.temperature, head.sampling.seed)

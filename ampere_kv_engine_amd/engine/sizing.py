@@ -21,7 +21,8 @@ class MemoryPlan:
     weight_bytes: int          # the model's tensors in the engine's arithmetic
     second_copy_bytes: int     # the row-major copies of the matrices that the library products read
     page_bytes: int            # one page of every cache group and layer
-    fixed_bytes: int           # residual stream, logits of recorded steps, activations of the largest step (estimate)
+    fixed_bytes: int           # residual stream, logits of recorded steps, activations of the largest step (estimate),
+                               # position tables
     num_pages: int             # pages that fit into what is left of `memory_bytes`
     page_size: int
 
@@ -34,7 +35,7 @@ def plan_memory(spec: ModelSpec, engine_config: EngineConfig, memory_bytes: int)
     """Pages of `engine_config.page_size` tokens that fit into `memory_bytes` of device memory beside the weights
     of `spec` and the engine's own buffers.  Raises ValueError when not even one page per request slot fits."""
     element = _ELEMENT_BYTES[engine_config.dtype]
-    model = Model(spec, dry_runtime())
+    model = Model(spec, dry_runtime(engine_config.max_seq_len, engine_config.page_size))
     tensors = [t for t in model.tensors() if not t.optional]
     weight_bytes = sum(_count(t.shape) for t in tensors) * element
     # (what a part keeps twice it says itself: a part with storage of its own is counted once)
@@ -54,6 +55,7 @@ def plan_memory(spec: ModelSpec, engine_config: EngineConfig, memory_bytes: int)
              + engine_config.max_seqs * spec.vocab_size * 4 * 2                       # logits, eager and recorded
              + engine_config.max_batched_tokens * widest * element * 18               # activations of a step, two arenas
              + 2 * largest                                                            # a matrix in flight while it is packed
+             + model.rt.shared_bytes()                                                # position tables, one per kind and size
              + (512 << 20))                                                           # timing spacer, library workspaces
     left = memory_bytes - weight_bytes - second - fixed
     num_pages = left // page_bytes if page_bytes else 0

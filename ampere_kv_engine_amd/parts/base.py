@@ -10,7 +10,7 @@ per-request state of fixed size, or nothing.
 
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Any, Callable
 
 import torch
@@ -55,9 +55,30 @@ class Runtime:
     device: torch.device
     max_seq_len: int
     page_size: int
+    _shared: dict = field(default_factory=dict, repr=False)
 
     def empty(self, *shape: int, dtype: torch.dtype | None = None) -> torch.Tensor:
         return torch.empty(shape, dtype=dtype or self.dtype, device=self.device)
+
+    def shared_buffer(self, key: tuple, shape: tuple[int, ...], dtype: torch.dtype,
+                      fill: Callable[[torch.Tensor], None]) -> torch.Tensor:
+        """A read-only buffer that follows from `key` alone (a kind, sizes, constants): built by `fill(buffer)` the
+        first time a part asks for the key and handed to every later part that asks for the same one - the layers of
+        a model share one position table instead of holding a copy each (the reference builds its inverse
+        frequencies once per model, ampere_kv/runner.py:41-44)."""
+        buffer = self._shared.get(key)
+        if buffer is None:
+            buffer = self.empty(*shape, dtype=dtype)
+            fill(buffer)
+            self._shared[key] = buffer
+        elif tuple(buffer.shape) != tuple(shape) or buffer.dtype != dtype:
+            raise ValueError(f"shared buffer {key!r} exists as {tuple(buffer.shape)} {buffer.dtype}, "
+                             f"asked for as {tuple(shape)} {dtype}")
+        return buffer
+
+    def shared_bytes(self) -> int:
+        """Device memory of the buffers that parts share (what the memory plan counts beside weights and pages)."""
+        return sum(b.numel() * b.element_size() for b in self._shared.values())
 
 
 # ---- what a mixer keeps between steps ----------------------------------------------------------------

@@ -19,9 +19,12 @@ class RotaryHalf(Part):
         # inverse frequencies exactly as the reference forms them (runner.py:42-43): float32 on the host
         exponent = torch.arange(0, self.head_dim, 2, dtype=torch.int64).float() / self.head_dim
         self.inv_freq = (1.0 / (self.theta ** exponent)).to(runtime.device)
-        # cos/sin of every position the engine can reach, float32 [max_seq_len, d/2, 2], built once
-        self.table = runtime.empty(runtime.max_seq_len, self.head_dim // 2, 2, dtype=torch.float32)
-        runtime.kernels.rope_table(self.inv_freq, self.table)
+        # cos/sin of every position the engine can reach, float32 [max_seq_len, d/2, 2]: built once per model - every
+        # layer with the same head size and theta is handed the same table (runner.py:41-44 builds inv_freq once)
+        self.table = runtime.shared_buffer(
+            ("rope_half", self.head_dim, self.theta, runtime.max_seq_len),
+            (runtime.max_seq_len, self.head_dim // 2, 2), torch.float32,
+            lambda table: runtime.kernels.rope_table(self.inv_freq, table))
 
     def apply(self, x: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
         """Rotate x [tokens, heads, head_dim] in place by each token's absolute position."""

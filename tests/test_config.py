@@ -128,3 +128,25 @@ def test_plan_memory_counts_a_second_copy_only_where_a_part_keeps_one():
     head = 97 * 32
     assert plan.second_copy_bytes == 2 * (2 * attention + dense + head)
     assert plan.weight_bytes >= 2 * (2 * attention + dense + experts + 2 * head)
+
+
+def test_layers_share_one_position_table_and_the_memory_plan_counts_it():
+    """Every layer's rotary part is handed the same cos/sin table (ampere_kv/runner.py:41-44 builds its inverse
+    frequencies once per model); `plan_memory` counts it once, sized by the longest sequence."""
+    from ampere_kv_engine_amd.config import EngineConfig, Qwen3Config
+    from ampere_kv_engine_amd.engine import plan_memory
+    from ampere_kv_engine_amd.engine.dry import dry_runtime
+    from ampere_kv_engine_amd.engine.model import Model
+    raw = dict(architectures=["Qwen3ForCausalLM"], vocab_size=1000, hidden_size=64, num_hidden_layers=5,
+               num_attention_heads=4, num_key_value_heads=2, head_dim=16, intermediate_size=128, rope_theta=1e4,
+               rms_norm_eps=1e-6, tie_word_embeddings=False, hidden_act="silu")
+    spec = Qwen3Config.from_dict(raw).to_model_spec()
+    runtime = dry_runtime(max_seq_len=4096, page_size=8)
+    model = Model(spec, runtime)
+    tables = {id(block.mixer.position.table) for block in model.blocks}
+    assert len(tables) == 1
+    assert runtime.shared_bytes() == 4096 * 8 * 2 * 4
+    sizes = dict(dtype="bfloat16", page_size=8, num_pages=1, max_seqs=2, max_batched_tokens=16)
+    short = plan_memory(spec, EngineConfig(max_seq_len=64, **sizes), 1 << 30)
+    long = plan_memory(spec, EngineConfig(max_seq_len=64 + 4096, **sizes), 1 << 30)
+    assert long.fixed_bytes - short.fixed_bytes == 4096 * 8 * 2 * 4

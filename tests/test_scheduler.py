@@ -391,3 +391,58 @@ def test_random_workloads_with_and_without_overlapped_decoding(name, model_folde
                 else:
                     cut = want[i].index(eos) + 1 if eos in want[i] else len(want[i])
                     assert request.output_ids == want[i][:cut], (trial, overlap, i, request.stop_reason)
+
+
+def test_decoding_overlaps_while_the_queue_is_blocked(model_folders):
+    """A pool so small that the second and third request wait until the one before has retired: while the head of
+    the queue cannot be admitted the decoding rounds still overlap, and when a request retires the next round admits
+    the head.  Tokens equal those of ordinary rounds; everything comes back."""
+    raw, _, page = TINY["A"]
+    folder = model_folders["A"]
+    prompts = [random_ids(raw["vocab_size"], n, seed=80 + i) for i, n in enumerate((20, 11, 25))]
+    limits = (12, 9, 7)
+    want = [alone(folder, page, p, n) for p, n in zip(prompts, limits)]
+    results = {}
+    for overlap in (False, True):
+        engine = make_engine(folder, page, num_pages=3)     # budgets of 3, 2 and 3 pages: one request at a time, two at most
+        scheduler = Scheduler(engine, overlap_decoding=overlap)
+        requests = [scheduler.submit(f"r{i}", p, n, ignore_eos=True) for i, (p, n) in enumerate(zip(prompts, limits))]
+        overlapped_while_waiting = 0
+        for _ in range(200):
+            if scheduler.idle:
+                break
+            before, waiting = scheduler.overlapped_rounds, len(scheduler.waiting)
+            scheduler.step()
+            if waiting and len(scheduler.waiting) == waiting and scheduler.overlapped_rounds > before:
+                overlapped_while_waiting += 1
+        assert scheduler.idle and scheduler.reserved_pages == [0]
+        assert engine.cache.num_free_pages == [3] and engine.cache.slots.num_free == 4
+        assert [r.output_ids for r in requests] == want
+        assert all(r.stop_reason == STOP_LIMIT for r in requests)
+        results[overlap] = (overlapped_while_waiting, scheduler.rounds)
+    assert results[False][0] == 0 and results[True][0] >= 10
+    assert results[True][1] <= results[False][1] + 4       # a round late per retirement, no more
+
+
+def test_a_cancelled_or_expired_waiting_request_ends_the_overlap(model_folders):
+    """A waiting request that was cancelled, or whose time has run out, is retired at the start of the next round
+    even while the running ones decode overlapped."""
+    raw, _, page = TINY["A"]
+    engine = make_engine(model_folders["A"], page, num_pages=3)
+    now = [0.0]
+    scheduler = Scheduler(engine, overlap_decoding=True, clock=lambda: now[0])
+    first = scheduler.submit("first", random_ids(raw["vocab_size"], 20, seed=1), 12, ignore_eos=True)
+    second = scheduler.submit("second", random_ids(raw["vocab_size"], 20, seed=2), 4, ignore_eos=True)
+    third = scheduler.submit("third", random_ids(raw["vocab_size"], 20, seed=3), 4, ignore_eos=True, deadline=5.0)
+    for _ in range(4):
+        scheduler.step()
+    assert scheduler.overlapped_rounds >= 2 and second.status == WAITING
+    scheduler.cancel(second)
+    finished, _ = scheduler.step()
+    assert second in finished and second.stop_reason == STOP_CANCELLED
+    now[0] = 6.0
+    finished, _ = scheduler.step()
+    assert third in finished and third.stop_reason == STOP_EXPIRED
+    scheduler.run_until_idle()
+    assert first.stop_reason == STOP_LIMIT and len(first.output_ids) == 12
+    assert engine.cache.num_free_pages == [3] and scheduler.reserved_pages == [0]
