@@ -31,7 +31,6 @@ import json
 import re
 import statistics
 import sys
-import tempfile
 
 import torch
 
@@ -265,14 +264,8 @@ def model_folder(args):
     """The folder of --model, or a temporary one written from --random-config (returned too, to be cleaned up)."""
     if args.random_config is None:
         return args.model, None
-    from .config import registry
-    from .weights.random import write_random_model
-    with open(args.random_config) as handle:
-        raw = json.load(handle)
-    scratch = tempfile.TemporaryDirectory()
-    with open(f"{scratch.name}/config.json", "w") as handle:
-        json.dump(raw, handle)
-    write_random_model(scratch.name, registry.load_config(scratch.name), args.weights_seed)
+    from .weights.random import random_model_folder
+    scratch = random_model_folder(args.random_config, args.weights_seed)
     return scratch.name, scratch
 
 

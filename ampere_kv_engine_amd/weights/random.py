@@ -77,6 +77,21 @@ def write_random_model(folder: str, config, seed: int, *, store_dtype: torch.dty
     return folder
 
 
+def random_model_folder(config_json: str, seed: int):
+    """A temporary model folder (config.json, model.safetensors) for the configuration in the file `config_json`,
+    filled with random weights from `seed`.  Returns the `tempfile.TemporaryDirectory`; its `name` is the folder, and
+    it is removed when the object is cleaned up or collected."""
+    import tempfile
+    from ..config import registry
+    with open(config_json) as handle:
+        raw = json.load(handle)
+    scratch = tempfile.TemporaryDirectory()
+    with open(os.path.join(scratch.name, "config.json"), "w") as handle:
+        json.dump(raw, handle)
+    write_random_model(scratch.name, registry.load_config(scratch.name), seed)
+    return scratch
+
+
 class RandomSource:
     """Hands out random tensors directly on a device, without a file: for measurements at sizes whose
     checkpoint would be tens of gigabytes.  Same laws as `write_random_model`, device generator."""

@@ -111,6 +111,40 @@ def test_trace_run_program(case, dtype, tmp_path):
                                       f"cutting {prefix} request {name}")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program_with_a_random_configuration_and_its_own_pool(case, dtype, tmp_path):
+    """bin/trace_run --random-config FILE --weights-seed S --page-size P --num-pages N --max-seqs M: the model is
+    written from the configuration and the seed (the same tensors as the case's folder), the pool has the model's own
+    page size (tiny-B: 8 tokens, tiny-C: 4) and so few pages that they are used again, four requests live at most."""
+    import numpy as np
+    from conftest import TINY
+    raw, seed, page = TINY[case["name"]]
+    config = tmp_path / "config.json"
+    config.write_text(json.dumps(raw))
+    requests = {k: case["requests"][k] for k in ("a", "b", "e", "f")}
+    pages = 192 // page
+    schedule = schedules.mixed(requests, PROMPTS, page, pages, seed=13)
+    records = schedules.to_trace(requests, schedule)
+    out = tmp_path / "out"
+    result = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--random-config", str(config), "--weights-seed",
+                             str(seed), "--dtype", dtype, "--out", str(out), "--max-tokens", "192", "--page-size",
+                             str(page), "--num-pages", str(pages), "--max-seqs", "4"],
+                            input="\n".join(json.dumps(r) for r in records) + "\n", capture_output=True, text=True,
+                            timeout=300)
+    assert result.returncode == 0, result.stderr[-2000:]
+    vocab = raw["vocab_size"]
+    collected = {}
+    for record in records:
+        data = np.fromfile(out / f"{record['step']}.f32", dtype="<f4").reshape(-1, vocab)
+        row = 0
+        for item in record["entries"]:
+            count = len(item["tokens"])
+            collected.setdefault(item["id"], []).append(torch.from_numpy(data[row:row + count].copy()))
+            row += count
+    for name in requests:
+        cases.assert_logits_close(torch.cat(collected[name]), case["expected"][name], dtype, "plain", f"request {name}")
+
+
 def test_recorded_decode_steps_of_many_requests(case):
     """More than 16 requests decode together: the products of such a step come from the BLAS library, also inside the
     recorded graph.  Every replay is checked against the plain implementation, with eager work between replays."""

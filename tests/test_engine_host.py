@@ -58,3 +58,37 @@ def test_branches_that_add_themselves_to_the_residual_sum_give_the_same_bits(cas
     assert calls["scaled"] == (2 * layers - 1) * small_steps      # every norm but the first, which meets no sums yet
     for name in want:
         assert (got[name] == want[name]).all(), name
+
+
+def test_replay_on_a_pool_of_its_own_page_size(case, tmp_path):
+    """The replay with the model's own page size (tiny-B: 8 tokens) and a pool given in pages, as `bin/trace_run
+    --page-size --num-pages --max-seqs` builds it: the mixed cutting, every position against the plain
+    implementation.  (On the host the torch double stands in for the kernels; the program itself runs on the GPU.)"""
+    import numpy as np
+    import torch
+    import schedules
+    from ampere_kv_engine_amd.engine.replay import build_engine, pool_pages, replay
+    page = case["page_size"]
+    assert pool_pages(192, 16) == 12 and pool_pages(192, 8) == 24 and pool_pages(65, 16) == 8
+    assert pool_pages(192, 24) == 9 and pool_pages(100, 256) == 1 and pool_pages(300, 128) == 3
+    requests = {k: case["requests"][k] for k in ("a", "b", "e", "f")}
+    pages = 192 // page
+    engine = build_engine(case["folder"], "float32", 192, page_size=page, num_pages=pages, max_seqs=4, device="cpu",
+                          kernels=TorchKernels())
+    assert engine.config.page_size == page and engine.config.num_pages == pages and engine.config.max_seqs == 4
+    records = schedules.to_trace(requests, schedules.mixed(requests, cases.PROMPTS, page, pages, seed=3))
+    import json
+    done = []
+    replay(engine, [json.dumps(r) for r in records], str(tmp_path), done.append)
+    assert done == [f"done {r['step']}" for r in records]
+    assert engine.cache.num_free_pages == [pages]
+    vocab = case["raw"]["vocab_size"]
+    collected = {}
+    for record in records:
+        data = np.fromfile(tmp_path / f"{record['step']}.f32", dtype="<f4").reshape(-1, vocab)
+        row = 0
+        for item in record["entries"]:
+            collected.setdefault(item["id"], []).append(torch.from_numpy(data[row:row + len(item["tokens"])].copy()))
+            row += len(item["tokens"])
+    for name in requests:
+        cases.assert_logits_close(torch.cat(collected[name]), case["expected"][name], "float32", "plain", name)
