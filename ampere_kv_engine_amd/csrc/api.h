@@ -57,5 +57,5 @@ int akv_linear_adds(const void* x, const void* wp, float* stream_out, float* sum
                     hipStream_t stream);
 int akv_linear_scaled(const float* stream_in, const float* sums, int sum_tiles, const float* gain, float eps,
                       const void* wp, void* y, float* pieces, unsigned int* arrivals, int exchange_tiles, int rows,
-                      int outs, int k, int n_tiles, int k_tiles, int gated, hipStream_t stream);
+                      int outs, int k, int n_tiles, int k_tiles, int gated, int row_tiles, hipStream_t stream);
 }

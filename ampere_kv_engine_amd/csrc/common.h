@@ -63,6 +63,37 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 
 enum DType : int { kF32 = 0, kBF16 = 1 };
 
+// Blocks of one launch that hand sums to each other through memory do it in three steps.  (1) The sums are written
+// with device-scope atomic stores (`publish`): such a store goes through to where every XCD sees it.  (2) The block
+// ticks a counter with `arrive`: first a wait until the wave's memory counters are at zero - every store it has
+// issued has been acknowledged -, then a device-scope read-modify-write; compiler-only fences on either side of both
+// keep the compiler from moving a store below the wait, the tick above it, or a later load above the tick (the wait
+// is an instruction, not a memory operation: by itself it orders nothing for the compiler).  (3) Whoever learns from
+// the counter that the others have been there reads their sums with device-scope atomic loads (`collect`), which do
+// not take a stale copy from a cache; they are issued after the tick has returned its value.  Nobody waits for
+// anybody.
+// Under the memory model alone the order would need the tick to be a release and an acquire at device scope, and
+// this device pays for those with a write-back of the XCD's L2 before the tick and its invalidation after (measured
+// with the tick written so: 28 -> 30 us and 43 -> 45 us for products of 128 rows whose k is cut over blocks, 20 ->
+// 27 us for a decode product whose row tiles straddle blocks) - although not one of the bytes concerned ever lies
+// in a cache that another XCD does not see.  What is relied on beyond the model is a fact of the hardware: a
+// device-scope store that has been acknowledged is seen by every later device-scope load or read-modify-write,
+// whichever XCD issues it.
+__device__ __forceinline__ void publish(float* at, float value) {
+  __hip_atomic_store(at, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float collect(const float* at) {
+  return __hip_atomic_load(at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ unsigned arrive(unsigned* counter) {
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
+  __builtin_amdgcn_s_waitcnt(0);       // every counter at zero: the wave's stores have arrived
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
+  const unsigned before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
+  return before;
+}
+
 }  // namespace akv
 
 // Expands `body` with `T` bound to the storage type named by `code`; unknown codes return -1.
@@ -80,3 +111,29 @@ enum DType : int { kF32 = 0, kBF16 = 1 };
   } while (0)
 
 #define AKV_LAUNCH_STATUS() static_cast<int>(hipGetLastError())
+
+namespace akv {
+
+// What the host needs to know of the device it launches on to cut work into blocks: asked of the runtime once per
+// device.  (The number of XCDs is not among a device's attributes: gfx950 parts have 8, each with an L2 of its own.)
+struct DeviceFacts {
+  int compute_units;
+  size_t lds_bytes;     // LDS of a compute unit: the most a block can ask for
+};
+constexpr int kXcds = 8;
+
+inline DeviceFacts device_facts() {
+  static DeviceFacts known[64] = {};
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return DeviceFacts{256, 160 * 1024};
+  if (known[device].compute_units == 0) {       // (two threads asking at once write the same values)
+    int units = 0, lds = 0;
+    if (hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || units <= 0) units = 256;
+    if (hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, device) != hipSuccess || lds <= 0)
+      lds = 160 * 1024;
+    known[device] = DeviceFacts{units, static_cast<size_t>(lds)};
+  }
+  return known[device];
+}
+
+}  // namespace akv

@@ -45,7 +45,6 @@ struct DecodeArgs {
 };
 
 constexpr int kGroup = 4;   // k-tiles per group of loads; two groups are in flight
-constexpr size_t kMaxLds = 160 * 1024;   // a compute unit's LDS: the most a block can have
 
 template <int RT, bool GATED, bool SCALED, bool ADDS>
 __global__ __launch_bounds__(768) void linear_decode_kernel(const DecodeArgs a) {
@@ -206,9 +205,9 @@ __global__ __launch_bounds__(768) void linear_decode_kernel(const DecodeArgs a) 
     // [lo, hi): every wave leaves its sums in LDS, the wave of unit lo adds them up.  Where the block holds the whole
     // wave-row that is the result.  Otherwise the wave-row's other parts lie in the neighbouring block (never in
     // more than two: a block has at least k_split waves): both leave their sums in `pieces` with device-scope
-    // stores - acknowledged when the wave's counters are back at zero - and tick `arrivals`; the second to arrive
-    // adds piece 0 + piece 1 (the same bits whichever it is), sets the counter back and goes on to the store.
-    // Nobody waits for anybody.
+    // stores and tick `arrivals` (a release and an acquire, see `arrive`); the second to arrive adds piece 0 +
+    // piece 1 (the same bits whichever it is), sets the counter back and goes on to the store.  Nobody waits for
+    // anybody.
     constexpr int kSet = RT * 4 * 64;
     if constexpr (SCALED) __syncthreads();   // the rows have been read: their memory takes the sums
     const int row_first = wave_row * a.k_split;
@@ -235,11 +234,10 @@ __global__ __launch_bounds__(768) void linear_decode_kernel(const DecodeArgs a) 
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          __hip_atomic_store(ours + (rt * 4 + i) * 64 + lane, acc[rt][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __builtin_amdgcn_s_waitcnt(0);   // every counter at zero: the stores above have arrived
+        for (int i = 0; i < 4; ++i) publish(ours + (rt * 4 + i) * 64 + lane, acc[rt][i]);
+      // the wave ticks as one: its lanes' stores precede the one read-modify-write, its lanes' loads follow it
       unsigned int before = 0;
-      if (lane == 0) before = __hip_atomic_fetch_add(a.arrivals + wave_row, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (lane == 0) before = arrive(a.arrivals + wave_row);
       before = __shfl(before, 0, kWave);
       if (before == 0u) return;        // the other block will finish this wave-row
       if (lane == 0) __hip_atomic_store(a.arrivals + wave_row, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
@@ -248,7 +246,7 @@ __global__ __launch_bounds__(768) void linear_decode_kernel(const DecodeArgs a) 
       for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float other = __hip_atomic_load(theirs + (rt * 4 + i) * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          const float other = collect(theirs + (rt * 4 + i) * 64 + lane);
           acc[rt][i] = piece == 0 ? acc[rt][i] + other : other + acc[rt][i];
         }
     }
@@ -320,7 +318,10 @@ DecodePlan plan_decode(int rt, int n_tiles, int k_tiles, int k, int normed_rows,
   // whole wave-rows: 320 wave-rows of 8 parts are 256 blocks of 10 waves, one and a quarter wave-rows each - the price
   // is the exchange of one wave-row's sums between two blocks, counted as 96 KB (measured: q/k/v of 6,144 x 4,096 gains
   // nothing from it, o of 5,120 x 8,192 goes from 26 to 20 us, down of 5,120 x 25,600 from 62 to 48).
-  constexpr int kUnits = 256, kMostWaves = 12;
+  constexpr int kMostWaves = 12;
+  const DeviceFacts device = device_facts();
+  const int kUnits = device.compute_units;
+  const size_t kMaxLds = device.lds_bytes;
   const size_t rows_bytes = normed_rows ? static_cast<size_t>(normed_rows) * k * 2 + (12 * 16 + 16) * 4 : 0;
   const double unit_bytes = static_cast<double>(rt) * ((k_tiles + k_split - 1) / k_split) * 1024;
   const double norm_bytes = 1.5 * normed_rows * k * 2, exchange_bytes = 96.0 * 1024;
@@ -352,6 +353,7 @@ int launch_decode(DecodeArgs a, hipStream_t stream) {
   a.k_split = k_split;
   a.red_floats = k_split > 1 ? waves * RT * 4 * 64 : 0;
   const size_t lds = max(static_cast<size_t>(a.red_floats) * 4, SCALED ? (12 * 16 + 16) * 4 + static_cast<size_t>(a.rows) * a.k * 2 : 0);
+  const size_t kMaxLds = device_facts().lds_bytes;
   if (lds > kMaxLds) return -2;
   if (lds > 64 * 1024) {   // more than a block may have without asking: asked once per kernel and device
     static std::mutex guard;
@@ -375,14 +377,15 @@ int launch_decode(DecodeArgs a, hipStream_t stream) {
 // stream_out [rows, outs] += bfloat16(x W^T) in place (float32); sums_out [n_tiles][16] receives, for every row tile of
 // 16 outputs and every row, the sum of squares of the new values (rows beyond `rows`: 0).  rows <= 16, k % 8 == 0.
 // `pieces` (exchange_tiles * 512 floats) and `arrivals` (exchange_tiles words, zero; left zero) may be null, or hold
-// fewer than n_tiles row tiles' worth, and are then not used: with them the product
+// fewer than n_tiles + 1 row tiles' worth (a wave's pair of row tiles may begin at the last tile), and are then not used: with them the product
 // may be cut into blocks that do not hold whole row tiles' parts of k (see plan_decode).  Launches that share them
 // follow each other on one stream.
-// What plan_decode makes of a product (for tests and measurements): out[0..3] = parts of k, waves per block, blocks,
-// whether row tiles may have their parts of k in two blocks.
+// What plan_decode makes of a product (for tests and measurements): out[0..4] = parts of k, waves per block, blocks,
+// whether row tiles may have their parts of k in two blocks, the busiest compute unit's work in KB.
 extern "C" int akv_linear_decode_plan(int rt, int n_tiles, int k_tiles, int k, int normed_rows, int may_straddle, int* out) {
   const DecodePlan plan = plan_decode(rt, n_tiles, k_tiles, k, normed_rows, may_straddle != 0);
   out[0] = plan.k_split, out[1] = plan.waves, out[2] = plan.blocks, out[3] = plan.straddles ? 1 : 0;
+  out[4] = static_cast<int>(plan.work / 1024.0);
   return 0;
 }
 
@@ -396,7 +399,7 @@ extern "C" int akv_linear_adds(const void* x, const void* wp, float* stream_out,
   a.wp = static_cast<const uintx4*>(wp);
   a.stream_out = stream_out;
   a.sums_out = sums_out;
-  if (pieces != nullptr && arrivals != nullptr && exchange_tiles >= n_tiles) a.pieces = pieces, a.arrivals = arrivals;
+  if (pieces != nullptr && arrivals != nullptr && exchange_tiles >= n_tiles + 1) a.pieces = pieces, a.arrivals = arrivals;
   a.rows = rows, a.outs = outs, a.k = k, a.k_tiles = k_tiles, a.n_tiles = n_tiles;
   return launch_decode<1, false, false, true>(a, stream);
 }
@@ -406,12 +409,15 @@ extern "C" int akv_linear_adds(const void* x, const void* wp, float* stream_out,
 // and the weight `gain` [k] - with the rows' sums of squares not formed here but taken from `sums`
 // [sum_tiles][16] (what akv_linear_adds left: sum_tiles = ceil(k / 16)).  rows <= 16, k % 8 == 0, and the normed rows
 // (rows * k bfloat16) fit into a compute unit's LDS (160 KB) beside 832 bytes; -2 otherwise.  `pieces`, `arrivals`: as
-// for akv_linear_adds.
+// for akv_linear_adds.  `row_tiles`: row tiles per wave of the plain product, 1 or 2; 0 leaves the choice to the sizes (a
+// gated product's waves always take a pair).
 extern "C" int akv_linear_scaled(const float* stream_in, const float* sums, int sum_tiles, const float* gain, float eps,
                                  const void* wp, void* y, float* pieces, unsigned int* arrivals, int exchange_tiles,
-                                 int rows, int outs, int k, int n_tiles, int k_tiles, int gated, hipStream_t stream) {
+                                 int rows, int outs, int k, int n_tiles, int k_tiles, int gated, int row_tiles,
+                                 hipStream_t stream) {
   if (rows <= 0 || outs <= 0) return 0;
   if (rows > 16 || (k & 7) != 0 || k_tiles * 32 < k || sum_tiles != (k + 15) / 16) return -2;
+  if (row_tiles < 0 || row_tiles > 2 || (gated && row_tiles == 1)) return -2;
   if (gated ? ((outs & 15) != 0 || n_tiles * 8 != outs) : n_tiles * 16 < outs) return -2;
   DecodeArgs a{};
   a.stream = stream_in;
@@ -421,7 +427,7 @@ extern "C" int akv_linear_scaled(const float* stream_in, const float* sums, int 
   a.eps = eps;
   a.wp = static_cast<const uintx4*>(wp);
   a.y = static_cast<bf16_t*>(y);
-  if (pieces != nullptr && arrivals != nullptr && exchange_tiles >= n_tiles) a.pieces = pieces, a.arrivals = arrivals;
+  if (pieces != nullptr && arrivals != nullptr && exchange_tiles >= n_tiles + 1) a.pieces = pieces, a.arrivals = arrivals;
   const bool may = a.pieces != nullptr;
   a.rows = rows, a.outs = outs, a.k = k, a.k_tiles = k_tiles, a.n_tiles = n_tiles;
   if (gated) return launch_decode<2, true, true, false>(a, stream);
@@ -429,7 +435,8 @@ extern "C" int akv_linear_scaled(const float* stream_in, const float* sums, int 
   // wave where one is faster (q/k/v at 4 rows: 19.4 -> 16.3 us, at 8: 20.3 -> 19.4; counted as 1.3 times the bytes, which puts the rule where the measurements are).
   // They pay where the normed rows fill so much LDS that a compute unit holds one block, and the blocks of one row tile
   // per wave would need a second round (16 rows of 4,096: 28.8 -> 23.0 us).
-  if (n_tiles >= 2 && plan_decode(2, n_tiles, k_tiles, k, rows, may).work * 1.3 < plan_decode(1, n_tiles, k_tiles, k, rows, may).work)
-    return launch_decode<2, false, true, false>(a, stream);
+  if (row_tiles == 0)
+    row_tiles = n_tiles >= 2 && plan_decode(2, n_tiles, k_tiles, k, rows, may).work * 1.3 < plan_decode(1, n_tiles, k_tiles, k, rows, may).work ? 2 : 1;
+  if (row_tiles == 2) return launch_decode<2, false, true, false>(a, stream);
   return launch_decode<1, false, true, false>(a, stream);
 }

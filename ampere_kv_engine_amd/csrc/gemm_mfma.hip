@@ -382,7 +382,7 @@ int dispatch_skinny(const void* x, const void* wp, void* y, int rows, int outs, 
 // bank conflicts.  Weights come from the packed layout straight into A operands, one k-tile ahead of their use.
 // Blocks are numbered so that the blocks sharing a band of 128 weight rows run on the same XCD (one L2 each: the
 // band is fetched from memory once), while XCDs work on different bands.
-constexpr int kWideN = 128, kWideK = 64, kXcds = 8;
+constexpr int kWideN = 128, kWideK = 64;
 
 // MW: token tiles per wave (8: 256 tokens per block; 4: 128 tokens per block, for products with few weight rows,
 // which would otherwise leave compute units without a block).

@@ -33,9 +33,7 @@ using namespace akv;
 namespace {
 
 constexpr int kHalves = 2;   // waves along k (A waves along the band of row tiles: 2, 3 or 4)
-constexpr int kXcds = 8;
 constexpr int kFetchers = 4;
-constexpr int kComputeUnits = 256;
 
 template <int MT> constexpr int kStage = MT <= 4 ? 4 : 2;     // k-tiles per stage and k half
 
@@ -56,8 +54,7 @@ __global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_ker
   constexpr int kLoads = kTiles / kFetchers;      // of which every fetching wave brings this many
   static_assert(kTiles % kFetchers == 0, "the stage's tiles are dealt to the fetching waves");
   static_assert(G % 2 == 0, "a ring position must always meet the same staging buffer");
-  extern __shared__ uintx4 staged[];              // [2][kTiles][64]; afterwards the sums of the second k half
-  __shared__ unsigned is_last;
+  extern __shared__ uintx4 staged[];              // [2][kTiles][64]; afterwards the sums of the second k half, then a flag
 
   // which work: blocks that share weights (same band and part of k, other rows) are neighbours on one XCD
   const int xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
@@ -210,9 +207,8 @@ __global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_ker
     // adds the parts in the order of their k ranges (whichever block that is, the bits are the same) and stores.
     const size_t block_floats = static_cast<size_t>(kAlong) * RT * MT * 256;
     float* band_parts = partial + (static_cast<size_t>(m_block) * bands + band) * parts * block_floats;
-    // No cache-wide write-back or invalidation is paid for this (a release and an acquire at device scope cost several
-    // microseconds per block here): the parts are stored and loaded with device scope themselves - such accesses go
-    // through to where all XCDs see them - and a wave's stores have been acknowledged when its vmcnt is back at zero.
+    // The parts are stored and loaded with device scope themselves - such accesses go through to where all XCDs see
+    // them -; the counter's tick is the release and the acquire that orders them (see `arrive` in common.h).
     if (half == 0) {
       float* mine = band_parts + part * block_floats + static_cast<size_t>(along) * RT * MT * 256;
 #pragma unroll
@@ -220,21 +216,17 @@ __global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_ker
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
-            __hip_atomic_store(mine + ((rt * MT + mt) * 4 + i) * 64 + lane, acc[rt][mt][i], __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
-      __builtin_amdgcn_s_waitcnt(0);   // every counter at zero: the stores above have arrived
+          for (int i = 0; i < 4; ++i) publish(mine + ((rt * MT + mt) * 4 + i) * 64 + lane, acc[rt][mt][i]);
     }
-    __syncthreads();                   // (the fetching waves have gone; all multiplying waves' stores have arrived)
+    __syncthreads();                   // (the fetching waves have gone; all multiplying waves have stored)
     if (threadIdx.x == 0) {
       unsigned* counter = counters + m_block * bands + band;
-      const unsigned before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const bool last = before == static_cast<unsigned>(parts - 1);
+      const bool last = arrive(counter) == static_cast<unsigned>(parts - 1);
       if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next launch
-      is_last = last ? 1u : 0u;
+      *reinterpret_cast<volatile unsigned*>(staged) = last ? 1u : 0u;   // (the sums that lay here have been read)
     }
     __syncthreads();
-    if (is_last == 0u) return;
+    if (*reinterpret_cast<volatile unsigned*>(staged) == 0u) return;
     if (half == 0) {
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt)
@@ -247,9 +239,7 @@ __global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_ker
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-              acc[rt][mt][i] += __hip_atomic_load(theirs + ((rt * MT + mt) * 4 + i) * 64 + lane, __ATOMIC_RELAXED,
-                                                  __HIP_MEMORY_SCOPE_AGENT);
+            for (int i = 0; i < 4; ++i) acc[rt][mt][i] += collect(theirs + ((rt * MT + mt) * 4 + i) * 64 + lane);
       }
     }
   }
@@ -288,6 +278,7 @@ constexpr size_t kMostPartialFloats = 8u << 20;   // 32 MB: more than that is no
 MidPlan plan_mid(int rows, int n_tiles, int k_tiles, bool gated, int along, int rt, int depth, int parts) {
   MidPlan best{};
   double best_cost = -1.0;
+  const int kComputeUnits = device_facts().compute_units;
   // tiles of 16 rows: up to eight a block, dealt evenly to the blocks (132 rows are two blocks of five tiles, not
   // one of eight and one that multiplies zeros)
   const int row_tiles = (rows + 15) / 16;

@@ -479,8 +479,10 @@ class HipKernels:
 
     def _reserve_exchange(self, n_tiles: int) -> None:
         """Called when a matrix is prepared: the memory through which two blocks of a decode product exchange the sums
-        of a row tile whose parts of k they share (512 floats and a counter per row tile; the counters are zero between
-        launches).  One pair of buffers for all products - they follow each other on the stream."""
+        of a row tile whose parts of k they share (512 floats and a counter per row tile, and one tile more: a wave's
+        pair of row tiles may begin at the last one; the counters are zero between launches).  One pair of buffers for
+        all products - they follow each other on the stream."""
+        n_tiles += 1
         if self._exchange_tiles < n_tiles:
             self._exchange_tiles = max(n_tiles, 4096)
             self._outgrown += [self._exchange_pieces, self._exchange_arrivals]
@@ -491,17 +493,17 @@ class HipKernels:
         """The exchange buffers if they serve a matrix of `n_tiles` row tiles (they do for every prepared matrix; they
         are never replaced inside a step, whose recording may hold their addresses) - else the product keeps whole
         row tiles in a block."""
-        if self._exchange_tiles < n_tiles:
+        if self._exchange_tiles < n_tiles + 1:
             return None, None
         return self._exchange_pieces, self._exchange_arrivals
 
     def decode_plan(self, weight, row_tiles_per_wave: int = 1, normed_rows: int = 0) -> dict:
         """How `linear_adds` / `linear_scaled` cut a product over this matrix into blocks (for tests and measurements)."""
         packed = weight.packed if isinstance(weight, GatedWeight) else weight
-        out = (ctypes.c_int * 4)()
+        out = (ctypes.c_int * 5)()
         may = 1 if self._exchange(packed.n_tiles)[0] is not None else 0
         self.lib.akv_linear_decode_plan(row_tiles_per_wave, packed.n_tiles, packed.k_tiles, packed.k, normed_rows, may, out)
-        return dict(k_split=out[0], waves=out[1], blocks=out[2], straddles=bool(out[3]))
+        return dict(k_split=out[0], waves=out[1], blocks=out[2], straddles=bool(out[3]), work_kb=out[4])
 
     def adds_to_stream(self, rows: int, weight, dtype) -> bool:
         return isinstance(weight, PackedWeight) and self.folds_norm(rows, weight.outs, dtype)
@@ -526,10 +528,11 @@ class HipKernels:
                                              rows, weight.outs, weight.k, weight.n_tiles,
                                              weight.k_tiles, self._stream()), "linear_adds")
 
-    def linear_scaled(self, stream, sums, norm_weight, eps, weight, out) -> None:
+    def linear_scaled(self, stream, sums, norm_weight, eps, weight, out, row_tiles: int = 0) -> None:
         """out = norm(stream) W^T (a `GatedWeight`: silu(. Wgate^T) * (. Wup^T)) with the norm of `add_rmsnorm`
         (scaled, rounded, times the weight, rounded) applied to the float32 rows as they become operands; the rows'
-        sums of squares are not formed but added up from `sums`, as `linear_adds` left them."""
+        sums of squares are not formed but added up from `sums`, as `linear_adds` left them.  `row_tiles` forces the
+        row tiles a wave of the plain product takes (1 or 2; for tests and measurements)."""
         gated = isinstance(weight, GatedWeight)
         packed = weight.packed if gated else weight
         rows, k = stream.shape
@@ -546,7 +549,7 @@ class HipKernels:
                                                ctypes.c_float(eps), _ptr(packed.data), _ptr(out), _ptr(pieces),
                                                _ptr(arrivals), self._exchange_tiles if pieces is not None else 0,
                                                rows, outs, k, packed.n_tiles, packed.k_tiles,
-                                               1 if gated else 0, self._stream()), "linear_scaled")
+                                               1 if gated else 0, row_tiles, self._stream()), "linear_scaled")
 
     STATIC_ROWS_ELEMENTS = 64 * 32768   # bfloat16 elements of the library's static device memory for repacked rows
 

@@ -377,7 +377,7 @@ def test_a_gated_product_norms_its_rows_from_the_sums_of_squares(hip, ref, rows,
     assert_close_but_for_flipped_roundings(got, want)
 
 
-@pytest.mark.parametrize("rows", [1, 8])
+@pytest.mark.parametrize("rows", [1, 8, 16])
 @pytest.mark.parametrize("outs,k", [(5120, 8192), (5120, 5120), (5136, 8200), (5120, 17416)])
 def test_row_tiles_whose_parts_of_k_lie_in_two_blocks(hip, ref, rows, outs, k, monkeypatch):
     """The decode products cut their work into equal blocks even where that splits a row tile's parts of k between two
@@ -428,6 +428,100 @@ def test_row_tiles_whose_parts_of_k_lie_in_two_blocks(hip, ref, rows, outs, k, m
         ref.add_rmsnorm(first[0].clone(), None, gain, 1e-6, normed)
         ref.linear(normed, back.unpack().cpu(), want_back)
         assert_close_but_for_flipped_roundings(got, want_back)
+
+
+@pytest.mark.parametrize("rows", [3, 16])
+@pytest.mark.parametrize("outs", [8208, 10256, 10272])      # 513, 641 and 642 row tiles: odd and even numbers of them
+def test_pairs_of_row_tiles_whose_parts_of_k_lie_in_two_blocks(hip, ref, rows, outs, monkeypatch):
+    """The product that norms its rows, with two row tiles a wave (forced: the sizes alone never choose it where
+    blocks share wave-rows) and so many row tiles that the blocks do not hold whole wave-rows: the exchange memory is
+    indexed by wave-row and holds two tiles for each - with an odd number of row tiles the last wave-row reaches one
+    tile beyond the matrix.  Against one row tile a wave (same sums, other order) and the double; twice, for the
+    counters; and nothing beyond the exchange memory's own end is touched."""
+    monkeypatch.setattr(hip, "fold_norms", True)
+    monkeypatch.setattr(hip, "FOLD_NORM_ROWS", 16)
+    k = 2048
+    w = rand(outs, k, dtype=torch.bfloat16, seed=61, scale=0.05)
+    packed = hip.prepare_linear(w.cuda())
+    plan = hip.decode_plan(packed, row_tiles_per_wave=2, normed_rows=rows)
+    assert plan["straddles"], plan
+    assert hip._exchange_tiles >= packed.n_tiles + 1
+    stream = rand(rows, k, seed=62, scale=2.0)
+    gain = 1 + rand(k, seed=63, scale=0.1)
+    sums = torch.zeros((k + 15) // 16, 16)
+    sums[:, :rows] = (stream * stream).view(rows, -1, 16).sum(-1).T
+    normed, want = torch.empty(rows, k, dtype=torch.bfloat16), torch.empty(rows, outs, dtype=torch.bfloat16)
+    ref.add_rmsnorm(stream.clone(), None, gain, 1e-6, normed)
+    ref.linear(normed, w, want)
+    guard = hip._exchange_pieces[(packed.n_tiles + 1) * 512:(packed.n_tiles + 1) * 512 + 4096]
+    guard.fill_(-77.0)
+
+    def scaled(row_tiles):
+        got = torch.full((rows, outs), float("nan"), dtype=torch.bfloat16, device="cuda")
+        hip.linear_scaled(stream.cuda(), sums.cuda(), gain.cuda(), 1e-6, packed, got, row_tiles=row_tiles)
+        return got.cpu()
+
+    pairs = scaled(2)
+    assert torch.equal(pairs, scaled(2)) and int(hip._exchange_arrivals.abs().sum()) == 0
+    assert bool((guard == -77.0).all()), "the exchange wrote beyond the tiles it was given"
+    assert_close_but_for_flipped_roundings(pairs, want)
+    assert_close_but_for_flipped_roundings(pairs, scaled(1))
+
+
+def test_exchanging_products_give_the_same_bits_two_hundred_times(hip, hip_own, monkeypatch):
+    """Products whose blocks hand sums to each other through memory (decode products whose row tiles straddle blocks;
+    mid-size products whose k is cut over blocks) are called 200 times back to back, each call on a copy of the matrix
+    that no cache holds, with other kernels' reads in between: every result equals the first bit for bit (the parts are
+    added in a fixed order whoever arrives last), and the counters are back at zero.  Stops at the first mismatch."""
+    monkeypatch.setattr(hip, "fold_norms", True)
+    monkeypatch.setattr(hip, "FOLD_NORM_ROWS", 16)
+    spacer = torch.zeros(96 << 20, dtype=torch.float32, device="cuda")       # 384 MB: more than the caches hold
+    cases = []
+    # decode: o and down at sizes whose 320 row tiles meet 256 compute units; the product that norms its rows likewise
+    for rows, outs, k in ((8, 5120, 8192), (16, 5120, 5120), (1, 5120, 17416)):
+        x = rand(rows, k, dtype=torch.bfloat16, seed=71).cuda()
+        copies = [hip.prepare_linear(rand(outs, k, dtype=torch.bfloat16, seed=72, scale=0.05).cuda()) for _ in range(3)]
+        assert hip.decode_plan(copies[0])["straddles"]
+        base = rand(rows, outs, seed=73, scale=2.0).cuda()
+
+        def adds(i, x=x, copies=copies, base=base, rows=rows, outs=outs):
+            stream, sums = base.clone(), torch.empty((outs + 15) // 16, 16, device="cuda")
+            hip.linear_adds(x, copies[i % 3], stream, sums)
+            return torch.cat((stream.view(-1), sums.view(-1)))
+        cases.append((f"adds {rows} x {outs} x {k}", adds))
+        if rows * outs * 2 <= hip.FOLD_NORM_BYTES:
+            back = [hip.prepare_linear(rand(5120, outs, dtype=torch.bfloat16, seed=74, scale=0.05).cuda()) for _ in range(3)]
+            sums = torch.rand((outs + 15) // 16, 16, device="cuda")
+            gain = (1 + rand(outs, seed=75, scale=0.1)).cuda()
+
+            def scaled(i, base=base, sums=sums, gain=gain, back=back, rows=rows):
+                out = torch.empty(rows, 5120, dtype=torch.bfloat16, device="cuda")
+                hip.linear_scaled(base, sums, gain, 1e-6, back[i % 3], out)
+                return out.view(-1).float()
+            cases.append((f"scaled {rows} x 5120 x {outs}", scaled))
+    # mid-size: the four products of a layer at 128 and 40 rows (their cuts divide k over blocks)
+    import ctypes
+    for rows in (128, 40):
+        for outs, k in ((6144, 4096), (4096, 4096), (4096, 12288)):
+            x = rand(rows, k, dtype=torch.bfloat16, seed=76).cuda()
+            copies = [hip_own.prepare_linear(rand(outs, k, dtype=torch.bfloat16, seed=77, scale=0.05).cuda()) for _ in range(3)]
+            need, words = ctypes.c_long(0), ctypes.c_long(0)
+            hip_own.lib.akv_linear_mid_workspace(rows, copies[0].n_tiles, copies[0].k_tiles, 0, 0, 0, 0, 0, ctypes.byref(need), ctypes.byref(words))
+            assert need.value > 0, "this product's k is not cut over blocks"
+
+            def mid(i, x=x, copies=copies, rows=rows, outs=outs):
+                out = torch.empty(rows, outs, dtype=torch.float32, device="cuda")
+                hip_own._mid(x, copies[i % 3], out, rows, outs, False)
+                return out.view(-1)
+            cases.append((f"mid {rows} x {outs} x {k}", mid))
+    for name, call in cases:
+        first = call(0).clone()
+        for turn in range(1, 201):      # (the copies hold the same values: every call must equal the first)
+            if turn % 2:
+                spacer.sum()            # other work between the calls, and the caches emptied
+            got = call(turn)
+            assert torch.equal(got, first), f"{name}: call {turn} differs from the first in {int((got != first).sum())} values"
+    assert int(hip._exchange_arrivals.abs().sum()) == 0 and int(hip_own._mid_counters.abs().sum()) == 0
 
 
 def test_decode_products_at_random_sizes(hip, ref, monkeypatch):
