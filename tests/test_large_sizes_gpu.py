@@ -120,7 +120,8 @@ def test_many_requests_decode_together_at_qwen3_8b_layer_sizes(two_layers, dtype
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_seventy_requests_through_the_scheduler_at_qwen3_8b_layer_sizes(two_layers, dtype):
     """More live requests than one launch of the decode attention takes (64): the scheduler decodes 70 together.
-    Every chosen token must be the plain implementation's best at its place, or within the arithmetic's reach of it."""
+    float32: every request generates the plain implementation's greedy tokens.  bfloat16: every chosen token must be
+    the plain implementation's best at its place, or within the arithmetic's reach of it."""
     import engine_cases as cases
     from ampere_kv_engine_amd.engine.scheduler import Scheduler
     folder, plain = two_layers
@@ -137,6 +138,9 @@ def test_seventy_requests_through_the_scheduler_at_qwen3_8b_layer_sizes(two_laye
     limit = cases.LIMITS[dtype, "plain"]["max"]
     for request, prompt in zip(requests, prompts):
         assert len(request.output_ids) == new and request.stop_reason == "reached limit"
+        if dtype == "float32":          # a row's arithmetic does not depend on its batch: the plain implementation's tokens
+            assert request.output_ids == plain.greedy(prompt, new), request.request_id
+            continue
         logits = plain.logits(prompt + request.output_ids[:-1])[len(prompt) - 1:]
         top = cases.scales(logits)[0]
         for place, token in enumerate(request.output_ids):

@@ -340,47 +340,26 @@ def test_random_workloads_with_and_without_overlapped_decoding(name, model_folde
     id some of them meet, portion sizes, pool sizes): whatever the rounds look like, a request that is not cancelled
     generates what it generates alone, a cancelled one a beginning of that, and pages, slots and reservations all
     come back."""
-    import random
+    import workloads
     raw, _, page = TINY[name]
     folder = model_folders[name]
     known = {}
     for trial in range(5):
-        rng = random.Random(trial * 31 + ord(name))
-        specs = [(random_ids(raw["vocab_size"], rng.randint(1, 40), seed=trial * 100 + i), rng.randint(1, 12),
-                  *rng.choice([(0.0, 0), (0.5, rng.randint(0, 99)), (1.0, rng.randint(0, 99))])) for i in range(rng.randint(1, 6))]
+        work = workloads.random_workload(raw["vocab_size"], trial, ord(name))
         want = []
-        for prompt, new, temperature, seed in specs:
+        for prompt, new, temperature, seed in work.specs:
             key = (tuple(prompt), new, temperature, seed)
             if key not in known:
                 known[key] = alone(folder, page, prompt, new, temperature=temperature, seed=seed)
             want.append(known[key])
-        pick = rng.choice(want)
-        eos = pick[len(pick) // 2] if rng.random() < 0.6 else None
-        num_pages = rng.randint(8, 40)
+        eos = want[work.eos_from[0]][work.eos_from[1]] if work.eos_from is not None else None
         for overlap in (False, True):
-            engine = make_engine(folder, page, num_pages=num_pages)
+            engine = make_engine(folder, page, num_pages=work.num_pages)
             if eos is not None:
-                engine.spec = type(engine.spec)(**{**engine.spec.__dict__, "eos_token_ids": (eos,)})
-            plan = random.Random(trial)
-            scheduler = Scheduler(engine, prefill_chunk_size=plan.choice([0, 5, 16]), overlap_decoding=overlap)
-            arrive = [plan.randint(0, 6) for _ in specs]
-            cancel_at = {i: plan.randint(1, 12) for i in range(len(specs)) if plan.random() < 0.2}
-            submitted = {}
-            for round_number in range(400):
-                for i, (prompt, new, temperature, seed) in enumerate(specs):
-                    if arrive[i] == round_number:
-                        try:
-                            submitted[i] = scheduler.submit(f"r{i}", prompt, new, temperature=temperature, seed=seed)
-                        except ValueError:
-                            submitted[i] = None               # it does not fit the pool at all: refused at once
-                for i, request in submitted.items():
-                    if request is not None and cancel_at.get(i) == round_number:
-                        scheduler.cancel(request)
-                if scheduler.idle and len(submitted) == len(specs):
-                    break
-                scheduler.step()
-            assert scheduler.idle and len(submitted) == len(specs), (trial, overlap)
-            assert engine.cache.num_free_pages == [num_pages] and engine.cache.slots.num_free == 4
+                workloads.with_eos(engine, eos)
+            scheduler = Scheduler(engine, prefill_chunk_size=work.chunk, overlap_decoding=overlap)
+            submitted = workloads.drive(scheduler, work)
+            assert engine.cache.num_free_pages == [work.num_pages] and engine.cache.slots.num_free == 4
             assert scheduler.reserved_pages == [0]
             for i, request in submitted.items():
                 if request is None:
@@ -391,7 +370,6 @@ def test_random_workloads_with_and_without_overlapped_decoding(name, model_folde
                 else:
                     cut = want[i].index(eos) + 1 if eos in want[i] else len(want[i])
                     assert request.output_ids == want[i][:cut], (trial, overlap, i, request.stop_reason)
-
 
 def test_decoding_overlaps_while_the_queue_is_blocked(model_folders):
     """A pool so small that the second and third request wait until the one before has retired: while the head of
