@@ -29,11 +29,20 @@ class EngineConfig:
     # are timed once, when the weights have been loaded (never inside a step), each decision is logged and the table
     # can be saved (`engine.kernels.save_product_choices(path)`).  Anything else: the path of such a saved table.
     product_choices: str = "fixed"
+    # Recorded steps (`decode_graphs`).  Steps with prompt portions are recorded up to `record_max_tokens` tokens:
+    # beyond that the device works longer on a step than the host needs to launch it.  A recording is made for block
+    # tables of a multiple of `graph_width_multiple` pages (a bound on the longest request's pages that sizes the
+    # launches: one recording serves every length under it).  Shapes met after `max_recordings` are run as they are
+    # (decode steps are always recorded).
+    record_max_tokens: int = 512
+    graph_width_multiple: int = 64
+    max_recordings: int = 512
 
     def __post_init__(self):
         if self.dtype not in DTYPES:
             raise ValueError(f"dtype must be one of {DTYPES}, got {self.dtype!r}")
-        for name in ("page_size", "num_pages", "max_seqs", "max_batched_tokens", "max_seq_len"):
+        for name in ("page_size", "num_pages", "max_seqs", "max_batched_tokens", "max_seq_len", "record_max_tokens",
+                     "graph_width_multiple", "max_recordings"):
             value = getattr(self, name)
             if not isinstance(value, int) or value <= 0:
                 raise ValueError(f"{name} must be a positive integer, got {value!r}")

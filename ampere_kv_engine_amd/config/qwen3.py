@@ -34,6 +34,7 @@ class Qwen3Config:
     rope_theta: float
     rms_norm_eps: float
     tie_word_embeddings: bool
+    attention_bias: bool
     max_position_embeddings: int | None
     eos_token_ids: tuple[int, ...]
 
@@ -77,8 +78,9 @@ class Qwen3Config:
                               "in every layer")
         if raw.get("rope_scaling") is not None:
             raise ConfigError("rope_scaling is set: only the unscaled rotary encoding is supported")
-        if raw.get("attention_bias", False):
-            raise ConfigError("attention_bias is set: projections with bias are not supported")
+        attention_bias = raw.get("attention_bias", False)
+        if not isinstance(attention_bias, bool):
+            raise ConfigError(f"attention_bias must be true or false, got {attention_bias!r}")
         if heads % kv_heads:
             raise ConfigError(f"num_attention_heads {heads} is not a multiple of num_key_value_heads {kv_heads}")
         if head_dim % 2:
@@ -103,6 +105,7 @@ class Qwen3Config:
             num_key_value_heads=kv_heads, head_dim=head_dim,
             intermediate_size=_positive_int(raw, "intermediate_size"), rope_theta=float(theta),
             rms_norm_eps=float(eps), tie_word_embeddings=bool(raw.get("tie_word_embeddings", False)),
+            attention_bias=attention_bias,
             max_position_embeddings=int(max_pos) if max_pos is not None else None, eos_token_ids=eos_ids,
         )
 
@@ -125,7 +128,7 @@ class Qwen3Config:
             "num_attention_heads": self.num_attention_heads, "num_key_value_heads": self.num_key_value_heads,
             "head_dim": self.head_dim, "intermediate_size": self.intermediate_size, "hidden_act": "silu",
             "rope_theta": self.rope_theta, "rope_scaling": None, "rms_norm_eps": self.rms_norm_eps,
-            "attention_bias": False, "use_sliding_window": False, "sliding_window": None,
+            "attention_bias": self.attention_bias, "use_sliding_window": False, "sliding_window": None,
             "tie_word_embeddings": self.tie_word_embeddings, "torch_dtype": "bfloat16",
         }
         if self.max_position_embeddings is not None:
@@ -137,7 +140,8 @@ class Qwen3Config:
     # ---- the model this configuration describes ---------------------------------------------------
     def to_model_spec(self) -> ModelSpec:
         """Every layer: pre-norm block, grouped-query attention with per-head q/k RMSNorm and half-split
-        rotary encoding, dense SwiGLU feed-forward (ampere_kv/runner.py:101-179)."""
+        rotary encoding (its four projections with biases if `attention_bias`), dense SwiGLU feed-forward
+        (ampere_kv/runner.py:101-179)."""
         norm = lambda size: part("rmsnorm", size=size, eps=self.rms_norm_eps)
         layers = []
         for index in range(self.num_hidden_layers):
@@ -148,7 +152,7 @@ class Qwen3Config:
                            kv_heads=self.num_key_value_heads, head_dim=self.head_dim, window=None,
                            qk_norm=norm(self.head_dim),
                            position=part("rope_half", head_dim=self.head_dim, theta=self.rope_theta),
-                           scale=self.head_dim ** -0.5, name="self_attn"),
+                           scale=self.head_dim ** -0.5, name="self_attn", bias=self.attention_bias),
                 feed_forward=part("swiglu", hidden_size=self.hidden_size,
                                   intermediate_size=self.intermediate_size, name="mlp"),
                 prefix=f"model.layers.{index}.",

@@ -33,15 +33,16 @@ int akv_qk_norm_rope_write(const void* qkv, const float* q_weight, const float* 
                            const float* table, int table_positions, const int* positions, const int* slot_map,
                            void* k_pages, void* v_pages, void* q_out, int dtype, long tokens, int q_heads,
                            int kv_heads, int dim, int page_size, long num_pages, hipStream_t stream);
+// Products y = x W^T (+ bias): `bias` [outs] float32 or null, added to the float32 sums before they are rounded.
 int akv_linear_tiled(const void* x, int x_dtype, const void* w, int w_dtype, void* y, int y_dtype, int rows, int outs,
-                     int k, hipStream_t stream);
+                     int k, const float* bias, hipStream_t stream);
 int akv_linear_packed(const void* x, const void* wp, void* y, int y_dtype, int rows, int outs, int k, int n_tiles,
-                      int k_tiles, int x_packed, hipStream_t stream);
+                      int k_tiles, int x_packed, const float* bias, hipStream_t stream);
 int akv_linear_packed_swiglu(const void* x, const void* wp, void* y, int y_dtype, int rows, int inter, int k,
                              int n_tiles, int k_tiles, int x_packed, hipStream_t stream);
 int akv_linear_packed_normed(const float* stream_in, const void* delta, const float* norm_weight, float eps,
                              float* stream_out, const void* wp, void* y, int rows, int outs, int k, int n_tiles,
-                             int k_tiles, int gated, hipStream_t stream);
+                             int k_tiles, int gated, const float* bias, hipStream_t stream);
 int akv_pack_rows(const void* x, void* xp, int rows, int k, hipStream_t stream);
 // No counterpart in the reference.  For callers that cannot allocate device memory (code under HIP graph capture,
 // tight serving loops, harnesses that forbid hipMalloc): akv_pack_rows + akv_linear_packed(x_packed = 1) as one call
@@ -54,8 +55,9 @@ int akv_linear_packed_static(const void* x, const void* wp, void* y, int y_dtype
 int akv_linear_decode_plan(int rt, int n_tiles, int k_tiles, int k, int normed_rows, int may_straddle, int* out);
 int akv_linear_adds(const void* x, const void* wp, float* stream_out, float* sums_out, float* pieces,
                     unsigned int* arrivals, int exchange_tiles, int rows, int outs, int k, int n_tiles, int k_tiles,
-                    hipStream_t stream);
+                    const float* bias, hipStream_t stream);
 int akv_linear_scaled(const float* stream_in, const float* sums, int sum_tiles, const float* gain, float eps,
                       const void* wp, void* y, float* pieces, unsigned int* arrivals, int exchange_tiles, int rows,
-                      int outs, int k, int n_tiles, int k_tiles, int gated, int row_tiles, hipStream_t stream);
+                      int outs, int k, int n_tiles, int k_tiles, int gated, int row_tiles, const float* bias,
+                      hipStream_t stream);
 }

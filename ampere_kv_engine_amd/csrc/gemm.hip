@@ -17,7 +17,8 @@ constexpr int kDepth = 16;  // k-tile
 
 template <typename TX, typename TW, typename TY>
 __global__ __launch_bounds__(256) void linear_tiled_kernel(const TX* __restrict__ x, const TW* __restrict__ w,
-                                                           TY* __restrict__ y, int rows, int outs, int k) {
+                                                           TY* __restrict__ y, int rows, int outs, int k,
+                                                           const float* __restrict__ bias) {
   __shared__ float xs[kDepth][kTile + 1];
   __shared__ float ws[kDepth][kTile + 1];
   const int row0 = blockIdx.y * kTile, out0 = blockIdx.x * kTile;
@@ -53,33 +54,34 @@ __global__ __launch_bounds__(256) void linear_tiled_kernel(const TX* __restrict_
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int o = out0 + tc * 4 + j;
-      if (o < outs) y[static_cast<size_t>(r) * outs + o] = from_float<TY>(acc[i][j]);
+      if (o < outs) y[static_cast<size_t>(r) * outs + o] = from_float<TY>(bias != nullptr ? acc[i][j] + bias[o] : acc[i][j]);
     }
   }
 }
 
 template <typename TX, typename TW, typename TY>
-int launch_tiled(const void* x, const void* w, void* y, int rows, int outs, int k, hipStream_t stream) {
+int launch_tiled(const void* x, const void* w, void* y, int rows, int outs, int k, const float* bias, hipStream_t stream) {
   dim3 grid((outs + kTile - 1) / kTile, (rows + kTile - 1) / kTile);
   linear_tiled_kernel<TX, TW, TY><<<grid, 256, 0, stream>>>(static_cast<const TX*>(x), static_cast<const TW*>(w),
-                                                            static_cast<TY*>(y), rows, outs, k);
+                                                            static_cast<TY*>(y), rows, outs, k, bias);
   return AKV_LAUNCH_STATUS();
 }
 
 }  // namespace
 
+// `bias` [outs] float32 or null: added to a sum after its last product, before it is rounded to y's type.
 extern "C" int akv_linear_tiled(const void* x, int x_dtype, const void* w, int w_dtype, void* y, int y_dtype, int rows,
-                                int outs, int k, hipStream_t stream) {
+                                int outs, int k, const float* bias, hipStream_t stream) {
   if (rows <= 0 || outs <= 0) return 0;
   if (((rows + kTile - 1) / kTile) > 65535) return -2;
   const int code = x_dtype * 4 + w_dtype * 2 + y_dtype;
   switch (code) {
-    case 0: return launch_tiled<float, float, float>(x, w, y, rows, outs, k, stream);
-    case 2: return launch_tiled<float, bf16_t, float>(x, w, y, rows, outs, k, stream);
-    case 4: return launch_tiled<bf16_t, float, float>(x, w, y, rows, outs, k, stream);
-    case 5: return launch_tiled<bf16_t, float, bf16_t>(x, w, y, rows, outs, k, stream);
-    case 6: return launch_tiled<bf16_t, bf16_t, float>(x, w, y, rows, outs, k, stream);
-    case 7: return launch_tiled<bf16_t, bf16_t, bf16_t>(x, w, y, rows, outs, k, stream);
+    case 0: return launch_tiled<float, float, float>(x, w, y, rows, outs, k, bias, stream);
+    case 2: return launch_tiled<float, bf16_t, float>(x, w, y, rows, outs, k, bias, stream);
+    case 4: return launch_tiled<bf16_t, float, float>(x, w, y, rows, outs, k, bias, stream);
+    case 5: return launch_tiled<bf16_t, float, bf16_t>(x, w, y, rows, outs, k, bias, stream);
+    case 6: return launch_tiled<bf16_t, bf16_t, float>(x, w, y, rows, outs, k, bias, stream);
+    case 7: return launch_tiled<bf16_t, bf16_t, bf16_t>(x, w, y, rows, outs, k, bias, stream);
     default: return -1;
   }
 }

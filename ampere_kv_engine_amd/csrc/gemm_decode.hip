@@ -38,6 +38,7 @@ struct DecodeArgs {
   bf16_t* y;                // not ADDS: [rows, outs]
   float* stream_out;        // ADDS: [rows, outs], updated in place
   float* sums_out;          // ADDS: [n_tiles][16]
+  const float* bias;        // [outs] or null: added to the sums over k before anything else is done with them (never GATED)
   float eps;
   int sum_tiles, rows, outs, k, k_tiles, n_tiles, k_split, red_floats;
   float* pieces;            // [wave-row][2][RT][4][64]: the sums of a wave-row whose parts of k lie in two blocks
@@ -252,6 +253,10 @@ __global__ __launch_bounds__(768) void linear_decode_kernel(const DecodeArgs a) 
     }
   }
   if (row_tile >= a.n_tiles) return;
+  if constexpr (!GATED) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) acc[rt] = plus_bias(acc[rt], a.bias, (row_tile + rt) * 16 + g * 4, a.outs);
+  }
   if constexpr (ADDS) {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
@@ -374,7 +379,7 @@ int launch_decode(DecodeArgs a, hipStream_t stream) {
 
 }  // namespace
 
-// stream_out [rows, outs] += bfloat16(x W^T) in place (float32); sums_out [n_tiles][16] receives, for every row tile of
+// stream_out [rows, outs] += bfloat16(x W^T (+ bias)) in place (float32; `bias` [outs] float32 or null); sums_out [n_tiles][16] receives, for every row tile of
 // 16 outputs and every row, the sum of squares of the new values (rows beyond `rows`: 0).  rows <= 16, k % 8 == 0.
 // `pieces` (exchange_tiles * 512 floats) and `arrivals` (exchange_tiles words, zero; left zero) may be null, or hold
 // fewer than n_tiles + 1 row tiles' worth (a wave's pair of row tiles may begin at the last tile), and are then not used: with them the product
@@ -391,7 +396,7 @@ extern "C" int akv_linear_decode_plan(int rt, int n_tiles, int k_tiles, int k, i
 
 extern "C" int akv_linear_adds(const void* x, const void* wp, float* stream_out, float* sums_out, float* pieces,
                                unsigned int* arrivals, int exchange_tiles, int rows, int outs, int k, int n_tiles,
-                               int k_tiles, hipStream_t stream) {
+                               int k_tiles, const float* bias, hipStream_t stream) {
   if (rows <= 0 || outs <= 0) return 0;
   if (rows > 16 || (k & 7) != 0 || n_tiles * 16 < outs || (n_tiles - 1) * 16 >= outs || k_tiles * 32 < k) return -2;
   DecodeArgs a{};
@@ -399,6 +404,7 @@ extern "C" int akv_linear_adds(const void* x, const void* wp, float* stream_out,
   a.wp = static_cast<const uintx4*>(wp);
   a.stream_out = stream_out;
   a.sums_out = sums_out;
+  a.bias = bias;
   if (pieces != nullptr && arrivals != nullptr && exchange_tiles >= n_tiles + 1) a.pieces = pieces, a.arrivals = arrivals;
   a.rows = rows, a.outs = outs, a.k = k, a.k_tiles = k_tiles, a.n_tiles = n_tiles;
   return launch_decode<1, false, false, true>(a, stream);
@@ -410,14 +416,14 @@ extern "C" int akv_linear_adds(const void* x, const void* wp, float* stream_out,
 // [sum_tiles][16] (what akv_linear_adds left: sum_tiles = ceil(k / 16)).  rows <= 16, k % 8 == 0, and the normed rows
 // (rows * k bfloat16) fit into a compute unit's LDS (160 KB) beside 832 bytes; -2 otherwise.  `pieces`, `arrivals`: as
 // for akv_linear_adds.  `row_tiles`: row tiles per wave of the plain product, 1 or 2; 0 leaves the choice to the sizes (a
-// gated product's waves always take a pair).
+// gated product's waves always take a pair).  `bias` [outs] float32 or null (never with `gated`): y = norm(stream) W^T + bias.
 extern "C" int akv_linear_scaled(const float* stream_in, const float* sums, int sum_tiles, const float* gain, float eps,
                                  const void* wp, void* y, float* pieces, unsigned int* arrivals, int exchange_tiles,
                                  int rows, int outs, int k, int n_tiles, int k_tiles, int gated, int row_tiles,
-                                 hipStream_t stream) {
+                                 const float* bias, hipStream_t stream) {
   if (rows <= 0 || outs <= 0) return 0;
   if (rows > 16 || (k & 7) != 0 || k_tiles * 32 < k || sum_tiles != (k + 15) / 16) return -2;
-  if (row_tiles < 0 || row_tiles > 2 || (gated && row_tiles == 1)) return -2;
+  if (row_tiles < 0 || row_tiles > 2 || (gated && (row_tiles == 1 || bias != nullptr))) return -2;
   if (gated ? ((outs & 15) != 0 || n_tiles * 8 != outs) : n_tiles * 16 < outs) return -2;
   DecodeArgs a{};
   a.stream = stream_in;
@@ -427,6 +433,7 @@ extern "C" int akv_linear_scaled(const float* stream_in, const float* sums, int 
   a.eps = eps;
   a.wp = static_cast<const uintx4*>(wp);
   a.y = static_cast<bf16_t*>(y);
+  a.bias = bias;
   if (pieces != nullptr && arrivals != nullptr && exchange_tiles >= n_tiles + 1) a.pieces = pieces, a.arrivals = arrivals;
   const bool may = a.pieces != nullptr;
   a.rows = rows, a.outs = outs, a.k = k, a.k_tiles = k_tiles, a.n_tiles = n_tiles;

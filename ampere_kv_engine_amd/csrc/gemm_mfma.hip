@@ -59,7 +59,7 @@ template <int MT, int RT, typename TY, bool GATED, bool NORMED = false>
 __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __restrict__ x, const uintx4* __restrict__ wp,
                                                             TY* __restrict__ y, int rows, int outs, int k,
                                                             int k_tiles, int n_tiles, int k_split, int x_packed,
-                                                            const NormIn norm) {
+                                                            const NormIn norm, const float* __restrict__ bias) {
   constexpr int U = kSkinnyGroup<MT, RT>;  // k-tiles per group; two groups are in flight
   extern __shared__ float red[];  // [wave, or group of waves with the same row tiles][RT][MT][4][64]
   const int lane = threadIdx.x & 63, waves = blockDim.x >> 6;
@@ -305,13 +305,15 @@ __global__ __launch_bounds__(512) void linear_skinny_kernel(const bf16_t* __rest
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
-        if (row_tile + rt < n_tiles) store_tile<TY>(y, acc[rt][mt], mt * 16 + r, (row_tile + rt) * 16 + g * 4, rows, outs);
+        if (row_tile + rt < n_tiles)
+          store_tile<TY>(y, plus_bias(acc[rt][mt], bias, (row_tile + rt) * 16 + g * 4, outs), mt * 16 + r,
+                         (row_tile + rt) * 16 + g * 4, rows, outs);
   }
 }
 
 template <int MT, int RT, typename TY, bool GATED, bool NORMED = false>
 int launch_skinny(const void* x, const void* wp, void* y, int rows, int outs, int k, int k_tiles, int n_tiles,
-                  int x_packed, hipStream_t stream, NormIn norm = NormIn{}) {
+                  int x_packed, hipStream_t stream, const float* bias = nullptr, NormIn norm = NormIn{}) {
   // Enough waves to keep every CU's memory pipe full: k is split over the waves of a block when there are few row
   // tiles - down to short parts of k while the waves are very few, and further only while a wave keeps enough k-tiles
   // for two rounds of its double-buffered loop (measured: 1,536 waves of 32 k-tiles beat 3,072 of 16).
@@ -336,40 +338,40 @@ int launch_skinny(const void* x, const void* wp, void* y, int rows, int outs, in
   }
   linear_skinny_kernel<MT, RT, TY, GATED, NORMED><<<blocks, waves * 64, lds, stream>>>(
       static_cast<const bf16_t*>(x), static_cast<const uintx4*>(wp), static_cast<TY*>(y), rows, outs, k, k_tiles,
-      n_tiles, k_split, x_packed, norm);
+      n_tiles, k_split, x_packed, norm, GATED ? nullptr : bias);
   return AKV_LAUNCH_STATUS();
 }
 
 template <typename TY, bool GATED>
 int dispatch_skinny(const void* x, const void* wp, void* y, int rows, int outs, int k, int k_tiles, int n_tiles,
-                    int x_packed, hipStream_t stream) {
+                    int x_packed, hipStream_t stream, const float* bias) {
   switch ((rows + 15) / 16) {
     case 1:
       // two row tiles per wave halve the activation loads per weight byte; that pays with several rows of x and
       // enough row tiles that the waves stay many (measured at 384 row tiles: 12.7 -> 11.5 us at 8 rows)
       if (GATED || (rows >= 4 && n_tiles >= 384 && n_tiles < 2048))
-        return launch_skinny<1, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
-      return launch_skinny<1, GATED ? 2 : 1, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
+        return launch_skinny<1, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream, bias);
+      return launch_skinny<1, GATED ? 2 : 1, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream, bias);
     // Several tiles of x rows.  Two tiles: a wave takes 2 row tiles of the weights, or 1 where there are so few that
     // the blocks would not even cover the compute units (4,096 outputs: 15.6 -> 13.1 us at k = 4,096).  Three and
     // four: 4 row tiles where that still leaves a thousand waves (the gated product is measured better with 2 up to
     // 2,048 row tiles: 68.7 -> 51.8 us at 64 rows), 2 otherwise.
     case 2:
       if (!GATED && n_tiles <= 256)
-        return launch_skinny<2, GATED ? 2 : 1, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
-      return launch_skinny<2, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
+        return launch_skinny<2, GATED ? 2 : 1, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream, bias);
+      return launch_skinny<2, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream, bias);
     case 3:
       if (!GATED && n_tiles <= 256)
-        return launch_skinny<3, GATED ? 2 : 1, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
+        return launch_skinny<3, GATED ? 2 : 1, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream, bias);
       return n_tiles >= (GATED ? 2048 : 512)
-                 ? launch_skinny<3, 4, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream)
-                 : launch_skinny<3, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
+                 ? launch_skinny<3, 4, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream, bias)
+                 : launch_skinny<3, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream, bias);
     case 4:
       if (!GATED && n_tiles <= 256)
-        return launch_skinny<4, GATED ? 2 : 1, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
+        return launch_skinny<4, GATED ? 2 : 1, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream, bias);
       return n_tiles >= (GATED ? 2048 : 512)
-                 ? launch_skinny<4, 4, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream)
-                 : launch_skinny<4, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
+                 ? launch_skinny<4, 4, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream, bias)
+                 : launch_skinny<4, 2, TY, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream, bias);
     default: return -2;
   }
 }
@@ -389,7 +391,8 @@ constexpr int kWideN = 128, kWideK = 64;
 template <typename TY, int MW, bool GATED>
 __global__ __launch_bounds__(256, 2) void linear_wide_kernel(const bf16_t* __restrict__ x, const uintx4* __restrict__ wp,
                                                           TY* __restrict__ y, int rows, int outs, int k, int k_tiles,
-                                                          int n_tiles, int n_blocks, int m_blocks) {
+                                                          int n_tiles, int n_blocks, int m_blocks,
+                                                          const float* __restrict__ bias) {
   constexpr int kWideM = 32 * MW;  // tokens per block
   __shared__ uintx4 xs[2][kWideK / 8][kWideM];  // 2 stages x 8 chunks x tokens x 16 B (64 KB for 256 tokens)
   const int lane = threadIdx.x & 63;
@@ -535,13 +538,14 @@ __global__ __launch_bounds__(256, 2) void linear_wide_kernel(const bf16_t* __res
     for (int n = 0; n < 4; ++n)
 #pragma unroll
       for (int m = 0; m < MW; ++m)
-        store_tile<TY>(y, acc[n][m], token0 + wave_m * (16 * MW) + m * 16 + r, (tile0 + n) * 16 + g * 4, rows, outs);
+        store_tile<TY>(y, plus_bias(acc[n][m], bias, (tile0 + n) * 16 + g * 4, outs), token0 + wave_m * (16 * MW) + m * 16 + r,
+                       (tile0 + n) * 16 + g * 4, rows, outs);
   }
 }
 
 template <typename TY, bool GATED>
 int launch_wide(const void* x, const void* wp, void* y, int rows, int outs, int k, int k_tiles, int n_tiles,
-                hipStream_t stream) {
+                hipStream_t stream, const float* bias) {
   const int n_blocks = (n_tiles * 16 + kWideN - 1) / kWideN;
   // 256 tokens per block when that still gives every compute unit its two blocks, else 128
   const bool tall = static_cast<long>(n_blocks) * ((rows + 255) / 256) >= 512;
@@ -552,11 +556,11 @@ int launch_wide(const void* x, const void* wp, void* y, int rows, int outs, int 
   if (tall)
     linear_wide_kernel<TY, 8, GATED><<<static_cast<unsigned>(blocks), 256, 0, stream>>>(
         static_cast<const bf16_t*>(x), static_cast<const uintx4*>(wp), static_cast<TY*>(y), rows, outs, k, k_tiles,
-        n_tiles, n_blocks, m_blocks);
+        n_tiles, n_blocks, m_blocks, GATED ? nullptr : bias);
   else
     linear_wide_kernel<TY, 4, GATED><<<static_cast<unsigned>(blocks), 256, 0, stream>>>(
         static_cast<const bf16_t*>(x), static_cast<const uintx4*>(wp), static_cast<TY*>(y), rows, outs, k, k_tiles,
-        n_tiles, n_blocks, m_blocks);
+        n_tiles, n_blocks, m_blocks, GATED ? nullptr : bias);
   return AKV_LAUNCH_STATUS();
 }
 
@@ -583,15 +587,15 @@ extern "C" int akv_pack_rows(const void* x, void* xp, int rows, int k, hipStream
 namespace {
 template <bool GATED>
 int linear_packed(const void* x, const void* wp, void* y, int y_dtype, int rows, int outs, int k, int n_tiles,
-                  int k_tiles, int x_packed, hipStream_t stream) {
+                  int k_tiles, int x_packed, hipStream_t stream, const float* bias = nullptr) {
   if (rows <= 64) {
-    if (y_dtype == kF32) return dispatch_skinny<float, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
-    if (y_dtype == kBF16) return dispatch_skinny<bf16_t, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream);
+    if (y_dtype == kF32) return dispatch_skinny<float, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream, bias);
+    if (y_dtype == kBF16) return dispatch_skinny<bf16_t, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, x_packed, stream, bias);
     return -1;
   }
   if (x_packed) return -2;  // only the products of up to 64 rows read packed activations
-  if (y_dtype == kF32) return launch_wide<float, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
-  if (y_dtype == kBF16) return launch_wide<bf16_t, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream);
+  if (y_dtype == kF32) return launch_wide<float, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream, bias);
+  if (y_dtype == kBF16) return launch_wide<bf16_t, GATED>(x, wp, y, rows, outs, k, k_tiles, n_tiles, stream, bias);
   return -1;
 }
 }  // namespace
@@ -599,11 +603,12 @@ int linear_packed(const void* x, const void* wp, void* y, int y_dtype, int rows,
 // x [rows, k] bfloat16 row-major; wp the packed weight of `n_tiles` x `k_tiles` tiles; y [rows, outs] bfloat16 or
 // float32.  k must be a multiple of 8 (a lane's 16-byte read of x must lie inside or outside the row as a whole).
 // `x_packed` (rows <= 64 only): x is not row-major but [tile of 16 rows][k / 8][16 rows][8], what akv_pack_rows writes.
+// `bias` [outs] float32 or null: added to the float32 sums before they are rounded.
 extern "C" int akv_linear_packed(const void* x, const void* wp, void* y, int y_dtype, int rows, int outs, int k,
-                                 int n_tiles, int k_tiles, int x_packed, hipStream_t stream) {
+                                 int n_tiles, int k_tiles, int x_packed, const float* bias, hipStream_t stream) {
   if (rows <= 0 || outs <= 0) return 0;
   if ((k & 7) != 0 || n_tiles * 16 < outs || k_tiles * 32 < k) return -2;
-  return linear_packed<false>(x, wp, y, y_dtype, rows, outs, k, n_tiles, k_tiles, x_packed, stream);
+  return linear_packed<false>(x, wp, y, y_dtype, rows, outs, k, n_tiles, k_tiles, x_packed, stream, bias);
 }
 
 namespace {
@@ -663,17 +668,18 @@ extern "C" int akv_linear_packed_swiglu(const void* x, const void* wp, void* y, 
 // The product of a few rows that are not computed yet: rows = norm(stream_in (+ delta)) as akv_add_rmsnorm norms them
 // (bfloat16 activations), normed by every block of the product for itself; stream_out [rows, k] receives
 // stream_in + delta and must be another buffer than stream_in.  `gated`: akv_linear_packed_swiglu's packing and result.
-// At most 4 rows; k a multiple of 8; -2 where the rows do not fit the block's LDS beside its sums.
+// At most 4 rows; k a multiple of 8; -2 where the rows do not fit the block's LDS beside its sums.  `bias` [outs] float32
+// or null (never with `gated`).
 extern "C" int akv_linear_packed_normed(const float* stream_in, const void* delta, const float* norm_weight, float eps,
                                         float* stream_out, const void* wp, void* y, int rows, int outs, int k,
-                                        int n_tiles, int k_tiles, int gated, hipStream_t stream) {
+                                        int n_tiles, int k_tiles, int gated, const float* bias, hipStream_t stream) {
   if (rows <= 0 || outs <= 0) return 0;
   if (rows > 4 || (k & 7) != 0 || k_tiles * 32 < k || stream_in == stream_out ||
       (gated ? ((outs & 15) != 0 || n_tiles * 8 != outs) : n_tiles * 16 < outs))
     return -2;
   NormIn norm{stream_in, static_cast<const bf16_t*>(delta), norm_weight, stream_out, eps, 0};
-  if (gated) return launch_skinny<1, 2, bf16_t, true, true>(nullptr, wp, y, rows, outs, k, k_tiles, n_tiles, 0, stream, norm);
+  if (gated) return launch_skinny<1, 2, bf16_t, true, true>(nullptr, wp, y, rows, outs, k, k_tiles, n_tiles, 0, stream, bias, norm);
   if (rows >= 4 && n_tiles >= 384 && n_tiles < 2048)
-    return launch_skinny<1, 2, bf16_t, false, true>(nullptr, wp, y, rows, outs, k, k_tiles, n_tiles, 0, stream, norm);
-  return launch_skinny<1, 1, bf16_t, false, true>(nullptr, wp, y, rows, outs, k, k_tiles, n_tiles, 0, stream, norm);
+    return launch_skinny<1, 2, bf16_t, false, true>(nullptr, wp, y, rows, outs, k, k_tiles, n_tiles, 0, stream, bias, norm);
+  return launch_skinny<1, 1, bf16_t, false, true>(nullptr, wp, y, rows, outs, k, k_tiles, n_tiles, 0, stream, bias, norm);
 }

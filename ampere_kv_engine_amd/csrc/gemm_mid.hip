@@ -47,7 +47,7 @@ __global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_ker
                                                               TY* __restrict__ y, float* __restrict__ partial,
                                                               unsigned* __restrict__ counters, int rows, int outs, int k,
                                                               int k_tiles, int n_tiles, int bands, int parts,
-                                                              int part_tiles, int m_blocks) {
+                                                              int part_tiles, int m_blocks, const float* __restrict__ bias) {
   constexpr int S = kStage<MT>;
   constexpr int kAlong = A, kMultipliers = A * kHalves;
   constexpr int kTiles = kHalves * S * MT;        // activation tiles of one stage
@@ -258,7 +258,9 @@ __global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_ker
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
-        if (tile0 + rt < n_tiles) store_tile<TY>(y, acc[rt][mt], row0 + mt * 16 + r, (tile0 + rt) * 16 + g * 4, rows, outs);
+        if (tile0 + rt < n_tiles)
+          store_tile<TY>(y, plus_bias(acc[rt][mt], bias, (tile0 + rt) * 16 + g * 4, outs), row0 + mt * 16 + r,
+                         (tile0 + rt) * 16 + g * 4, rows, outs);
   }
 }
 
@@ -327,7 +329,7 @@ MidPlan plan_mid(int rows, int n_tiles, int k_tiles, bool gated, int along, int 
 
 template <int A, int MT, int RT, int G, bool GATED, typename TY>
 int launch_mid(const MidPlan& p, const void* x, const void* wp, void* y, float* partial, unsigned* counters, int rows,
-               int outs, int k, int k_tiles, int n_tiles, hipStream_t stream) {
+               int outs, int k, int k_tiles, int n_tiles, const float* bias, hipStream_t stream) {
   constexpr size_t lds = 2 * kHalves * kStage<MT> * MT * 1024;
   static_assert(lds >= static_cast<size_t>(A) * RT * MT * 1024, "the sums of a k half must fit the staging memory");
   static_assert(lds <= 64 * 1024, "the staging memory is taken without asking for more than a block may have by default");
@@ -336,16 +338,16 @@ int launch_mid(const MidPlan& p, const void* x, const void* wp, void* y, float* 
   if (blocks > 0x7fffffffL) return -2;
   linear_mid_kernel<A, MT, RT, G, GATED, TY><<<static_cast<unsigned>(blocks), (A * kHalves + kFetchers) * 64, lds, stream>>>(
       static_cast<const bf16_t*>(x), static_cast<const uintx4*>(wp), static_cast<TY*>(y), partial, counters, rows, outs,
-      k, k_tiles, n_tiles, p.bands, p.parts, p.part_tiles, p.m_blocks);
+      k, k_tiles, n_tiles, p.bands, p.parts, p.part_tiles, p.m_blocks, GATED ? nullptr : bias);
   return AKV_LAUNCH_STATUS();
 }
 
 template <bool GATED, typename TY>
 int dispatch_mid(const MidPlan& p, const void* x, const void* wp, void* y, float* partial, unsigned* counters, int rows,
-                 int outs, int k, int k_tiles, int n_tiles, hipStream_t stream) {
+                 int outs, int k, int k_tiles, int n_tiles, const float* bias, hipStream_t stream) {
 #define AKV_MID(A_, MT_, RT_, G_) \
   if (p.along == A_ && p.mt == MT_ && p.rt == RT_ && p.depth == G_) \
-    return launch_mid<A_, MT_, RT_, G_, GATED, TY>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, stream)
+    return launch_mid<A_, MT_, RT_, G_, GATED, TY>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, bias, stream)
 #define AKV_MID_ROWS(A_, RT_, G_) \
   AKV_MID(A_, 2, RT_, G_); AKV_MID(A_, 3, RT_, G_); AKV_MID(A_, 4, RT_, G_); AKV_MID(A_, 5, RT_, G_); \
   AKV_MID(A_, 6, RT_, G_); AKV_MID(A_, 7, RT_, G_); AKV_MID(A_, 8, RT_, G_)
@@ -377,24 +379,27 @@ extern "C" int akv_linear_mid_workspace(int rows, int n_tiles, int k_tiles, int 
 // akv_linear_packed_swiglu).  `along` (waves along a band: 2..4), `rt` (row tiles per wave, 1 or 2), `depth`
 // (register sets of the weight ring: 2 with rt = 2, 4 with rt = 1) and `parts` (blocks along k, a power of two) may be 0: chosen here.
 // `partial_floats` and `counter_words` say how much `partial` and `counters` hold: a cut that needs more
-// (akv_linear_mid_workspace tells) is refused with -3 and nothing is launched.
+// (akv_linear_mid_workspace tells) is refused with -3 and nothing is launched.  `bias` [outs] float32 or null (never with
+// `gated`): added to the float32 sums before they are rounded.
 extern "C" int akv_linear_mid(const void* x, const void* wp, void* y, int y_dtype, float* partial, long partial_floats,
                               unsigned* counters, long counter_words, int rows, int outs, int k, int n_tiles,
-                              int k_tiles, int gated, int along, int rt, int depth, int parts, hipStream_t stream) {
+                              int k_tiles, int gated, int along, int rt, int depth, int parts, const float* bias,
+                              hipStream_t stream) {
   if (rows <= 0 || outs <= 0) return 0;
   if ((k & 7) != 0 || k_tiles * 32 < k) return -2;
   if (gated ? ((outs & 15) != 0 || n_tiles * 8 != outs) : n_tiles * 16 < outs) return -2;
+  if (gated && bias != nullptr) return -2;
   if (along < 0 || along == 1 || along > 4 || rt < 0 || rt > 2 || depth < 0 || parts < 0 || (parts & (parts - 1)) != 0) return -2;
   const MidPlan p = plan_mid(rows, n_tiles, k_tiles, gated != 0, along, rt, depth, parts);
   if (p.along == 0) return -2;
   if (p.parts > 1 && (partial == nullptr || counters == nullptr)) return -2;
   if (p.parts > 1 && (static_cast<long>(p.partial_floats) > partial_floats || static_cast<long>(p.counters) > counter_words)) return -3;
   if (gated) {
-    if (y_dtype == kF32) return dispatch_mid<true, float>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, stream);
-    if (y_dtype == kBF16) return dispatch_mid<true, bf16_t>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, stream);
+    if (y_dtype == kF32) return dispatch_mid<true, float>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, bias, stream);
+    if (y_dtype == kBF16) return dispatch_mid<true, bf16_t>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, bias, stream);
     return -1;
   }
-  if (y_dtype == kF32) return dispatch_mid<false, float>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, stream);
-  if (y_dtype == kBF16) return dispatch_mid<false, bf16_t>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, stream);
+  if (y_dtype == kF32) return dispatch_mid<false, float>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, bias, stream);
+  if (y_dtype == kBF16) return dispatch_mid<false, bf16_t>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, bias, stream);
   return -1;
 }

@@ -54,6 +54,17 @@ __device__ __forceinline__ void store_tile(TY* y, floatx4 acc, int token, int fe
   }
 }
 
+// The tile's four values plus the bias of their features; `bias` [outs] may be null: then nothing is added.  (A product
+// with a bias is x W^T + b formed in float32 and rounded once, as torch.nn.functional.linear forms it.)
+__device__ __forceinline__ floatx4 plus_bias(floatx4 acc, const float* __restrict__ bias, int feature, int outs) {
+  if (bias != nullptr) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (feature + i < outs) acc[i] += bias[feature + i];
+  }
+  return acc;
+}
+
 __device__ __forceinline__ floatx4 silu_times(floatx4 gate, floatx4 up) {
   floatx4 v;
 #pragma unroll

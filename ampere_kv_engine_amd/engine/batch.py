@@ -120,6 +120,9 @@ class StepContext:
     spare_buffer: torch.Tensor | None = None    # float32 [a few rows, hidden]: where a small step may move it
     stream: torch.Tensor | None = None          # the step's residual sum, wherever it is now
     spare_stream: torch.Tensor | None = None    # the other buffer's rows, or None where the step has too many
+    # set by the model's pass and by blocks around every branch: the branch may add its output to the residual sum in
+    # its last product and return `StreamSums` (see `parts.base.Part`)
+    fold_into_stream: bool = False
     # the device's persistent integer state (slot words, block tables) and what this step changes in it
     table_pages: int = 0                        # bound on the pages of the step's longest request (sizes launches)
     patches: torch.Tensor | None = None         # int32 [2 * patch_room]: (offset into slot_state, value) pairs

@@ -4,10 +4,10 @@ from __future__ import annotations
 
 import torch
 
-from ..parts.base import Runtime
+from ..parts.base import KernelSet, Runtime
 
 
-class _NoKernels:
+class _NoKernels(KernelSet):
     def __getattr__(self, name):
         return lambda *args, **kwargs: None
 

@@ -91,7 +91,7 @@ class Engine:
     def _loaded(self) -> None:
         """The weights are in place: what is decided once per model is decided now, not inside a step."""
         self.loaded = True
-        if self.config.product_choices == "measure" and hasattr(self.kernels, "measure_products"):
+        if self.config.product_choices == "measure":
             self.kernels.measure_products()
 
     # ---- requests ---------------------------------------------------------------------------------
@@ -170,11 +170,8 @@ class Engine:
                                  f"of {vocab}")
 
     # ---- steps as recorded graphs -----------------------------------------------------------------------------
-    SPARE_STREAM_ROWS = 1         # steps of up to this many tokens may move the residual sum between two buffers
-    GRAPH_WIDTH_MULTIPLE = 64     # block tables of a recorded step are this many pages wide, or a multiple
-    RECORD_MAX_TOKENS = 512       # steps with prompt portions are recorded up to this many tokens: beyond it the
-                                  # device works longer on a step than the host needs to launch it
-    MAX_RECORDINGS = 512          # shapes met after this many are run as they are
+    SPARE_STREAM_ROWS = 1         # steps of up to this many tokens may move the residual sum between two buffers (what
+                                  # the one-row product that norms its own row needs: a fact of that kernel, not a setting)
 
     def _recordable_shape(self, entries: list[StepEntry]):
         """(tokens per request in the step's order - single tokens first -, wanted rows), or None for a step that
@@ -184,7 +181,7 @@ class Engine:
         wanted = sum(len(e.want) for e in entries)
         if wanted == 0 or wanted > self.config.max_seqs or any(e.extra for e in entries):
             return None
-        if counts[-1] != 1 and sum(counts) > self.RECORD_MAX_TOKENS:
+        if counts[-1] != 1 and sum(counts) > self.config.record_max_tokens:
             return None
         return counts, wanted
 
@@ -197,7 +194,7 @@ class Engine:
         serves all lengths under it.  The logits are written to a buffer that all recordings share: the next
         recorded step overwrites them (`step` hands out a copy unless the caller asked to borrow the buffer)."""
         counts, wanted = shape
-        ctx, _ = self.builder.build(entries, width_multiple=self.GRAPH_WIDTH_MULTIPLE)
+        ctx, _ = self.builder.build(entries, width_multiple=self.config.graph_width_multiple)
         ctx.stream_buffer, ctx.spare_buffer = self.stream_buffer, self.spare_buffer
         self._last_step = ctx
         width = ctx.table_pages        # the longest request's pages, rounded up: a bound the recording is made for
@@ -213,7 +210,7 @@ class Engine:
         graph = self._graphs.get(key, False)
         if graph is False:              # first met: run as it is (this also settles the arenas)
             self.model.forward(ctx, self.cache.layer_cache, logits)
-            if len(self._graphs) < self.MAX_RECORDINGS or counts[-1] == 1:   # (decode steps are always remembered)
+            if len(self._graphs) < self.config.max_recordings or counts[-1] == 1:   # (decode steps are always remembered)
                 self._graphs[key] = None
             return logits
         if graph is None:               # met again: record

@@ -10,8 +10,7 @@ from __future__ import annotations
 import torch
 
 from ..config.specs import ModelSpec
-from ..parts.base import PagedKV, Runtime, SlotState, build_part
-from ..parts.norm import StreamSums
+from ..parts.base import PagedKV, Runtime, SlotState, StreamSums, build_part
 from ..weights.spec import TensorSpec
 
 
@@ -84,9 +83,9 @@ class Model:
         arenas = ctx.arenas
         # the residual sum; a block may move it to the step's spare buffer (`ctx.spare_stream`) and says so in `ctx.stream`
         ctx.stream = ctx.stream_buffer[:ctx.num_tokens]
-        spare = getattr(ctx, "spare_buffer", None)
+        spare = ctx.spare_buffer
         ctx.spare_stream = spare[:ctx.num_tokens] if spare is not None and ctx.num_tokens <= spare.shape[0] else None
-        if getattr(ctx, "slot_state", None) is not None:
+        if ctx.slot_state is not None:
             k.step_prologue(ctx)        # block-table changes and new lengths reach the device's persistent state
         self.embedding.forward(ctx.token_ids, ctx.stream, ctx)
         pending = None
@@ -97,7 +96,7 @@ class Model:
             # a block's last branch may add its output to the residual sum itself and hand on the rows' sums of squares
             # instead, if whoever reads `pending` next knows what to make of that: the next block, or the end below
             following = self.blocks[order[step_index + 1].layer] if step_index + 1 < len(order) else None
-            ctx.fold_into_stream = following is None or getattr(following, "takes_stream_sums", False)
+            ctx.fold_into_stream = following is None or following.takes_stream_sums
             pending = self.blocks[entry.layer].forward(ctx.stream, pending, ctx, layer_cache[entry.cache_layer],
                                                        entry.writes_cache)
         if isinstance(pending, StreamSums):      # the last branch's output is in the residual sum already

@@ -12,6 +12,7 @@ import ctypes
 import torch
 
 from ..csrc.build import ensure_attention, ensure_built
+from ..parts.base import KernelSet
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 MAX_HEAD_DIM = 256
@@ -86,7 +87,7 @@ def _ptr(t: torch.Tensor | None):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
 
 
-class HipKernels:
+class HipKernels(KernelSet):
     name = "hip-gfx950"
     OWN_SKINNY_ROWS = 64            # the most rows the engine's own decode product takes
 
@@ -346,7 +347,7 @@ class HipKernels:
             return "library"
         return "mid" if (rows > 64 or outs <= k) else "library"
 
-    def _mid(self, x, packed: PackedWeight, out, rows: int, outs: int, gated: bool) -> None:
+    def _mid(self, x, packed: PackedWeight, out, rows: int, outs: int, gated: bool, bias=None) -> None:
         """The mid-size product (`csrc/gemm_mid.hip`).  Where it cuts k over blocks it needs room for partial sums
         and a few counters; both belong to this kernel set and serve one launch at a time (one stream)."""
         partial_floats, counters = ctypes.c_long(0), ctypes.c_long(0)
@@ -367,7 +368,7 @@ class HipKernels:
         self._check(self.lib.akv_linear_mid(_ptr(x), _ptr(packed.data), _ptr(out), _code(out), _ptr(self._mid_partial),
                                             held(self._mid_partial), _ptr(self._mid_counters), held(self._mid_counters),
                                             rows, outs, packed.k, packed.n_tiles,
-                                            packed.k_tiles, 1 if gated else 0, 0, 0, 0, 0, self._stream()),
+                                            packed.k_tiles, 1 if gated else 0, 0, 0, 0, 0, _ptr(bias), self._stream()),
                     "mid-size product")
 
     MEASURED_ROWS = (32, 48, 64, 128, 256, 512)
@@ -439,31 +440,52 @@ class HipKernels:
             table[kind, int(outs), int(k), int(tiles)] = choice
         return table
 
-    def linear(self, x, weight, out):
+    def _bias(self, bias, outs: int):
+        if bias is not None:
+            self._dense(bias, "bias", torch.float32, (outs,))
+        return bias
+
+    def linear(self, x, weight, out, bias=None):
+        """out = x W^T (+ bias): `bias` [outs] float32 is added to the float32 sums before they are rounded to
+        `out`'s type - one rounding, as torch.nn.functional.linear makes."""
         if isinstance(weight, PackedWeight):
             rows, k = x.shape
             self._dense(x, "x", torch.bfloat16, (rows, weight.k))
             self._dense(out, "out", None, (rows, weight.outs))
             self._dense(weight.data, "packed weight", torch.bfloat16)
+            self._bias(bias, weight.outs)
             route = "own" if rows <= 16 else self._route("linear", weight.outs, weight.k, rows,
                                                          weight.row_major is not None, out.dtype)
             if route == "library":
-                torch.mm(x, weight.row_major.t(), out=out)
+                if bias is None:
+                    torch.mm(x, weight.row_major.t(), out=out)
+                else:       # (the library adds the bias to its float32 sums too; it wants the bias in the result's type)
+                    torch.addmm(self._library_bias(bias), x, weight.row_major.t(), out=out)
             elif route == "mid":
-                self._mid(x, weight, out, rows, weight.outs, False)
+                self._mid(x, weight, out, rows, weight.outs, False, bias)
             else:
                 operand, packed_rows = self._operand_rows(x, rows, weight.k)
                 self._check(self.lib.akv_linear_packed(_ptr(operand), _ptr(weight.data), _ptr(out), _code(out), rows,
                                                        weight.outs, weight.k, weight.n_tiles, weight.k_tiles,
-                                                       packed_rows, self._stream()), "linear")
+                                                       packed_rows, _ptr(bias), self._stream()), "linear")
             return
         rows, k = x.shape
         outs = weight.shape[0]
         self._dense(x, "x")
         self._dense(weight, "weight", None, (outs, k))
         self._dense(out, "out", None, (rows, outs))
+        self._bias(bias, outs)
         self._check(self.lib.akv_linear_tiled(_ptr(x), _code(x), _ptr(weight), _code(weight), _ptr(out), _code(out),
-                                              rows, outs, k, self._stream()), "linear")
+                                              rows, outs, k, _ptr(bias), self._stream()), "linear")
+
+    def _library_bias(self, bias: torch.Tensor) -> torch.Tensor:
+        """The bias as the library's product wants it: bfloat16, made once per bias and kept (a bias read from a
+        16-bit checkpoint is exact in bfloat16)."""
+        known = self.__dict__.setdefault("_library_biases", {})
+        key = bias.data_ptr()
+        if key not in known or known[key][0] is not bias:
+            known[key] = (bias, bias.to(torch.bfloat16))
+        return known[key][1]
 
     # ---- decode steps: the residual sum and the norm inside the products -----------------------------------------
     FOLD_NORM_ROWS = 16             # steps of up to this many rows fold the residual sum and the norm into products
@@ -512,8 +534,8 @@ class HipKernels:
         packed = weight.packed if isinstance(weight, GatedWeight) else weight
         return isinstance(packed, PackedWeight) and self.folds_norm(rows, packed.k, dtype)
 
-    def linear_adds(self, x, weight: PackedWeight, stream, sums) -> None:
-        """stream [rows, outs] (float32) += bfloat16(x W^T), in place; sums [ceil(outs / 16), 16] (float32) receives
+    def linear_adds(self, x, weight: PackedWeight, stream, sums, bias=None) -> None:
+        """stream [rows, outs] (float32) += bfloat16(x W^T (+ bias)), in place; sums [ceil(outs / 16), 16] (float32) receives
         per tile of 16 outputs and row the sum of squares of the new values."""
         rows = x.shape[0]
         if not isinstance(weight, PackedWeight) or rows > 16:
@@ -526,9 +548,10 @@ class HipKernels:
         self._check(self.lib.akv_linear_adds(_ptr(x), _ptr(weight.data), _ptr(stream), _ptr(sums), _ptr(pieces),
                                              _ptr(arrivals), self._exchange_tiles if pieces is not None else 0,
                                              rows, weight.outs, weight.k, weight.n_tiles,
-                                             weight.k_tiles, self._stream()), "linear_adds")
+                                             weight.k_tiles, _ptr(self._bias(bias, weight.outs)), self._stream()),
+                    "linear_adds")
 
-    def linear_scaled(self, stream, sums, norm_weight, eps, weight, out, row_tiles: int = 0) -> None:
+    def linear_scaled(self, stream, sums, norm_weight, eps, weight, out, row_tiles: int = 0, bias=None) -> None:
         """out = norm(stream) W^T (a `GatedWeight`: silu(. Wgate^T) * (. Wup^T)) with the norm of `add_rmsnorm`
         (scaled, rounded, times the weight, rounded) applied to the float32 rows as they become operands; the rows'
         sums of squares are not formed but added up from `sums`, as `linear_adds` left them.  `row_tiles` forces the
@@ -544,12 +567,15 @@ class HipKernels:
         outs = weight.inter if gated else packed.outs
         self._dense(out, "out", torch.bfloat16, (rows, outs))
         self._dense(packed.data, "packed weight", torch.bfloat16)
+        if bias is not None and gated:
+            raise KernelError("the gated product takes no bias")
+        self._bias(bias, outs)
         pieces, arrivals = self._exchange(packed.n_tiles)
         self._check(self.lib.akv_linear_scaled(_ptr(stream), _ptr(sums), (k + 15) // 16, _ptr(norm_weight),
                                                ctypes.c_float(eps), _ptr(packed.data), _ptr(out), _ptr(pieces),
                                                _ptr(arrivals), self._exchange_tiles if pieces is not None else 0,
                                                rows, outs, k, packed.n_tiles, packed.k_tiles,
-                                               1 if gated else 0, row_tiles, self._stream()), "linear_scaled")
+                                               1 if gated else 0, row_tiles, _ptr(bias), self._stream()), "linear_scaled")
 
     STATIC_ROWS_ELEMENTS = 64 * 32768   # bfloat16 elements of the library's static device memory for repacked rows
 
@@ -585,7 +611,7 @@ class HipKernels:
         return (self.norm_in_products and 0 < rows <= self.NORM_IN_PRODUCT_ROWS and dtype == torch.bfloat16
                 and isinstance(packed, PackedWeight) and packed.k % 8 == 0 and rows * packed.k * 2 <= 48 * 1024)
 
-    def linear_after_norm(self, stream, delta, norm_weight, eps, stream_out, weight, out):
+    def linear_after_norm(self, stream, delta, norm_weight, eps, stream_out, weight, out, bias=None):
         """out = norm(stream (+ delta)) W^T (a `GatedWeight`: silu(. Wgate^T) * (. Wup^T)) without a kernel for the
         norm: every block of the product adds, norms and rounds the few rows itself, as `add_rmsnorm` would, while its
         first weights are on their way.  stream [rows, k] float32 is not changed; stream_out [rows, k], another
@@ -607,8 +633,8 @@ class HipKernels:
         self._dense(packed.data, "packed weight", torch.bfloat16)
         self._check(self.lib.akv_linear_packed_normed(
             _ptr(stream), _ptr(delta), _ptr(norm_weight), ctypes.c_float(eps), _ptr(stream_out), _ptr(packed.data),
-            _ptr(out), rows, outs, k, packed.n_tiles, packed.k_tiles, 1 if gated else 0, self._stream()),
-            "linear_after_norm")
+            _ptr(out), rows, outs, k, packed.n_tiles, packed.k_tiles, 1 if gated else 0,
+            _ptr(self._bias(bias, outs) if not gated else None), self._stream()), "linear_after_norm")
 
     def prepare_gated_linear(self, gate: torch.Tensor, up: torch.Tensor):
         """The packing for `gated_linear`, or None where the two matrices have to stay a stacked product followed by

@@ -1,7 +1,7 @@
 """Grouped-query attention over the paged cache (ampere_kv/runner.py:60-77, :121, :128-132, :164-165;
 scores, mask and softmax ampere_kv/kv_cache.py:76-94).
 
-Order per token: stacked q/k/v projection -> head split -> optional per-head norm of q and k over head_dim
+Order per token: stacked q/k/v projection (with biases where the specification's `bias` says so) -> head split -> optional per-head norm of q and k over head_dim
 (v is never normed) -> position encoding of q and k -> k (encoded) and v written to the token's cache slot
 -> every query attends the keys of its own request up to its own position (optionally only the last
 `window`) -> heads merged -> output projection.  Query head h reads kv head h // (q_heads / kv_heads).
@@ -33,9 +33,10 @@ class Attention(Part):
         if self.window is not None and int(self.window) <= 0:
             raise ValueError(f"window must be positive or None, got {self.window}")
         self.q_size, self.kv_size = self.q_heads * self.head_dim, self.kv_heads * self.head_dim
+        bias = bool(spec.get("bias", False))        # q, k, v and o each with a bias vector (runner.py:64-66, :165)
         self.qkv = Linear(runtime, self.hidden, [self.q_size, self.kv_size, self.kv_size],
-                          ["q_proj.weight", "k_proj.weight", "v_proj.weight"])
-        self.out = Linear(runtime, self.q_size, [self.hidden], ["o_proj.weight"])
+                          ["q_proj.weight", "k_proj.weight", "v_proj.weight"], bias=bias)
+        self.out = Linear(runtime, self.q_size, [self.hidden], ["o_proj.weight"], bias=bias)
         norm_spec = spec.get("qk_norm")
         self.q_norm = build_part("norm", norm_spec, runtime) if norm_spec is not None else None
         self.k_norm = build_part("norm", norm_spec, runtime) if norm_spec is not None else None
@@ -94,7 +95,7 @@ class Attention(Part):
             self._encode_with_parts(qkv, q, ctx, meta, cache, writes_cache)
             k.attention(q, cache.k, cache.v, ctx, meta, self.q_heads, self.kv_heads, self.head_dim,
                         self.scale, self.window, merged)
-        if getattr(ctx, "fold_into_stream", False):     # the output product adds itself to the residual sum
+        if ctx.fold_into_stream:     # the output product adds itself to the residual sum
             sums = self.out.add_to_stream(merged, ctx)
             if sums is not None:
                 return sums
@@ -117,7 +118,7 @@ class Attention(Part):
         else:
             k.copy_heads(q_in, q3)
             k.copy_heads(k_in, k3)
-        if getattr(self.position, "wants_context", False):     # an encoding of more than the position: it reads the step
+        if self.position.wants_context:     # an encoding of more than the position: it reads the step
             self.position.apply(q3, ctx.positions, ctx)
             self.position.apply(k3, ctx.positions, ctx)
         else:

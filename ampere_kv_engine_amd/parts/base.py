@@ -101,11 +101,40 @@ class SlotState:
 
 
 class Part:
-    """Base of all parts: tensors expected under a name prefix, and their adoption."""
+    """Base of all parts: tensors expected under a name prefix, their adoption - and the flags through which a part
+    says what it can take.  Every flag has a default here; a part that says nothing is handed plain tensors.
+
+    The fold protocol (steps of few rows; see `parts/block.py`).  Between a branch of a block and the norm that
+    follows it three things can be handed on instead of a tensor, each only to a part that has declared that it
+    knows it:
+
+      * `StreamSums` - a branch's last product has already added the branch's output to the residual sum
+        (`Linear.add_to_stream`) and left the rows' sums of squares.  Handed on as a block's `pending` only when
+        `ctx.fold_into_stream` is set, which the model's pass sets when whoever reads `pending` next - the next block
+        in the run order, or the model's end - has `takes_stream_sums = True`.  A mixer or feed-forward asks
+        `ctx.fold_into_stream` before its last product and otherwise returns a tensor.
+      * `UnnormedRows` (`PendingNorm`, `ScaledNorm` of `parts/norm.py`) - the rows norm(stream [+ delta]) before
+        anybody has computed them.  A block hands them to a mixer or feed-forward with `takes_pending_norm = True`,
+        which promises to read its input exactly once and through `Linear.forward` or the kernel set's gated product:
+        that product norms the rows itself where the kernel set can (`UnnormedRows.product`), else the rows are
+        normed first (`UnnormedRows.rows`).  A norm offers them through `Norm.pending` / `Norm.scaled`, which return
+        None for a norm that can only be computed at once.
+      * nothing else: a part without these flags gets and returns tensors `[tokens, width]` in `runtime.dtype`.
+
+    The kernel set's side of the protocol is `KernelSet` below: capabilities that default to "no".
+    """
 
     # True if the part's launches depend on nothing but the step's shape (number of requests and tokens, table
     # width): everything else it reads on the device.  Only then may a step that runs it be recorded and replayed.
     graph_safe = False
+    # (mixers, feed-forwards) the input is read exactly once, through a `Linear` or the gated product: it may arrive
+    # as `UnnormedRows`
+    takes_pending_norm = False
+    # (blocks) `pending` may be a `StreamSums`: the residual sum then already holds the branch's output
+    takes_stream_sums = False
+    # (position encodings) `apply(x, positions, ctx)` instead of `apply(x, positions)`: the encoding reads further
+    # integers per token from the step (`ctx.extra`)
+    wants_context = False
 
     def tensors(self, prefix: str) -> list[TensorSpec]:
         return []
@@ -116,3 +145,80 @@ class Part:
     def weight_bytes(self) -> int:
         """Bytes of weights one step reads (for roofline accounting)."""
         return 0
+
+
+class Norm(Part):
+    """What a block asks of a norm.  `forward` and `forward_residual` compute at once; `pending` and `scaled` offer
+    the result before it is computed, for a reader whose first product can compute it (`UnnormedRows`) - None, the
+    default, says that this norm cannot be put off."""
+
+    def forward(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+    def forward_residual(self, stream: torch.Tensor, delta: torch.Tensor | None, out: torch.Tensor) -> torch.Tensor:
+        """stream (float32, the residual sum) += delta, in place; out = norm(stream)."""
+        raise NotImplementedError
+
+    def pending(self, stream, delta, stream_out, arena) -> "UnnormedRows | None":
+        """norm(stream + delta) not yet computed, the new residual sum to be left in `stream_out`."""
+        return None
+
+    def scaled(self, stream, sums: "StreamSums", arena) -> "UnnormedRows | None":
+        """norm(stream) not yet computed, for a stream whose rows' sums of squares are in `sums`."""
+        return None
+
+
+class StreamSums:
+    """What a branch hands on instead of its output when its last product has already added that output to the
+    residual sum (`Linear.add_to_stream`): the partial sums of squares of the new residual rows, float32
+    `[ceil(width / 16), 16]`, from which the next norm's scale follows without a pass over the rows."""
+
+    def __init__(self, sums: torch.Tensor):
+        self.sums = sums
+
+
+class UnnormedRows:
+    """Rows that are still to be normed (see `Part`).  `shape` and `dtype` are those of the normed rows.  Read once:
+    either `product(weight, out, bias)` - out = norm(rows) times `weight` (a prepared matrix or a gated pair), plus
+    `bias` if there is one, inside one kernel; False if the kernel set has no such product for these sizes, and then
+    nothing has happened - or `rows()`,
+    the normed rows as a tensor.  After a product that moved the residual sum to another buffer `moved` is True and
+    `stream_out` is where it now lies."""
+
+    shape: tuple
+    dtype: torch.dtype
+    moved = False
+    stream_out = None
+
+    def product(self, weight, out: torch.Tensor, bias: torch.Tensor | None = None) -> bool:
+        raise NotImplementedError
+
+    def rows(self) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class KernelSet:
+    """The optional capabilities a kernel set may offer to the fold protocol; the defaults say "no", and the parts
+    then launch the norm's and the product's own kernels.  (The operations every kernel set must have - `linear`,
+    `add_rmsnorm`, `attention`, ... - are those `kernels/hip.py` defines.)"""
+
+    def folds_norm(self, rows: int, hidden: int, dtype) -> bool:
+        """A step of `rows` rows may let branches add themselves to the residual sum (`linear_adds`) and the next
+        product norm its rows from the sums left there (`linear_scaled`)."""
+        return False
+
+    def adds_to_stream(self, rows: int, weight, dtype) -> bool:
+        """`linear_adds(x, weight, stream, sums, bias=)` exists for this product."""
+        return False
+
+    def norms_rows_in_product(self, rows: int, weight, dtype) -> bool:
+        """`linear_scaled(stream, sums, norm_weight, eps, weight, out, bias=)` exists for this product."""
+        return False
+
+    def norm_in_product(self, rows: int, weight, dtype) -> bool:
+        """`linear_after_norm(stream, delta, norm_weight, eps, stream_out, weight, out, bias=)` exists for this product."""
+        return False
+
+    def measure_products(self, *args, **kwargs) -> dict:
+        """Times the candidates for every prepared product once (`EngineConfig.product_choices = "measure"`)."""
+        return {}

@@ -8,7 +8,7 @@ may instead add its output to the stream inside its last product and hand on the
 from __future__ import annotations
 
 from .base import Part, build_part, register_part
-from .norm import StreamSums
+from .base import StreamSums
 
 
 class PreNormBlock(Part):
@@ -42,9 +42,8 @@ class PreNormBlock(Part):
     def forward(self, stream, pending, ctx, cache, writes_cache=True):
         """stream [tokens, hidden] float32 (updated in place); pending: the previous branch's output, not
         yet added, or None.  Returns this block's own pending output."""
-        folds = getattr(self.rt.kernels, "folds_norm", None)
-        fold = folds is not None and folds(stream.shape[0], self.hidden, self.rt.dtype)
-        later = ctx.fold_into_stream if hasattr(ctx, "fold_into_stream") else False   # whoever comes next takes sums
+        fold = bool(self.rt.kernels.folds_norm(stream.shape[0], self.hidden, self.rt.dtype))
+        later = ctx.fold_into_stream        # whoever reads this block's `pending` takes sums
         normed, unnormed = self._normed(self.mixer_norm, self.mixer, stream, pending, ctx, fold)
         ctx.fold_into_stream = fold         # the mixer's output meets this block's own second norm
         mixed = self.mixer.forward(normed, ctx, cache, writes_cache)
@@ -61,17 +60,18 @@ class PreNormBlock(Part):
         buffer for the residual sum), handed on unnormed to a reader that can take that, whose first product may
         norm the rows itself: one launch less."""
         if isinstance(delta, StreamSums):    # the stream holds the branch's output already; its sums of squares are known
-            if getattr(reader, "takes_pending_norm", False) and hasattr(norm, "scaled"):
-                unnormed = norm.scaled(stream, delta, ctx.arena)
+            unnormed = norm.scaled(stream, delta, ctx.arena) if reader.takes_pending_norm else None
+            if unnormed is not None:
                 return unnormed, unnormed
             normed = ctx.arena.take((stream.shape[0], self.hidden), self.rt.dtype)
             norm.forward_residual(stream, None, normed)
             return normed, None
         # (while branches add themselves to the stream it stays in its buffer: a branch finds it through the context)
-        spare = None if fold else getattr(ctx, "spare_stream", None)
-        if spare is not None and getattr(reader, "takes_pending_norm", False) and hasattr(norm, "pending"):
+        spare = None if fold else ctx.spare_stream
+        if spare is not None and reader.takes_pending_norm:
             unnormed = norm.pending(stream, delta, spare, ctx.arena)
-            return unnormed, unnormed
+            if unnormed is not None:
+                return unnormed, unnormed
         normed = ctx.arena.take((stream.shape[0], self.hidden), self.rt.dtype)
         norm.forward_residual(stream, delta, normed)
         return normed, None

@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import torch
 
-from .base import Part, register_part
+from .base import Part, UnnormedRows, register_part
 from .linear import Linear
 
 
@@ -47,10 +47,10 @@ class SwiGLU(Part):
         """x [tokens, hidden] -> [tokens, hidden], both in the activation dtype."""
         tokens = x.shape[0]
         act = ctx.arena.take((tokens, self.inter), self.rt.dtype)
-        if self.gated is not None and hasattr(x, "product") and x.product(self.gated, act):
+        if self.gated is not None and isinstance(x, UnnormedRows) and x.product(self.gated, act):
             pass                    # the product normed the rows itself
         elif self.gated is not None:
-            if hasattr(x, "rows"):
+            if isinstance(x, UnnormedRows):
                 x = x.rows()
             shape = self.rt.kernels.gated_scratch(self.gated, tokens, self.rt.dtype)
             scratch = ctx.arena.take(shape, self.rt.dtype) if shape is not None else None
@@ -59,7 +59,7 @@ class SwiGLU(Part):
             gate_up = ctx.arena.take((tokens, 2 * self.inter), self.rt.dtype)
             self.gate_up.forward(x, gate_up)
             self.rt.kernels.swiglu(gate_up, act)
-        if getattr(ctx, "fold_into_stream", False):     # the down product adds itself to the residual sum
+        if ctx.fold_into_stream:     # the down product adds itself to the residual sum
             sums = self.down.add_to_stream(act, ctx)
             if sums is not None:
                 return sums

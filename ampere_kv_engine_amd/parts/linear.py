@@ -1,18 +1,26 @@
-"""A weight matrix [out, in] used as y = x W^T (ampere_kv/runner.py:64).  Several matrices that read the
-same input may be stacked along `out` at load; a row of W keeps its own reduction, so stacking changes no
-value."""
+"""A weight matrix [out, in] used as y = x W^T, with a bias [out] where the model has one: y = x W^T + b, formed in
+float32 and rounded once (torch.nn.functional.linear, ampere_kv/runner.py:64-66, :165).  Several matrices that read
+the same input may be stacked along `out` at load, their biases with them; a row of W keeps its own reduction, so
+stacking changes no value."""
 
 from __future__ import annotations
 
 import torch
 
-from ..weights.spec import MATRIX, TensorSpec
-from .base import Part
+from ..weights.spec import BIAS, MATRIX, TensorSpec
+from .base import Part, StreamSums, UnnormedRows
 
 
 class Linear(Part):
-    def __init__(self, runtime, in_features: int, out_features: list[int], names: list[str], role: str = MATRIX):
+    def __init__(self, runtime, in_features: int, out_features: list[int], names: list[str], role: str = MATRIX,
+                 bias: bool = False):
+        """`names`: the matrices' tensor names, each ending in ".weight"; with `bias` every matrix has a vector
+        under the same name ending in ".bias"."""
         self.rt = runtime
+        self.has_bias = bool(bias)
+        self.bias = None            # float32 [sum of outs] (a widening of what the file stores), or None
+        if bias and not all(name.endswith(".weight") for name in names):
+            raise ValueError(f"a bias is named after its matrix, whose name must end in '.weight': {names}")
         self.in_features = in_features
         self.out_features = list(out_features)
         self.names = list(names)
@@ -24,12 +32,23 @@ class Linear(Part):
     def total_out(self) -> int:
         return sum(self.out_features)
 
-    def tensors(self, prefix: str):
+    def _matrices(self, prefix: str):
         return [TensorSpec(prefix + name, (out, self.in_features), self.role, library_copy=True)
                 for name, out in zip(self.names, self.out_features)]
 
+    def _biases(self, prefix: str):
+        if not self.has_bias:
+            return []
+        return [TensorSpec(prefix + name[:-len("weight")] + "bias", (out,), BIAS)
+                for name, out in zip(self.names, self.out_features)]
+
+    def tensors(self, prefix: str):
+        return self._matrices(prefix) + self._biases(prefix)
+
     def load(self, fetch, prefix: str):
-        pieces = [fetch(spec) for spec in self.tensors(prefix)]
+        if self.has_bias:
+            self.bias = torch.cat([fetch(spec).to(torch.float32) for spec in self._biases(prefix)]).contiguous()
+        pieces = [fetch(spec) for spec in self._matrices(prefix)]
         dtypes = {p.dtype for p in pieces}
         if len(dtypes) != 1:
             raise ValueError(f"matrices stacked into one product are stored in different dtypes: "
@@ -41,7 +60,7 @@ class Linear(Part):
         self._adopt(weight)
 
     def _adopt(self, matrix: torch.Tensor):
-        self._bytes = matrix.numel() * matrix.element_size()
+        self._bytes = matrix.numel() * matrix.element_size() + (self.bias.numel() * 4 if self.bias is not None else 0)
         # the kernel set may re-lay the matrix for its matrix cores; the row-major original is then let go
         self.weight = self.rt.kernels.prepare_linear(matrix)
 
@@ -53,20 +72,18 @@ class Linear(Part):
         has a product that does that for a step of this size: returns the `StreamSums` the product left, or None -
         then the caller computes `forward` and hands its output on as before."""
         kernels = self.rt.kernels
-        can = getattr(kernels, "adds_to_stream", None)
-        stream = getattr(ctx, "stream", None)
-        if can is None or stream is None or not can(x.shape[0], self.weight, self.rt.dtype) or stream.shape[1] != self.total_out:
+        stream = ctx.stream
+        if stream is None or stream.shape[1] != self.total_out or not kernels.adds_to_stream(x.shape[0], self.weight, self.rt.dtype):
             return None
-        from .norm import StreamSums
         sums = ctx.arena.take(((self.total_out + 15) // 16, 16), torch.float32)
-        kernels.linear_adds(x, self.weight, stream, sums)
+        kernels.linear_adds(x, self.weight, stream, sums, bias=self.bias)
         return StreamSums(sums)
 
     def forward(self, x, out: torch.Tensor) -> torch.Tensor:
-        """x: [rows, in] in the activation dtype, or rows that are still to be normed (`PendingNorm`)."""
-        if hasattr(x, "product"):
-            if x.product(self.weight, out):
+        """x: [rows, in] in the activation dtype, or rows that are still to be normed (`UnnormedRows`)."""
+        if isinstance(x, UnnormedRows):
+            if x.product(self.weight, out, bias=self.bias):
                 return out
             x = x.rows()
-        self.rt.kernels.linear(x, self.weight, out)
+        self.rt.kernels.linear(x, self.weight, out, bias=self.bias)
         return out

@@ -7,10 +7,10 @@ from __future__ import annotations
 import torch
 
 from ..weights.spec import NORM, TensorSpec
-from .base import Part, register_part
+from .base import Norm, StreamSums, UnnormedRows, register_part  # noqa: F401  (StreamSums is found here too)
 
 
-class RMSNorm(Part):
+class RMSNorm(Norm):
     def __init__(self, spec, runtime):
         self.size = int(spec["size"])
         self.eps = float(spec["eps"])
@@ -48,16 +48,7 @@ class RMSNorm(Part):
         return ScaledNorm(self, stream, sums, arena)
 
 
-class StreamSums:
-    """What a branch hands on instead of its output when its last product has already added that output to the
-    residual sum (`Linear.add_to_stream`): the partial sums of squares of the new residual rows, float32
-    `[ceil(width / 16), 16]`, from which the next norm's scale follows without a pass over the rows."""
-
-    def __init__(self, sums: torch.Tensor):
-        self.sums = sums
-
-
-class ScaledNorm:
+class ScaledNorm(UnnormedRows):
     """norm(stream) for a stream whose sums of squares are at hand, before anybody has computed it.  Like
     `PendingNorm` it is read exactly once, through a `Linear` or the gated product: where the kernel set's product
     norms its rows itself (`linear_scaled`) it does; otherwise the rows are normed by the norm's own kernel."""
@@ -75,13 +66,12 @@ class ScaledNorm:
             raise RuntimeError("rows that were handed on unnormed can be read once")
         self._used = True
 
-    def product(self, weight, out: torch.Tensor) -> bool:
+    def product(self, weight, out: torch.Tensor, bias: torch.Tensor | None = None) -> bool:
         kernels = self.norm.rt.kernels
-        can = getattr(kernels, "norms_rows_in_product", None)
-        if can is None or not can(self.shape[0], weight, out.dtype):
+        if not kernels.norms_rows_in_product(self.shape[0], weight, out.dtype):
             return False
         self._once()
-        kernels.linear_scaled(self.stream, self.sums.sums, self.norm.weight, self.norm.eps, weight, out)
+        kernels.linear_scaled(self.stream, self.sums.sums, self.norm.weight, self.norm.eps, weight, out, bias=bias)
         return True
 
     def rows(self) -> torch.Tensor:
@@ -90,7 +80,7 @@ class ScaledNorm:
         return self.norm.forward_residual(self.stream, None, out)
 
 
-class PendingNorm:
+class PendingNorm(UnnormedRows):
     """The rows norm(stream + delta) before anybody has computed them.  A part that `takes_pending_norm` reads them
     exactly once, through a `Linear` or the kernel set's gated product: where the kernel set's product can norm a few
     rows itself (`norm_in_product`), it does, and the new residual sum is then in `stream_out` (`moved` tells the
@@ -108,15 +98,15 @@ class PendingNorm:
             raise RuntimeError("rows that were handed on unnormed can be read once")
         self._used = True
 
-    def product(self, weight, out: torch.Tensor) -> bool:
-        """out = these rows times `weight` (a packed matrix or a gated pair) if the kernel set computes the norm inside
-        that product; False if the caller has to ask for `rows()` and multiply itself."""
+    def product(self, weight, out: torch.Tensor, bias: torch.Tensor | None = None) -> bool:
+        """out = these rows times `weight` (a packed matrix or a gated pair), plus `bias`, if the kernel set computes
+        the norm inside that product; False if the caller has to ask for `rows()` and multiply itself."""
         kernels = self.norm.rt.kernels
-        can = getattr(kernels, "norm_in_product", None)
-        if can is None or not can(self.shape[0], weight, out.dtype):
+        if not kernels.norm_in_product(self.shape[0], weight, out.dtype):
             return False
         self._once()
-        kernels.linear_after_norm(self.stream, self.delta, self.norm.weight, self.norm.eps, self.stream_out, weight, out)
+        kernels.linear_after_norm(self.stream, self.delta, self.norm.weight, self.norm.eps, self.stream_out, weight, out,
+                                  bias=bias)
         self.moved = True
         return True
 

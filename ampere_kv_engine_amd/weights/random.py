@@ -1,7 +1,7 @@
 """Random-weights mode: draw a model's tensors from a seed and write a model folder.
 
-Laws, by the role a part gives its tensor: matrices and embeddings N(0, 0.02); norm weights 1 + N(0, 0.1); integer
-tables zero.  A part whose tensors follow another law names a role of its own and registers the law
+Laws, by the role a part gives its tensor: matrices, embeddings and biases N(0, 0.02); norm weights 1 + N(0, 0.1);
+integer tables zero.  A part whose tensors follow another law names a role of its own and registers the law
 (`register_init_law`).  Every tensor is drawn in float32 on the host by its own generator, seeded from the folder's
 seed and the tensor's name, so a tensor's values depend on neither the order nor the presence of others; values are
 rounded to bfloat16 once and stored so.
@@ -16,7 +16,7 @@ import os
 import torch
 from safetensors.torch import save_file
 
-from .spec import EMBEDDING, INT_TABLE, MATRIX, NORM, TensorSpec  # noqa: F401
+from .spec import BIAS, EMBEDDING, INT_TABLE, MATRIX, NORM, TensorSpec  # noqa: F401
 
 MATRIX_STD = 0.02
 NORM_STD = 0.1
@@ -37,6 +37,7 @@ _INIT_LAWS = {
     MATRIX: _normal(0.0, MATRIX_STD),
     EMBEDDING: _normal(0.0, MATRIX_STD),
     NORM: _normal(1.0, NORM_STD),
+    BIAS: _normal(0.0, MATRIX_STD),
     INT_TABLE: lambda shape, generator, device: torch.zeros(shape, dtype=torch.int32, device=device),
 }
 

@@ -4,7 +4,7 @@ from __future__ import annotations
 
 from dataclasses import dataclass
 
-MATRIX, NORM, EMBEDDING, INT_TABLE = "matrix", "norm", "embedding", "int_table"
+MATRIX, NORM, EMBEDDING, INT_TABLE, BIAS = "matrix", "norm", "embedding", "int_table", "bias"
 
 
 @dataclass(frozen=True)

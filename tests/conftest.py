@@ -28,7 +28,12 @@ TINY_B = dict(architectures=["Qwen3ForCausalLM"], vocab_size=379, hidden_size=96
 TINY_C = dict(architectures=["Qwen3ForCausalLM"], vocab_size=211, hidden_size=72, num_hidden_layers=2,
               num_attention_heads=6, num_key_value_heads=3, head_dim=64, intermediate_size=104, rope_theta=500000.0,
               rms_norm_eps=1e-6, tie_word_embeddings=False, hidden_act="silu")
-TINY = {"A": (TINY_A, 0, 16), "B": (TINY_B, 1, 8), "C": (TINY_C, 2, 4)}   # config, weight seed, page size
+# A fourth whose attention projections carry biases (`attention_bias`), with widths that are multiples of neither 16 nor
+# 32 where the configuration allows it (heads of 48, a feed-forward of 152).
+TINY_D = dict(architectures=["Qwen3ForCausalLM"], vocab_size=301, hidden_size=80, num_hidden_layers=2,
+              num_attention_heads=4, num_key_value_heads=2, head_dim=48, intermediate_size=152, rope_theta=20000.0,
+              rms_norm_eps=1e-6, tie_word_embeddings=True, attention_bias=True, hidden_act="silu")
+TINY = {"A": (TINY_A, 0, 16), "B": (TINY_B, 1, 8), "C": (TINY_C, 2, 4), "D": (TINY_D, 3, 16)}   # config, weight seed, page size
 
 
 @pytest.fixture(scope="session")

@@ -82,17 +82,19 @@ def attention_mixer(x: torch.Tensor, positions: torch.Tensor, w: dict, *, q_head
                     head_dim: int, eps: float, inv_freq: torch.Tensor, window: int | None = None) -> torch.Tensor:
     """Projection, head split, per-head q/k RMSNorm over d (v is not normed), rotation of q and k after the
     norm, causal attention, head merge, output projection.  ampere_kv/runner.py:64-77 (projection, split,
-    q/k norm), :121 (rotation after the norm), :164-165 (merge and o_proj)."""
+    q/k norm), :121 (rotation after the norm), :164-165 (merge and o_proj).  A projection's bias, where `w` holds
+    one ("q_bias", ...), is added to its product (runner.py:64-66, :165 hand `module.bias` to F.linear)."""
     tokens = x.shape[0]
-    q = (x @ w["q_proj"].T).reshape(tokens, q_heads, head_dim)
-    k = (x @ w["k_proj"].T).reshape(tokens, kv_heads, head_dim)
-    v = (x @ w["v_proj"].T).reshape(tokens, kv_heads, head_dim)
+    project = lambda name: x @ w[name + "_proj"].T + (w[name + "_bias"] if name + "_bias" in w else 0.0)
+    q = project("q").reshape(tokens, q_heads, head_dim)
+    k = project("k").reshape(tokens, kv_heads, head_dim)
+    v = project("v").reshape(tokens, kv_heads, head_dim)
     q = rms_norm(q, w["q_norm"], eps)
     k = rms_norm(k, w["k_norm"], eps)
     q = rope(q, positions, inv_freq)
     k = rope(k, positions, inv_freq)
     merged = causal_attention(q, k, v, window=window).reshape(tokens, q_heads * head_dim)
-    return merged @ w["o_proj"].T
+    return merged @ w["o_proj"].T + (w["o_bias"] if "o_bias" in w else 0.0)
 
 
 def decoder_block(h: torch.Tensor, positions: torch.Tensor, w: dict, **attention_sizes) -> torch.Tensor:
@@ -139,7 +141,11 @@ class PlainQwen3:
             "q_norm": "self_attn.q_norm.weight", "k_norm": "self_attn.k_norm.weight",
             "gate_proj": "mlp.gate_proj.weight", "up_proj": "mlp.up_proj.weight", "down_proj": "mlp.down_proj.weight",
         }
-        return {key: self.w[p + name] for key, name in names.items()}
+        found = {key: self.w[p + name] for key, name in names.items()}
+        for key in "qkvo":              # biases of the four projections, where the file holds them (attention_bias)
+            if f"{p}self_attn.{key}_proj.bias" in self.w:
+                found[key + "_bias"] = self.w[f"{p}self_attn.{key}_proj.bias"]
+        return found
 
     def hidden_states(self, token_ids, run_order=None) -> torch.Tensor:
         ids = torch.as_tensor(token_ids, dtype=torch.long)

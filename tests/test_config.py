@@ -33,7 +33,7 @@ def test_a_missing_size_is_an_error_not_a_default(key):
 
 @pytest.mark.parametrize("change,match", [
     ({"hidden_act": "gelu"}, "hidden_act"), ({"use_sliding_window": True, "sliding_window": 128}, "sliding"),
-    ({"rope_scaling": {"type": "yarn"}}, "rope_scaling"), ({"attention_bias": True}, "attention_bias"),
+    ({"rope_scaling": {"type": "yarn"}}, "rope_scaling"), ({"attention_bias": "yes"}, "attention_bias"),
     ({"num_key_value_heads": 4}, "multiple"), ({"head_dim": 31}, "odd"), ({"vocab_size": -1}, "vocab_size"),
     ({"num_hidden_layers": 2.5}, "num_hidden_layers"), ({"rope_theta": 0}, "rope_theta")])
 def test_unsupported_options_are_refused(change, match):
@@ -150,3 +150,24 @@ def test_layers_share_one_position_table_and_the_memory_plan_counts_it():
     short = plan_memory(spec, EngineConfig(max_seq_len=64, **sizes), 1 << 30)
     long = plan_memory(spec, EngineConfig(max_seq_len=64 + 4096, **sizes), 1 << 30)
     assert long.fixed_bytes - short.fixed_bytes == 4096 * 8 * 2 * 4
+
+
+def test_attention_bias_adds_the_four_bias_vectors_to_every_layer():
+    """`attention_bias: true` (ampere_kv/runner.py:64-66, :165 hand each projection's bias to F.linear): every layer
+    expects q/k/v/o biases beside the 11 tensors, 15 L + 3 in all; the key reads back from `to_dict`."""
+    from ampere_kv_engine_amd.config import Qwen3Config
+    from ampere_kv_engine_amd.engine.model import expected_tensors
+    raw = dict(architectures=["Qwen3ForCausalLM"], vocab_size=100, hidden_size=64, num_hidden_layers=3,
+               num_attention_heads=4, num_key_value_heads=2, head_dim=16, intermediate_size=128, rope_theta=1e4,
+               rms_norm_eps=1e-6, tie_word_embeddings=False, hidden_act="silu", attention_bias=True)
+    config = Qwen3Config.from_dict(raw)
+    assert config.attention_bias and config.to_dict()["attention_bias"] is True
+    assert Qwen3Config.from_dict(config.to_dict()) == config
+    specs = {t.name: t for t in expected_tensors(config.to_model_spec())}
+    assert len(specs) == 15 * 3 + 3
+    assert specs["model.layers.1.self_attn.q_proj.bias"].shape == (64,)
+    assert specs["model.layers.1.self_attn.k_proj.bias"].shape == (32,)
+    assert specs["model.layers.2.self_attn.o_proj.bias"].shape == (64,) and specs["model.layers.2.self_attn.o_proj.bias"].role == "bias"
+    assert not any("mlp" in name and name.endswith("bias") for name in specs)
+    plain = Qwen3Config.from_dict({**raw, "attention_bias": False})
+    assert len(expected_tensors(plain.to_model_spec())) == 11 * 3 + 3

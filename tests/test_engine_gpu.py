@@ -17,7 +17,7 @@ from engine_cases import PROMPTS, tolerance
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(scope="module", params=["A", "B", "C"])
+@pytest.fixture(scope="module", params=["A", "B", "C", "D"])
 def case(request, model_folders):
     return cases.make_case(request.param, model_folders)
 

@@ -7,7 +7,7 @@ import engine_cases as cases
 from torch_kernels import TorchKernels
 
 
-@pytest.fixture(scope="module", params=["A", "B"])
+@pytest.fixture(scope="module", params=["A", "B", "D"])
 def case(request, model_folders):
     return cases.make_case(request.param, model_folders)
 
@@ -39,13 +39,13 @@ def test_branches_that_add_themselves_to_the_residual_sum_give_the_same_bits(cas
     calls = {"adds": 0, "scaled": 0}
 
     class Counting(TorchKernels):
-        def linear_adds(self, *args):
+        def linear_adds(self, *args, **kwargs):
             calls["adds"] += 1
-            return super().linear_adds(*args)
+            return super().linear_adds(*args, **kwargs)
 
-        def linear_scaled(self, *args):
+        def linear_scaled(self, *args, **kwargs):
             calls["scaled"] += 1
-            return super().linear_scaled(*args)
+            return super().linear_scaled(*args, **kwargs)
 
     ordinary = cases.make_engine(case, "bfloat16", "cpu", kernels=TorchKernels())
     folding = cases.make_engine(case, "bfloat16", "cpu", kernels=Counting(fold_rows=16))

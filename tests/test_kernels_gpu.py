@@ -178,6 +178,68 @@ def test_linear_packed(hip_either, ref, y_dtype, rows, outs, k):
     torch.testing.assert_close(got.cpu().float(), want.float(), **t)
 
 
+@pytest.mark.parametrize("outs,k", [(379, 96), (4096, 4096), (1040, 1000), (5136, 2048)])
+def test_products_with_a_bias(hip_either, ref, outs, k, monkeypatch):
+    """y = x W^T + b with the bias added to the float32 sums before they are rounded (one rounding, as
+    torch.nn.functional.linear makes it), through every kernel a product can take: the plain float32 kernel; the
+    engine's own kernels at 1 to 64 rows, the mid-size one, the library or the wide one beyond; the decode products
+    that add themselves to the residual sum, norm their rows (one and two row tiles a wave) or norm their single
+    row.  The bias is large beside the products, so a kernel that drops it, or adds it to the wrong feature, fails."""
+    hip = hip_either
+    monkeypatch.setattr(hip, "fold_norms", True)
+    monkeypatch.setattr(hip, "FOLD_NORM_ROWS", 16)
+    w = rand(outs, k, dtype=torch.bfloat16, seed=36, scale=0.05)
+    bias = rand(outs, dtype=torch.bfloat16, seed=37, scale=0.7).float()     # (as read from a 16-bit file: exact in bfloat16)
+    packed = hip.prepare_linear(w.cuda())
+    for rows in (1, 9, 16, 17, 40, 64, 100, 200, 300, 600):
+        x = rand(rows, k, dtype=torch.bfloat16, seed=38)
+        for y_dtype in DTYPES:
+            want = torch.empty(rows, outs, dtype=y_dtype)
+            ref.linear(x, w, want, bias)
+            got = torch.full((rows, outs), float("nan"), dtype=y_dtype, device="cuda")
+            hip.linear(x.cuda(), packed, got, bias=bias.cuda())
+            t = dict(rtol=2e-4, atol=2e-5 * k ** 0.5) if y_dtype == torch.float32 else tol(torch.bfloat16)
+            torch.testing.assert_close(got.cpu().float(), want.float(), **t, msg=lambda m: f"{rows} rows into {y_dtype}: {m}")
+    # the plain kernel, float32 throughout
+    x32, w32 = rand(70, k, seed=39), w.float()
+    want = torch.empty(70, outs)
+    ref.linear(x32, w32, want, bias)
+    got = torch.empty(70, outs, device="cuda")
+    hip.linear(x32.cuda(), w32.cuda(), got, bias=bias.cuda())
+    torch.testing.assert_close(got.cpu(), want, rtol=1e-4, atol=1e-6 * k ** 0.5)     # (sums of k float32 products)
+    # the decode products
+    for rows in (1, 5, 16):
+        x = rand(rows, k, dtype=torch.bfloat16, seed=40)
+        stream = rand(rows, outs, seed=41, scale=2.0)
+        y = torch.empty(rows, outs, dtype=torch.bfloat16)
+        ref.linear(x, w, y, bias)
+        residual, sums = stream.cuda(), torch.full(((outs + 15) // 16, 16), float("nan"), device="cuda")
+        hip.linear_adds(x.cuda(), packed, residual, sums, bias=bias.cuda())
+        torch.testing.assert_close(residual.cpu(), stream + y.float(), rtol=0, atol=2.0 ** -7 * y.float().abs().max().item())
+        torch.testing.assert_close(sums.cpu().sum(0)[:rows].double(), residual.cpu().double().pow(2).sum(-1), rtol=1e-5, atol=1e-6)
+        if rows * k * 2 > hip.FOLD_NORM_BYTES:
+            continue
+        rows_in = rand(rows, k, seed=42, scale=2.0)
+        gain = 1 + rand(k, seed=43, scale=0.1)
+        squares = torch.zeros((k + 15) // 16, 16)
+        padded = torch.zeros(rows, squares.shape[0] * 16)
+        padded[:, :k] = rows_in
+        squares[:, :rows] = (padded * padded).view(rows, -1, 16).sum(-1).T
+        normed, want = torch.empty(rows, k, dtype=torch.bfloat16), torch.empty(rows, outs, dtype=torch.bfloat16)
+        ref.add_rmsnorm(rows_in.clone(), None, gain, 1e-6, normed)
+        ref.linear(normed, w, want, bias)
+        for row_tiles in (0, 1, 2):
+            got = torch.full((rows, outs), float("nan"), dtype=torch.bfloat16, device="cuda")
+            hip.linear_scaled(rows_in.cuda(), squares.cuda(), gain.cuda(), 1e-6, packed, got, row_tiles=row_tiles, bias=bias.cuda())
+            assert_close_but_for_flipped_roundings(got, want)
+        if rows == 1 and k * 2 <= 48 * 1024:
+            new = torch.empty(rows, k, device="cuda")
+            got = torch.full((rows, outs), float("nan"), dtype=torch.bfloat16, device="cuda")
+            hip.linear_after_norm(rows_in.cuda(), None, gain.cuda(), 1e-6, new, packed, got, bias=bias.cuda())
+            assert_close_but_for_flipped_roundings(got, want)
+    assert int(hip._exchange_arrivals.abs().sum()) == 0
+
+
 def test_linear_packed_rows_do_not_depend_on_the_batch(hip_own):
     hip = hip_own
     """A row's result is bit-identical alone and among up to 64 rows (one kernel), and among more (the other)."""
@@ -634,12 +696,16 @@ def test_mid_size_product(hip_own, ref, rows, outs, k):
     counters = torch.zeros(4096, dtype=torch.int32, device="cuda")
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     xd = x.cuda()
+    bias = rand(outs, seed=83, scale=0.5)
+    bias_d = bias.cuda()
+    plain_want = want
     for along, rt, depth, parts in ((0, 0, 0, 0), (2, 1, 4, 1), (3, 2, 2, 2), (4, 1, 4, 4), (4, 2, 2, 8), (3, 1, 0, 1), (2, 2, 0, 2)):
         for code, dtype in ((1, torch.bfloat16), (0, torch.float32)):
-            for _ in range(2):
+            for with_bias in (False, True):     # (twice: a launch that cuts k over blocks leaves its counters at zero)
+                want = plain_want + bias if with_bias else plain_want
                 got = torch.full((rows, outs), float("nan"), dtype=dtype, device="cuda")
                 status = lib.akv_linear_mid(_ptr(xd), _ptr(packed.data), _ptr(got), code, _ptr(partial), ctypes.c_long(partial.numel()), _ptr(counters), ctypes.c_long(counters.numel()), rows,
-                                            outs, k, packed.n_tiles, packed.k_tiles, 0, along, rt, depth, parts, stream)
+                                            outs, k, packed.n_tiles, packed.k_tiles, 0, along, rt, depth, parts, _ptr(bias_d) if with_bias else None, stream)
                 assert status == 0, (along, rt, depth, parts, status)
                 limits = tol(dtype) if dtype == torch.bfloat16 else dict(rtol=2e-5, atol=2e-5 * float(want.abs().max()))
                 torch.testing.assert_close(got.cpu().float(), want if dtype == torch.float32 else want.bfloat16().float(), **limits,
@@ -650,17 +716,17 @@ def test_mid_size_product(hip_own, ref, rows, outs, k):
     again = torch.empty((rows, outs), dtype=torch.float32, device="cuda")
     for target in (first, again):
         assert lib.akv_linear_mid(_ptr(xd), _ptr(packed.data), _ptr(target), 0, _ptr(partial), ctypes.c_long(partial.numel()), _ptr(counters), ctypes.c_long(counters.numel()), rows, outs, k,
-                                  packed.n_tiles, packed.k_tiles, 0, 4, 1, 4, 4, stream) == 0
+                                  packed.n_tiles, packed.k_tiles, 0, 4, 1, 4, 4, None, stream) == 0
     assert torch.equal(first, again)
     # a ring depth that the row tiles per wave do not allow is refused
     assert lib.akv_linear_mid(_ptr(xd), _ptr(packed.data), _ptr(first), 0, _ptr(partial), ctypes.c_long(partial.numel()), _ptr(counters),
-                              ctypes.c_long(counters.numel()), rows, outs, k, packed.n_tiles, packed.k_tiles, 0, 2, 2, 4, 1, stream) == -2
+                              ctypes.c_long(counters.numel()), rows, outs, k, packed.n_tiles, packed.k_tiles, 0, 2, 2, 4, 1, None, stream) == -2
     # a workspace that is too small for the cut is refused before anything is launched
     need, words = ctypes.c_long(0), ctypes.c_long(0)
     lib.akv_linear_mid_workspace(rows, packed.n_tiles, packed.k_tiles, 0, 4, 1, 4, 4, ctypes.byref(need), ctypes.byref(words))
     assert lib.akv_linear_mid(_ptr(xd), _ptr(packed.data), _ptr(first), 0, _ptr(partial), ctypes.c_long(16), _ptr(counters),
                               ctypes.c_long(counters.numel()), rows, outs, k, packed.n_tiles, packed.k_tiles, 0, 4, 1, 4, 4,
-                              stream) == (-3 if need.value > 16 else 0)
+                              None, stream) == (-3 if need.value > 16 else 0)
 
 
 @pytest.mark.parametrize("rows,inter,k", [(40, 208, 264), (64, 512, 2048), (130, 208, 520), (17, 16, 8), (256, 1024, 1024),
@@ -680,7 +746,7 @@ def test_mid_size_gated_product(hip_own, ref, rows, inter, k):
     for along, parts in ((0, 0), (2, 1), (3, 2), (4, 4)):
         got = torch.full((rows, inter), float("nan"), dtype=torch.bfloat16, device="cuda")
         assert lib.akv_linear_mid(_ptr(x.cuda()), _ptr(weight.packed.data), _ptr(got), 1, _ptr(partial), ctypes.c_long(partial.numel()), _ptr(counters), ctypes.c_long(counters.numel()), rows,
-                                  inter, k, weight.packed.n_tiles, weight.packed.k_tiles, 1, along, 2, 2, parts, stream) == 0
+                                  inter, k, weight.packed.n_tiles, weight.packed.k_tiles, 1, along, 2, 2, parts, None, stream) == 0
         torch.testing.assert_close(got.cpu().float(), want.float(), **tol(torch.bfloat16))
     assert int(counters.abs().sum()) == 0
 

@@ -139,7 +139,9 @@ def test_seventy_requests_through_the_scheduler_at_qwen3_8b_layer_sizes(two_laye
     for request, prompt in zip(requests, prompts):
         assert len(request.output_ids) == new and request.stop_reason == "reached limit"
         if dtype == "float32":          # a row's arithmetic does not depend on its batch: the plain implementation's tokens
-            assert request.output_ids == plain.greedy(prompt, new), request.request_id
+            # (each token is the plain implementation's best given the tokens before it: by induction its greedy tokens)
+            best = plain.logits(prompt + request.output_ids[:-1])[len(prompt) - 1:].argmax(-1).tolist()
+            assert request.output_ids == best, request.request_id
             continue
         logits = plain.logits(prompt + request.output_ids[:-1])[len(prompt) - 1:]
         top = cases.scales(logits)[0]

@@ -179,6 +179,33 @@ def test_v_is_neither_normed_nor_rotated_and_q_k_are_normed_per_head(plain_b):
     torch.testing.assert_close(moved, base, rtol=1e-4, atol=1e-7)
 
 
+def test_projection_biases_enter_before_the_norm_and_after_the_output_product():
+    """With `attention_bias` the four projections are torch.nn.functional.linear(x, W, b) (ampere_kv/runner.py:64-66,
+    :165).  Pinned by special cases: zero matrices for q, k and v leave the biases alone - every key is then the same
+    vector, every position's weights are uniform and the mixer returns o(b_v) + b_o, whatever x is; a q bias enters
+    before the per-head norm, so scaling W_q and b_q together changes nothing; and the o bias is added once, not per
+    head."""
+    torch.manual_seed(3)
+    q_heads, kv_heads, d, hidden = 4, 2, 8, 24
+    sizes = dict(q_heads=q_heads, kv_heads=kv_heads, head_dim=d, eps=1e-30, inv_freq=P.rope_inverse_frequencies(d, 1e4))
+    w = {"q_proj": torch.randn(q_heads * d, hidden, dtype=torch.float64), "k_proj": torch.randn(kv_heads * d, hidden, dtype=torch.float64),
+         "v_proj": torch.randn(kv_heads * d, hidden, dtype=torch.float64), "o_proj": torch.randn(hidden, q_heads * d, dtype=torch.float64),
+         "q_norm": torch.ones(d, dtype=torch.float64), "k_norm": torch.ones(d, dtype=torch.float64),
+         "q_bias": torch.randn(q_heads * d, dtype=torch.float64), "k_bias": torch.randn(kv_heads * d, dtype=torch.float64),
+         "v_bias": torch.randn(kv_heads * d, dtype=torch.float64), "o_bias": torch.randn(hidden, dtype=torch.float64)}
+    x, positions = torch.randn(7, hidden, dtype=torch.float64), torch.arange(7)
+    zeroed = {**w, "q_proj": 0 * w["q_proj"], "k_proj": 0 * w["k_proj"], "v_proj": 0 * w["v_proj"]}
+    values = w["v_bias"].view(kv_heads, d).repeat_interleave(q_heads // kv_heads, dim=0).reshape(-1)   # head h reads kv head h // 2
+    want = torch.nn.functional.linear(values, w["o_proj"], w["o_bias"])
+    torch.testing.assert_close(P.attention_mixer(x, positions, zeroed, **sizes), want.expand(7, -1))
+    base = P.attention_mixer(x, positions, w, **sizes)
+    torch.testing.assert_close(P.attention_mixer(x, positions, {**w, "q_proj": 3 * w["q_proj"], "q_bias": 3 * w["q_bias"]}, **sizes), base)
+    assert not torch.allclose(P.attention_mixer(x, positions, {**w, "q_bias": 3 * w["q_bias"]}, **sizes), base)
+    without = {k: v for k, v in w.items() if not k.endswith("_bias")}
+    only_o = P.attention_mixer(x, positions, {**without, "o_bias": w["o_bias"]}, **sizes)
+    torch.testing.assert_close(only_o, P.attention_mixer(x, positions, without, **sizes) + w["o_bias"])
+
+
 # ---- whole model ------------------------------------------------------------------------------------------------------
 def test_logits_are_causal_and_tied_head_is_the_embedding(model_folders):
     raw_a = TINY["A"][0]

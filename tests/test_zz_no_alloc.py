@@ -34,7 +34,7 @@ def test_the_product_without_allocation_equals_the_one_with_a_buffer():
             got = torch.full((rows, outs), float("nan"), dtype=dtype, device="cuda")
             assert lib.akv_pack_rows(_pointer(x), _pointer(staged), rows, k, stream) == 0
             assert lib.akv_linear_packed(_pointer(staged), _pointer(weight.data), _pointer(want), code, rows, outs, k,
-                                         weight.n_tiles, weight.k_tiles, 1, stream) == 0
+                                         weight.n_tiles, weight.k_tiles, 1, None, stream) == 0
             torch.cuda.synchronize()
             before = torch.cuda.memory_stats()["allocation.all.allocated"]
             assert lib.akv_linear_packed_static(_pointer(x), _pointer(weight.data), _pointer(got), code, rows, outs, k,

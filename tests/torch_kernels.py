@@ -13,12 +13,14 @@ import math
 import numpy as np
 import torch
 
+from ampere_kv_engine_amd.parts.base import KernelSet
+
 
 def _round(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     return x.to(dtype)
 
 
-class TorchKernels:
+class TorchKernels(KernelSet):
     name = "torch-double"
 
     def __init__(self, fold_rows: int = 0):
@@ -74,8 +76,9 @@ class TorchKernels:
     def prepare_linear(self, matrix):
         return matrix
 
-    def linear(self, x, weight, out):
-        out.copy_((x.float() @ weight.float().T).to(out.dtype))
+    def linear(self, x, weight, out, bias=None):
+        y = x.float() @ weight.float().T
+        out.copy_((y if bias is None else y + bias.float()).to(out.dtype))
 
     def prepare_gated_linear(self, gate, up):
         return (gate, up)
@@ -91,9 +94,9 @@ class TorchKernels:
         matrix = weight[0] if isinstance(weight, tuple) else weight
         return isinstance(matrix, torch.Tensor) and self.folds_norm(rows, matrix.shape[1], dtype)
 
-    def linear_adds(self, x, weight, stream, sums):
+    def linear_adds(self, x, weight, stream, sums, bias=None):
         y = torch.empty(x.shape[0], weight.shape[0], dtype=x.dtype)
-        self.linear(x, weight, y)
+        self.linear(x, weight, y, bias)
         stream += y.float()
         rows, outs = stream.shape
         padded = torch.zeros(rows, sums.shape[0] * 16)
@@ -101,14 +104,14 @@ class TorchKernels:
         sums.zero_()
         sums[:, :rows] = (padded * padded).view(rows, -1, 16).sum(-1).T
 
-    def linear_scaled(self, stream, sums, norm_weight, eps, weight, out):
+    def linear_scaled(self, stream, sums, norm_weight, eps, weight, out, bias=None):
         rows, k = stream.shape
         scale = torch.rsqrt(sums.sum(0)[:rows, None] / k + eps)
         normed = _round(_round(stream * scale, out.dtype).float() * norm_weight, out.dtype)
         if isinstance(weight, tuple):
             self.gated_linear(normed, weight, out)
         else:
-            self.linear(normed, weight, out)
+            self.linear(normed, weight, out, bias)
 
     def gated_scratch(self, weight, rows, dtype):
         return None
