@@ -9,6 +9,8 @@ extern "C" {
 
 int akv_embed(const int* ids, const void* table, int table_dtype, float* out, int tokens, int hidden, int vocab,
               const int* seq_of_token, const int* seq_slots, const int* slot_words, hipStream_t stream);
+// out[0..7]: words per slot and the indices of its named words, as the kernels were compiled (see common.h)
+int akv_slot_layout(int* out);
 int akv_step_prologue(int* state, long state_size, const int* patches, const int* count, int capacity,
                       const int* seq_slots, const int* seq_lens, int seqs, hipStream_t stream);
 int akv_add_rmsnorm(float* stream_buf, const void* delta, const float* weight, float eps, void* out, int dtype,

@@ -63,6 +63,19 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 
 enum DType : int { kF32 = 0, kBF16 = 1 };
 
+// Per-request state of fixed size on the device: kSlotWords 32-bit words per slot.  This is the one definition for
+// the kernels; the host's (cache/slots.py) is checked against it when the library is loaded (akv_slot_layout).
+constexpr int kSlotWords = 8;
+enum SlotWord : int {
+  kSlotLength = 0,       // tokens held
+  kSlotLastToken = 1,    // the token chosen last (-1: none yet)
+  kSlotTemperature = 2,  // float bits
+  kSlotSeedLow = 3,
+  kSlotSeedHigh = 4,
+  kSlotDraws = 5,        // draws made so far
+  kSlotTaken = 6,        // whether a request holds the slot
+};
+
 // Blocks of one launch that hand sums to each other through memory do it in three steps.  (1) The sums are written
 // with device-scope atomic stores (`publish`): such a store goes through to where every XCD sees it.  (2) The block
 // ticks a counter with `arrive`: first a wait until the wave's memory counters are at zero - every store it has

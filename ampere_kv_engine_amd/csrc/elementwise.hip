@@ -11,11 +11,7 @@ using namespace akv;
 
 namespace {
 
-// ---- per-request state of fixed size: SLOT_WORDS 32-bit words per slot -----------------------------------------
-// word 0 tokens held, 1 the token chosen last (-1: none yet), 2 temperature (float bits), 3 and 4 the seed's low
-// and high half, 5 draws made so far, 6 whether a request holds the slot.
-constexpr int kSlotWords = 8;
-constexpr int kSlotLength = 0, kSlotLastToken = 1;
+// ---- per-request state of fixed size: kSlotWords 32-bit words per slot (the words are named in common.h) -----------
 
 // What a step changes in the persistent integer state before its first kernel reads it: `count` (offset, value) pairs
 // - block-table entries of pages the step's requests were given or gave back - and the requests' new lengths.
@@ -658,3 +654,11 @@ int akv_qk_norm_rope_write(const void* qkv, const float* q_weight, const float* 
 }
 
 }  // extern "C"
+
+// The slot layout the kernels were compiled with: out[0] = words per slot, out[1..7] = the indices of length, last
+// token, temperature, seed low, seed high, draws, taken.  The host checks its own layout against this at load.
+extern "C" int akv_slot_layout(int* out) {
+  out[0] = kSlotWords, out[1] = kSlotLength, out[2] = kSlotLastToken, out[3] = kSlotTemperature, out[4] = kSlotSeedLow;
+  out[5] = kSlotSeedHigh, out[6] = kSlotDraws, out[7] = kSlotTaken;
+  return 0;
+}

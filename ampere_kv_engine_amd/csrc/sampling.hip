@@ -33,8 +33,8 @@ __device__ __forceinline__ uint32_t philox_first(uint32_t c0, uint32_t c1, uint3
 
 // SLOTS: the sampling state is not handed in row by row but read from (and written to) the slot of the row's request:
 // the row's token row is rows_of[row], its request seq_of_token[...], its slot seq_slots[...]; slot words 2..5 hold
-// temperature, seed and draws made so far, word 1 receives the chosen token and word 5 counts the draw.
-constexpr int kSlotWords = 8;
+// temperature, seed and draws made so far, word 1 receives the chosen token and word 5 counts the draw (the words are
+// named in common.h).
 
 template <bool SLOTS>
 __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ logits,
@@ -57,10 +57,10 @@ __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ 
   int* words = nullptr;
   if constexpr (SLOTS) {
     words = slot_words + static_cast<size_t>(seq_slots[seq_of_token[rows_of[row]]]) * kSlotWords;
-    t = __int_as_float(words[2]);
-    k0 = static_cast<uint32_t>(words[3]);
-    k1 = static_cast<uint32_t>(words[4]);
-    draw = static_cast<uint32_t>(words[5]);
+    t = __int_as_float(words[kSlotTemperature]);
+    k0 = static_cast<uint32_t>(words[kSlotSeedLow]);
+    k1 = static_cast<uint32_t>(words[kSlotSeedHigh]);
+    draw = static_cast<uint32_t>(words[kSlotDraws]);
     __syncthreads();   // every thread has read the state before thread 0 writes it below
   } else {
     t = temperature != nullptr ? temperature[row] : 0.f;
@@ -132,8 +132,8 @@ __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ 
     const int token = (index < vocab && any_nan == 0) ? index : -1;
     out[row] = token;
     if constexpr (SLOTS) {
-      words[1] = token;
-      words[5] = static_cast<int>(draw + 1u);
+      words[kSlotLastToken] = token;
+      words[kSlotDraws] = static_cast<int>(draw + 1u);
     }
   }
 }

@@ -115,6 +115,7 @@ class StepContext:
     host_seq_slots: list[int] = field(default_factory=list)
     max_seq_len: int = 0           # longest request of the step, after the step
     max_new_tokens: int = 0        # longest portion of the step
+    most_wanted: int = 0           # the most places any one request wants logits at
     arenas: tuple = ()             # two arenas used by alternate layers (a layer's output outlives its own arena's reset)
     stream_buffer: torch.Tensor | None = None   # float32 [max tokens, hidden]: the residual sum
     spare_buffer: torch.Tensor | None = None    # float32 [a few rows, hidden]: where a small step may move it
@@ -298,6 +299,7 @@ class BatchBuilder:
             host_q_start=[int(x) for x in q_start[:r + 1]], host_seq_lens=[int(x) for x in seq_lens[:r]],
             host_seq_slots=[int(x) for x in seq_slots[:r]],
             max_seq_len=int(seq_lens[:r].max()), max_new_tokens=max(len(e.tokens) for e in ordered),
+            most_wanted=max(len(e.want) for e in ordered),
             arenas=self.arenas, table_pages=width, patches=dev(s_pa), patch_count=dev(s_pc), patch_room=patch_room,
             slot_state=arrays.state if arrays is not None else None,
             slot_words=arrays.words if arrays is not None else None,

@@ -131,7 +131,8 @@ class Engine:
         drawn, by the temperature, seed and draw count that the row's request keeps in its slot on the device.  The
         kernel leaves the chosen token and the new draw count in the slot - `StepEntry(seq, LAST_TOKEN)` feeds that
         token without the host sending it - and nothing is uploaded for the choice; one copy brings the tokens to
-        the host.  `NO_TOKEN` (-1) for a row that holds a NaN or no finite logit.  At most one wanted row per request."""
+        the host.  `NO_TOKEN` (-1) for a row that holds a NaN or no finite logit.  At most one wanted row per request
+        (more are refused)."""
         ctx = getattr(self, "_last_step", None)
         if ctx is None or logits is None or logits.shape[0] != ctx.logit_rows.shape[0]:
             raise ValueError("choose() takes the logits of the step that was run last")

@@ -142,6 +142,19 @@ class HipKernels(KernelSet):
                      "akv_linear_adds", "akv_linear_scaled", "akv_linear_decode_plan", "akv_read_probe",
                      "akv_attention_rows", "akv_decode_plan", "akv_sample", "akv_sample_slots", "akv_step_prologue"):
             getattr(self.lib, name).restype = ctypes.c_int
+        self._check_slot_layout()
+
+    def _check_slot_layout(self) -> None:
+        """The words of a request's slot are laid out once for the kernels (csrc/common.h) and once for the host
+        (cache/slots.py): a library built from another layout would read a seed as a temperature, so it is refused."""
+        from ..cache import slots
+        layout = (ctypes.c_int * 8)()
+        self.lib.akv_slot_layout(layout)
+        host = (slots.SLOT_WORDS, slots.WORD_LENGTH, slots.WORD_LAST_TOKEN, slots.WORD_TEMPERATURE, slots.WORD_SEED_LOW,
+                slots.WORD_SEED_HIGH, slots.WORD_DRAWS, slots.WORD_TAKEN)
+        if tuple(layout) != host:
+            raise KernelError(f"the kernel library lays a request's slot out as {tuple(layout)} (words, then the indices of "
+                              f"length, last token, temperature, seed low, seed high, draws, taken); the host as {host}")
 
     # ---- helpers -----------------------------------------------------------------------------------------
     def _stream(self):
@@ -285,6 +298,10 @@ class HipKernels(KernelSet):
     def prepare_linear(self, matrix: torch.Tensor):
         """bfloat16 matrices whose k is a multiple of 8 are packed for the MFMA kernels; others stay row-major and
         go through the plain tiled kernel."""
+        if matrix.dtype == torch.bfloat16 and matrix.shape[1] % 8 != 0:
+            self._warn_once(("k", matrix.shape[1]), f"a bfloat16 matrix of {matrix.shape[0]} x {matrix.shape[1]}: its inner width is no "
+                            "multiple of 8, so its products run in the plain float32 kernel instead of the matrix cores "
+                            "(correct, and many times slower)")
         if matrix.dtype == torch.bfloat16 and matrix.shape[1] % 8 == 0:
             weight = PackedWeight(matrix, keep_row_major=self.library_products_above is not None)
             self._products.setdefault(("linear", weight.outs, weight.k), weight)
@@ -882,8 +899,20 @@ class HipKernels(KernelSet):
         return blocks >= 2 * units and (ctx.max_seq_len >= 4096 or 2 * blocks >= 5 * units)
 
     def _matrix_core_attention(self, dtype, page_size) -> bool:
-        return (dtype == torch.bfloat16 and page_size >= 4 and page_size & (page_size - 1) == 0
-                and not self.one_wave_per_head)
+        fits = page_size >= 4 and page_size & (page_size - 1) == 0
+        if dtype == torch.bfloat16 and not fits and not self.one_wave_per_head:
+            self._warn_once(("page", page_size), f"cache pages of {page_size} tokens: the matrix-core attention takes pages of "
+                            "4 tokens or more whose size is a power of two, so bfloat16 attention runs in the plain kernel, "
+                            "one wave per token and head (correct, and many times slower)")
+        return dtype == torch.bfloat16 and fits and not self.one_wave_per_head
+
+    def _warn_once(self, key, message: str) -> None:
+        """A kernel choice that keeps results right and costs much speed is said once, not silently made."""
+        told = self.__dict__.setdefault("_told", set())
+        if key not in told:
+            told.add(key)
+            import warnings
+            warnings.warn(message, RuntimeWarning, stacklevel=3)
 
     def encode_and_attend(self, qkv, q_weight, k_weight, eps, table, positions, slot_map, k_pages, v_pages, q, ctx,
                           meta, q_heads, kv_heads, head_dim, scale, window, out):

@@ -94,6 +94,11 @@ class SlotSampler:
         rows = logits.shape[0]
         if rows > self.max_rows:
             raise ValueError(f"{rows} rows to choose from; the sampler was built for {self.max_rows}")
+        if ctx.most_wanted > 1:
+            # (the kernel reads and advances a request's draw count and last token once per row: two rows of one
+            # request would race on them and draw with the same counter)
+            raise ValueError("a request wants logits at several places of this step: a token can be chosen for one "
+                             "place per request")
         out = self._out[:rows]
         self.kernels.sample_slots(logits, ctx, out)
         if self.device.type != "cuda":

@@ -193,3 +193,16 @@ def test_a_step_is_checked_in_the_order_its_requests_register():
     builder.build([StepEntry(young, [0], [0])])
     m.close(old), m.close(young)
     assert m.num_free_pages == [5]
+
+
+def test_the_kernels_and_the_host_lay_a_slot_out_alike():
+    """The words of a request's slot are named once for the kernels (csrc/common.h) and once for the host
+    (cache/slots.py); the library reports its layout and the kernel set refuses one that differs from the host's."""
+    import ctypes
+    from ampere_kv_engine_amd.cache import slots
+    from ampere_kv_engine_amd.csrc.build import ensure_built
+    lib = ctypes.CDLL(ensure_built())
+    layout = (ctypes.c_int * 8)()
+    assert lib.akv_slot_layout(layout) == 0
+    assert tuple(layout) == (slots.SLOT_WORDS, slots.WORD_LENGTH, slots.WORD_LAST_TOKEN, slots.WORD_TEMPERATURE,
+                             slots.WORD_SEED_LOW, slots.WORD_SEED_HIGH, slots.WORD_DRAWS, slots.WORD_TAKEN)

@@ -424,3 +424,18 @@ def test_a_cancelled_or_expired_waiting_request_ends_the_overlap(model_folders):
     scheduler.run_until_idle()
     assert first.stop_reason == STOP_LIMIT and len(first.output_ids) == 12
     assert engine.cache.num_free_pages == [3] and scheduler.reserved_pages == [0]
+
+
+def test_a_token_is_chosen_for_one_place_per_request(model_folders):
+    """`Engine.choose` advances a request's draw count and last token once per wanted row; two wanted rows of one
+    request would race on them, so such a choice is refused on the host."""
+    from ampere_kv_engine_amd.engine import StepEntry
+    raw, _, page = TINY["A"]
+    engine = make_engine(model_folders["A"], page, 8)
+    seq = engine.open("r")
+    logits = engine.step([StepEntry(seq, random_ids(raw["vocab_size"], 6, seed=1), [2, 5])])
+    with pytest.raises(ValueError, match="one\\s+place per request"):
+        engine.choose(logits)
+    logits = engine.step([StepEntry(seq, [7], [0])])
+    assert len(engine.choose(logits)) == 1
+    engine.close(seq)
