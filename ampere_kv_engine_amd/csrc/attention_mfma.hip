@@ -1064,16 +1064,12 @@ __global__ __launch_bounds__(64 * kSharedWaves, D <= 128 ? (NQ == 1 ? 3 : 2) : 1
   const int calm_from = a.window > 0 ? (max(range_lo, last_pos - a.window + 1) + 31) & ~31 : first_base;
   // base < calm_to: base + 95 <= range_hi, and base + 31 <= the block's first position
   const int calm_to = same_page ? min(range_hi - 94, t.first_pos - 30) : first_base;
-  int buffer = 0;
-  for (int base = first_base; base <= range_hi; base += 32, buffer ^= 1) {
-    if (base >= calm_from && base < calm_to) {
-      fetch_inside(base + 32, pages, kst, vst);
-      lookup(base + 64, pages, unchecked);
-      if (wave_active) step(base, buffer, unchecked);
-      stash(buffer ^ 1, kst, vst);
-      __syncthreads();
-      continue;
-    }
+  // Three loops, one after the other, instead of one with a test per step: steps before the calm ones (a window's
+  // first steps), the calm ones, and those after.  In a loop of its own the calm step's sums stay in their registers
+  // from step to step (in a loop shared with the other kinds of step the compiler copied all of them at every turn);
+  // a wave without tokens runs the same loops without the arithmetic.
+  int buffer = 0, base = first_base;
+  auto ordinary_step = [&](int base, int buffer) {
     const bool more = base + 32 <= range_hi;
     if (more) fetch_step(base + 32);
     if (base + 64 <= range_hi) lookup_step(base + 64);
@@ -1086,7 +1082,25 @@ __global__ __launch_bounds__(64 * kSharedWaves, D <= 128 ? (NQ == 1 ? 3 : 2) : 1
     }
     if (more) stash(buffer ^ 1, kst, vst);
     __syncthreads();
+  };
+  for (; base <= range_hi && base < calm_from; base += 32, buffer ^= 1) ordinary_step(base, buffer);
+  if (wave_active) {
+    for (; base < calm_to; base += 32, buffer ^= 1) {
+      fetch_inside(base + 32, pages, kst, vst);
+      lookup(base + 64, pages, unchecked);
+      step(base, buffer, unchecked);
+      stash(buffer ^ 1, kst, vst);
+      __syncthreads();
+    }
+  } else {
+    for (; base < calm_to; base += 32, buffer ^= 1) {
+      fetch_inside(base + 32, pages, kst, vst);
+      lookup(base + 64, pages, unchecked);
+      stash(buffer ^ 1, kst, vst);
+      __syncthreads();
+    }
   }
+  for (; base <= range_hi; base += 32, buffer ^= 1) ordinary_step(base, buffer);
   if (bad) bad_page = 1;
   __syncthreads();
   const bool poisoned = bad_page != 0;

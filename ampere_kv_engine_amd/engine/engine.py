@@ -57,7 +57,7 @@ class Engine:
                                         device=self.device)
         self.loaded = False
         self._chooser = None
-        self._graphs: dict[tuple, object] = {}               # (tokens per request, wanted rows, table width) -> graph
+        self._graphs: dict[tuple, object] = {}               # (tokens per request, wanted rows, table width, portions' bound) -> graph
         self._graph_logits = None                            # [max_seqs, vocab] float32, where recorded steps write
         self._recordable = (engine_config.decode_graphs and self.device.type == "cuda" and all(
             part.graph_safe for block in self.model.blocks for part in (block, block.mixer, block.feed_forward)))
@@ -171,6 +171,7 @@ class Engine:
                                  f"of {vocab}")
 
     # ---- steps as recorded graphs -----------------------------------------------------------------------------
+    PORTION_BOUND = 1024          # recorded steps: the smallest bound on the length of a request that brings a portion
     SPARE_STREAM_ROWS = 1         # steps of up to this many tokens may move the residual sum between two buffers (what
                                   # the one-row product that norms its own row needs: a fact of that kernel, not a setting)
 
@@ -199,11 +200,21 @@ class Engine:
         ctx.stream_buffer, ctx.spare_buffer = self.stream_buffer, self.spare_buffer
         self._last_step = ctx
         width = ctx.table_pages        # the longest request's pages, rounded up: a bound the recording is made for
-        key = (counts, wanted, width)
-        # sizes of launches come from the bound, not from this step's lengths
+        # sizes of launches come from bounds, not from this step's lengths: single tokens from the longest request's
+        # bound; prompt portions from a bound of their own - the longest of them rounded up to a power of two (from
+        # PORTION_BOUND tokens on) - so that a short prompt arriving beside long decoding requests is not cut into
+        # segments, and given partial results, as if it had their history
         bound = max(width * self.config.page_size, 1)
+        decodes = ctx.num_decode_seqs
+        portion_bound = None
+        if decodes < ctx.num_seqs:
+            portion_bound = self.PORTION_BOUND
+            while portion_bound < max(ctx.host_seq_lens[decodes:]):
+                portion_bound *= 2
+            portion_bound = min(portion_bound, bound)
+        key = (counts, wanted, width, portion_bound)
         ctx.max_seq_len = bound
-        ctx.host_seq_lens = [bound] * ctx.num_seqs
+        ctx.host_seq_lens = [bound] * decodes + [portion_bound] * (ctx.num_seqs - decodes)
         if self._graph_logits is None:  # one buffer for every recording: a recorded step's logits are its first rows
             self._graph_logits = torch.empty((self.config.max_seqs, self.spec.vocab_size), dtype=torch.float32,
                                              device=self.device)

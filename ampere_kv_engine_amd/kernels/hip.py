@@ -872,7 +872,9 @@ class HipKernels(KernelSet):
     def _few_portion_blocks(self, ctx, first, q_heads, kv_heads) -> bool:
         """Whether the prompt portions of the step are so short, and their histories so long, that blocks of four
         tiles would leave most compute units idle while each walks thousands of keys: then a wave takes a tile and a
-        segment of the keys, as in decoding.  Measured at Qwen3-8B sizes, blocks of four tiles against cut keys:
+        segment of the keys, as in decoding.  The histories are those of the portions' own requests (in a recorded
+        step a bound on them), not of the single tokens beside them.  Measured at Qwen3-8B sizes, blocks of four tiles
+        against cut keys:
         128 tokens after 4,096: 114 / 63 us; 64 after 8,192: 221 / 65; 32 after 16,384: 437 / 70; but 256 after
         2,048: 67 / 77, 128 after 1,024: 37 / 41, 512 after 4,096: 128 / 195."""
         group = q_heads // kv_heads
@@ -881,7 +883,7 @@ class HipKernels(KernelSet):
         starts = ctx.host_q_start
         blocks = sum((starts[r + 1] - starts[r] + per_block - 1) // per_block for r in range(first, ctx.num_seqs))
         blocks *= kv_heads * ((group + heads_per_tile - 1) // heads_per_tile)
-        return 4 * blocks <= self.compute_units and ctx.max_seq_len >= 2048
+        return 4 * blocks <= self.compute_units and max(ctx.host_seq_lens[first:ctx.num_seqs]) > 2048
 
     def _wide_shared_tiles(self, ctx, first, q_heads, kv_heads) -> bool:
         """Whether the prompt portions of the step go to blocks of 4 x 32 columns rather than 4 x 16.  The wide
@@ -896,7 +898,7 @@ class HipKernels(KernelSet):
         blocks = sum((starts[r + 1] - starts[r] + per_block - 1) // per_block for r in range(first, ctx.num_seqs))
         blocks *= kv_heads * ((group + heads_per_tile - 1) // heads_per_tile)
         units = self.compute_units
-        return blocks >= 2 * units and (ctx.max_seq_len >= 4096 or 2 * blocks >= 5 * units)
+        return blocks >= 2 * units and (max(ctx.host_seq_lens[first:ctx.num_seqs]) >= 4096 or 2 * blocks >= 5 * units)
 
     def _matrix_core_attention(self, dtype, page_size) -> bool:
         fits = page_size >= 4 and page_size & (page_size - 1) == 0

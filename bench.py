@@ -11,7 +11,9 @@ with random keys and values: what they hold does not change the time a step take
   value     decoded tokens per second at the default batch
   prefill   one request's 2,048-token prompt fed whole: tokens/s, ms, and flops / time / bf16 MFMA peak
   roofline  bytes a decode step has to read (every weight once + the live requests' cache) / its time / HBM peak
-  points    decoded tokens per second at batch 1 and 64; milliseconds of a step that feeds 120 tokens of a prompt beside
+  points    decoded tokens per second at batch 1 and 64; the same three batch sizes with caches of 2,048 tokens, where the
+            weights are most of what a step reads, each with its bytes / time / HBM peak (`..._frac`); milliseconds of a
+            step that feeds 120 tokens of a prompt beside
             the batch's decoding requests; prefill tokens per second with every product in the engine's
             own kernels (by default bfloat16 products of more than 16 rows go to the BLAS library); hbm_read_gbs,
             what a kernel that only reads draws from this device's memory (the ceiling to hold `roofline` against)
@@ -45,6 +47,7 @@ QWEN3_8B = dict(architectures=["Qwen3ForCausalLM"], num_hidden_layers=36, hidden
 QWEN3_14B = dict(QWEN3_8B, num_hidden_layers=40, hidden_size=5120, num_attention_heads=40, intermediate_size=17408)
 QWEN3_32B = dict(QWEN3_8B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, intermediate_size=25600)
 PAGE_SIZE, CONTEXT, PREFILL_TOKENS = 16, 8192, 2048
+SHORT_CONTEXT = 2048    # decoding right after such a prompt is timed too (points decode_b*_ctx2048)
 PRIMING = 3   # untimed steps before the warm-up steps: the first runs eagerly, the second is recorded, the third replays
 HBM_PEAK_GBS, BF16_PEAK_FLOPS = 8000.0, 2.5e15
 
@@ -210,12 +213,12 @@ def main() -> int:
     generator = torch.Generator().manual_seed(0)
     sync = lambda: torch.cuda.synchronize(engine.device)
 
-    def decode(batch: int, steps: int, warmup: int) -> tuple[float, list[float]]:
-        """Seconds for `steps` decode steps of `batch` requests whose caches hold `context` tokens, and the moments
-        (seconds since the start) at which each step's tokens were on the host."""
+    def decode(batch: int, steps: int, warmup: int, context: int | None = None) -> tuple[float, list[float]]:
+        """Seconds for `steps` decode steps of `batch` requests whose caches hold `context` tokens (default: the
+        run's), and the moments (seconds since the start) at which each step's tokens were on the host."""
         seqs = [engine.open(f"b{batch}_{i}") for i in range(batch)]
         for index, seq in enumerate(seqs):
-            engine.cache.reserve(seq, (contexts[index] if contexts is not None else args.context) - 1)
+            engine.cache.reserve(seq, (context or (contexts[index] if contexts is not None else args.context)) - 1)
         first = torch.randint(0, config.vocab_size, (batch,), generator=generator).tolist()
         logits = engine.step([StepEntry(seq, [token], [0]) for seq, token in zip(seqs, first)], borrow_logits=True)
         engine.choose(logits)
@@ -311,8 +314,14 @@ def main() -> int:
     value = args.batch * args.steps / elapsed
     weight_bytes = engine.model.weight_bytes_per_step()
     held = sum(contexts) if contexts is not None else args.batch * args.context
-    kv_bytes = (held + args.batch * (PRIMING + args.warmup + args.steps // 2)) * engine.cache.bytes_per_token()
-    achieved = (weight_bytes + kv_bytes) / (ms_per_step / 1000) / 1e9
+
+    def read_rate(held_tokens: int, batch: int, steps: int, warmup: int, seconds_per_step: float) -> float:
+        """GB/s of a decode step: every weight it uses once and the cache of the live requests (at the middle of the
+        timed steps), over its time."""
+        kv_bytes = (held_tokens + batch * (PRIMING + warmup + steps // 2)) * engine.cache.bytes_per_token()
+        return (weight_bytes + kv_bytes) / seconds_per_step / 1e9
+
+    achieved = read_rate(held, args.batch, args.steps, args.warmup, ms_per_step / 1000)
     record = {
         "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2,048 tokens (Qwen3-8B bf16)",
         "value": round(value, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -336,6 +345,16 @@ def main() -> int:
             steps = max(8, args.steps // 2) if batch > args.batch else args.steps
             seconds, _ = decode(batch, steps, max(2, args.warmup // 2))
             record["points"][f"decode_b{batch}"] = round(batch * steps / seconds, 2)
+        # Decoding right after a 2,048-token prompt, where the weights are most of what a step reads (the reference's
+        # own decode figures are taken at short histories, docs/DEVLOG.md:314-319): tokens a second, and the step's
+        # bytes over its time as a fraction of the 8 TB/s.
+        if contexts is None and args.context > SHORT_CONTEXT:
+            for batch in sorted(set([args.batch] + points)):
+                steps, warmup = max(8, args.steps // 2), max(2, args.warmup // 2)
+                seconds, _ = decode(batch, steps, warmup, context=SHORT_CONTEXT)
+                record["points"][f"decode_b{batch}_ctx{SHORT_CONTEXT}"] = round(batch * steps / seconds, 2)
+                record["points"][f"decode_b{batch}_ctx{SHORT_CONTEXT}_frac"] = round(
+                    read_rate(batch * SHORT_CONTEXT, batch, steps, warmup, seconds / steps) / HBM_PEAK_GBS, 4)
     if not args.no_prefill:
         seconds, prefill_samples = prefill()
         layer_params = sum(engine.model.blocks[e.layer].mixer.weight_bytes() + engine.model.blocks[e.layer].feed_forward.weight_bytes()

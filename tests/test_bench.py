@@ -97,3 +97,16 @@ def test_the_products_beside_a_bare_read():
         else:
             assert record["routed_to"] in ("mid", "library", "own")
             assert all(record[key] > 0 for key in ("routed_us", "mid_us", "library_us", "own_us"))
+
+
+@pytest.mark.gpu
+def test_the_points_at_caches_of_2048_tokens():
+    """With a context above 2,048 tokens the line also times decoding at caches of 2,048 tokens, where the weights are
+    most of what a step reads, for every batch size it times, each with its fraction of the memory peak."""
+    result = subprocess.run([sys.executable, BENCH, "--layers", "1", "--steps", "3", "--warmup", "1", "--points", "1",
+                             "--context", "2100", "--no-prefill"], capture_output=True, text=True, timeout=600, cwd=ROOT)
+    assert result.returncode == 0, result.stderr[-2000:]
+    points = json.loads(result.stdout.strip().splitlines()[-1])["points"]
+    for batch in (1, 8):
+        assert points[f"decode_b{batch}_ctx2048"] > 0 and 0 < points[f"decode_b{batch}_ctx2048_frac"] < 1
+    assert points["decode_b8_ctx2048"] > points["decode_b1_ctx2048"]

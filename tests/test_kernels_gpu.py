@@ -1060,8 +1060,11 @@ def test_short_portion_after_a_long_history_has_its_keys_cut(hip, ref):
     q, k_pages, v_pages, ctx, meta, _, _ = _attention_case(torch.bfloat16, 8, 2, 128, 16, portions, None, 33)
     ctx.num_decode_seqs = 1
     assert hip._few_portion_blocks(ctx, 1, 8, 2)
-    long_portion = SimpleNamespace(host_q_start=[0, 1, 2049], num_seqs=2, max_seq_len=4096)
+    long_portion = SimpleNamespace(host_q_start=[0, 1, 2049], num_seqs=2, max_seq_len=4096, host_seq_lens=[700, 4096])
     assert not hip._few_portion_blocks(long_portion, 1, 8, 2)
+    # the history that counts is the portion's own request's, not that of a single token beside it
+    beside_long = SimpleNamespace(host_q_start=[0, 1, 17], num_seqs=2, max_seq_len=9000, host_seq_lens=[9000, 500])
+    assert not hip._few_portion_blocks(beside_long, 1, 8, 2)
     want = torch.empty_like(q)
     ref.attention(q, k_pages, v_pages, ctx, meta, 8, 2, 128, 128 ** -0.5, None, want)
     cctx, cmeta = _to_cuda(ctx, meta)
