@@ -171,7 +171,8 @@ class Engine:
                                  f"of {vocab}")
 
     # ---- steps as recorded graphs -----------------------------------------------------------------------------
-    PORTION_BOUND = 1024          # recorded steps: the smallest bound on the length of a request that brings a portion
+    PORTION_BOUND = 2048          # recorded steps: the smallest bound on the length of a request that brings a portion
+                                  # (up to it a portion's launches are the same whatever the length: no smaller bound pays)
     SPARE_STREAM_ROWS = 1         # steps of up to this many tokens may move the residual sum between two buffers (what
                                   # the one-row product that norms its own row needs: a fact of that kernel, not a setting)
 

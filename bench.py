@@ -166,6 +166,8 @@ def main() -> int:
                         help="every step is launched kernel by kernel instead of replayed from a recording (for counter "
                              "collection; the host's launches then show in the time)")
     parser.add_argument("--prefill-only", action="store_true", help="time the prefill alone (for kernel profiles)")
+    parser.add_argument("--mixed-only", action="store_true",
+                        help="time the step of 120 prompt tokens beside the batch's decoding requests alone (for kernel profiles)")
     parser.add_argument("--workload", choices=["decode", "serving-14b", "batch-32b", "offline-512-32"], default="decode",
                         help="decode: the headline measurement; the others run a set of requests through the scheduler")
     parser.add_argument("--library-above", type=int, default=16,
@@ -304,6 +306,10 @@ def main() -> int:
             engine.close(seq)
         return elapsed / steps * 1000
 
+    if args.mixed_only:
+        print(json.dumps({"mixed_step_120_beside_batch_ms": round(mixed_step(), 3), "batch": args.batch,
+                          "context": args.context, "layers": args.layers}))
+        return 0
     if args.prefill_only:
         seconds, _ = prefill()
         print(json.dumps({"prefill_ms": round(seconds * 1000, 3), "tokens": PREFILL_TOKENS,
