@@ -3,11 +3,12 @@ group, and slots for per-request state of fixed size.
 
 The reference keeps one pool and one tensor pair per layer and lets every request hold one table per layer
 that all grow in lock-step (ampere_kv/scheduler.py:63-69, ampere_kv/paged_cache.py:10-62).  Here layers whose
-mixers ask for the same thing (`PagedKV(kv_heads, head_dim, window)`) form a group with ONE pool, ONE table
-per request and one tensor `[layers, 2, pages, kv_heads, page_size * head_dim]`, so a page id is valid for
-every layer of its group.  Within a page, keys lie `[page_size, head_dim]` and values `[head_dim, page_size]`:
-scores contract over head_dim and the weighted sum over keys, and each reaches the matrix cores with its
-contracted axis contiguous.  Groups with a window give pages back while the request lives.  Mixers that ask
+mixers ask for the same thing (`PagedKV(kv_heads, head_dim, window, value_dim)`) form a group with ONE pool, ONE
+table per request and one tensor `[layers, elements of a layer]` - a layer's keys `[pages, kv_heads, page_size,
+head_dim]`, then its values `[pages, kv_heads, value_dim, page_size]` -, so a page id is valid for every layer of
+its group.  Within a page, keys lie `[page_size, head_dim]` and values `[value_dim, page_size]`: scores contract
+over head_dim and the weighted sum over keys, and each reaches the matrix cores with its contracted axis
+contiguous.  Keys and values need not be equally wide, and a mixer may ask for no values at all.  Groups with a window give pages back while the request lives.  Mixers that ask
 for `SlotState` get a tensor `[slots, *shape]` per layer, zeroed (or set by the mixer's own `init`) when a request
 takes the slot.
 
@@ -32,10 +33,10 @@ class PagedGroup:
     layers: list[int]                 # cache-layer ids, in the order of the tensor's first axis
     allocator: PageAllocator
     page_size: int
-    pages: torch.Tensor | None = None  # [len(layers), 2, num_pages, kv_heads, page_size * head_dim]
+    pages: torch.Tensor | None = None  # [len(layers), num_pages * kv_heads * page_size * (head_dim + value_dim)]
 
     def bytes_per_token(self, element_size: int) -> int:
-        return 2 * len(self.layers) * self.need.kv_heads * self.need.head_dim * element_size
+        return len(self.layers) * self.need.kv_heads * (self.need.head_dim + self.need.v_dim) * element_size
 
 
 @dataclass
@@ -43,7 +44,7 @@ class LayerCache:
     """What one cache layer's mixer sees: its group id and its own key and value pages, or its state."""
     group: int | None = None
     k: torch.Tensor | None = None      # [num_pages, kv_heads, page_size, head_dim]
-    v: torch.Tensor | None = None      # [num_pages, kv_heads, head_dim, page_size]
+    v: torch.Tensor | None = None      # [num_pages, kv_heads, value_dim, page_size]; None where the mixer keeps none
     state: torch.Tensor | None = None  # [slots, *shape]
 
 
@@ -80,15 +81,16 @@ class CacheManager:
                     self.groups.append(by_need[need])
                 by_need[need].layers.append(layer)
         for group in self.groups:
+            heads, k_dim, v_dim = group.need.kv_heads, group.need.head_dim, group.need.v_dim
+            k_elements, v_elements = num_pages * heads * page_size * k_dim, num_pages * heads * page_size * v_dim
             if allocate_tensors:
-                group.pages = torch.empty((len(group.layers), 2, num_pages, group.need.kv_heads,
-                                           page_size * group.need.head_dim), dtype=dtype, device=device)
+                group.pages = torch.empty((len(group.layers), k_elements + v_elements), dtype=dtype, device=device)
             for row, layer in enumerate(group.layers):
                 view = LayerCache(group=group.index)
                 if group.pages is not None:
-                    heads, dim = group.need.kv_heads, group.need.head_dim
-                    view.k = group.pages[row, 0].view(num_pages, heads, page_size, dim)
-                    view.v = group.pages[row, 1].view(num_pages, heads, dim, page_size)
+                    view.k = group.pages[row, :k_elements].view(num_pages, heads, page_size, k_dim)
+                    if v_dim:
+                        view.v = group.pages[row, k_elements:].view(num_pages, heads, v_dim, page_size)
                 self.layer_cache[layer] = view
         for layer in sorted(needs):
             need = needs[layer]

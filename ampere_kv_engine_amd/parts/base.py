@@ -85,10 +85,17 @@ class Runtime:
 
 @dataclass(frozen=True)
 class PagedKV:
-    """Keys and values of every token (or of the last `window` tokens) in pages."""
+    """Keys and values of every token (or of the last `window` tokens) in pages.  Keys are `head_dim` wide; values
+    `value_dim` (None: as wide as the keys; 0: the mixer keeps one record per token and head and no values - a
+    compressed latent, say - and its layer's view of the cache has no `v`)."""
     kv_heads: int
     head_dim: int
     window: int | None = None
+    value_dim: int | None = None
+
+    @property
+    def v_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
 
 @dataclass(frozen=True)

@@ -67,11 +67,30 @@ def _manager(**kw):
 def test_groups_by_need_and_tensor_shapes():
     m = _manager()
     assert [g.layers for g in m.groups] == [[0, 1], [2]]
-    assert m.groups[0].pages.shape == (2, 2, 24, 2, 4 * 16) and m.groups[1].pages.shape == (1, 2, 24, 2, 4 * 16)
-    assert m.layer_cache[1].k.shape == (24, 2, 4, 16) and m.layer_cache[1].k.data_ptr() == m.groups[0].pages[1, 0].data_ptr()
-    assert m.layer_cache[1].v.shape == (24, 2, 16, 4) and m.layer_cache[1].v.data_ptr() == m.groups[0].pages[1, 1].data_ptr()
+    plane = 24 * 2 * 4 * 16                      # pages x heads x page size x width
+    assert m.groups[0].pages.shape == (2, 2 * plane) and m.groups[1].pages.shape == (1, 2 * plane)
+    assert m.layer_cache[1].k.shape == (24, 2, 4, 16) and m.layer_cache[1].k.data_ptr() == m.groups[0].pages[1].data_ptr()
+    assert m.layer_cache[1].v.shape == (24, 2, 16, 4) and m.layer_cache[1].v.data_ptr() == m.groups[0].pages[1, plane:].data_ptr()
     assert m.layer_cache[3].state.shape == (3, 3, 5) and m.layer_cache[4].group is None
     assert m.bytes_per_token() == (2 * 2 + 2 * 1) * 2 * 16 * 4
+
+
+def test_keys_and_values_of_different_widths_and_keys_alone():
+    """A mixer's values may be narrower (or wider) than its keys, or absent: each such need is a group of its own, its
+    layers' views have the widths asked for and do not overlap, and a token's bytes count both widths."""
+    needs = {0: PagedKV(2, 16), 1: PagedKV(2, 16, value_dim=8), 2: PagedKV(3, 24, value_dim=0), 3: PagedKV(2, 16, value_dim=16),
+             4: PagedKV(2, 16, value_dim=8)}
+    m = CacheManager(needs, page_size=4, num_pages=6, max_seqs=2, dtype=torch.float32)
+    assert [g.layers for g in m.groups] == [[0], [1, 4], [2], [3]]      # (an explicit width equal to the keys' is another need)
+    narrow, alone = m.layer_cache[4], m.layer_cache[2]
+    assert narrow.k.shape == (6, 2, 4, 16) and narrow.v.shape == (6, 2, 8, 4)
+    assert alone.k.shape == (6, 3, 4, 24) and alone.v is None
+    assert m.groups[1].pages.shape == (2, 6 * 2 * 4 * (16 + 8)) and m.groups[2].pages.shape == (1, 6 * 3 * 4 * 24)
+    m.groups[1].pages.zero_()
+    narrow.k.fill_(1.0), narrow.v.fill_(2.0)
+    assert float(m.groups[1].pages[0].abs().sum()) == 0.0                                  # the other layer of the group
+    assert float(m.groups[1].pages[1].sum()) == 6 * 2 * 4 * (16 * 1.0 + 8 * 2.0)           # every element once
+    assert m.bytes_per_token() == (2 * 32 + 2 * 2 * 24 + 3 * 24 + 2 * 32) * 4
 
 
 def test_slots_are_zeroed_when_taken_again():

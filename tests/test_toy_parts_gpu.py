@@ -408,3 +408,127 @@ def test_a_position_encoding_of_two_axes_reads_further_integers_of_the_step(tmp_
             engine.step([StepEntry(a, [1, 2], [], extra={"axes": [[0, 0], [0, 1]]}), StepEntry(b, [3], [])])
         finally:
             engine.close(a), engine.close(b)
+
+
+# ---- a mixer whose values are narrower than its keys, and one that keeps keys alone -------------------------------
+
+class NarrowValueAttention(Part):
+    """One head.  Keys 16 wide, values `value_dim` wide; with `value_dim` 0 the mixer keeps one record per token and
+    reads it as key and as value (as a compressed latent would be).  Written with torch on the pages that the cache
+    manager hands it: a new token's record goes where the step's slot map says, a request's history is gathered
+    through its row of the group's block table."""
+
+    def __init__(self, spec, runtime):
+        self.rt, self.hidden, self.value_dim = runtime, int(spec["hidden_size"]), int(spec["value_dim"])
+        self.out_dim = self.value_dim or 16
+        self.w = {}
+
+    def tensors(self, prefix):
+        shapes = {"q": (16, self.hidden), "k": (16, self.hidden), "o": (self.hidden, self.out_dim)}
+        if self.value_dim:
+            shapes["v"] = (self.value_dim, self.hidden)
+        return [TensorSpec(f"{prefix}narrow.{name}.weight", shape, "matrix") for name, shape in shapes.items()]
+
+    def load(self, fetch, prefix):
+        self.w = {spec.name.split(".")[-2]: fetch(spec).float() for spec in self.tensors(prefix)}
+
+    def cache_request(self):
+        from ampere_kv_engine_amd.parts import PagedKV
+        return PagedKV(1, 16, None, value_dim=self.value_dim)
+
+    def forward(self, x, ctx, cache, writes_cache=True):
+        meta, page = ctx.paged[cache.group], cache.k.shape[2]
+        xf = x.float()
+        q, k = xf @ self.w["q"].T, xf @ self.w["k"].T
+        slots = meta.slot_map.long()
+        if writes_cache:
+            cache.k[slots // page, 0, slots % page, :] = k.to(cache.k.dtype)
+            if self.value_dim:
+                cache.v[slots // page, 0, :, slots % page] = (xf @ self.w["v"].T).to(cache.v.dtype)
+        out = ctx.arena.take(tuple(x.shape), self.rt.dtype)
+        for r in range(ctx.num_seqs):
+            first, last, length = ctx.host_q_start[r], ctx.host_q_start[r + 1], ctx.host_seq_lens[r]
+            row = ctx.host_seq_slots[r] if meta.rows is None else int(meta.rows[r])
+            pages = meta.block_table[row, :(length + page - 1) // page].long()
+            keys = cache.k[pages, 0].reshape(-1, 16)[:length].float()                         # [length, 16]
+            values = cache.v[pages, 0].permute(0, 2, 1).reshape(-1, self.value_dim)[:length].float() if self.value_dim else keys
+            scores = q[first:last] @ keys.T * 0.25
+            place = torch.arange(length - (last - first), length, device=x.device)[:, None]   # the new tokens' positions
+            scores = scores.masked_fill(torch.arange(length, device=x.device)[None, :] > place, float("-inf"))
+            out[first:last] = (torch.softmax(scores, dim=-1) @ values @ self.w["o"].T).to(self.rt.dtype)
+        return out
+
+
+@dataclass(frozen=True)
+class NarrowConfig(ToyConfig):
+    architecture = "ToyNarrowValuesForCausalLM"
+
+    def to_model_spec(self):
+        h = self.hidden_size
+        block = part("prenorm", hidden_size=h, norm=part("rmsnorm", size=h, eps=self.eps))
+        ff = part("swiglu", hidden_size=h, intermediate_size=40, name="mlp")
+        attention = part("attention", hidden_size=h, q_heads=2, kv_heads=1, head_dim=16, window=None,
+                         qk_norm=part("rmsnorm", size=16, eps=self.eps),
+                         position=part("rope_half", head_dim=16, theta=1e4), scale=0.25, name="self_attn")
+        layers = (LayerSpec(block, part("narrow_values", hidden_size=h, value_dim=8), ff, "model.layers.0."),
+                  LayerSpec(block, attention, ff, "model.layers.1."),
+                  LayerSpec(block, part("narrow_values", hidden_size=h, value_dim=0), ff, "model.layers.2."),
+                  LayerSpec(block, part("narrow_values", hidden_size=h, value_dim=8), ff, "model.layers.3."))
+        return ModelSpec(self.architecture, self.vocab_size, h,
+                         part("embedding", vocab_size=self.vocab_size, hidden_size=h, name="model.embed_tokens.weight"),
+                         layers, tuple(RunEntry(i, i) for i in range(4)),
+                         part("rmsnorm", size=h, eps=self.eps, name="model.norm.weight"),
+                         part("linear_head", vocab_size=self.vocab_size, hidden_size=h, name="lm_head.weight", tied_to=None))
+
+
+def plain_narrow_logits(folder, config, ids):
+    from safetensors.torch import load_file
+    w = {k: v.float() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    n = len(ids)
+    h = w["model.embed_tokens.weight"][torch.tensor(ids)]
+    for index, value_dim in enumerate((8, None, 0, 8)):
+        p = f"model.layers.{index}."
+        x = P.rms_norm(h, w[p + "input_layernorm.weight"], config.eps)
+        if value_dim is None:
+            aw = {k: w[p + "self_attn." + k + ".weight"] for k in ("q_proj", "k_proj", "v_proj", "o_proj", "q_norm", "k_norm")}
+            h = h + P.attention_mixer(x, torch.arange(n), aw, q_heads=2, kv_heads=1, head_dim=16, eps=config.eps,
+                                      inv_freq=P.rope_inverse_frequencies(16, 1e4))
+        else:
+            q, k = x @ w[p + "narrow.q.weight"].T, x @ w[p + "narrow.k.weight"].T
+            v = x @ w[p + "narrow.v.weight"].T if value_dim else k
+            scores = (q @ k.T * 0.25).masked_fill(torch.ones(n, n).triu(1).bool(), float("-inf"))
+            h = h + torch.softmax(scores, dim=-1) @ v @ w[p + "narrow.o.weight"].T
+        x = P.rms_norm(h, w[p + "post_attention_layernorm.weight"], config.eps)
+        h = h + P.swiglu_feed_forward(x, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    return P.rms_norm(h, w["model.norm.weight"], config.eps) @ w["lm_head.weight"].T
+
+
+def test_a_mixer_with_values_narrower_than_its_keys_and_one_with_keys_alone(tmp_path):
+    """The cache manager gives pages of the widths a mixer asks for: three groups here (keys 16 with values 8 - two
+    layers -, the framework's attention, keys alone), each with its own pool and block tables.  Two requests, whole and
+    in portions beside each other, with so few pages that the second pass writes into pages the first gave back."""
+    register_part("mixer", "narrow_values", NarrowValueAttention, replace=True)
+    register_architecture(NarrowConfig.architecture, NarrowConfig, replace=True)
+    config = NarrowConfig(vocab_size=83, hidden_size=32, decay=0.0, eps=1e-5)
+    folder = write_random_model(str(tmp_path / "narrow"), config, seed=17)
+    engine = Engine.from_folder(folder, EngineConfig(dtype="float32", page_size=4, num_pages=9, max_seqs=2,
+                                                     max_batched_tokens=64, max_seq_len=32, device="cuda:0"))
+    assert [len(g.layers) for g in engine.cache.groups] == [2, 1, 1]
+    views = engine.cache.layer_cache
+    assert views[3].v.shape == (9, 1, 8, 4) and views[1].v.shape == (9, 1, 16, 4) and views[2].v is None
+    a_ids, b_ids = random_ids(83, 22, seed=18), random_ids(83, 11, seed=19)
+    want_a, want_b = plain_narrow_logits(folder, config, a_ids), plain_narrow_logits(folder, config, b_ids)
+    for group in engine.cache.groups:
+        group.pages.fill_(float("nan"))            # whatever a page held before must not matter
+    a = engine.open("a")
+    torch.testing.assert_close(engine.step([StepEntry(a, a_ids, list(range(22)))]).cpu(), want_a, rtol=1e-4, atol=1e-5)
+    engine.close(a)
+    a, b, got_a, got_b = engine.open("b2"), engine.open("a2"), [], []
+    plan = [((0, 7), (0, 2)), ((7, 9), (2, 5)), ((9, 10), (5, 6)), ((10, 22), (6, 11))]
+    for (a0, a1), (b0, b1) in plan:
+        out = engine.step([StepEntry(a, a_ids[a0:a1], list(range(a1 - a0))), StepEntry(b, b_ids[b0:b1], list(range(b1 - b0)))]).cpu()
+        got_a.append(out[:a1 - a0]), got_b.append(out[a1 - a0:])
+    engine.close(a), engine.close(b)
+    torch.testing.assert_close(torch.cat(got_a), want_a, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(torch.cat(got_b), want_b, rtol=1e-4, atol=1e-5)
+    assert engine.cache.num_free_pages == [9, 9, 9]
