@@ -247,3 +247,64 @@ def test_many_requests_decode_together_at_qwen3_32b_layer_sizes(one_wide_layer, 
     for seq in seqs:
         engine.close(seq)
     assert engine.cache.num_free_pages == [2 * live]
+
+
+# ---- (d) the portions' attention on a second stream, beside the single tokens' --------------------------------------
+
+@pytest.mark.parametrize("name", ["A", "B", "D"])
+def test_portions_beside_single_tokens_give_the_same_bits_as_one_after_the_other(name, model_folders):
+    """A bfloat16 step of single tokens and prompt portions launches the portions' encoding and attention on a second
+    stream (two branches of the graph where the step is recorded).  The kernels are the same and touch different
+    requests, so every logit must have the same bits as with one stream - eager, recorded, and on every replay of a
+    recording, with other steps (eager ones among them) and reads of the results in between."""
+    from ampere_kv_engine_amd.kernels.hip import HipKernels
+    raw, _, page = TINY[name]
+    folder, vocab = model_folders[name], raw["vocab_size"]
+    engines = {}
+    for beside in (True, False):
+        for graphs in (True, False):
+            kernels = HipKernels("cuda:0")
+            kernels.portions_beside_single_tokens = beside
+            engines[beside, graphs] = Engine.from_folder(folder, EngineConfig(
+                dtype="bfloat16", page_size=page, num_pages=2400 // page, max_seqs=6, max_batched_tokens=1024,
+                max_seq_len=1024, device="cuda:0", decode_graphs=graphs), kernels=kernels)
+    ids = {key: random_ids(vocab, 900, seed=500 + i) for i, key in enumerate("abcdef")}
+    fed = {key: 0 for key in ids}
+    seqs = {mode: {} for mode in engines}
+    mixed_steps = 0
+
+    def step(parts):
+        nonlocal mixed_steps
+        outs = {}
+        for mode, engine in engines.items():
+            entries = []
+            for key, count, want in parts:
+                if key not in seqs[mode]:
+                    seqs[mode][key] = engine.open(key)
+                entries.append(StepEntry(seqs[mode][key], ids[key][fed[key]:fed[key] + count], want))
+            outs[mode] = engine.step(entries).cpu()          # (read at once: a synchronization between the steps)
+        for key, count, _ in parts:
+            fed[key] += count
+        first = outs[True, True]
+        for mode, out in outs.items():
+            assert torch.equal(out, first), f"{mode} differs from (True, True) in a step of {[p[1] for p in parts]}"
+        counts = [p[1] for p in parts]
+        mixed_steps += 1 in counts and max(counts) > 1
+
+    step([("a", 150, [149]), ("b", 40, [39])])
+    step([("c", 300, [299])])
+    for turn in range(7):                                  # met, recorded, replayed five times
+        step([("a", 1, [0]), ("b", 1, [0]), ("c", 1, [0]), ("d", 23, [22, 0])])
+    step([("e", 600, [599])])                              # an eager step in between
+    for turn in range(5):                                  # the same shape, other lengths; two portions
+        step([("a", 1, [0]), ("e", 1, [0]), ("b", 1, [0]), ("f", 23, [5]), ("d", 2, [1])])
+    for turn in range(3):
+        step([("c", 1, [0]), ("f", 70, [69])])
+    assert mixed_steps == 15
+    recorded = engines[True, True]
+    assert any(graph is not None for graph in recorded._graphs.values())
+    assert recorded.kernels._beside_stream is not None and engines[False, True].kernels._beside_stream is None
+    for mode, engine in engines.items():
+        for seq in seqs[mode].values():
+            engine.close(seq)
+        assert engine.cache.num_free_pages == [2400 // page]
