@@ -46,6 +46,7 @@ QWEN3_8B = dict(architectures=["Qwen3ForCausalLM"], num_hidden_layers=36, hidden
 # the layer sizes of the two larger dense models (Qwen3-14B, Qwen3-32B)
 QWEN3_14B = dict(QWEN3_8B, num_hidden_layers=40, hidden_size=5120, num_attention_heads=40, intermediate_size=17408)
 QWEN3_32B = dict(QWEN3_8B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=64, intermediate_size=25600)
+SIZES = {"8b": ("Qwen3-8B", QWEN3_8B), "14b": ("Qwen3-14B", QWEN3_14B), "32b": ("Qwen3-32B", QWEN3_32B)}
 PAGE_SIZE, CONTEXT, PREFILL_TOKENS = 16, 8192, 2048
 SHORT_CONTEXT = 2048    # decoding right after such a prompt is timed too (points decode_b*_ctx2048)
 PRIMING = 3   # untimed steps before the warm-up steps: the first runs eagerly, the second is recorded, the third replays
@@ -156,7 +157,9 @@ def main() -> int:
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--context", type=int, default=CONTEXT)
-    parser.add_argument("--layers", type=int, default=QWEN3_8B["num_hidden_layers"],
+    parser.add_argument("--sizes", choices=sorted(SIZES), default="8b",
+                        help="layer sizes of the decode and prefill measurements (the default is the record's)")
+    parser.add_argument("--layers", type=int, default=None,
                         help="fewer layers than the configuration has, where memory or time needs it")
     parser.add_argument("--points", default="1,64", help="further batch sizes to time (comma separated, '' for none)")
     parser.add_argument("--contexts", default="", help="requests of different context lengths in one batch, e.g. "
@@ -179,9 +182,9 @@ def main() -> int:
         return 2
 
     if args.workload == "offline-512-32":
-        return offline_workload(args.layers if args.layers != QWEN3_8B["num_hidden_layers"] else None)
+        return offline_workload(args.layers)
     if args.workload != "decode":
-        return scheduler_workload(args.workload, args.layers if args.layers != QWEN3_8B["num_hidden_layers"] else None,
+        return scheduler_workload(args.workload, args.layers,
                                   library_above)
 
     import torch
@@ -197,7 +200,9 @@ def main() -> int:
         args.batch, args.context, args.points, args.no_prefill = len(contexts), max(contexts), "", True
     points = [int(p) for p in args.points.split(",") if p]
     max_batch = max([args.batch] + points)
-    raw = dict(QWEN3_8B, num_hidden_layers=args.layers)
+    model_name, sizes = SIZES[args.sizes]
+    args.layers = args.layers or sizes["num_hidden_layers"]
+    raw = dict(sizes, num_hidden_layers=args.layers)
     config = Qwen3Config.from_dict(raw)
     tokens_per_request = args.context + PRIMING + args.warmup + args.steps + 2
     pages = max_batch * ((tokens_per_request + PAGE_SIZE - 1) // PAGE_SIZE) + PREFILL_TOKENS // PAGE_SIZE + 2
@@ -329,12 +334,12 @@ def main() -> int:
 
     achieved = read_rate(held, args.batch, args.steps, args.warmup, ms_per_step / 1000)
     record = {
-        "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2,048 tokens (Qwen3-8B bf16)",
+        "metric": f"decode tok/s at batch 1/8/64; prefill tok/s at 2,048 tokens ({model_name} bf16)",
         "value": round(value, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "samples": fifths(moments), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic: random-init weights N(0, 0.02), uniform random token ids, random cache",
-        "config": {"model": "Qwen3-8B layer sizes", "global_batch": args.batch, "seq_len": args.context,
-                   "parallelism": "single GPU", "layers": args.layers, "layers_of_config": QWEN3_8B["num_hidden_layers"],
+        "config": {"model": f"{model_name} layer sizes", "global_batch": args.batch, "seq_len": args.context,
+                   "parallelism": "single GPU", "layers": args.layers, "layers_of_config": sizes["num_hidden_layers"],
                    "hidden": config.hidden_size, "q_heads": config.num_attention_heads,
                    "kv_heads": config.num_key_value_heads, "head_dim": config.head_dim,
                    "intermediate": config.intermediate_size, "vocab": config.vocab_size, "page_size": PAGE_SIZE,
