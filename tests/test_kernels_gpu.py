@@ -1232,6 +1232,36 @@ def test_attention_finds_a_far_key(hip, ref, dtype):
         torch.testing.assert_close(picked[3], values[r][at, 1].float(), rtol=0.05, atol=0.05)
 
 
+@pytest.mark.parametrize("portions,spike", [
+    ([(120_000, 1), (300, 1), (70_001, 1)], (0, 5)),        # single tokens: 128 segments of a thousand keys; a far, early key
+    ([(120_000, 1), (300, 1), (70_001, 1)], (2, 69_999)),   # ... and one in another request's last segment but one
+    ([(60_000, 48)], (0, 59_000)),                          # a short portion after a long history: its keys are cut
+    ([(0, 3_000)], (0, 7)),                                 # a long prompt whole: blocks of four waves, ninety calm steps
+    ([(2_500, 700), (0, 40)], (0, 2_499)),                  # a long portion after a history, the key at the history's end
+])
+def test_attention_at_long_contexts_finds_a_far_key(hip, ref, portions, spike):
+    """Qwen3-8B's head shape (four query heads to a key head of 128) at lengths far beyond the other tests', where a
+    launch's cut of the keys, the calm steps of a long prompt and 32-bit offsets into a request's table are not what
+    they are at a few hundred tokens.  The queries of the spiked request match one far key: their output is that
+    key's value, and everything equals the torch double within the attention's limits."""
+    q_heads, kv_heads, dim, page_size = 4, 1, 128, 16
+    q, k_pages, v_pages, ctx, meta, keys, values = _attention_case(torch.bfloat16, q_heads, kv_heads, dim, page_size,
+                                                                   portions, None, 31, spike)
+    ctx.num_decode_seqs = sum(1 for _, n in portions if n == 1) if all(n == 1 for _, n in portions) else 0
+    want = torch.empty_like(q)
+    ref.attention(q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, dim, dim ** -0.5, None, want)
+    cctx, cmeta = _to_cuda(ctx, meta)
+    got = torch.full_like(q, float("nan"), device="cuda")
+    hip.attention(q.cuda(), k_pages.cuda(), v_pages.cuda(), cctx, cmeta, q_heads, kv_heads, dim, dim ** -0.5, None, got)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **attention_tol(torch.bfloat16))
+    r, at = spike
+    rows = range(ctx.host_q_start[r], ctx.host_q_start[r + 1])
+    seen = [row for row in rows if int(ctx.positions[row]) >= at]           # (earlier tokens of a prompt cannot see it)
+    assert seen
+    for row in (seen[0], seen[-1]):
+        torch.testing.assert_close(got.cpu().float()[row].reshape(q_heads, dim)[2], values[r][at, 0].float(), rtol=0.05, atol=0.05)
+
+
 @pytest.mark.parametrize("vocab", [1531, 1532, 40004])     # single loads; 16-byte loads; more than one round of them
 def test_sample(hip, vocab):
     import numpy as np

@@ -308,3 +308,65 @@ def test_portions_beside_single_tokens_give_the_same_bits_as_one_after_the_other
         for seq in seqs[mode].values():
             engine.close(seq)
         assert engine.cache.num_free_pages == [2400 // page]
+
+
+# ---- (e) long requests: many pages, recordings for several table widths -----------------------------------------------
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_a_long_request_beside_short_ones_across_the_widths_of_the_block_table(name, dtype, model_folders):
+    """A request of 3,100 tokens (hundreds of pages of 8 or 4 tokens), fed in portions of up to 512 beside two short
+    requests that decode meanwhile, then decoded itself for 40 tokens across a boundary of the recorded steps' table
+    width (a multiple of 64 pages): every fed position against the plain implementation, and every step bit for bit
+    against an engine that records nothing."""
+    from ampere_kv_engine_amd.kernels.hip import HipKernels
+    raw, _, page = TINY[name]
+    folder, vocab = model_folders[name], raw["vocab_size"]
+    boundary = 64 * page * (3072 // (64 * page))                    # a width boundary near 3,072 tokens
+    long_ids = random_ids(vocab, boundary + 24, seed=901)
+    prompt = boundary - 16                                            # decoding starts 16 tokens before the boundary
+    short = {"s": random_ids(vocab, 90, seed=902), "t": random_ids(vocab, 61, seed=903)}
+    plain = PlainQwen3(folder)
+    want = {"long": plain.logits(long_ids), **{key: plain.logits(ids) for key, ids in short.items()}}
+    kernels = HipKernels("cuda:0")
+    pages = (len(long_ids) + 200) // page + 8
+    engines = [Engine.from_folder(folder, EngineConfig(dtype=dtype, page_size=page, num_pages=pages, max_seqs=3,
+                                                       max_batched_tokens=600, max_seq_len=len(long_ids) + page,
+                                                       device="cuda:0", decode_graphs=graphs), kernels=kernels)
+               for graphs in (True, False)]
+    seqs = [{key: engine.open(key) for key in ("long", "s", "t")} for engine in engines]
+    fed = {"long": 0, "s": 0, "t": 0}
+    ids = {"long": long_ids, **short}
+    got = {key: [] for key in ids}
+
+    def step(counts):
+        outs = []
+        for engine, mine in zip(engines, seqs):
+            entries = [StepEntry(mine[key], ids[key][fed[key]:fed[key] + count], list(range(count))) for key, count in counts.items()]
+            outs.append(engine.step(entries).cpu())
+        assert torch.equal(outs[0], outs[1]), f"recorded and eager steps differ at {fed}"
+        row = 0
+        for key, count in counts.items():
+            got[key].append(outs[0][row:row + count])
+            row += count
+            fed[key] += count
+
+    step({"s": 30, "t": 20})
+    portions = [512, 7, 512, 512, 300, 512, 2, 512]
+    portions.append(prompt - sum(portions))
+    assert portions[-1] > 0
+    for size in portions:                                             # the short ones decode beside every portion
+        counts = {key: 1 for key in ("s", "t") if fed[key] < len(ids[key])}
+        step({**counts, "long": size})
+    while fed["long"] < len(long_ids):                                # single tokens, across the boundary
+        counts = {key: 1 for key in ("s", "t") if fed[key] < len(ids[key])}
+        step({**counts, "long": 1})
+    widths = {key[2] for key, graph in engines[0]._graphs.items() if graph is not None}
+    assert len(widths) >= 2, f"the recorded steps saw one table width only: {widths}"
+    for key in ids:
+        logits = torch.cat(got[key])
+        cases.assert_logits_close(logits, want[key][:len(logits)], dtype, "plain", f"{name}/{dtype} request {key}")
+    for engine, mine in zip(engines, seqs):
+        for seq in mine.values():
+            engine.close(seq)
+        assert engine.cache.num_free_pages == [pages]
