@@ -80,40 +80,53 @@ __global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_ker
     const int f = wave - kMultipliers;
     constexpr int kRowsPerLoad = 16 / S;
     const int row_in_load = lane / (4 * S), piece = lane % (4 * S);   // piece = k-tile of the stage * 4 + chunk of 8
+    // Every load is issued whatever it asks for - rows beyond the last, k beyond this half's part are asked for at an
+    // address that exists - and what must count as zero is zeroed when it is filed: with a test per load the compiler
+    // cannot count the loads between a tile and its use and waits for the stage after it as well.
     uintx4 fetched[2][kLoads];
-    auto fetch_rows = [&](int stage, uintx4 (&into)[kLoads]) {
+    unsigned there[2];             // bit j: load j of the set brought something that exists
+    auto fetch_rows = [&](int stage, uintx4 (&into)[kLoads], unsigned& exists) {
+      exists = 0u;
 #pragma unroll
       for (int j = 0; j < kLoads; ++j) {
         const int i = f + kFetchers * j;
         const int h = i / (S * MT), group = i % (S * MT);
         const int kt = kb0 + h * per_half + stage * S + piece / 4;
         const int row = row0 + group * kRowsPerLoad + row_in_load, col = kt * 32 + (piece % 4) * 8;
-        const bool there = kt < min(kb1, kb0 + (h + 1) * per_half) && row < rows && col < k;
-        into[j] = there ? *reinterpret_cast<const uintx4*>(x + static_cast<size_t>(row) * k + col) : zero;
+        const bool real = kt < min(kb1, kb0 + (h + 1) * per_half) && row < rows && col < k;
+        exists |= real ? 1u << j : 0u;
+        into[j] = *reinterpret_cast<const uintx4*>(x + static_cast<size_t>(min(row, rows - 1)) * k + min(col, k - 8));
       }
     };
-    auto file_rows = [&](int buffer, const uintx4 (&from)[kLoads]) {
+    auto file_rows = [&](int buffer, const uintx4 (&from)[kLoads], unsigned exists) {
 #pragma unroll
       for (int j = 0; j < kLoads; ++j) {
         const int i = f + kFetchers * j;
         const int h = i / (S * MT), group = i % (S * MT);
         const int row = group * kRowsPerLoad + row_in_load;          // of the block's MT * 16
         const int u = piece / 4, g = piece % 4;
-        staged[(buffer * kTiles + (h * S + u) * MT + row / 16) * 64 + slot_of(u, g, row % 16)] = from[j];
+        staged[(buffer * kTiles + (h * S + u) * MT + row / 16) * 64 + slot_of(u, g, row % 16)] = (exists >> j & 1u) ? from[j] : zero;
       }
     };
-    fetch_rows(0, fetched[0]);
-    if (1 < stages) fetch_rows(1, fetched[1]);
-    for (int first = 0; first < stages; first += 2) {
+    fetch_rows(0, fetched[0], there[0]);
+    fetch_rows(1, fetched[1], there[1]);
+    __builtin_amdgcn_sched_barrier(0);
+    int first = 0;
+    for (; first + 2 <= stages; first += 2) {       // (pairs of stages, no test inside)
 #pragma unroll
       for (int d = 0; d < 2; ++d) {
-        const int stage = first + d;
-        if (stage < stages) {
-          file_rows(d, fetched[d]);
-          if (stage + 2 < stages) fetch_rows(stage + 2, fetched[d]);
-          __syncthreads();
-        }
+        // (the fences keep the zeroing of a set's pieces where it is written - behind the other set's loads -: moved
+        // up by the compiler it waits for loads that were meant to have a stage's time)
+        file_rows(d, fetched[d], there[d]);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_rows(first + d + 2, fetched[d], there[d]);
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
       }
+    }
+    if (first < stages) {
+      file_rows(0, fetched[0], there[0]);
+      __syncthreads();
     }
     return;
   }
@@ -129,26 +142,20 @@ __global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_ker
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  auto fetch_weights = [&](int stage, uintx4 (&a)[RT][S]) {
+  // The loads of a stage's weight tiles are the same instructions at every turn, with no test among them: tiles
+  // beyond the matrix or beyond this wave's part of k are asked for at the last tile that exists instead - their
+  // sums are never stored, or meet activation tiles that the fetching waves have filled with zeros.  (With a test
+  // per load the compiler cannot count how many younger loads stand between a tile and its use, and waits for ALL
+  // loads - the ones just issued for a later stage included - before it multiplies: the ring was never ahead.)
+  auto fetch_weights = [&](int stage, uintx4 (&a)[RT][S], auto once) {
     const int kt = mine0 + stage * S;
-    const uintx4* at = wp + lane;
-    if (kt + S <= mine1 && tile0 + RT <= n_tiles) {   // the whole group exists: no test per load
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt)
+    for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-        for (int u = 0; u < S; ++u) {
-          const uintx4* from = at + tile_index<GATED>(tile0 + rt, kt + u, k_tiles) * 64;
-          a[rt][u] = shared_weights ? *from : load_once(from);
-        }
-    } else {
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-        for (int u = 0; u < S; ++u) {
-          const uintx4* from = at + tile_index<GATED>(tile0 + rt, kt + u, k_tiles) * 64;
-          a[rt][u] = (kt + u < mine1 && tile0 + rt < n_tiles) ? (shared_weights ? *from : load_once(from)) : zero;
-        }
-    }
+      for (int u = 0; u < S; ++u) {
+        const uintx4* from = wp + lane + tile_index<GATED>(min(tile0 + rt, n_tiles - 1), min(kt + u, k_tiles - 1), k_tiles) * 64;
+        a[rt][u] = decltype(once)::value ? load_once(from) : *from;
+      }
   };
   auto multiply = [&](int buffer, const uintx4 (&a)[RT][S]) {
     const uintx4* tiles = staged + (buffer * kTiles + half * S * MT) * 64;
@@ -165,21 +172,34 @@ __global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_ker
     }
   };
 
-  uintx4 a[G][RT][S];
+  // The turns of the ring: G stages a turn, no test inside a turn; what is left after the last whole turn (fewer than
+  // G stages) runs with tests.  Loads for stages beyond the last one bring a tile that exists and nobody multiplies.
+  auto stream = [&](auto once) {
+    uintx4 a[G][RT][S];
 #pragma unroll
-  for (int d = 0; d < G - 1; ++d)
-    if (d < stages) fetch_weights(d, a[d]);
-  for (int first = 0; first < stages; first += G) {
+    for (int d = 0; d < G - 1; ++d) fetch_weights(d, a[d], once);
+    int first = 0;
+    for (; first + G <= stages; first += G) {
 #pragma unroll
-    for (int d = 0; d < G; ++d) {
-      const int stage = first + d;
-      if (stage < stages) {
+      for (int d = 0; d < G; ++d) {
         __syncthreads();          // the stage's activations are in LDS
-        if (stage + G - 1 < stages) fetch_weights(stage + G - 1, a[(d + G - 1) % G]);
+        fetch_weights(first + d + G - 1, a[(d + G - 1) % G], once);
+        __builtin_amdgcn_sched_barrier(0);   // (left alone the compiler moves these loads behind the products: no ring)
         multiply(d & 1, a[d]);
       }
     }
-  }
+#pragma unroll
+    for (int d = 0; d < G - 1; ++d) {
+      if (first + d < stages) {
+        __syncthreads();
+        fetch_weights(first + d + G - 1, a[(d + G - 1) % G], once);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(d & 1, a[d]);
+      }
+    }
+  };
+  if (shared_weights) stream(std::false_type{});
+  else stream(std::true_type{});
 
   // the two k halves: the second hands its sums over through LDS, the first adds them to its own
   __syncthreads();
