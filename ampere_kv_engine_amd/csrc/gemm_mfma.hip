@@ -414,7 +414,12 @@ __global__ __launch_bounds__(256, 2) void linear_wide_kernel(const bf16_t* __res
     for (int m = 0; m < MW; ++m) acc[n][m] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   // staging: a thread moves 8 chunks of 16 B per stage; chunk c = e % 8 of token e / 8, so that 8 consecutive threads
-  // read 128 consecutive bytes of one row of x
+  // read 128 consecutive bytes of one row of x.
+  // No load of the loop stands behind a test: tokens beyond the last, k beyond the matrix and stages beyond the last
+  // are asked for at the nearest address that exists, and what has to count as zero is zeroed when it is written to
+  // LDS (weights beyond the matrix meet such zeros, or feed sums that are never stored).  With a test per load the
+  // compiler cannot tell how many younger loads stand between a load and its use, and waits for all of them - those
+  // it has just issued for the next stage included.
   const char* x_bytes = reinterpret_cast<const char*>(x);
   constexpr int PX = MW;  // 16-byte chunks a thread stages: tokens * 8 / 256
   uint32_t x_at[PX];
@@ -423,38 +428,32 @@ __global__ __launch_bounds__(256, 2) void linear_wide_kernel(const bf16_t* __res
   for (int p = 0; p < PX; ++p) {
     const int e = p * 256 + threadIdx.x, token = token0 + e / 8;
     x_row[p] = token < rows;
-    x_at[p] = static_cast<uint32_t>(token) * static_cast<uint32_t>(k) * 2u + (e % 8) * 16u;
+    x_at[p] = static_cast<uint32_t>(min(token, rows - 1)) * static_cast<uint32_t>(k) * 2u;
   }
-  auto fetch = [&](int stage, uintx4 (&moving)[PX]) {
-    const char* at = x_bytes + static_cast<size_t>(stage) * (kWideK * 2);
+  auto fetch = [&](int stage, uintx4 (&moving)[PX], unsigned& exists) {
+    exists = 0u;
 #pragma unroll
     for (int p = 0; p < PX; ++p) {
       const int e = p * 256 + threadIdx.x;
-      const bool inside = stage * kWideK + (e % 8) * 8 < k;
-      moving[p] = (x_row[p] && inside) ? *reinterpret_cast<const uintx4*>(at + x_at[p]) : zero;
+      const int col = stage * kWideK + (e % 8) * 8;
+      exists |= (x_row[p] && col < k) ? 1u << p : 0u;
+      moving[p] = *reinterpret_cast<const uintx4*>(x_bytes + x_at[p] + static_cast<uint32_t>(min(col, k - 8)) * 2u);
     }
   };
-  auto stash = [&](int buffer, const uintx4 (&moving)[PX]) {
+  auto stash = [&](int buffer, const uintx4 (&moving)[PX], unsigned exists) {
 #pragma unroll
     for (int p = 0; p < PX; ++p) {
       const int e = p * 256 + threadIdx.x, c = e % 8, t = e / 8;
-      xs[buffer][c][t ^ (c << 1)] = moving[p];
+      xs[buffer][c][t ^ (c << 1)] = (exists >> p & 1u) ? moving[p] : zero;
     }
   };
   // weights: the wave's 4 row tiles of one k-tile
   const char* w_bytes = reinterpret_cast<const char*>(wp);
-  uint32_t w_at[4];
-  bool w_row[4];
-#pragma unroll
-  for (int n = 0; n < 4; ++n) {
-    w_row[n] = tile0 + n < n_tiles;
-    w_at[n] = lane * 16u;
-  }
   auto weights = [&](int kt, uintx4 (&a)[4]) {
 #pragma unroll
     for (int n = 0; n < 4; ++n) {
-      const char* at = w_bytes + tile_index<GATED>(tile0 + n, kt, k_tiles) * 1024;
-      a[n] = (w_row[n] && kt < k_tiles) ? *reinterpret_cast<const uintx4*>(at + w_at[n]) : zero;
+      const char* at = w_bytes + tile_index<GATED>(min(tile0 + n, n_tiles - 1), min(kt, k_tiles - 1), k_tiles) * 1024;
+      a[n] = *reinterpret_cast<const uintx4*>(at + lane * 16u);
     }
   };
   auto multiply = [&](int buffer, int half, const uintx4 (&a)[4]) {
@@ -480,49 +479,60 @@ __global__ __launch_bounds__(256, 2) void linear_wide_kernel(const bf16_t* __res
     __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
   };
 
+  // (the fences: left alone, the compiler moves the loads behind the products that were to hide them, and the zeroing
+  // of what has arrived up to where it waits for loads that were meant to have a stage's time)
   if constexpr (MW <= 4) {
     // Registers allow two sets of everything: the weights of a whole stage (two k-tiles) are fetched one stage ahead,
     // the activations two stages ahead (they wait in registers for one stage, then go to the LDS buffer that the
     // stage before has just finished reading).
     uintx4 a0[2][4], a1[2][4], m0[PX], m1[PX];
+    unsigned e0, e1;
     auto run_stage = [&](int stage, const uintx4 (&cur)[2][4], uintx4 (&next)[2][4], uintx4 (&arriving)[PX],
-                         const uintx4 (&arrived)[PX]) {
+                         unsigned& arriving_exists, const uintx4 (&arrived)[PX], unsigned arrived_exists) {
       const int buffer = stage & 1;
-      if (stage + 2 < stages) fetch(stage + 2, arriving);
-      if (stage + 1 < stages) {
-        weights(stage * 2 + 2, next[0]);
-        weights(stage * 2 + 3, next[1]);
-      }
+      fetch(stage + 2, arriving, arriving_exists);
+      weights(stage * 2 + 2, next[0]);
+      weights(stage * 2 + 3, next[1]);
+      __builtin_amdgcn_sched_barrier(0);
       multiply(buffer, 0, cur[0]);
       multiply(buffer, 1, cur[1]);
-      if (stage + 1 < stages) stash(buffer ^ 1, arrived);
+      __builtin_amdgcn_sched_barrier(0);
+      stash(buffer ^ 1, arrived, arrived_exists);
       __syncthreads();
     };
-    fetch(0, m0);
-    stash(0, m0);
-    if (stages > 1) fetch(1, m1);
+    fetch(0, m0, e0);
+    stash(0, m0, e0);
+    fetch(1, m1, e1);
     weights(0, a0[0]);
     weights(1, a0[1]);
+    __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
-    for (int stage = 0; stage < stages; stage += 2) {
-      run_stage(stage, a0, a1, m0, m1);
-      if (stage + 1 < stages) run_stage(stage + 1, a1, a0, m1, m0);
+    int stage = 0;
+    for (; stage + 2 <= stages; stage += 2) {
+      run_stage(stage, a0, a1, m0, e0, m1, e1);
+      run_stage(stage + 1, a1, a0, m1, e1, m0, e0);
     }
+    if (stage < stages) run_stage(stage, a0, a1, m0, e0, m1, e1);
   } else {
     // weights are fetched one k-tile ahead, activations one stage ahead
     uintx4 a0[4], a1[4], moving[PX];
-    fetch(0, moving);
-    stash(0, moving);
+    unsigned exists;
+    fetch(0, moving, exists);
+    stash(0, moving, exists);
     weights(0, a0);
     __syncthreads();
     for (int stage = 0; stage < stages; ++stage) {
       const int buffer = stage & 1;
-      if (stage + 1 < stages) fetch(stage + 1, moving);
+      fetch(stage + 1, moving, exists);
       weights(stage * 2 + 1, a1);
+      __builtin_amdgcn_sched_barrier(0);
       multiply(buffer, 0, a0);
+      __builtin_amdgcn_sched_barrier(0);
       weights(stage * 2 + 2, a0);
+      __builtin_amdgcn_sched_barrier(0);
       multiply(buffer, 1, a1);
-      if (stage + 1 < stages) stash(buffer ^ 1, moving);
+      __builtin_amdgcn_sched_barrier(0);
+      stash(buffer ^ 1, moving, exists);
       __syncthreads();
     }
   }

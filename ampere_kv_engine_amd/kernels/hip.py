@@ -340,14 +340,15 @@ class HipKernels(KernelSet):
         """Which kernel takes a bfloat16 product of more than 16 rows: "own" (the skinny kernel up to 64 rows, the
         wide one above), "mid" (17..512 rows: the block's waves share the activations through LDS) or "library".
         The table of choices decides where it names the product; otherwise a fixed rule, from measurements at
-        Qwen3-8B, -14B and -32B shapes (cold weights, 24 to 256 rows; `bench_products --rows ...` repeats them):
-        the library where there is one, except for the gated product up to 64 rows (the mid-size kernel is 8-28 %
-        faster; beyond, the library is as fast at Qwen3-8B shapes and 2-15 % faster at the larger ones), plain
-        products with outs <= k up to 64 rows (the stacked q/k/v product, outs > k, is 2-6 % faster in the library
-        there) and every plain product from 65 to 256 rows (from 4 % slower to three times faster; the library's
-        times jump with the row count - q/k/v of 7,168 x 5,120: 36 / 50 / 63 us at 128 / 192 / 256 rows, the
-        mid-size kernel 36 / 41 / 42).  Without the library: the skinny kernel up to
-        64 rows, the mid-size one up to 512, the wide one beyond."""
+        Qwen3-8B, -14B and -32B shapes (cold weights, 32 to 512 rows; `bench_products --rows ...` repeats them):
+        plain products go to the mid-size kernel up to 256 rows (q/k/v, o, down at 128 rows: 26.8 / 21.6 / 36.8 us
+        against the library's 28.5 / 27.4 / 69.7 at Qwen3-8B shapes, 36.9 / 31.8 / 70.1 against 44.6 / 47.2 / 185.7
+        at Qwen3-32B's; the library's times jump with the row count), and up to 512 where k is at least twice the
+        outputs (the down product: 69 against 84 us at 512 rows; the others are within a few percent either way
+        there); the gated product up to 64 rows, and up to 128 where the two matrices hold no more than 64 M elements
+        (Qwen3-8B: 47 against 57 us with the library's activation pass; Qwen3-14B: 100 / 101; Qwen3-32B: 126 / 112).
+        Beyond, the library.  Without the library: the mid-size kernel up to 512 rows (it is faster than the skinny
+        one from 17 rows on), the wide one beyond."""
         library = (has_row_major and self.library_products_above is not None and rows > self.library_products_above
                    and out_dtype == torch.bfloat16)
         bucket = self._row_bucket(rows)
@@ -359,12 +360,12 @@ class HipKernels(KernelSet):
         if choice is not None:
             return choice
         if not library:
-            return "own" if rows <= self.OWN_SKINNY_ROWS else "mid"
+            return "mid"
         if kind == "gated":
-            return "mid" if rows <= 64 else "library"
-        if rows > 256:
-            return "library"
-        return "mid" if (rows > 64 or outs <= k) else "library"
+            return "mid" if rows <= 64 or (rows <= 128 and outs * k <= 64 << 20) else "library"
+        if rows <= 256 or k >= 2 * outs:
+            return "mid"
+        return "library"
 
     def _mid(self, x, packed: PackedWeight, out, rows: int, outs: int, gated: bool, bias=None) -> None:
         """The mid-size product (`csrc/gemm_mid.hip`).  Where it cuts k over blocks it needs room for partial sums
