@@ -191,11 +191,11 @@ __global__ __launch_bounds__(768) void linear_decode_kernel(const DecodeArgs a) 
       multiply(kt, w0, x0);
       fetch_weights(kt + 2 * U, w0);
       fetch_rows(kt + 2 * U, x0);
+      __builtin_amdgcn_sched_barrier(0);      // (the loads stay where they are written: ahead of the other group's products)
       multiply(kt + U, w1, x1);
-      if (kt + 3 * U < kt1) {
-        fetch_weights(kt + 3 * U, w1);
-        fetch_rows(kt + 3 * U, x1);
-      }
+      fetch_weights(kt + 3 * U, w1);          // (beyond the part: the last tile again, never multiplied - no test, so
+      fetch_rows(kt + 3 * U, x1);             //  that the waits above can count the loads behind them)
+      __builtin_amdgcn_sched_barrier(0);
     }
     multiply(kt, w0, x0);
     if (kt + U < kt1) multiply(kt + U, w1, x1);
