@@ -257,9 +257,16 @@ __device__ __forceinline__ void encode_head(uintx4 (&reg)[KT], bool normed, floa
 // ONCE: no other block of the launch reads these keys and values (single tokens, one block per kv head and segment):
 // the loads are marked read-once.  A bare reader with this kernel's lanes and depth draws 7.1 TB/s from 2 GB of
 // pages with the mark and 6.5 TB/s without.
+// (The kernel's text is a function of where a wave stands in the grid, so that another kernel can run it beside the
+// prompt portions' blocks: see `attention_pair_kernel`.)
+struct Where {
+  int bx, by, bz, gx, gy;   // the wave's block and the grid, as blockIdx and gridDim would name them
+  int lane;
+};
+
 template <int NQ, bool SPLIT, bool PIPE, bool FRESH, bool ONCE>
-__global__ __launch_bounds__(64, (SPLIT && NQ == 1 && D <= 128) ? 2 : 1) void attention_mfma_kernel(const Args a) {
-  const int lane = threadIdx.x, r16 = lane & 15, g = lane >> 4;
+__device__ __forceinline__ void attention_mfma_body(const Args& a, const Where at) {
+  const int lane = at.lane, r16 = lane & 15, g = lane >> 4;
   auto from_pages = [](const char* at) {
     const uintx4* p = reinterpret_cast<const uintx4*>(at);
     return ONCE ? __builtin_nontemporal_load(p) : *p;
@@ -270,14 +277,13 @@ __global__ __launch_bounds__(64, (SPLIT && NQ == 1 && D <= 128) ? 2 : 1) void at
   // (FRESH launches hold single tokens, whose tiles have nothing to balance: one tile per block, like SPLIT.)
   constexpr bool kOneTile = SPLIT || FRESH;
   for (int pass = 0; pass < (kOneTile ? 1 : 2); ++pass) {
-  const int slot = kOneTile ? static_cast<int>(blockIdx.x)
-                            : (pass == 0 ? a.tiles - 1 - static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x));
+  const int slot = kOneTile ? at.bx : (pass == 0 ? a.tiles - 1 - at.bx : at.bx);
   if (!kOneTile && pass == 1 && slot >= a.tiles - 1 - slot) break;  // the middle tile was the first pass's
   Tile t{};
   int seg_lo = 0, seg_hi = 0x7fffffff;     // SPLIT: the keys of this block's segment
   long part = 0;                           // SPLIT: index of its partial result's tile
-  if (SPLIT && a.plan != nullptr) {        // item blockIdx.y of the plan: a request and a segment of its keys
-    const int item = static_cast<int>(blockIdx.y);
+  if (SPLIT && a.plan != nullptr) {        // item `by` of the plan: a request and a segment of its keys
+    const int item = at.by;
     if (item >= a.plan[0]) return;
     const int4 record = *reinterpret_cast<const int4*>(a.plan + 132 + 4 * item);
     t.request = a.seq_first + record.x;
@@ -287,17 +293,17 @@ __global__ __launch_bounds__(64, (SPLIT && NQ == 1 && D <= 128) ? 2 : 1) void at
     t.found = true;
     seg_lo = record.y;
     seg_hi = record.w;
-    part = static_cast<long>(item) * gridDim.x + blockIdx.x;
+    part = static_cast<long>(item) * at.gx + at.bx;
   } else {
     t = find_tile(a, slot, a.tokens_per_tile);
     if (!t.found) continue;
     if (SPLIT) {
-      seg_lo = static_cast<int>(blockIdx.z) * a.seg_keys;
+      seg_lo = at.bz * a.seg_keys;
       seg_hi = seg_lo + a.seg_keys - 1;
-      part = (static_cast<long>(blockIdx.x) * gridDim.y + blockIdx.y) * a.num_splits + blockIdx.z;
+      part = (static_cast<long>(at.bx) * at.gy + at.by) * a.num_splits + at.bz;
     }
   }
-  const int head_block = (SPLIT && a.plan != nullptr) ? blockIdx.x : blockIdx.y;  // (kv head, group of its query heads)
+  const int head_block = (SPLIT && a.plan != nullptr) ? at.bx : at.by;  // (kv head, group of its query heads)
   const int kvh = head_block / a.head_groups, hg = head_block % a.head_groups;
   const uintx4 zero = uintx4{0u, 0u, 0u, 0u};
   const int page_size = 1 << a.page_shift, page_mask = page_size - 1;
@@ -663,6 +669,13 @@ __global__ __launch_bounds__(64, (SPLIT && NQ == 1 && D <= 128) ? 2 : 1) void at
   }  // pass
 }
 
+template <int NQ, bool SPLIT, bool PIPE, bool FRESH, bool ONCE>
+__global__ __launch_bounds__(64, (SPLIT && NQ == 1 && D <= 128) ? 2 : 1) void attention_mfma_kernel(const Args a) {
+  attention_mfma_body<NQ, SPLIT, PIPE, FRESH, ONCE>(
+      a, Where{static_cast<int>(blockIdx.x), static_cast<int>(blockIdx.y), static_cast<int>(blockIdx.z),
+               static_cast<int>(gridDim.x), static_cast<int>(gridDim.y), static_cast<int>(threadIdx.x)});
+}
+
 // ---- prompt portions: four waves share every key and value through LDS ------------------------------------------------
 // A block of 4 waves works on 4 consecutive tiles of one request and one kv head (4 * 16 * NQ columns).  The keys and
 // values of a step of 32 keys are fetched from the pages ONCE per block - every thread moves a few 16-byte pieces into
@@ -683,18 +696,18 @@ constexpr float kLazy = 8.f;  // the exponentials' reference point trails the ma
 // SP: pages per step of 32 keys (4: pages of 8 tokens, 2: of 16, 1: of 32 or more) - with it the page arithmetic of a
 // step is known when compiling.
 template <int NQ, int SP>
-__global__ __launch_bounds__(64 * kSharedWaves, D <= 128 ? (NQ == 1 ? 3 : 2) : 1) void attention_shared_kernel(const Args a) {
+__device__ __forceinline__ void attention_shared_body(const Args& a, const int block, const int thread) {
   const int page_shift = SP == 4 ? 3 : (SP == 2 ? 4 : a.page_shift);
   __shared__ __align__(16) bf16_t k_lds[2][32 * KROW];
   __shared__ __align__(16) bf16_t v_lds[2][D * VROW];
   __shared__ int bad_page;
-  const int tid = threadIdx.x, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+  const int tid = thread, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   // Late tiles of a prompt see the most keys.  Blocks are ranked longest first, and the ranks are dealt out to the
   // compute units like cards in a snake: the first `units` blocks take the longest, the next `units` blocks the
   // following ranks in ascending order, so that the two blocks that share a unit add up to about the same work.
   const int heads = a.kv_heads * a.head_groups, round = 2 * a.units;
-  const int turn = static_cast<int>(blockIdx.x) / round, within = static_cast<int>(blockIdx.x) % round;
+  const int turn = block / round, within = block % round;
   const int total = a.tiles * heads, in_round = min(round, total - turn * round);
   // a short last round has in_round < round blocks: its second part, if any, mirrors onto the ranks that exist
   const int rank = turn * round + (within < a.units ? within : in_round - 1 - (within - a.units));
@@ -1119,6 +1132,37 @@ __global__ __launch_bounds__(64 * kSharedWaves, D <= 128 ? (NQ == 1 ? 3 : 2) : 1
   }
 }
 
+template <int NQ, int SP>
+__global__ __launch_bounds__(64 * kSharedWaves, D <= 128 ? (NQ == 1 ? 3 : 2) : 1) void attention_shared_kernel(const Args a) {
+  attention_shared_body<NQ, SP>(a, static_cast<int>(blockIdx.x), static_cast<int>(threadIdx.x));
+}
+
+// ---- single tokens and short prompt portions in one launch ---------------------------------------------------------------
+// A step that decodes some requests and feeds a short portion of another's prompt has two attention launches that do
+// not depend on each other and do not fill the device: the single tokens' keys stream from memory, the portion's few
+// blocks wait for one load after the other.  One after the other they take the sum of their times; on two streams
+// they run beside each other, and the two waits between the streams cost most of what that saves.  Here they are one
+// grid: the first `portion_blocks` blocks are the portion's (they walk the longest, so they start first), every block
+// after them is four independent waves of the single tokens' kernel, wave w of block b standing where block
+// 4 b + w of that kernel's own grid (kv heads x items of the plan) would.  The text of either kernel is the same as in
+// its own launch, so the bits are.  Registers are the larger of the two (two waves a SIMD, which the single tokens'
+// kernel has anyway); every block holds the portion kernel's LDS.
+template <bool ONCE, int SP>
+__global__ __launch_bounds__(64 * kSharedWaves, 2) void attention_pair_kernel(const Args single, const Args portion,
+                                                                              const int portion_blocks) {
+  if constexpr (D % 64 == 0) {
+    if (static_cast<int>(blockIdx.x) < portion_blocks) {
+      attention_shared_body<1, SP>(portion, static_cast<int>(blockIdx.x), static_cast<int>(threadIdx.x));
+    } else {
+      const int gx = single.kv_heads * single.head_groups, gy = single.items_grid;
+      const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6);
+      const int unit = (static_cast<int>(blockIdx.x) - portion_blocks) * kSharedWaves + wave;
+      if (unit >= gx * gy) return;
+      attention_mfma_body<1, true, true, true, ONCE>(single, Where{unit % gx, unit / gx, 0, gx, gy, static_cast<int>(threadIdx.x) & 63});
+    }
+  }
+}
+
 // Merge of the segments' partial results: out = sum_z 2^(m_z - M) O_z / sum_z 2^(m_z - M) l_z, M = max_z m_z
 // (csrc/paged_decode.cu:528-544 of the reference has the same rule in base e).  One block of kMergeWaves waves per
 // (tile, head group, column); a lane owns dims lane, lane + 64, ...; wave w sums the segments w, w + kMergeWaves, ...
@@ -1265,6 +1309,74 @@ int launch(const Args& a, int tiles, bool shared, hipStream_t stream) {
   return AKV_LAUNCH_STATUS();
 }
 
+// The pair launch (see attention_pair_kernel), then the single tokens' merge.
+int launch_pair(const Args& single, const Args& portion, int portion_tiles, hipStream_t stream) {
+  if constexpr (D % 64 == 0) {
+    const long portion_blocks = static_cast<long>(portion_tiles) * portion.kv_heads * portion.head_groups;
+    const long units = static_cast<long>(single.kv_heads) * single.head_groups * single.items_grid;
+    const long blocks = portion_blocks + (units + kSharedWaves - 1) / kSharedWaves;
+    if (blocks > 0x7fffffffL) return -2;
+    const bool once = single.head_groups == 1;
+    const dim3 grid(static_cast<unsigned>(blocks));
+    const int first = static_cast<int>(portion_blocks);
+#define AKV_PAIR(SP_) \
+    do { \
+      if (once) attention_pair_kernel<true, SP_><<<grid, 64 * kSharedWaves, 0, stream>>>(single, portion, first); \
+      else attention_pair_kernel<false, SP_><<<grid, 64 * kSharedWaves, 0, stream>>>(single, portion, first); \
+    } while (0)
+    if (portion.page_shift >= 5) AKV_PAIR(1);
+    else if (portion.page_shift == 4) AKV_PAIR(2);
+    else if (portion.page_shift == 3) AKV_PAIR(4);
+    else return -2;
+#undef AKV_PAIR
+    const dim3 merge_grid(single.seq_count, single.kv_heads * single.head_groups, single.heads_per_tile);
+    attention_merge_kernel<1><<<merge_grid, 64 * kMergeWaves, 0, stream>>>(single);
+    return AKV_LAUNCH_STATUS();
+  } else {
+    return -2;
+  }
+}
+
+// What every launch of a step shares, checked and put into `a`; 0 or an error code.
+int common_args(Args& a, const void* q, const void* k_pages, const void* v_pages, void* out, const int* q_start,
+                const int* seq_lens, const int* block_table, const int* table_rows, int table_width, int q_heads,
+                int kv_heads, int page_size, long num_pages, float scale, int window) {
+  int page_shift = 0;
+  while ((1 << page_shift) < page_size) ++page_shift;
+  if (page_size < 4 || (1 << page_shift) != page_size || kv_heads <= 0 || q_heads % kv_heads != 0) return -2;
+  a.q = static_cast<const bf16_t*>(q);
+  a.k_pages = static_cast<const bf16_t*>(k_pages);
+  a.v_pages = static_cast<const bf16_t*>(v_pages);
+  a.out = static_cast<bf16_t*>(out);
+  a.q_start = q_start;
+  a.seq_lens = seq_lens;
+  a.block_table = block_table;
+  a.table_rows = table_rows;
+  a.table_width = table_width;
+  a.q_heads = q_heads;
+  a.kv_heads = kv_heads;
+  a.group = q_heads / kv_heads;
+  a.page_shift = page_shift;
+  a.num_pages = num_pages;
+  a.scale_log2 = scale * kLog2e;
+  a.window = window;
+  a.units = 1;
+  return 0;
+}
+
+// The compute units of the current device (asked once per device); 0 on an error.
+int units_of_device() {
+  static int units_of[64] = {0};
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 0;
+  if (units_of[device] == 0) {
+    int count = 0;
+    if (hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count <= 0) return 0;
+    units_of[device] = count;
+  }
+  return units_of[device];
+}
+
 }  // namespace
 
 #define AKV_CONCAT2(a, b) a##b
@@ -1294,44 +1406,27 @@ extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
     const float* q_weight, const float* k_weight, float eps, const float* rope_table, int table_positions,
     const int* plan, int items_grid, hipStream_t stream) {
   if (tiles <= 0 || seq_count <= 0) return 0;
-  int page_shift = 0;
-  while ((1 << page_shift) < page_size) ++page_shift;
-  if (page_size < 4 || (1 << page_shift) != page_size || q_heads % kv_heads != 0 ||
-      heads_per_tile * tokens_per_tile > 16 * nq || kv_heads * head_groups > 65535 || num_splits > 65535 ||
+  if (heads_per_tile * tokens_per_tile > 16 * nq || kv_heads * head_groups > 65535 || num_splits > 65535 ||
       num_splits < 1 || (single_tokens && tiles != seq_count) || (shared && (page_size < 8 || num_splits != 1)) ||
       (qkv != nullptr && (shared || !single_tokens || nq != 1 || D % 64 != 0 || (q_weight == nullptr) != (k_weight == nullptr))) ||
       (plan != nullptr && (shared || !single_tokens || seq_count > 64 || items_grid < 1 || items_grid > 65535)))
     return -2;
   Args a;
-  a.q = static_cast<const bf16_t*>(q);
-  a.k_pages = static_cast<const bf16_t*>(k_pages);
-  a.v_pages = static_cast<const bf16_t*>(v_pages);
-  a.out = static_cast<bf16_t*>(out);
+  const int status = common_args(a, q, k_pages, v_pages, out, q_start, seq_lens, block_table, table_rows, table_width,
+                                 q_heads, kv_heads, page_size, num_pages, scale, window);
+  if (status != 0) return status;
   a.partial = partial;
-  a.q_start = q_start;
-  a.seq_lens = seq_lens;
-  a.block_table = block_table;
-  a.table_rows = table_rows;
-  a.table_width = table_width;
   a.seq_first = seq_first;
   a.seq_count = seq_count;
   a.tiles = tiles;
-  a.q_heads = q_heads;
-  a.kv_heads = kv_heads;
-  a.group = q_heads / kv_heads;
   a.heads_per_tile = heads_per_tile;
   a.head_groups = head_groups;
   a.tokens_per_tile = tokens_per_tile;
-  a.page_shift = page_shift;
   a.single_tokens = single_tokens;
-  a.num_pages = num_pages;
-  a.scale_log2 = scale * kLog2e;
-  a.window = window;
   a.seg_keys = seg_keys;
   a.num_splits = num_splits;
   a.plan = plan;
   a.items_grid = items_grid;
-  a.units = 1;
   a.qkv = static_cast<const bf16_t*>(qkv);
   a.q_weight = q_weight;
   a.k_weight = k_weight;
@@ -1339,15 +1434,8 @@ extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
   a.table_positions = table_positions;
   a.eps = eps;
   if (shared) {
-    static int units_of[64] = {0};  // compute units per device, asked once
-    int device = 0;
-    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return -3;
-    if (units_of[device] == 0) {
-      int count = 0;
-      if (hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count <= 0) return -3;
-      units_of[device] = count;
-    }
-    a.units = units_of[device];
+    a.units = units_of_device();
+    if (a.units == 0) return -3;
     if (static_cast<long>(tiles) * kv_heads * head_groups > 0x7fffffffL) return -2;
   }
   switch (nq) {
@@ -1355,4 +1443,71 @@ extern "C" int AKV_CONCAT(akv_attention_mfma_d, AKV_HEAD_DIM)(
     case 2: return launch<2>(a, tiles, shared != 0, stream);
     default: return -2;
   }
+}
+
+// Single tokens and prompt portions of one step in ONE launch (see attention_pair_kernel), then the single tokens'
+// merge.  The single tokens are requests single_first .. + single_count - 1 (at most 64), with their raw projections
+// `qkv` and a plan of their keys as for the launch above with `qkv` and `plan` (so head sizes are multiples of 64);
+// the portions are requests portion_first .. + portion_count - 1 in blocks of four tiles of 16 columns that share keys
+// and values (`shared`, nq = 1; pages of 8 tokens and more), `portion_tiles` such blocks of tokens.  What the two
+// write and read is as in their own launches.
+extern "C" int AKV_CONCAT(akv_attention_pair_d, AKV_HEAD_DIM)(
+    const void* q, const void* k_pages, const void* v_pages, void* out, const int* q_start, const int* seq_lens,
+    const int* block_table, const int* table_rows, int table_width, int q_heads, int kv_heads, int page_size,
+    long num_pages, float scale, int window,
+    int single_first, int single_count, int single_heads_per_tile, int single_head_groups, float* partial,
+    const int* plan, int items_grid, const void* qkv, const float* q_weight, const float* k_weight, float eps,
+    const float* rope_table, int table_positions,
+    int portion_first, int portion_count, int portion_tiles, int portion_heads_per_tile, int portion_head_groups,
+    int portion_tokens_per_tile, hipStream_t stream) {
+  if (single_count <= 0 || portion_count <= 0 || portion_tiles <= 0) return -2;
+  if (D % 64 != 0 || page_size < 8 || single_count > 64 || plan == nullptr || qkv == nullptr || partial == nullptr ||
+      items_grid < 1 || items_grid > 65535 || (q_weight == nullptr) != (k_weight == nullptr) ||
+      single_heads_per_tile > 16 || portion_heads_per_tile * portion_tokens_per_tile > 16 ||
+      kv_heads * single_head_groups > 65535)
+    return -2;
+  Args single, portion;
+  int status = common_args(single, q, k_pages, v_pages, out, q_start, seq_lens, block_table, table_rows, table_width,
+                           q_heads, kv_heads, page_size, num_pages, scale, window);
+  if (status != 0) return status;
+  portion = single;
+  single.partial = partial;
+  single.seq_first = single_first;
+  single.seq_count = single_count;
+  single.tiles = single_count;
+  single.heads_per_tile = single_heads_per_tile;
+  single.head_groups = single_head_groups;
+  single.tokens_per_tile = 16 / single_heads_per_tile;
+  single.single_tokens = 1;
+  single.seg_keys = 0;
+  single.num_splits = 1;
+  single.plan = plan;
+  single.items_grid = items_grid;
+  single.qkv = static_cast<const bf16_t*>(qkv);
+  single.q_weight = q_weight;
+  single.k_weight = k_weight;
+  single.rope_table = rope_table;
+  single.table_positions = table_positions;
+  single.eps = eps;
+  portion.partial = nullptr;
+  portion.seq_first = portion_first;
+  portion.seq_count = portion_count;
+  portion.tiles = portion_tiles;
+  portion.heads_per_tile = portion_heads_per_tile;
+  portion.head_groups = portion_head_groups;
+  portion.tokens_per_tile = portion_tokens_per_tile;
+  portion.single_tokens = 0;
+  portion.seg_keys = 0;
+  portion.num_splits = 1;
+  portion.plan = nullptr;
+  portion.items_grid = 0;
+  portion.qkv = nullptr;
+  portion.q_weight = nullptr;
+  portion.k_weight = nullptr;
+  portion.rope_table = nullptr;
+  portion.table_positions = 0;
+  portion.eps = 0.f;
+  portion.units = units_of_device();
+  if (portion.units == 0) return -3;
+  return launch_pair(single, portion, portion_tiles, stream);
 }

@@ -134,7 +134,8 @@ class HipKernels(KernelSet):
         self.norm_in_products = True    # steps of a few rows: the products that follow a norm compute it themselves
         self.wide_prompt_tiles = None   # such blocks with 32 columns per wave instead of 16: None = by the step's size
         self.split_prompt_keys = None   # prompt portions on one wave per tile and key segment: None = by the step's size
-        self.portions_beside_single_tokens = True   # a step of both: the portions' attention on a second stream
+        self.pair_launch = True         # a step of single tokens and short portions: their attention as one launch,
+        self.portions_beside_single_tokens = True   # or, where that does not fit, the portions' on a second stream
         self._beside_stream = None
         self.compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
         for name in ("akv_embed", "akv_add_rmsnorm", "akv_rmsnorm_rows", "akv_copy_rows", "akv_gather_rows",
@@ -780,6 +781,61 @@ class HipKernels(KernelSet):
             self._attention_entry[head_dim] = entry
         return self._attention_entry[head_dim]
 
+    def _attention_pair_entry(self, head_dim: int):
+        key = ("pair", head_dim)
+        if key not in self._attention_entry:
+            self._attention_mfma_entry(head_dim)            # (loads the head size's library)
+            lib = ctypes.CDLL(ensure_attention(head_dim))
+            entry = getattr(lib, f"akv_attention_pair_d{head_dim}")
+            entry.restype = ctypes.c_int
+            self._attention_entry[key] = entry
+        return self._attention_entry[key]
+
+    def _pair_fits(self, ctx, decodes, q_heads, kv_heads, head_dim, page_size, fresh) -> bool:
+        """Whether a step's single tokens and prompt portions can go into one launch: the single tokens' kernel takes
+        raw projections and cuts the keys on the device (at most 64 requests, some history beyond one segment), the
+        portions are so short that their blocks of four narrow tiles do not fill the device, and no history of theirs
+        is so long that its keys would be cut."""
+        if not (self.pair_launch and fresh is not None and 0 < decodes <= 64 and head_dim % 64 == 0 and page_size >= 8
+                and self.share_prompt_tiles and self.cut_keys_on_device and self.split_prompt_keys is not True
+                and self.wide_prompt_tiles is not True):
+            return False
+        if max(ctx.host_seq_lens[:decodes]) <= self.decode_min_segment:
+            return False
+        if self._portion_blocks(ctx, decodes, q_heads, kv_heads) > self.compute_units:
+            return False
+        return not self._few_portion_blocks(ctx, decodes, q_heads, kv_heads)
+
+    def _attention_pair(self, q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out,
+                        page_size, num_pages, decodes, fresh):
+        """Requests 0 .. decodes - 1 (single tokens, raw projections in `fresh`) and the prompt portions behind them in
+        one launch of `akv_attention_pair`, then the single tokens' merge."""
+        group = q_heads // kv_heads
+        heads_per_tile = min(group, 16)
+        head_groups = (group + heads_per_tile - 1) // heads_per_tile
+        tokens_per_tile = 16 // heads_per_tile
+        starts = ctx.host_q_start
+        per_block = 4 * tokens_per_tile
+        portion_tiles = sum((starts[r + 1] - starts[r] + per_block - 1) // per_block for r in range(decodes, ctx.num_seqs))
+        # (the portions' blocks - four waves each - stand beside the single tokens' waves: together they are what one
+        # round of the device holds, or the single tokens' last blocks wait for a second round)
+        portion_waves = 4 * portion_tiles * kv_heads * head_groups
+        waves = max(self.decode_wave_target // 2, self.decode_wave_target - portion_waves)
+        plan, items_grid = self._decode_plan(ctx, 0, decodes, window, kv_heads * head_groups, waves)
+        count = items_grid * kv_heads * head_groups * 16 * (head_dim + 4)
+        arena = getattr(ctx, "arena", None)
+        partial = (arena.take((count,), torch.float32) if arena is not None
+                   else torch.empty(count, dtype=torch.float32, device=self.device))
+        qkv, q_weight, k_weight, eps, table = fresh
+        self._check(self._attention_pair_entry(head_dim)(
+            _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(out), _ptr(ctx.q_start), _ptr(ctx.seq_lens),
+            _ptr(meta.block_table), _ptr(getattr(meta, "rows", None)), meta.width, q_heads, kv_heads, page_size,
+            ctypes.c_long(num_pages), ctypes.c_float(scale), int(window) if window is not None else 0,
+            0, decodes, heads_per_tile, head_groups, _ptr(partial), _ptr(plan), items_grid, _ptr(qkv), _ptr(q_weight),
+            _ptr(k_weight), ctypes.c_float(eps), _ptr(table), table.shape[0] if table is not None else 0,
+            decodes, ctx.num_seqs - decodes, portion_tiles, heads_per_tile, head_groups, tokens_per_tile,
+            self._stream()), "attention")
+
     def _attention_mfma(self, q, k_pages, v_pages, ctx, meta, q_heads, kv_heads, head_dim, scale, window, out,
                         page_size, num_pages, seq_first, seq_count, nq, split, shared=False, fresh=None, single=None):
         """Requests seq_first .. seq_first + seq_count - 1 of the step on the MFMA kernel, in tiles of 16 * nq
@@ -831,13 +887,13 @@ class HipKernels(KernelSet):
 
     PLAN_ENTRIES = 132          # ints of a plan before its items (4 per item)
 
-    def _decode_plan(self, ctx, seq_first, seq_count, window, head_blocks):
+    def _decode_plan(self, ctx, seq_first, seq_count, window, head_blocks, waves=None):
         """The cut of the keys of requests seq_first .. + seq_count - 1 (single tokens) into (request, segment) items:
         segments of one size for all requests - about `decode_wave_target` waves in all, no segment shorter than
         `decode_min_segment` unless it is a request's only one - worked out by a one-wave kernel from the lengths on
         the device.  The cut depends on the lengths alone, so the layers of a step share one plan: it is remembered on
         the step's context.  Returns the plan and the bound on the number of items that sizes grids and buffers."""
-        items = max(1, self.decode_wave_target // head_blocks)
+        items = max(1, (waves if waves is not None else self.decode_wave_target) // head_blocks)
         key = (seq_first, seq_count, int(window) if window is not None else 0, items, self.decode_min_segment)
         plans = getattr(ctx, "decode_plans", None)
         if plans is None:
@@ -981,10 +1037,11 @@ class HipKernels(KernelSet):
         nothing else).
         A step of single tokens and short prompt portions: the two kinds read and write different requests' pages
         and different rows of `q` and `out`, and neither fills the device - the single tokens' keys stream from
-        memory, the portions' few blocks (no more than there are compute units) wait for one load after the other -
-        so the portions' launches go to a second stream and the two run beside each other.  (Measured in a recorded
-        step of 120 prompt tokens beside 8 x 8,192: 6.5 + 27 + 48 + 5 us one after the other, 66 us beside each
-        other and about 15 us for the two waits between the streams.)"""
+        memory, the portions' few blocks (no more than there are compute units) wait for one load after the other.
+        Where the two kernels can share a grid (`_pair_fits`) they are ONE launch, the portions' blocks first
+        (`akv_attention_pair`); otherwise the portions' launches go to a second stream and the two run beside each
+        other.  (Measured in a recorded step of 120 prompt tokens beside 8 x 8,192: 6.5 + 27 + 48 + 5 us one after
+        the other; on two streams 66 us beside each other and about 15 us for the two waits between the streams.)"""
         tokens = q.shape[0]
         self._dense(q, "q", None, (tokens, q_heads * head_dim))
         self._dense(out, "out", q.dtype, (tokens, q_heads * head_dim))
@@ -1028,6 +1085,11 @@ class HipKernels(KernelSet):
                     nq = 2 if wide else 1
                 self._attention_mfma(*common, decodes, ctx.num_seqs - decodes, nq, False, shared=shared)
 
+            if ctx.num_seqs > decodes and self._pair_fits(ctx, decodes, q_heads, kv_heads, head_dim, page_size, fresh):
+                if encode_portions is not None:
+                    encode_portions()
+                self._attention_pair(*common, decodes, fresh)
+                return
             beside = None
             if ctx.num_seqs > decodes:
                 if (decodes > 0 and self.portions_beside_single_tokens

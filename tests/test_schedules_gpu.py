@@ -265,6 +265,7 @@ def test_portions_beside_single_tokens_give_the_same_bits_as_one_after_the_other
         for graphs in (True, False):
             kernels = HipKernels("cuda:0")
             kernels.portions_beside_single_tokens = beside
+            kernels.pair_launch = False                    # (the one launch for both has its own test below)
             engines[beside, graphs] = Engine.from_folder(folder, EngineConfig(
                 dtype="bfloat16", page_size=page, num_pages=2400 // page, max_seqs=6, max_batched_tokens=1024,
                 max_seq_len=1024, device="cuda:0", decode_graphs=graphs), kernels=kernels)
@@ -370,3 +371,73 @@ def test_a_long_request_beside_short_ones_across_the_widths_of_the_block_table(n
         for seq in mine.values():
             engine.close(seq)
         assert engine.cache.num_free_pages == [pages]
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16"])
+def test_single_tokens_and_a_portion_in_one_launch_give_the_same_bits_at_qwen3_8b_layer_sizes(two_layers, dtype):
+    """Heads of 128 in groups of four: the single tokens' attention (raw projections, keys cut on the device) and a
+    short portion's attention (blocks of four waves) as ONE launch, against the same two kernels launched one after the
+    other - the same text runs, so every logit must have the same bits - eager, recorded, replayed; with histories
+    long enough that the single tokens' keys are cut, a portion with and without a history, and steps the launch does
+    not fit (a portion alone, single tokens alone, a portion whose blocks fill the device) in between."""
+    from ampere_kv_engine_amd.kernels.hip import HipKernels
+    folder, plain = two_layers
+    engines, calls = {}, {}
+    for pair in (True, False):
+        for graphs in (True, False):
+            kernels = HipKernels("cuda:0")
+            kernels.pair_launch, kernels.portions_beside_single_tokens = pair, False
+            counted = calls[pair, graphs] = [0]
+            inner = kernels._attention_pair
+            kernels._attention_pair = lambda *a, _inner=inner, _n=counted, **kw: (_n.__setitem__(0, _n[0] + 1), _inner(*a, **kw))[1]
+            engines[pair, graphs] = Engine.from_folder(folder, EngineConfig(
+                dtype=dtype, page_size=16, num_pages=200, max_seqs=8, max_batched_tokens=2048, max_seq_len=2048,
+                device="cuda:0", decode_graphs=graphs), kernels=kernels)
+    ids = {key: random_ids(1000, 1500, seed=700 + i) for i, key in enumerate("abcdefg")}
+    fed = {key: 0 for key in ids}
+    seqs = {mode: {} for mode in engines}
+    kept = {}
+
+    def step(parts, keep=None):
+        outs = {}
+        for mode, engine in engines.items():
+            entries = []
+            for key, count, want in parts:
+                if key not in seqs[mode]:
+                    seqs[mode][key] = engine.open(key)
+                entries.append(StepEntry(seqs[mode][key], ids[key][fed[key]:fed[key] + count], want))
+            outs[mode] = engine.step(entries).cpu()
+        first = outs[True, True]
+        for mode, out in outs.items():
+            assert torch.equal(out, first), f"{mode} differs from (True, True) in a step of {[p[1] for p in parts]}"
+        if keep is not None:
+            kept[keep] = (first, [(key, fed[key], count, want) for key, count, want in parts])
+        for key, count, _ in parts:
+            fed[key] += count
+
+    step([("a", 300, [299]), ("b", 170, [169])])                   # histories beyond one segment of 128 keys
+    step([("c", 140, [139])])
+    for turn in range(6):                                          # met, recorded, replayed: a portion without a history first
+        step([("a", 1, [0]), ("b", 1, [0]), ("c", 1, [0]), ("d", 40, [39, 0])], keep="mixed" if turn == 5 else None)
+    step([("e", 700, [699])])                                      # a portion alone
+    for turn in range(4):                                          # other requests, two portions, one with a history
+        step([("e", 1, [0]), ("a", 1, [0]), ("d", 24, [23]), ("f", 9, [8])])
+    step([("a", 1, [0]), ("b", 1, [0]), ("g", 1100, [1099])])      # a portion whose blocks fill the device: two launches
+    step([("a", 1, [0]), ("b", 1, [0]), ("c", 1, [0])])            # single tokens alone
+    layers = 2                                                     # (a call per layer of every step that fits)
+    assert calls[True, True][0] >= 2 * layers and calls[True, False][0] == 10 * layers
+    assert calls[False, True][0] == calls[False, False][0] == 0
+    # and the numbers are right: the last mixed step of the first kind against the plain implementation, in the root
+    # mean square (at these widths a single logit's limit is met by rounding alone, see test_large_sizes_gpu.py)
+    logits, parts = kept["mixed"]
+    row = 0
+    for key, start, count, want in parts:
+        expected = plain.logits(ids[key][:start + count])
+        for place in want:
+            _, _, by_rms = cases.error_of(logits[row][None], expected[start + place][None], dtype, "plain")
+            assert by_rms <= 1.0, f"request {key}: rms error {by_rms:.2f} of its limit against the plain implementation"
+            row += 1
+    for mode, engine in engines.items():
+        for seq in seqs[mode].values():
+            engine.close(seq)
+        assert engine.cache.num_free_pages == [200]
