@@ -24,6 +24,9 @@
 // GATED: the packed matrix alternates gate and up tiles (RT = 2 gives a wave one pair); what is stored is
 // silu(gate) * up from the float32 sums.
 
+#include <mutex>
+#include <type_traits>
+
 #include "common.h"
 #include "mfma_tiles.h"
 #include "api.h"
@@ -34,6 +37,31 @@ namespace {
 
 constexpr int kHalves = 2;   // waves along k (A waves along the band of row tiles: 2, 3 or 4)
 constexpr int kFetchers = 4;
+
+// What a product does beyond y = x W^T in a step of many rows that keeps the residual sum and the norm between two
+// branches out of kernels of their own (all pointers null: nothing).
+//   ADDS (`stream`; never gated, y bfloat16): the branch's last product rounds its result to bfloat16, adds it to the
+//   float32 residual sum in place, stores the new sum times the weight of the norm that follows (`gain`) as y, and
+//   leaves, per band of its row tiles and row, the sum of squares of the band's new values in `sums_out`.
+//   ROWSCALED (`sums_in`): x holds such rows - the residual sum times the norm's weight, not yet divided by the
+//   rows' root mean square.  The division commutes with the product: every float32 sum is multiplied by
+//   rsqrt(mean of squares + eps) of its row before bias, activation and rounding; the row's sum of squares is added
+//   up from the `groups_in` partial sums that the ADDS product left (in the order of the bands, by the fetching waves,
+//   who asked for them before the stream began).  Against a norm kernel's rows (scaled, rounded, times the weight,
+//   rounded) the operand is rounded once and the scale stays in float32.
+struct MidFold {
+  float* stream;          // ADDS: [rows, outs]
+  const float* gain;      // ADDS: [outs]
+  float* sums_out;        // ADDS: [bands][sum_stride]
+  const float* sums_in;   // ROWSCALED: [groups_in][sum_stride]
+  int groups_in;
+  int sum_stride;         // rows of the step, rounded up to a multiple of 16
+  float eps, inv_k;       // ROWSCALED: 1 / width of the normed rows (this product's k)
+};
+constexpr int kMostSums = 40;   // partial sums of a row that one fetching thread adds up (it holds them in registers)
+// threads of the fetching waves that share a row's partial sums
+template <int MT> constexpr int kSumChunks = (kFetchers * 64) / (MT * 16);
+constexpr int kExtraFloats = 256 + 4 * 128;   // LDS behind the staging memory: the rows' sums by chunk; squares by wave
 
 template <int MT> constexpr int kStage = MT <= 4 ? 4 : 2;     // k-tiles per stage and k half
 
@@ -47,14 +75,18 @@ __global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_ker
                                                               TY* __restrict__ y, float* __restrict__ partial,
                                                               unsigned* __restrict__ counters, int rows, int outs, int k,
                                                               int k_tiles, int n_tiles, int bands, int parts,
-                                                              int part_tiles, int m_blocks, const float* __restrict__ bias) {
+                                                              int part_tiles, int m_blocks, const float* __restrict__ bias,
+                                                              const MidFold fold) {
   constexpr int S = kStage<MT>;
+  constexpr int kBlockRows = MT * 16, kChunks = kSumChunks<MT>;
+  const bool rowscaled = fold.sums_in != nullptr;
   constexpr int kAlong = A, kMultipliers = A * kHalves;
   constexpr int kTiles = kHalves * S * MT;        // activation tiles of one stage
   constexpr int kLoads = kTiles / kFetchers;      // of which every fetching wave brings this many
   static_assert(kTiles % kFetchers == 0, "the stage's tiles are dealt to the fetching waves");
   static_assert(G % 2 == 0, "a ring position must always meet the same staging buffer");
   extern __shared__ uintx4 staged[];              // [2][kTiles][64]; afterwards the sums of the second k half, then a flag
+  float* extra = reinterpret_cast<float*>(staged + 2 * kTiles * 64);   // [kExtraFloats]
 
   // which work: blocks that share weights (same band and part of k, other rows) are neighbours on one XCD
   const int xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
@@ -108,6 +140,17 @@ __global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_ker
         staged[(buffer * kTiles + (h * S + u) * MT + row / 16) * 64 + slot_of(u, g, row % 16)] = (exists >> j & 1u) ? from[j] : zero;
       }
     };
+    // ROWSCALED: thread (chunk, row) asks for the partial sums chunk, chunk + kChunks, ... of its row before anything
+    // else (loads come back in the order they were asked for: asked for later, they would stand between the first
+    // stages' activations and their filing) and adds them up when the stream is over.
+    const int ft = threadIdx.x - kMultipliers * 64, sum_row = ft % kBlockRows, sum_chunk = ft / kBlockRows;
+    float partials[kMostSums];
+    if (rowscaled) {
+      const float* from = fold.sums_in + min(row0 + sum_row, fold.sum_stride - 1);
+#pragma unroll
+      for (int i = 0; i < kMostSums; ++i)
+        partials[i] = from[static_cast<size_t>(min(sum_chunk + kChunks * i, fold.groups_in - 1)) * fold.sum_stride];
+    }
     fetch_rows(0, fetched[0], there[0]);
     fetch_rows(1, fetched[1], there[1]);
     __builtin_amdgcn_sched_barrier(0);
@@ -127,6 +170,14 @@ __global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_ker
     if (first < stages) {
       file_rows(0, fetched[0], there[0]);
       __syncthreads();
+    }
+    if (rowscaled) {
+      float total = 0.f;
+#pragma unroll
+      for (int i = 0; i < kMostSums; ++i)
+        if (sum_chunk + kChunks * i < fold.groups_in) total += partials[i];
+      if (sum_chunk < kChunks) extra[sum_chunk * kBlockRows + sum_row] = total;
+      __syncthreads();   // (the multiplying waves meet it when their stream is over)
     }
     return;
   }
@@ -264,6 +315,89 @@ __global__ __launch_bounds__((A * kHalves + kFetchers) * 64) void linear_mid_ker
     }
   }
   if (half != 0) return;
+  if (rowscaled) {   // every sum times its row's 1 / root mean square
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      float total = 0.f;
+#pragma unroll
+      for (int c = 0; c < kChunks; ++c) total += extra[c * kBlockRows + mt * 16 + r];
+      const float scale = rsqrtf(total * fold.inv_k + fold.eps);
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[rt][mt][i] *= scale;
+    }
+  }
+  constexpr bool kMayAdd = !GATED && std::is_same<TY, bf16_t>::value;
+  if constexpr (kMayAdd) {
+    if (fold.stream != nullptr) {
+      // What the sums are added to - the residual sum's values at this wave's outputs, and the norm's weight there -
+      // is asked for in one go, every load whatever its place (places beyond the matrix or the rows ask at one that
+      // exists and are not used): loads behind tests would be waited for one by one, a trip to memory each.  (Asked
+      // for before the exchanges of sums, which would hide their way, they take the registers that the exchange
+      // needs to have its own loads in flight together: 24 -> 83 us at 128 rows.)
+      const bool whole_quads = (outs & 3) == 0;
+      float4 held[RT][MT], weight_held[RT];
+      if (whole_quads) {
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          const int feature = max(0, min((tile0 + rt) * 16 + g * 4, outs - 4));
+          weight_held[rt] = *reinterpret_cast<const float4*>(fold.gain + feature);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            held[rt][mt] = *reinterpret_cast<const float4*>(fold.stream + static_cast<size_t>(min(row0 + mt * 16 + r, rows - 1)) * outs + feature);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      float squares[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        squares[mt] = 0.f;
+        const int row = row0 + mt * 16 + r;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+          const int feature = (tile0 + rt) * 16 + g * 4;
+          if (tile0 + rt >= n_tiles || row >= rows || feature >= outs) continue;
+          const floatx4 product = plus_bias(acc[rt][mt], bias, feature, outs);
+          float* sum_at = fold.stream + static_cast<size_t>(row) * outs + feature;
+          if (whole_quads) {     // (then feature + 3 < outs: the features of a quad exist together)
+            const float4 before = held[rt][mt], weight = weight_held[rt];
+            floatx4 now = {before.x + rounded<bf16_t>(product[0]), before.y + rounded<bf16_t>(product[1]),
+                           before.z + rounded<bf16_t>(product[2]), before.w + rounded<bf16_t>(product[3])};
+            *reinterpret_cast<float4*>(sum_at) = make_float4(now[0], now[1], now[2], now[3]);
+            squares[mt] += now[0] * now[0] + now[1] * now[1] + now[2] * now[2] + now[3] * now[3];
+            store4<bf16_t>(y + static_cast<size_t>(row) * outs + feature,
+                           floatx4{now[0] * weight.x, now[1] * weight.y, now[2] * weight.z, now[3] * weight.w});
+          } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (feature + i < outs) {
+                const float now = sum_at[i] + rounded<bf16_t>(product[i]);
+                sum_at[i] = now;
+                squares[mt] += now * now;
+                y[static_cast<size_t>(row) * outs + feature + i] = from_float<bf16_t>(now * fold.gain[feature + i]);
+              }
+          }
+        }
+        squares[mt] += __shfl_xor(squares[mt], 16, kWave);
+        squares[mt] += __shfl_xor(squares[mt], 32, kWave);
+      }
+      // the band's sum per row: the waves along the band, added in their order
+      float* by_wave = extra + 256;
+      if (g == 0) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) by_wave[along * kBlockRows + mt * 16 + r] = squares[mt];
+      }
+      __syncthreads();   // (only the first k half's waves are left)
+      for (int row = along * 64 + lane; row < kBlockRows; row += kAlong * 64) {
+        float total = 0.f;
+#pragma unroll
+        for (int w = 0; w < kAlong; ++w) total += by_wave[w * kBlockRows + row];
+        if (row0 + row < fold.sum_stride) fold.sums_out[static_cast<size_t>(band) * fold.sum_stride + row0 + row] = total;
+      }
+      return;
+    }
+  }
   if constexpr (GATED) {
     static_assert(RT % 2 == 0, "a wave must own gate and up tiles in pairs");
 #pragma unroll
@@ -349,25 +483,41 @@ MidPlan plan_mid(int rows, int n_tiles, int k_tiles, bool gated, int along, int 
 
 template <int A, int MT, int RT, int G, bool GATED, typename TY>
 int launch_mid(const MidPlan& p, const void* x, const void* wp, void* y, float* partial, unsigned* counters, int rows,
-               int outs, int k, int k_tiles, int n_tiles, const float* bias, hipStream_t stream) {
-  constexpr size_t lds = 2 * kHalves * kStage<MT> * MT * 1024;
-  static_assert(lds >= static_cast<size_t>(A) * RT * MT * 1024, "the sums of a k half must fit the staging memory");
-  static_assert(lds <= 64 * 1024, "the staging memory is taken without asking for more than a block may have by default");
+               int outs, int k, int k_tiles, int n_tiles, const float* bias, const MidFold& fold, hipStream_t stream) {
+  constexpr size_t staging = 2 * kHalves * kStage<MT> * MT * 1024;
+  static_assert(staging >= static_cast<size_t>(A) * RT * MT * 1024, "the sums of a k half must fit the staging memory");
+  static_assert(staging <= 64 * 1024, "the staging memory of a block");
+  static_assert(kSumChunks<MT> * MT * 16 <= 256 && A * MT * 16 <= 4 * 128, "what lies behind the staging memory");
+  constexpr size_t lds = staging + kExtraFloats * 4;
+  if (fold.sums_in != nullptr && fold.groups_in > kSumChunks<MT> * kMostSums) return -2;
+  if (lds > 64 * 1024) {   // more than a block may have without asking: asked once per kernel and device
+    static std::mutex guard;
+    static bool asked[64] = {};
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return -2;
+    std::lock_guard<std::mutex> lock(guard);
+    if (!asked[device]) {
+      const hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_mid_kernel<A, MT, RT, G, GATED, TY>),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+      if (status != hipSuccess) return static_cast<int>(status);
+      asked[device] = true;
+    }
+  }
   const long items = static_cast<long>(p.bands) * p.parts;
   const long blocks = (items + kXcds - 1) / kXcds * kXcds * p.m_blocks;
   if (blocks > 0x7fffffffL) return -2;
   linear_mid_kernel<A, MT, RT, G, GATED, TY><<<static_cast<unsigned>(blocks), (A * kHalves + kFetchers) * 64, lds, stream>>>(
       static_cast<const bf16_t*>(x), static_cast<const uintx4*>(wp), static_cast<TY*>(y), partial, counters, rows, outs,
-      k, k_tiles, n_tiles, p.bands, p.parts, p.part_tiles, p.m_blocks, GATED ? nullptr : bias);
+      k, k_tiles, n_tiles, p.bands, p.parts, p.part_tiles, p.m_blocks, GATED ? nullptr : bias, fold);
   return AKV_LAUNCH_STATUS();
 }
 
 template <bool GATED, typename TY>
 int dispatch_mid(const MidPlan& p, const void* x, const void* wp, void* y, float* partial, unsigned* counters, int rows,
-                 int outs, int k, int k_tiles, int n_tiles, const float* bias, hipStream_t stream) {
+                 int outs, int k, int k_tiles, int n_tiles, const float* bias, const MidFold& fold, hipStream_t stream) {
 #define AKV_MID(A_, MT_, RT_, G_) \
   if (p.along == A_ && p.mt == MT_ && p.rt == RT_ && p.depth == G_) \
-    return launch_mid<A_, MT_, RT_, G_, GATED, TY>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, bias, stream)
+    return launch_mid<A_, MT_, RT_, G_, GATED, TY>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, bias, fold, stream)
 #define AKV_MID_ROWS(A_, RT_, G_) \
   AKV_MID(A_, 2, RT_, G_); AKV_MID(A_, 3, RT_, G_); AKV_MID(A_, 4, RT_, G_); AKV_MID(A_, 5, RT_, G_); \
   AKV_MID(A_, 6, RT_, G_); AKV_MID(A_, 7, RT_, G_); AKV_MID(A_, 8, RT_, G_)
@@ -401,10 +551,10 @@ extern "C" int akv_linear_mid_workspace(int rows, int n_tiles, int k_tiles, int 
 // `partial_floats` and `counter_words` say how much `partial` and `counters` hold: a cut that needs more
 // (akv_linear_mid_workspace tells) is refused with -3 and nothing is launched.  `bias` [outs] float32 or null (never with
 // `gated`): added to the float32 sums before they are rounded.
-extern "C" int akv_linear_mid(const void* x, const void* wp, void* y, int y_dtype, float* partial, long partial_floats,
-                              unsigned* counters, long counter_words, int rows, int outs, int k, int n_tiles,
-                              int k_tiles, int gated, int along, int rt, int depth, int parts, const float* bias,
-                              hipStream_t stream) {
+namespace {
+int linear_mid(const void* x, const void* wp, void* y, int y_dtype, float* partial, long partial_floats,
+               unsigned* counters, long counter_words, int rows, int outs, int k, int n_tiles, int k_tiles, int gated,
+               int along, int rt, int depth, int parts, const float* bias, const MidFold& fold, hipStream_t stream) {
   if (rows <= 0 || outs <= 0) return 0;
   if ((k & 7) != 0 || k_tiles * 32 < k) return -2;
   if (gated ? ((outs & 15) != 0 || n_tiles * 8 != outs) : n_tiles * 16 < outs) return -2;
@@ -415,11 +565,60 @@ extern "C" int akv_linear_mid(const void* x, const void* wp, void* y, int y_dtyp
   if (p.parts > 1 && (partial == nullptr || counters == nullptr)) return -2;
   if (p.parts > 1 && (static_cast<long>(p.partial_floats) > partial_floats || static_cast<long>(p.counters) > counter_words)) return -3;
   if (gated) {
-    if (y_dtype == kF32) return dispatch_mid<true, float>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, bias, stream);
-    if (y_dtype == kBF16) return dispatch_mid<true, bf16_t>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, bias, stream);
+    if (y_dtype == kF32) return dispatch_mid<true, float>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, bias, fold, stream);
+    if (y_dtype == kBF16) return dispatch_mid<true, bf16_t>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, bias, fold, stream);
     return -1;
   }
-  if (y_dtype == kF32) return dispatch_mid<false, float>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, bias, stream);
-  if (y_dtype == kBF16) return dispatch_mid<false, bf16_t>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, bias, stream);
+  if (y_dtype == kF32) return dispatch_mid<false, float>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, bias, fold, stream);
+  if (y_dtype == kBF16) return dispatch_mid<false, bf16_t>(p, x, wp, y, partial, counters, rows, outs, k, k_tiles, n_tiles, bias, fold, stream);
   return -1;
+}
+}  // namespace
+
+extern "C" int akv_linear_mid(const void* x, const void* wp, void* y, int y_dtype, float* partial, long partial_floats,
+                              unsigned* counters, long counter_words, int rows, int outs, int k, int n_tiles,
+                              int k_tiles, int gated, int along, int rt, int depth, int parts, const float* bias,
+                              hipStream_t stream) {
+  return linear_mid(x, wp, y, y_dtype, partial, partial_floats, counters, counter_words, rows, outs, k, n_tiles, k_tiles,
+                    gated, along, rt, depth, parts, bias, MidFold{}, stream);
+}
+
+// The bands of row tiles into which akv_linear_mid_adds cuts this product (one partial sum of squares per band and
+// row), and the most partial sums per row that akv_linear_mid_rowscaled adds up for a step of `rows` rows.
+extern "C" int akv_linear_mid_bands(int rows, int n_tiles, int k_tiles) {
+  return plan_mid(rows, n_tiles, k_tiles, false, 0, 0, 0, 0).bands;
+}
+extern "C" int akv_linear_mid_most_groups(int rows) {
+  const int row_tiles = (rows + 15) / 16, m_blocks = (row_tiles + 7) / 8;
+  const int mt = row_tiles < 2 ? 2 : (row_tiles + m_blocks - 1) / m_blocks;
+  return (kFetchers * 64) / (mt * 16) * kMostSums;
+}
+
+// A branch's last product in a step of many rows (see `MidFold`): stream_sum [rows, outs] float32 += bfloat16(x W^T (+
+// bias)) in place; y [rows, outs] bfloat16 receives the new sum times `gain` [outs]; sums_out [bands][sum_stride]
+// float32 the bands' sums of squares per row (bands: akv_linear_mid_bands; sum_stride >= rows, a multiple of 16).
+extern "C" int akv_linear_mid_adds(const void* x, const void* wp, void* y, float* partial, long partial_floats,
+                                   unsigned* counters, long counter_words, int rows, int outs, int k, int n_tiles,
+                                   int k_tiles, const float* bias, float* stream_sum, const float* gain, float* sums_out,
+                                   int sum_stride, hipStream_t stream) {
+  if (stream_sum == nullptr || gain == nullptr || sums_out == nullptr || sum_stride < rows || (sum_stride & 15) != 0) return -2;
+  MidFold fold{};
+  fold.stream = stream_sum, fold.gain = gain, fold.sums_out = sums_out, fold.sum_stride = sum_stride;
+  return linear_mid(x, wp, y, kBF16, partial, partial_floats, counters, counter_words, rows, outs, k, n_tiles, k_tiles, 0,
+                    0, 0, 0, 0, bias, fold, stream);
+}
+
+// The product that reads rows left by akv_linear_mid_adds: y = (x W^T) * rsqrt(sum of squares of the row / k + eps) (+
+// bias; gated: silu of the scaled gate times the scaled up), the row's sum added up from sums_in [groups][sum_stride].
+// Refused with -2 where `groups` exceeds akv_linear_mid_most_groups(rows).
+extern "C" int akv_linear_mid_rowscaled(const void* x, const void* wp, void* y, int y_dtype, float* partial,
+                                        long partial_floats, unsigned* counters, long counter_words, int rows, int outs,
+                                        int k, int n_tiles, int k_tiles, int gated, const float* bias,
+                                        const float* sums_in, int groups, int sum_stride, float eps, hipStream_t stream) {
+  if (sums_in == nullptr || groups <= 0 || sum_stride < rows) return -2;
+  MidFold fold{};
+  fold.sums_in = sums_in, fold.groups_in = groups, fold.sum_stride = sum_stride, fold.eps = eps;
+  fold.inv_k = 1.f / static_cast<float>(k);
+  return linear_mid(x, wp, y, y_dtype, partial, partial_floats, counters, counter_words, rows, outs, k, n_tiles, k_tiles,
+                    gated, 0, 0, 0, 0, bias, fold, stream);
 }

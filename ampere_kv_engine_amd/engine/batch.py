@@ -124,6 +124,8 @@ class StepContext:
     # set by the model's pass and by blocks around every branch: the branch may add its output to the residual sum in
     # its last product and return `StreamSums` (see `parts.base.Part`)
     fold_into_stream: bool = False
+    # ... and the weight of the norm that will read what the branch leaves, where that norm has one (`Norm.fold_gain`)
+    fold_gain: object = None
     # the device's persistent integer state (slot words, block tables) and what this step changes in it
     table_pages: int = 0                        # bound on the pages of the step's longest request (sizes launches)
     patches: torch.Tensor | None = None         # int32 [2 * patch_room]: (offset into slot_state, value) pairs

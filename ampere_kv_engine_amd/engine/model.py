@@ -97,6 +97,7 @@ class Model:
             # instead, if whoever reads `pending` next knows what to make of that: the next block, or the end below
             following = self.blocks[order[step_index + 1].layer] if step_index + 1 < len(order) else None
             ctx.fold_into_stream = following is None or following.takes_stream_sums
+            ctx.fold_gain = following.entry_gain() if following is not None and following.takes_stream_sums else None
             pending = self.blocks[entry.layer].forward(ctx.stream, pending, ctx, layer_cache[entry.cache_layer],
                                                        entry.writes_cache)
         if isinstance(pending, StreamSums):      # the last branch's output is in the residual sum already

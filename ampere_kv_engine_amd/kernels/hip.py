@@ -142,6 +142,7 @@ class HipKernels(KernelSet):
                      "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
                      "akv_linear_tiled", "akv_linear_packed", "akv_linear_packed_swiglu", "akv_linear_packed_normed",
                      "akv_pack_rows", "akv_linear_packed_static", "akv_linear_mid", "akv_linear_mid_workspace",
+                     "akv_linear_mid_adds", "akv_linear_mid_rowscaled", "akv_linear_mid_bands", "akv_linear_mid_most_groups",
                      "akv_linear_adds", "akv_linear_scaled", "akv_linear_decode_plan", "akv_read_probe",
                      "akv_attention_rows", "akv_decode_plan", "akv_sample", "akv_sample_slots", "akv_step_prologue"):
             getattr(self.lib, name).restype = ctypes.c_int
@@ -368,9 +369,11 @@ class HipKernels(KernelSet):
             return "mid"
         return "library"
 
-    def _mid(self, x, packed: PackedWeight, out, rows: int, outs: int, gated: bool, bias=None) -> None:
+    def _mid(self, x, packed: PackedWeight, out, rows: int, outs: int, gated: bool, bias=None, adds=None, scaled=None) -> None:
         """The mid-size product (`csrc/gemm_mid.hip`).  Where it cuts k over blocks it needs room for partial sums
-        and a few counters; both belong to this kernel set and serve one launch at a time (one stream)."""
+        and a few counters; both belong to this kernel set and serve one launch at a time (one stream).
+        `adds` = (stream, gain, sums): the product adds itself to the residual sum (`add_to_stream`); `scaled` =
+        (sums, eps): its results are divided by the rows' root mean square (`linear_rowscaled`)."""
         partial_floats, counters = ctypes.c_long(0), ctypes.c_long(0)
         self.lib.akv_linear_mid_workspace(rows, packed.n_tiles, packed.k_tiles, 1 if gated else 0, 0, 0, 0, 0,
                                           ctypes.byref(partial_floats), ctypes.byref(counters))
@@ -386,6 +389,23 @@ class HipKernels(KernelSet):
                 self._outgrown.append(self._mid_counters)
                 self._mid_counters = torch.zeros(max(counters.value, 1 << 16), dtype=torch.int32, device=self.device)
         held = lambda buffer: ctypes.c_long(buffer.numel() if buffer is not None else 0)
+        if adds is not None:
+            stream, gain, sums = adds
+            self._check(self.lib.akv_linear_mid_adds(_ptr(x), _ptr(packed.data), _ptr(out), _ptr(self._mid_partial),
+                                                     held(self._mid_partial), _ptr(self._mid_counters), held(self._mid_counters),
+                                                     rows, outs, packed.k, packed.n_tiles, packed.k_tiles, _ptr(bias),
+                                                     _ptr(stream), _ptr(gain), _ptr(sums), sums.shape[1], self._stream()),
+                        "mid-size product that adds to the residual sum")
+            return
+        if scaled is not None:
+            sums, eps = scaled
+            self._check(self.lib.akv_linear_mid_rowscaled(_ptr(x), _ptr(packed.data), _ptr(out), _code(out), _ptr(self._mid_partial),
+                                                          held(self._mid_partial), _ptr(self._mid_counters), held(self._mid_counters),
+                                                          rows, outs, packed.k, packed.n_tiles, packed.k_tiles, 1 if gated else 0,
+                                                          _ptr(bias), _ptr(sums), sums.shape[0], sums.shape[1],
+                                                          ctypes.c_float(eps), self._stream()),
+                        "mid-size product of rows to be scaled")
+            return
         self._check(self.lib.akv_linear_mid(_ptr(x), _ptr(packed.data), _ptr(out), _code(out), _ptr(self._mid_partial),
                                             held(self._mid_partial), _ptr(self._mid_counters), held(self._mid_counters),
                                             rows, outs, packed.k, packed.n_tiles,
@@ -513,12 +533,19 @@ class HipKernels(KernelSet):
                                     # (measured from 1 to 16 rows at Qwen3-8B sizes: 5 to 14 us less per layer)
     FOLD_NORM_BYTES = 160 * 1024 - 832   # ... while the normed rows fit into a compute unit's LDS beside the scales
     fold_norms = True
+    FOLD_MID_ROWS = 512             # ... and steps of up to this many, where the mid-size kernel takes the products:
+    fold_mid = True                 # (a layer launches two norm kernels less: 5 us each and the gaps around them)
 
     def folds_norm(self, rows: int, hidden: int, dtype) -> bool:
         """Whether a step of `rows` rows may let a branch's last product add itself to the residual sum
-        (`linear_adds`) and the next product norm its rows itself from the sums left there (`linear_scaled`)."""
-        return (self.fold_norms and 0 < rows <= self.FOLD_NORM_ROWS and dtype == torch.bfloat16 and hidden % 8 == 0
-                and rows * hidden * 2 <= self.FOLD_NORM_BYTES)
+        (`add_to_stream`) and the next product take the norm upon itself: up to 16 rows it norms the rows from the
+        sums left there (`linear_scaled`); up to 512 it reads rows that the adding product left multiplied by the
+        norm's weight and divides its results by the rows' root mean square (`linear_rowscaled`)."""
+        if dtype != torch.bfloat16 or hidden % 8 != 0:
+            return False
+        if 0 < rows <= self.FOLD_NORM_ROWS:
+            return self.fold_norms and rows * hidden * 2 <= self.FOLD_NORM_BYTES
+        return self.fold_mid and rows <= self.FOLD_MID_ROWS
 
     def _reserve_exchange(self, n_tiles: int) -> None:
         """Called when a matrix is prepared: the memory through which two blocks of a decode product exchange the sums
@@ -548,12 +575,66 @@ class HipKernels(KernelSet):
         self.lib.akv_linear_decode_plan(row_tiles_per_wave, packed.n_tiles, packed.k_tiles, packed.k, normed_rows, may, out)
         return dict(k_split=out[0], waves=out[1], blocks=out[2], straddles=bool(out[3]), work_kb=out[4])
 
-    def adds_to_stream(self, rows: int, weight, dtype) -> bool:
-        return isinstance(weight, PackedWeight) and self.folds_norm(rows, weight.outs, dtype)
+    def adds_to_stream(self, rows: int, weight, dtype, gain=None) -> bool:
+        if not isinstance(weight, PackedWeight) or not self.folds_norm(rows, weight.outs, dtype):
+            return False
+        if rows <= self.FOLD_NORM_ROWS:
+            return True
+        # many rows: the mid-size kernel, which must know the weight of the norm that follows
+        return gain is not None and self._route("linear", weight.outs, weight.k, rows, weight.row_major is not None,
+                                                torch.bfloat16) == "mid"
+
+    def add_to_stream(self, x, weight: PackedWeight, stream, arena, bias=None, gain=None):
+        """stream [rows, outs] (float32) += bfloat16(x W^T (+ bias)) in place; returns what the product left for the
+        norm that follows (`StreamSums`): the rows' partial sums of squares, and in steps of more than 16 rows the
+        new rows times `gain` as well."""
+        from ..parts.base import StreamSums
+        rows = x.shape[0]
+        if rows <= self.FOLD_NORM_ROWS:
+            sums = arena.take(((weight.outs + 15) // 16, 16), torch.float32)
+            self.linear_adds(x, weight, stream, sums, bias=bias)
+            return StreamSums(sums)
+        self._dense(x, "x", torch.bfloat16, (rows, weight.k))
+        self._dense(stream, "stream", torch.float32, (rows, weight.outs))
+        self._dense(gain, "norm weight", torch.float32, (weight.outs,))
+        self._dense(weight.data, "packed weight", torch.bfloat16)
+        self._bias(bias, weight.outs)
+        bands = self.lib.akv_linear_mid_bands(rows, weight.n_tiles, weight.k_tiles)
+        sums = arena.take((bands, (rows + 15) // 16 * 16), torch.float32)
+        left = arena.take((rows, weight.outs), torch.bfloat16)
+        self._mid(x, weight, left, rows, weight.outs, False, bias, adds=(stream, gain, sums))
+        return StreamSums(sums, rows=left, gain=gain)
+
+    def scales_rows_in_product(self, rows: int, weight, dtype, sums) -> bool:
+        gated = isinstance(weight, GatedWeight)
+        packed = weight.packed if gated else weight
+        if (not isinstance(packed, PackedWeight) or sums.rows is None or not self.FOLD_NORM_ROWS < rows <= self.FOLD_MID_ROWS
+                or dtype != torch.bfloat16 or sums.sums.shape[0] > self.lib.akv_linear_mid_most_groups(rows)):
+            return False
+        if gated:
+            return self._route("gated", weight.inter, packed.k, rows, weight.stacked is not None, dtype) == "mid"
+        return self._route("linear", packed.outs, packed.k, rows, packed.row_major is not None, dtype) == "mid"
+
+    def linear_rowscaled(self, x, sums, eps, weight, out, bias=None) -> None:
+        """out = (x W^T) with every row divided by sqrt(mean of squares + eps), plus `bias` (a `GatedWeight`: silu of
+        the scaled gate times the scaled up): x [rows, k] are rows that `add_to_stream` left - the residual sum times
+        the norm's weight -, sums [groups, rows rounded up to 16] the partial sums of squares of the residual rows."""
+        gated = isinstance(weight, GatedWeight)
+        packed = weight.packed if gated else weight
+        rows = x.shape[0]
+        outs = weight.inter if gated else packed.outs
+        self._dense(x, "x", torch.bfloat16, (rows, packed.k))
+        self._dense(sums, "sums", torch.float32, (sums.shape[0], (rows + 15) // 16 * 16))
+        self._dense(out, "out", torch.bfloat16, (rows, outs))
+        self._dense(packed.data, "packed weight", torch.bfloat16)
+        if bias is not None and gated:
+            raise KernelError("the gated product takes no bias")
+        self._bias(bias, outs)
+        self._mid(x, packed, out, rows, outs, gated, bias, scaled=(sums, eps))
 
     def norms_rows_in_product(self, rows: int, weight, dtype) -> bool:
         packed = weight.packed if isinstance(weight, GatedWeight) else weight
-        return isinstance(packed, PackedWeight) and self.folds_norm(rows, packed.k, dtype)
+        return isinstance(packed, PackedWeight) and rows <= self.FOLD_NORM_ROWS and self.folds_norm(rows, packed.k, dtype)
 
     def linear_adds(self, x, weight: PackedWeight, stream, sums, bias=None) -> None:
         """stream [rows, outs] (float32) += bfloat16(x W^T (+ bias)), in place; sums [ceil(outs / 16), 16] (float32) receives

@@ -119,7 +119,10 @@ class Part:
         (`Linear.add_to_stream`) and left the rows' sums of squares.  Handed on as a block's `pending` only when
         `ctx.fold_into_stream` is set, which the model's pass sets when whoever reads `pending` next - the next block
         in the run order, or the model's end - has `takes_stream_sums = True`.  A mixer or feed-forward asks
-        `ctx.fold_into_stream` before its last product and otherwise returns a tensor.
+        `ctx.fold_into_stream` before its last product and otherwise returns a tensor.  Beside the flag the context
+        names the weight of the norm that will read the sums where it has one (`ctx.fold_gain`, from
+        `Norm.fold_gain` / a block's `entry_gain`): in steps of many rows the product leaves the new rows times
+        that weight too (`StreamSums.rows`), and the reading product only scales its results by the rows' 1 / rms.
       * `UnnormedRows` (`PendingNorm`, `ScaledNorm` of `parts/norm.py`) - the rows norm(stream [+ delta]) before
         anybody has computed them.  A block hands them to a mixer or feed-forward with `takes_pending_norm = True`,
         which promises to read its input exactly once and through `Linear.forward` or the kernel set's gated product:
@@ -142,6 +145,10 @@ class Part:
     # (position encodings) `apply(x, positions, ctx)` instead of `apply(x, positions)`: the encoding reads further
     # integers per token from the step (`ctx.extra`)
     wants_context = False
+
+    def entry_gain(self):
+        """(blocks) The weight of the norm that reads this block's input - see `Norm.fold_gain` - or None."""
+        return None
 
     def tensors(self, prefix: str) -> list[TensorSpec]:
         return []
@@ -174,14 +181,23 @@ class Norm(Part):
         """norm(stream) not yet computed, for a stream whose rows' sums of squares are in `sums`."""
         return None
 
+    def fold_gain(self):
+        """The float32 vector w of a norm of the form x / rms(x) * w, for a product that leaves rows already
+        multiplied by it (`StreamSums.rows`); None for any other norm."""
+        return None
+
 
 class StreamSums:
     """What a branch hands on instead of its output when its last product has already added that output to the
-    residual sum (`Linear.add_to_stream`): the partial sums of squares of the new residual rows, float32
-    `[ceil(width / 16), 16]`, from which the next norm's scale follows without a pass over the rows."""
+    residual sum (`Linear.add_to_stream`): the partial sums of squares of the new residual rows, float32, from which
+    the next norm's scale follows without a pass over the rows - `[ceil(width / 16), 16]` in steps of up to 16 rows,
+    `[groups, rows rounded up to 16]` in larger ones.  There the product leaves `rows` as well: the new residual
+    rows times `gain`, the weight of the norm that reads them, in the activation dtype - what is still missing
+    from the normed rows is the division by each row's root mean square, which the reading product applies to its
+    results (`KernelSet.scales_rows_in_product`)."""
 
-    def __init__(self, sums: torch.Tensor):
-        self.sums = sums
+    def __init__(self, sums: torch.Tensor, rows: torch.Tensor | None = None, gain: torch.Tensor | None = None):
+        self.sums, self.rows, self.gain = sums, rows, gain
 
 
 class UnnormedRows:
@@ -214,8 +230,14 @@ class KernelSet:
         product norm its rows from the sums left there (`linear_scaled`)."""
         return False
 
-    def adds_to_stream(self, rows: int, weight, dtype) -> bool:
-        """`linear_adds(x, weight, stream, sums, bias=)` exists for this product."""
+    def adds_to_stream(self, rows: int, weight, dtype, gain=None) -> bool:
+        """`add_to_stream(x, weight, stream, arena, bias=, gain=)` exists for this product: stream += x W^T (+ bias),
+        rounded to `dtype` first; returns the `StreamSums`.  `gain`: the weight of the norm that follows, if known."""
+        return False
+
+    def scales_rows_in_product(self, rows: int, weight, dtype, sums: "StreamSums") -> bool:
+        """`linear_rowscaled(sums.rows, sums.sums, eps, weight, out, bias=)` exists for this product: out = the product
+        of `sums.rows`, every row divided by sqrt(its mean of squares + eps), the mean taken from `sums.sums`."""
         return False
 
     def norms_rows_in_product(self, rows: int, weight, dtype) -> bool:

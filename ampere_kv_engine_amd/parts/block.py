@@ -43,17 +43,22 @@ class PreNormBlock(Part):
         """stream [tokens, hidden] float32 (updated in place); pending: the previous branch's output, not
         yet added, or None.  Returns this block's own pending output."""
         fold = bool(self.rt.kernels.folds_norm(stream.shape[0], self.hidden, self.rt.dtype))
-        later = ctx.fold_into_stream        # whoever reads this block's `pending` takes sums
+        later, later_gain = ctx.fold_into_stream, ctx.fold_gain     # whoever reads this block's `pending` takes sums
         normed, unnormed = self._normed(self.mixer_norm, self.mixer, stream, pending, ctx, fold)
         ctx.fold_into_stream = fold         # the mixer's output meets this block's own second norm
+        ctx.fold_gain = self.feed_forward_norm.fold_gain()
         mixed = self.mixer.forward(normed, ctx, cache, writes_cache)
         stream = self._after(unnormed, stream, ctx)
         normed, unnormed = self._normed(self.feed_forward_norm, self.feed_forward, stream, mixed, ctx, fold)
         ctx.fold_into_stream = fold and later
+        ctx.fold_gain = later_gain
         out = self.feed_forward.forward(normed, ctx)
         ctx.fold_into_stream = later
         self._after(unnormed, stream, ctx)
         return out
+
+    def entry_gain(self):
+        return self.mixer_norm.fold_gain()
 
     def _normed(self, norm, reader, stream, delta, ctx, fold=False):
         """norm(stream + delta) for `reader`: computed now - or, in steps of few rows (the context then has a spare

@@ -8,7 +8,7 @@ from __future__ import annotations
 import torch
 
 from ..weights.spec import BIAS, MATRIX, TensorSpec
-from .base import Part, StreamSums, UnnormedRows
+from .base import Part, UnnormedRows
 
 
 class Linear(Part):
@@ -73,11 +73,10 @@ class Linear(Part):
         then the caller computes `forward` and hands its output on as before."""
         kernels = self.rt.kernels
         stream = ctx.stream
-        if stream is None or stream.shape[1] != self.total_out or not kernels.adds_to_stream(x.shape[0], self.weight, self.rt.dtype):
+        if (stream is None or stream.shape[1] != self.total_out
+                or not kernels.adds_to_stream(x.shape[0], self.weight, self.rt.dtype, ctx.fold_gain)):
             return None
-        sums = ctx.arena.take(((self.total_out + 15) // 16, 16), torch.float32)
-        kernels.linear_adds(x, self.weight, stream, sums, bias=self.bias)
-        return StreamSums(sums)
+        return kernels.add_to_stream(x, self.weight, stream, ctx.arena, bias=self.bias, gain=ctx.fold_gain)
 
     def forward(self, x, out: torch.Tensor) -> torch.Tensor:
         """x: [rows, in] in the activation dtype, or rows that are still to be normed (`UnnormedRows`)."""

@@ -42,6 +42,9 @@ class RMSNorm(Norm):
         """`forward_residual` not yet computed: for a consumer whose first product can compute it itself."""
         return PendingNorm(self, stream, delta, stream_out, arena)
 
+    def fold_gain(self):
+        return self.weight
+
     def scaled(self, stream: torch.Tensor, sums: "StreamSums", arena) -> "ScaledNorm":
         """The norm of a residual sum whose rows' sums of squares are already known (`StreamSums`): for a consumer
         whose first product can norm its rows itself from them."""
@@ -68,6 +71,12 @@ class ScaledNorm(UnnormedRows):
 
     def product(self, weight, out: torch.Tensor, bias: torch.Tensor | None = None) -> bool:
         kernels = self.norm.rt.kernels
+        if self.sums.rows is not None:      # a step of many rows: the rows times this norm's weight are at hand
+            if self.sums.gain is not self.norm.weight or not kernels.scales_rows_in_product(self.shape[0], weight, out.dtype, self.sums):
+                return False
+            self._once()
+            kernels.linear_rowscaled(self.sums.rows, self.sums.sums, self.norm.eps, weight, out, bias=bias)
+            return True
         if not kernels.norms_rows_in_product(self.shape[0], weight, out.dtype):
             return False
         self._once()

@@ -45,6 +45,45 @@ def test_cutting_with_the_norm_kernels_of_their_own(case, cutting):
     getattr(cases, "case_" + cutting)(engine, case)
 
 
+@pytest.mark.parametrize("cutting", ["whole", "mixed_with_pages_used_again"])
+def test_steps_of_many_rows_without_norm_kernels_and_with_them(case, cutting):
+    """Steps of 17 to 512 bfloat16 rows run without norm kernels inside the layers too: a branch's last product (the
+    mid-size kernel) adds itself to the residual sum and leaves the new rows times the next norm's weight, and the
+    product that reads them divides its results by the rows' root mean square.  Counted here: in every such step
+    every branch but the last layer's second takes that path; and with the path switched off
+    (`fold_mid`) the layers go through `add_rmsnorm` as before - the same limits against the plain implementation
+    hold either way."""
+    engine = cases.make_engine(case, "bfloat16", "cuda:0")
+    kernels = engine.kernels
+    calls = {"adds": 0, "scaled": 0, "steps": 0}
+    add_to_stream, linear_rowscaled, step = kernels.add_to_stream, kernels.linear_rowscaled, engine.step
+
+    def counting_adds(x, *args, **kwargs):
+        left = add_to_stream(x, *args, **kwargs)
+        calls["adds"] += left.rows is not None
+        return left
+
+    def counting_scaled(*args, **kwargs):
+        calls["scaled"] += 1
+        return linear_rowscaled(*args, **kwargs)
+
+    def counting_step(entries, *args, **kwargs):
+        calls["steps"] += 16 < sum(len(entry.tokens) for entry in entries) <= kernels.FOLD_MID_ROWS
+        return step(entries, *args, **kwargs)
+
+    kernels.add_to_stream, kernels.linear_rowscaled, engine.step = counting_adds, counting_scaled, counting_step
+    engine._recordable = False           # (a replayed step calls no Python: every step runs as it is and is counted)
+    getattr(cases, "case_" + cutting)(engine, case)
+    layers = case["raw"]["num_hidden_layers"]
+    assert calls["steps"] > 0 and calls["adds"] == calls["steps"] * (2 * layers - 1)
+    # (a reader that goes to the BLAS library - the gated product of more than 128 rows - norms its rows with the
+    # norm's kernel from the residual sum instead; every other one takes the rows as they were left)
+    assert 0 < calls["scaled"] <= calls["adds"]
+    plain = cases.make_engine(case, "bfloat16", "cuda:0")
+    plain.kernels.fold_mid = False
+    getattr(cases, "case_" + cutting)(plain, case)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("cutting", ["last_32_one_by_one", "portions_down_to_two_tokens", "mixed_with_pages_used_again"])
 def test_cutting_with_one_page_a_request(case, dtype, cutting):

@@ -60,6 +60,32 @@ def test_branches_that_add_themselves_to_the_residual_sum_give_the_same_bits(cas
         assert (got[name] == want[name]).all(), name
 
 
+def test_branches_of_many_rows_leave_rows_for_a_product_that_scales_its_results(case):
+    """Steps of more than 16 rows: a branch's last product adds itself to the residual sum and leaves the new rows
+    times the next norm's weight with the rows' partial sums of squares; the product that reads them divides its
+    results by the rows' root mean square (what the HIP kernel set's mid-size products do).  With a double that offers
+    the two, the parts take that path in every step of 17 rows and more - prompts whole, and the mixed cutting with
+    pages used again - and every position agrees with the plain implementation as the ordinary path does."""
+    calls = {"adds": 0, "scaled": 0}
+
+    class Counting(TorchKernels):
+        def add_to_stream(self, x, *args, **kwargs):
+            left = super().add_to_stream(x, *args, **kwargs)
+            calls["adds"] += left.rows is not None
+            return left
+
+        def linear_rowscaled(self, *args, **kwargs):
+            calls["scaled"] += 1
+            return super().linear_rowscaled(*args, **kwargs)
+
+    engine = cases.make_engine(case, "bfloat16", "cpu", kernels=Counting(fold_rows=16, fold_many_rows=512))
+    cases.case_whole(engine, case)
+    layers = case["raw"]["num_hidden_layers"]
+    assert calls["adds"] > 0 and calls["adds"] % (2 * layers - 1) == 0      # every branch but the last layer's second
+    assert calls["scaled"] == calls["adds"]                                 # and every one met the product that reads it
+    cases.case_mixed_with_pages_used_again(engine, case)
+
+
 def test_replay_on_a_pool_of_its_own_page_size(case, tmp_path):
     """The replay with the model's own page size (tiny-B: 8 tokens) and a pool given in pages, as `bin/trace_run
     --page-size --num-pages --max-seqs` builds it: the mixed cutting, every position against the plain

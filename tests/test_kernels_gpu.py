@@ -757,6 +757,77 @@ def test_mid_size_gated_product(hip_own, ref, rows, inter, k):
     assert int(counters.abs().sum()) == 0
 
 
+@pytest.mark.parametrize("rows,hidden,k,inter", [(17, 96, 72, 64), (40, 304, 520, 208), (64, 1024, 2048, 512), (100, 4096, 4096, 1024),
+                                                 (128, 520, 1032, 208), (132, 4096, 512, 512), (300, 1000, 2048, 256),
+                                                 (512, 1536, 512, 128), (90, 5120, 256, 64), (200, 8192, 64, 32)])
+def test_mid_size_products_keep_the_residual_sum_and_the_norm(hip_own, ref, rows, hidden, k, inter):
+    """Steps of 17 to 512 rows: `add_to_stream` (stream += bfloat16(x W^T + b); leaves the new rows times the next
+    norm's weight and, per band of its row tiles, the rows' sums of squares) and `linear_rowscaled` (the product of
+    such rows, every result divided by its row's root mean square; plain with a bias, and gated) - each against its
+    formula, the pair against the norm kernel followed by the ordinary products, and twice: the second call finds
+    the counters of the first at zero and gives the same bits."""
+    from ampere_kv_engine_amd.engine.batch import Arena
+    eps = 1e-5
+    w = rand(hidden, k, dtype=torch.bfloat16, seed=301, scale=0.05)
+    x = rand(rows, k, dtype=torch.bfloat16, seed=302)
+    bias = rand(hidden, seed=303, scale=0.5)
+    before = rand(rows, hidden, seed=304, scale=2.0)
+    gain = rand(hidden, seed=305).abs() + 0.5
+    packed = hip_own.prepare_linear(w.cuda())
+    arena = Arena("cuda:0")
+    assert hip_own.adds_to_stream(rows, packed, torch.bfloat16, gain.cuda())
+    assert not hip_own.adds_to_stream(rows, packed, torch.bfloat16, None)      # without the next norm's weight: no
+    assert not hip_own.adds_to_stream(513, packed, torch.bfloat16, gain.cuda())
+    stream = before.clone().cuda()
+    left = hip_own.add_to_stream(x.cuda(), packed, stream, arena, bias=bias.cuda(), gain=gain.cuda())
+    product = (x.float() @ w.float().T + bias).bfloat16().float()
+    torch.testing.assert_close((stream.cpu() - before), product, rtol=1.6e-2, atol=2e-3)   # (a sum's low bits go when it is added to 2.0)
+    now = stream.cpu()
+    assert torch.equal(left.rows.cpu(), (now * gain).bfloat16())                # the rows it left, from the sum it left
+    assert left.gain is not None and left.sums.shape[1] == (rows + 15) // 16 * 16
+    totals = left.sums.sum(0).cpu()
+    torch.testing.assert_close(totals[:rows], (now * now).sum(-1), rtol=1e-5, atol=1e-6)
+    assert float(totals[rows:].abs().sum()) == 0.0
+    again = before.clone().cuda()
+    left_again = hip_own.add_to_stream(x.cuda(), packed, again, arena, bias=bias.cuda(), gain=gain.cuda())
+    assert torch.equal(again, stream) and torch.equal(left_again.rows, left.rows) and torch.equal(left_again.sums, left.sums)
+
+    # the products that read such rows
+    scale = torch.rsqrt(totals[:rows, None] / hidden + eps)
+    rows_left = left.rows.cpu().float()
+    normed = torch.empty(rows, hidden, dtype=torch.bfloat16)
+    ref.add_rmsnorm(now.clone(), None, gain, eps, normed)                      # what a norm kernel would hand on
+    second = rand(inter, hidden, dtype=torch.bfloat16, seed=306, scale=0.05)
+    second_bias = rand(inter, seed=307, scale=0.5)
+    plain = hip_own.prepare_linear(second.cuda())
+    most = hip_own.lib.akv_linear_mid_most_groups(rows)
+    assert hip_own.scales_rows_in_product(rows, plain, torch.bfloat16, left) == (left.sums.shape[0] <= most)
+    if left.sums.shape[0] > most:       # more partial sums a row than the reading product's fetching waves hold:
+        return                          # the parts then norm the rows with the norm's own kernel
+    for with_bias in (False, True):
+        got = torch.full((rows, inter), float("nan"), dtype=torch.bfloat16, device="cuda")
+        hip_own.linear_rowscaled(left.rows, left.sums, eps, plain, got, bias=second_bias.cuda() if with_bias else None)
+        want = rows_left @ second.float().T * scale + (second_bias if with_bias else 0.0)
+        torch.testing.assert_close(got.cpu().float(), want.bfloat16().float(), **tol(torch.bfloat16))
+        # against the ordinary pair (rows normed, rounded, weighted, rounded; then the product): every operand is
+        # rounded elsewhere, so single outputs differ by what bfloat16 operands allow - over all of them, little
+        ordinary = (normed.float() @ second.float().T + (second_bias if with_bias else 0.0)).bfloat16().float()
+        apart = got.cpu().float() - ordinary
+        assert float(apart.pow(2).mean().sqrt()) <= 2.0 ** -7 * float(ordinary.pow(2).mean().sqrt())
+        assert float(apart.abs().max()) <= 2.0 ** -4 * float(ordinary.pow(2).mean().sqrt())
+    gate, up = (rand(inter, hidden, dtype=torch.bfloat16, seed=308 + i, scale=0.05) for i in range(2))
+    gated = hip_own.prepare_gated_linear(gate.cuda(), up.cuda())
+    assert hip_own.scales_rows_in_product(rows, gated, torch.bfloat16, left)
+    got = torch.full((rows, inter), float("nan"), dtype=torch.bfloat16, device="cuda")
+    hip_own.linear_rowscaled(left.rows, left.sums, eps, gated, got)
+    g, u = rows_left @ gate.float().T * scale, rows_left @ up.float().T * scale
+    torch.testing.assert_close(got.cpu().float(), (g * torch.sigmoid(g) * u).bfloat16().float(), **tol(torch.bfloat16))
+    first = got.clone()
+    hip_own.linear_rowscaled(left.rows, left.sums, eps, gated, got)
+    assert torch.equal(first, got)
+    assert int(hip_own._mid_counters.abs().sum()) == 0 if hip_own._mid_counters is not None else True
+
+
 def test_linear_keeps_other_weights_row_major(hip):
     assert isinstance(hip.prepare_linear(torch.zeros(4, 12, dtype=torch.bfloat16, device="cuda")), torch.Tensor)   # k % 8
     assert isinstance(hip.prepare_linear(torch.zeros(4, 16, device="cuda")), torch.Tensor)                         # float32

@@ -23,10 +23,14 @@ def _round(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
 class TorchKernels(KernelSet):
     name = "torch-double"
 
-    def __init__(self, fold_rows: int = 0):
+    def __init__(self, fold_rows: int = 0, fold_many_rows: int = 0):
         """`fold_rows`: steps of up to this many rows let a branch's last product add itself to the residual sum and
-        the next product norm its rows itself, as the HIP kernel set does in decode steps (0: never)."""
+        the next product norm its rows from the sums of squares left there, as the HIP kernel set does in decode
+        steps (0: never).  `fold_many_rows`: steps of more rows, up to this many, do the same the way the HIP
+        kernel set's mid-size products do: the adding product leaves the new rows times the next norm's weight, and
+        the reading product divides its results by the rows' root mean square."""
         self.fold_rows = fold_rows
+        self.fold_many_rows = fold_many_rows
 
     def check_attention_sizes(self, q_heads, kv_heads, head_dim, page_size):
         if q_heads % kv_heads:
@@ -85,10 +89,46 @@ class TorchKernels(KernelSet):
 
     # ---- the residual sum and the norm inside the products (decode steps) -------------------------------
     def folds_norm(self, rows, hidden, dtype):
-        return 0 < rows <= self.fold_rows and dtype == torch.bfloat16
+        return 0 < rows <= max(self.fold_rows, self.fold_many_rows) and dtype == torch.bfloat16
 
-    def adds_to_stream(self, rows, weight, dtype):
-        return isinstance(weight, torch.Tensor) and self.folds_norm(rows, weight.shape[0], dtype)
+    def adds_to_stream(self, rows, weight, dtype, gain=None):
+        if not isinstance(weight, torch.Tensor) or dtype != torch.bfloat16:
+            return False
+        if 0 < rows <= self.fold_rows:
+            return True
+        return gain is not None and rows <= self.fold_many_rows
+
+    def add_to_stream(self, x, weight, stream, arena, bias=None, gain=None):
+        from ampere_kv_engine_amd.parts.base import StreamSums
+        rows, outs = x.shape[0], weight.shape[0]
+        if rows <= self.fold_rows:
+            sums = arena.take(((outs + 15) // 16, 16), torch.float32)
+            self.linear_adds(x, weight, stream, sums, bias=bias)
+            return StreamSums(sums)
+        # many rows: the new rows times the next norm's weight, and three groups of partial sums per row
+        y = torch.empty(rows, outs, dtype=x.dtype)
+        self.linear(x, weight, y, bias)
+        stream += y.float()
+        sums = arena.take((3, (rows + 15) // 16 * 16), torch.float32)
+        sums.zero_()
+        for group, columns in enumerate(torch.arange(outs).chunk(3)):
+            sums[group, :rows] = (stream[:, columns] ** 2).sum(-1)
+        left = arena.take((rows, outs), x.dtype)
+        left.copy_((stream * gain).to(x.dtype))
+        return StreamSums(sums, rows=left, gain=gain)
+
+    def scales_rows_in_product(self, rows, weight, dtype, sums):
+        return sums.rows is not None and self.fold_rows < rows <= self.fold_many_rows and dtype == torch.bfloat16
+
+    def linear_rowscaled(self, x, sums, eps, weight, out, bias=None):
+        rows, k = x.shape
+        scale = torch.rsqrt(sums.sum(0)[:rows, None] / k + eps)
+        if isinstance(weight, tuple):
+            g, u = x.float() @ weight[0].float().T * scale, x.float() @ weight[1].float().T * scale
+            out.copy_((g * torch.sigmoid(g) * u).to(out.dtype))
+        else:
+            y = x.float() @ weight.float().T * scale
+            out.copy_((y if bias is None else y + bias.float()).to(out.dtype))
 
     def norms_rows_in_product(self, rows, weight, dtype):
         matrix = weight[0] if isinstance(weight, tuple) else weight
