@@ -1201,12 +1201,18 @@ __global__ __launch_bounds__(64 * kMergeWaves) void attention_merge_kernel(const
   };
   float ahead[8][PER] = {};
   if (mine > 0) fetch8(0, 0, min(64, mine), ahead);
-  // every wave finds the maximum over all segments (a lane per segment)
-  float top = -INFINITY;
+  // every wave finds the maximum over all segments (a lane per segment).  A segment's maximum and sum are asked for
+  // together and whatever the lane (a lane beyond the last segment reads the last one's): the first 64 segments'
+  // are handed to the lanes that weigh them by a shuffle instead of a second trip to memory.
+  float top = -INFINITY, first_m = -INFINITY, first_l = 0.f;
   bool poisoned = false;
   for (int z0 = 0; z0 < splits; z0 += 64) {
     const int z = z0 + lane;
-    const float mz = z < splits ? src[z * split_stride + D] : -INFINITY;
+    const long at = static_cast<long>(max(0, min(z, splits - 1))) * split_stride;
+    float mz = src[at + D];
+    const float lz = src[at + D + 1];
+    if (z >= splits) mz = -INFINITY;
+    if (z0 == 0) first_m = mz, first_l = lz;
     poisoned = poisoned || mz != mz;
     top = fmaxf(top, mz);
   }
@@ -1218,11 +1224,15 @@ __global__ __launch_bounds__(64 * kMergeWaves) void attention_merge_kernel(const
   for (int i0 = 0; i0 < mine; i0 += 64) {
     const int i = i0 + lane;
     float w = 0.f;
+    const long z = wave + static_cast<long>(kMergeWaves) * i;
+    float mz = __shfl(first_m, static_cast<int>(z & 63), 64), lz = __shfl(first_l, static_cast<int>(z & 63), 64);
+    if (i < mine && z >= 64) {
+      mz = src[z * split_stride + D];
+      lz = src[z * split_stride + D + 1];
+    }
     if (i < mine) {
-      const long z = wave + static_cast<long>(kMergeWaves) * i;
-      const float mz = src[z * split_stride + D];
       w = (mz == -INFINITY || mz != mz) ? 0.f : __builtin_amdgcn_exp2f(mz - top);
-      denom += w * src[z * split_stride + D + 1];
+      denom += w * lz;
     }
     const int count = min(64, mine - i0);
     for (int ii0 = 0; ii0 < count; ii0 += 8) {  // ascending segments

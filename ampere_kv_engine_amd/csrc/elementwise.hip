@@ -78,26 +78,30 @@ __global__ __launch_bounds__(256) void add_rmsnorm_kernel(float* __restrict__ st
   T* o = out + base;
   float acc = 0.f;
   if ((hidden & 3) == 0 && hidden <= 256 * 4 * GROUPS) {
-    float4 kept[GROUPS];
+    // Every group's loads go out before anything waits, whatever the row's width (a group beyond the row reads its
+    // last four values and counts for nothing): behind a test per group the compiler waits for each group's loads,
+    // and for its store, before it asks for the next - eight trips to memory a row instead of one.
+    float4 kept[GROUPS], added[GROUPS], gain[GROUPS];
 #pragma unroll
-    for (int j = 0; j < GROUPS; ++j) {
-      const int i = (j * 256 + threadIdx.x) * 4;
-      if (i < hidden) {
-        float4 v = load4<float>(s + i);
-        if (delta != nullptr) {
-          const float4 d = load4<T>(delta + base + i);
-          v = make_float4(v.x + d.x, v.y + d.y, v.z + d.z, v.w + d.w);
-          store4<float>(s + i, v);
-        }
-        kept[j] = v;
-        acc += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-      }
+    for (int j = 0; j < GROUPS; ++j) kept[j] = load4<float>(s + min((j * 256 + static_cast<int>(threadIdx.x)) * 4, hidden - 4));
+#pragma unroll
+    for (int j = 0; j < GROUPS; ++j) gain[j] = load4<float>(weight + min((j * 256 + static_cast<int>(threadIdx.x)) * 4, hidden - 4));
+    if (delta != nullptr) {   // (last: what is widened to float32 as it arrives is waited for at once)
+#pragma unroll
+      for (int j = 0; j < GROUPS; ++j) added[j] = load4<T>(delta + base + min((j * 256 + static_cast<int>(threadIdx.x)) * 4, hidden - 4));
     }
-    float4 gain[GROUPS];  // asked for before the sum, so that they arrive while it is formed
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < GROUPS; ++j) {
       const int i = (j * 256 + threadIdx.x) * 4;
-      if (i < hidden) gain[j] = load4<float>(weight + i);
+      float4 v = kept[j];
+      if (delta != nullptr) {
+        const float4 d = added[j];
+        v = make_float4(v.x + d.x, v.y + d.y, v.z + d.z, v.w + d.w);
+        if (i < hidden) store4<float>(s + i, v);
+      }
+      kept[j] = v;
+      if (i < hidden) acc += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
     }
     const float scale = rsqrtf(block_sum(acc, scratch) / static_cast<float>(hidden) + eps);
 #pragma unroll
@@ -297,6 +301,26 @@ template <> __device__ __forceinline__ void load8<bf16_t>(const bf16_t* p, float
     v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
   }
 }
+// The same in two steps - the registers as they come from memory, and their eight values -, for code that wants all
+// its loads on their way before the first of them is looked at.
+template <typename T> struct Raw8;
+template <> struct Raw8<float> { float4 a, b; };
+template <> struct Raw8<bf16_t> { uint4 u; };
+__device__ __forceinline__ Raw8<float> fetch8(const float* p) {
+  return Raw8<float>{*reinterpret_cast<const float4*>(p), *reinterpret_cast<const float4*>(p + 4)};
+}
+__device__ __forceinline__ Raw8<bf16_t> fetch8(const bf16_t* p) { return Raw8<bf16_t>{*reinterpret_cast<const uint4*>(p)}; }
+__device__ __forceinline__ void unpack8(const Raw8<float>& r, float (&v)[8]) {
+  v[0] = r.a.x; v[1] = r.a.y; v[2] = r.a.z; v[3] = r.a.w; v[4] = r.b.x; v[5] = r.b.y; v[6] = r.b.z; v[7] = r.b.w;
+}
+__device__ __forceinline__ void unpack8(const Raw8<bf16_t>& r, float (&v)[8]) {
+  const uint32_t w[4] = {r.u.x, r.u.y, r.u.z, r.u.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = __uint_as_float(w[i] << 16);
+    v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
 template <typename T> __device__ __forceinline__ void store8(T* p, const float (&v)[8]);
 template <> __device__ __forceinline__ void store8<float>(float* p, const float (&v)[8]) {
   *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
@@ -329,24 +353,28 @@ __device__ __forceinline__ void write_values_by_eights(const T* __restrict__ qkv
   long slot[8];
   bool together = (page_size & 7) == 0 && sizeof(T) == 2;
 #pragma unroll
+  for (int t = 0; t < 8; ++t) slot[t] = slot_map[min(n0 + t, tokens - 1)];   // (all eight asked for at once)
+#pragma unroll
   for (int t = 0; t < 8; ++t) {
-    slot[t] = n0 + t < tokens ? slot_map[n0 + t] : -1;
-    if (slot[t] < 0 || slot[t] >= num_slots) slot[t] = -1;  // host checks the map; never write outside the pool
+    if (n0 + t >= tokens || slot[t] < 0 || slot[t] >= num_slots) slot[t] = -1;  // host checks the map; never write outside the pool
     together = together && slot[t] >= 0 && slot[t] == slot[0] + t;
   }
   together = together && (slot[0] & 7) == 0;
-  const T* src = qkv + n0 * row + static_cast<long>(q_heads + kv_heads + h) * dim;
+  const T* src = qkv + static_cast<long>(q_heads + kv_heads + h) * dim;
   for (int d = 2 * lane; d < dim; d += 2 * kWave) {
+    // All eight tokens' loads go out together, whatever their slots (a token beyond the last reads the last one's
+    // row; what has no slot is set to zero afterwards): behind a test each, they are waited for one by one - eight
+    // trips to memory instead of one.
     T pair[8][2];
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
-      if (slot[t] >= 0) {
-        pair[t][0] = src[t * row + d];
-        pair[t][1] = src[t * row + d + 1];
-      } else {
-        pair[t][0] = pair[t][1] = T{};
-      }
+      const T* from = src + min(n0 + t, tokens - 1) * row + d;
+      pair[t][0] = from[0];
+      pair[t][1] = from[1];
     }
+#pragma unroll
+    for (int t = 0; t < 8; ++t)
+      if (slot[t] < 0) pair[t][0] = pair[t][1] = T{};
     if constexpr (sizeof(T) == 2) {
       if (together) {
         const long page = slot[0] / page_size, offset = slot[0] % page_size;
@@ -377,19 +405,23 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
     const T* __restrict__ qkv, const float* __restrict__ q_weight, const float* __restrict__ k_weight, float eps,
     const float* __restrict__ table, int table_positions, const int* __restrict__ positions,
     const int* __restrict__ slot_map, T* __restrict__ k_pages, T* __restrict__ v_pages, T* __restrict__ q_out,
-    long tokens, int q_heads, int kv_heads, int dim, int page_size, long num_slots, unsigned value_blocks_from) {
+    long tokens, int q_heads, int kv_heads, int dim, int page_size, long num_slots, unsigned value_blocks) {
   const int waves = blockDim.x / kWave, wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
-  if (blockIdx.x >= value_blocks_from) {  // the blocks that write values, eight tokens at a time (see below)
+  // value_blocks: 0xffffffff - values are written like keys, by the lanes of their heads; else the first so many
+  // blocks write them, eight tokens at a time (see above; they take longest, so they start first)
+  const bool values_apart = value_blocks != 0xffffffffu;
+  if (values_apart && blockIdx.x < value_blocks) {
     write_values_by_eights<T>(qkv, slot_map, v_pages, tokens, q_heads, kv_heads, dim, page_size, num_slots,
-                              static_cast<long>(blockIdx.x - value_blocks_from) * waves + wave, lane);
+                              static_cast<long>(blockIdx.x) * waves + wave, lane);
     return;
   }
+  const unsigned block = values_apart ? blockIdx.x - value_blocks : blockIdx.x;
   const int lanes_per_head = dim / 16, heads_per_wave = kWave / lanes_per_head;
   // with blocks of their own for the values, the heads of this part are the query and key heads alone
   const int row_heads = q_heads + 2 * kv_heads;
-  const int heads = value_blocks_from == 0xffffffffu ? row_heads : q_heads + kv_heads;
+  const int heads = values_apart ? q_heads + kv_heads : row_heads;
   const int groups = (heads + heads_per_wave - 1) / heads_per_wave;
-  const long item = static_cast<long>(blockIdx.x) * waves + wave;
+  const long item = static_cast<long>(block) * waves + wave;
   if (item >= tokens * groups) return;
   const long n = item / groups;
   const int sub = lane / lanes_per_head, part = lane % lanes_per_head;
@@ -400,48 +432,56 @@ __global__ __launch_bounds__(256) void qk_norm_rope_write_kernel(
   const float nan = __uint_as_float(0x7fc00000u);
   const bool normed = q_weight != nullptr;
 
-  long slot = -1;
-  if (slot_map != nullptr) {
-    slot = slot_map[n];
-    if (slot < 0 || slot >= num_slots) slot = -1;  // host checks the map; never write outside the pool
+  // Every load goes out before anything waits, and none stands behind a test of what a lane is: a lane without a
+  // head reads the row's last head, a position without angles the table's first row, and what must not count is
+  // dropped afterwards.  (Behind tests the compiler waits for each group of loads where the paths meet again: a
+  // trip to memory for the row, one for the position, one for the angles, one for the weights.)  The tests left are
+  // those of the launch - no table, no norm, no cache -, the same for every lane.
+  const int h_read = min(h, row_heads - 1);
+  const T* src = qkv + (n * row_heads + h_read) * dim;
+  const Raw8<T> raw_lo = fetch8(src + j0), raw_hi = fetch8(src + half + j0);
+  long slot = (slot_map != nullptr ? slot_map : positions)[n];   // (no cache: any integer of the token, dropped below)
+  const int pos = positions[n];
+  Raw8<float> raw_w_lo{}, raw_w_hi{};
+  if (normed) {
+    const float* w = is_q ? q_weight : k_weight;
+    raw_w_lo = fetch8(w + j0);
+    raw_w_hi = fetch8(w + half + j0);
   }
+  float4 angles[4] = {};
+  const bool known = pos >= 0 && pos < table_positions;
+  if (table != nullptr) {
+    const float* at = table + (static_cast<long>(known ? pos : 0) * half + j0) * 2;  // (cos, sin) pairs of 8 consecutive j
+#pragma unroll
+    for (int q = 0; q < 4; ++q) angles[q] = *reinterpret_cast<const float4*>(at + 4 * q);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  if (slot_map == nullptr || slot < 0 || slot >= num_slots) slot = -1;  // host checks the map; never write outside the pool
   const long page = slot >= 0 ? slot / page_size : 0, offset = slot >= 0 ? slot % page_size : 0;
   const bool works = active && (is_q || slot >= 0);  // keys and values of a token without a slot go nowhere
-
-  // every load goes out before anything waits: the row's pieces, the pair's cos/sin, the norm weights
+  const bool turns = works && !is_v;  // a query or key head: normed and rotated
   float lo[8], hi[8], cs[8], sn[8], w_lo[8], w_hi[8];
+  unpack8(raw_lo, lo);
+  unpack8(raw_hi, hi);
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    lo[e] = hi[e] = sn[e] = 0.f;
+    if (!works) lo[e] = hi[e] = 0.f;
+    sn[e] = 0.f;
     cs[e] = w_lo[e] = w_hi[e] = 1.f;
   }
-  const bool turns = works && !is_v;  // a query or key head: normed and rotated
-  if (works) {
-    const T* src = qkv + (n * row_heads + h) * dim;
-    load8<T>(src + j0, lo);
-    load8<T>(src + half + j0, hi);
-  }
-  if (turns && table != nullptr) {
-    const int pos = positions[n];
-    if (pos < 0 || pos >= table_positions) {
+  if (table != nullptr) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) cs[e] = sn[e] = nan;
-    } else {
-      const float* at = table + (static_cast<long>(pos) * half + j0) * 2;  // (cos, sin) pairs of 8 consecutive j
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const float4 pair = *reinterpret_cast<const float4*>(at + 4 * q);
-        cs[2 * q] = pair.x;
-        sn[2 * q] = pair.y;
-        cs[2 * q + 1] = pair.z;
-        sn[2 * q + 1] = pair.w;
-      }
+    for (int q = 0; q < 4; ++q) {
+      cs[2 * q] = known ? angles[q].x : nan;
+      sn[2 * q] = known ? angles[q].y : nan;
+      cs[2 * q + 1] = known ? angles[q].z : nan;
+      sn[2 * q + 1] = known ? angles[q].w : nan;
     }
   }
-  if (turns && normed) {
-    const float* w = is_q ? q_weight : k_weight;
-    load8<float>(w + j0, w_lo);
-    load8<float>(w + half + j0, w_hi);
+  if (normed) {
+    unpack8(raw_w_lo, w_lo);
+    unpack8(raw_w_hi, w_hi);
   }
   if (works && is_v) {  // value: copied as it is, into the [dim, page_size] layout
     T* dst = v_pages + (page * kv_heads + (h - q_heads - kv_heads)) * dim * page_size + offset;
@@ -649,7 +689,7 @@ int akv_qk_norm_rope_write(const void* qkv, const float* q_weight, const float* 
                qk_norm_rope_write_kernel<T><<<first + more, 256, 0, stream>>>(
                    static_cast<const T*>(qkv), q_weight, k_weight, eps, table, table_positions, positions, slot_map,
                    static_cast<T*>(k_pages), static_cast<T*>(v_pages), static_cast<T*>(q_out), tokens, q_heads,
-                   kv_heads, dim, page_size, num_pages * page_size, values_apart ? first : 0xffffffffu));
+                   kv_heads, dim, page_size, num_pages * page_size, values_apart ? more : 0xffffffffu));
   return AKV_LAUNCH_STATUS();
 }
 
