@@ -62,4 +62,10 @@ int akv_linear_scaled(const float* stream_in, const float* sums, int sum_tiles, 
                       const void* wp, void* y, float* pieces, unsigned int* arrivals, int exchange_tiles, int rows,
                       int outs, int k, int n_tiles, int k_tiles, int gated, int row_tiles, const float* bias,
                       hipStream_t stream);
+int akv_linear_adds_rows(const void* x, const void* wp, float* stream_out, float* sums_out, float* pieces,
+                         unsigned int* arrivals, int exchange_tiles, int rows, int outs, int k, int n_tiles, int k_tiles,
+                         const float* bias, void* rows_out, const float* gain, hipStream_t stream);
+int akv_linear_rowscaled(const void* x, const float* sums, int sum_tiles, float eps, const void* wp, void* y,
+                         float* pieces, unsigned int* arrivals, int exchange_tiles, int rows, int outs, int k,
+                         int n_tiles, int k_tiles, int gated, int row_tiles, const float* bias, hipStream_t stream);
 }

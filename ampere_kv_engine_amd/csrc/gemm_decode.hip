@@ -10,6 +10,13 @@
 //           rsqrt(mean + eps); then every thread norms pieces of 8 values as the norm kernel does - scaled, rounded,
 //           times the weight, rounded - and puts them where the matrix cores' operand wants them.
 //
+//   ROWSCALED  the same reader another way round: the adding product has also left the new rows times the norm's
+//           weight as bfloat16 (`rows_out`), and since the division by a row's root mean square commutes with the
+//           product, this one multiplies those rows as they are and scales its float32 sums by rsqrt(mean + eps) of
+//           their row - the blocks read 2 bytes a value instead of 4 and the weight, and norm nothing (q/k/v at 8
+//           rows 19.4 -> 17.5 us, gate and up 40.0 -> 36.7 on cold weights).  Against SCALED an operand is rounded
+//           once instead of twice and the scale stays in float32: the same up to roundings, not the same bits.
+//
 // Otherwise this is the skinny kernel of gemm_mfma.hip for one tile of rows: a wave owns RT row tiles of the packed
 // weight and a part of k, streams its tiles once (two groups of registers in turn, loads marked as read-once), the
 // parts of k are summed through LDS in a fixed order.  GATED as there (a pair of gate and up tiles, RT = 2).
@@ -30,14 +37,16 @@ using namespace akv;
 namespace {
 
 struct DecodeArgs {
-  const bf16_t* x;          // not SCALED: [rows, k]
+  const bf16_t* x;          // not SCALED: [rows, k] (ROWSCALED: the residual rows times the norm's weight)
   const float* stream;      // SCALED: [rows, k], the residual sum
-  const float* sums;        // SCALED: [sum_tiles][16] partial sums of squares of the residual rows
+  const float* sums;        // SCALED, ROWSCALED: [sum_tiles][16] partial sums of squares of the residual rows
   const float* gain;        // SCALED: [k], the norm's weight
   const uintx4* wp;         // the packed weight
   bf16_t* y;                // not ADDS: [rows, outs]
   float* stream_out;        // ADDS: [rows, outs], updated in place
   float* sums_out;          // ADDS: [n_tiles][16]
+  bf16_t* rows_out;         // ADDS: [rows, outs] or null: the new residual sum times `gain_out`, for a ROWSCALED reader
+  const float* gain_out;    // ADDS: [outs], the weight of the norm that follows (with rows_out)
   const float* bias;        // [outs] or null: added to the sums over k before anything else is done with them (never GATED)
   float eps;
   int sum_tiles, rows, outs, k, k_tiles, n_tiles, k_split, red_floats;
@@ -47,9 +56,10 @@ struct DecodeArgs {
 
 constexpr int kGroup = 4;   // k-tiles per group of loads; two groups are in flight
 
-template <int RT, bool GATED, bool SCALED, bool ADDS>
+template <int RT, bool GATED, bool SCALED, bool ADDS, bool ROWSCALED = false>
 __global__ __launch_bounds__(768) void linear_decode_kernel(const DecodeArgs a) {
   static_assert(!(GATED && ADDS) && (!GATED || RT == 2), "the gated pair is a wave's two row tiles");
+  static_assert(!(ROWSCALED && (SCALED || ADDS)), "a product scales its sums, or norms its rows, or adds itself");
   constexpr int U = kGroup;
   extern __shared__ float red[];   // [wave][RT][4][64] for the sum over the parts of k - SCALED: before that, the rows' scales and the normed rows
   const int lane = threadIdx.x & 63, waves = blockDim.x >> 6;
@@ -87,7 +97,22 @@ __global__ __launch_bounds__(768) void linear_decode_kernel(const DecodeArgs a) 
   uintx4* rows_lds = reinterpret_cast<uintx4*>(red + (SCALED ? kScaleFloats : 0));
   fetch_weights(kt0, w0);       // two groups on their way while the rows are normed
   fetch_weights(kt0 + U, w1);
-  if constexpr (SCALED) {
+  // ADDS: what the sums will be added to, and the next norm's weight there, are asked for now - in the epilogue they
+  // would cost the block's last wave a trip to memory.  (Every output has one owner: nobody changes them meanwhile.)
+  float4 held[ADDS ? RT : 1], gain_held[ADDS ? RT : 1];
+  const bool quads = (a.outs & 3) == 0;
+  if constexpr (ADDS) {
+    if (quads) {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        const int feature = max(0, min((min(row_tile + rt, a.n_tiles - 1)) * 16 + g * 4, a.outs - 4));
+        held[rt] = *reinterpret_cast<const float4*>(a.stream_out + static_cast<size_t>(min(r, a.rows - 1)) * a.outs + feature);
+        gain_held[rt] = *reinterpret_cast<const float4*>((a.gain_out != nullptr ? a.gain_out : a.stream_out) + feature);
+      }
+    }
+  }
+  float my_scale = 1.f;         // ROWSCALED: 1 / rms of this lane's row
+  if constexpr (SCALED || ROWSCALED) {
     // (Asking for what the norm needs BEFORE the first weights - a wave's loads come back in the order in which they
     // were asked for - was measured and is no gain: 15.0 -> 16.0 us at one row, 23.1 -> 22.8 at eight, q/k/v.)
     // The rows' sums of squares: sum_tiles x 16 partial sums.  The waves share the tiles; a lane adds up quads of
@@ -120,6 +145,10 @@ __global__ __launch_bounds__(768) void linear_decode_kernel(const DecodeArgs a) 
       scales[threadIdx.x] = static_cast<int>(threadIdx.x) < a.rows ? rsqrtf(total / static_cast<float>(a.k) + a.eps) : 0.f;
     }
     __syncthreads();
+    if constexpr (ROWSCALED) my_scale = scales[r];
+  }
+  if constexpr (SCALED) {
+    float* scales = red + 12 * 16;
     auto normed = [&](float4 lo, float4 hi, float4 g0, float4 g1, float scale) {
       const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
       const float gains[8] = {g0.x, g0.y, g0.z, g0.w, g1.x, g1.y, g1.z, g1.w};
@@ -210,7 +239,7 @@ __global__ __launch_bounds__(768) void linear_decode_kernel(const DecodeArgs a) 
     // piece 1 (the same bits whichever it is), sets the counter back and goes on to the store.  Nobody waits for
     // anybody.
     constexpr int kSet = RT * 4 * 64;
-    if constexpr (SCALED) __syncthreads();   // the rows have been read: their memory takes the sums
+    if constexpr (SCALED || ROWSCALED) __syncthreads();   // the rows (the scales) have been read: their memory takes the sums
     const int row_first = wave_row * a.k_split;
     const int lo = max(first_unit, row_first), hi = min(first_unit + waves, row_first + a.k_split);
     float* mine = red + static_cast<size_t>(wave) * kSet;
@@ -253,6 +282,12 @@ __global__ __launch_bounds__(768) void linear_decode_kernel(const DecodeArgs a) 
     }
   }
   if (row_tile >= a.n_tiles) return;
+  if constexpr (ROWSCALED) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[rt][i] *= my_scale;
+  }
   if constexpr (!GATED) {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) acc[rt] = plus_bias(acc[rt], a.bias, (row_tile + rt) * 16 + g * 4, a.outs);
@@ -266,14 +301,18 @@ __global__ __launch_bounds__(768) void linear_decode_kernel(const DecodeArgs a) 
       float squares = 0.f;
       if (r < a.rows) {
         float* at = a.stream_out + static_cast<size_t>(r) * a.outs + feature;
-        if (feature + 3 < a.outs && (a.outs & 3) == 0) {
-          float4 s = *reinterpret_cast<float4*>(at);
+        if (quads && feature < a.outs) {      // (then feature + 3 < outs: the features of a quad exist together)
+          float4 s = held[rt];
           s.x += rounded<bf16_t>(acc[rt][0]);
           s.y += rounded<bf16_t>(acc[rt][1]);
           s.z += rounded<bf16_t>(acc[rt][2]);
           s.w += rounded<bf16_t>(acc[rt][3]);
           *reinterpret_cast<float4*>(at) = s;
           squares = s.x * s.x + s.y * s.y + s.z * s.z + s.w * s.w;
+          if (a.rows_out != nullptr) {
+            const float4 w = gain_held[rt];
+            store4<bf16_t>(a.rows_out + static_cast<size_t>(r) * a.outs + feature, floatx4{s.x * w.x, s.y * w.y, s.z * w.z, s.w * w.w});
+          }
         } else {
 #pragma unroll
           for (int i = 0; i < 4; ++i)
@@ -281,6 +320,7 @@ __global__ __launch_bounds__(768) void linear_decode_kernel(const DecodeArgs a) 
               const float s = at[i] + rounded<bf16_t>(acc[rt][i]);
               at[i] = s;
               squares += s * s;
+              if (a.rows_out != nullptr) a.rows_out[static_cast<size_t>(r) * a.outs + feature + i] = from_float<bf16_t>(s * a.gain_out[feature + i]);
             }
         }
       }
@@ -351,13 +391,14 @@ DecodePlan plan_decode(int rt, int n_tiles, int k_tiles, int k, int normed_rows,
   return plan;
 }
 
-template <int RT, bool GATED, bool SCALED, bool ADDS>
+template <int RT, bool GATED, bool SCALED, bool ADDS, bool ROWSCALED = false>
 int launch_decode(DecodeArgs a, hipStream_t stream) {
   const DecodePlan plan = plan_decode(RT, a.n_tiles, a.k_tiles, a.k, SCALED ? a.rows : 0, a.pieces != nullptr);
   const int k_split = plan.k_split, waves = plan.waves, blocks = plan.blocks;
   a.k_split = k_split;
   a.red_floats = k_split > 1 ? waves * RT * 4 * 64 : 0;
-  const size_t lds = max(static_cast<size_t>(a.red_floats) * 4, SCALED ? (12 * 16 + 16) * 4 + static_cast<size_t>(a.rows) * a.k * 2 : 0);
+  const size_t lds = max(static_cast<size_t>(a.red_floats) * 4,
+                         SCALED ? (12 * 16 + 16) * 4 + static_cast<size_t>(a.rows) * a.k * 2 : (ROWSCALED ? (12 * 16 + 16) * 4 : 0));
   const size_t kMaxLds = device_facts().lds_bytes;
   if (lds > kMaxLds) return -2;
   if (lds > 64 * 1024) {   // more than a block may have without asking: asked once per kernel and device
@@ -367,13 +408,13 @@ int launch_decode(DecodeArgs a, hipStream_t stream) {
     if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return -2;
     std::lock_guard<std::mutex> lock(guard);
     if (!asked[device]) {
-      const hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_decode_kernel<RT, GATED, SCALED, ADDS>),
+      const hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void*>(&linear_decode_kernel<RT, GATED, SCALED, ADDS, ROWSCALED>),
                                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kMaxLds));
       if (status != hipSuccess) return static_cast<int>(status);
       asked[device] = true;
     }
   }
-  linear_decode_kernel<RT, GATED, SCALED, ADDS><<<blocks, waves * 64, lds, stream>>>(a);
+  linear_decode_kernel<RT, GATED, SCALED, ADDS, ROWSCALED><<<blocks, waves * 64, lds, stream>>>(a);
   return AKV_LAUNCH_STATUS();
 }
 
@@ -394,20 +435,74 @@ extern "C" int akv_linear_decode_plan(int rt, int n_tiles, int k_tiles, int k, i
   return 0;
 }
 
-extern "C" int akv_linear_adds(const void* x, const void* wp, float* stream_out, float* sums_out, float* pieces,
-                               unsigned int* arrivals, int exchange_tiles, int rows, int outs, int k, int n_tiles,
-                               int k_tiles, const float* bias, hipStream_t stream) {
+namespace {
+int linear_adds(const void* x, const void* wp, float* stream_out, float* sums_out, float* pieces,
+                unsigned int* arrivals, int exchange_tiles, int rows, int outs, int k, int n_tiles,
+                int k_tiles, const float* bias, void* rows_out, const float* gain, hipStream_t stream) {
   if (rows <= 0 || outs <= 0) return 0;
   if (rows > 16 || (k & 7) != 0 || n_tiles * 16 < outs || (n_tiles - 1) * 16 >= outs || k_tiles * 32 < k) return -2;
+  if ((rows_out == nullptr) != (gain == nullptr)) return -2;
   DecodeArgs a{};
   a.x = static_cast<const bf16_t*>(x);
   a.wp = static_cast<const uintx4*>(wp);
   a.stream_out = stream_out;
   a.sums_out = sums_out;
+  a.rows_out = static_cast<bf16_t*>(rows_out);
+  a.gain_out = gain;
   a.bias = bias;
   if (pieces != nullptr && arrivals != nullptr && exchange_tiles >= n_tiles + 1) a.pieces = pieces, a.arrivals = arrivals;
   a.rows = rows, a.outs = outs, a.k = k, a.k_tiles = k_tiles, a.n_tiles = n_tiles;
   return launch_decode<1, false, false, true>(a, stream);
+}
+}  // namespace
+
+extern "C" int akv_linear_adds(const void* x, const void* wp, float* stream_out, float* sums_out, float* pieces,
+                               unsigned int* arrivals, int exchange_tiles, int rows, int outs, int k, int n_tiles,
+                               int k_tiles, const float* bias, hipStream_t stream) {
+  return linear_adds(x, wp, stream_out, sums_out, pieces, arrivals, exchange_tiles, rows, outs, k, n_tiles, k_tiles, bias,
+                     nullptr, nullptr, stream);
+}
+
+// The same, and rows_out [rows, outs] bfloat16 receives the new residual sum times `gain` [outs] (the weight of the
+// norm that follows): what akv_linear_rowscaled reads.
+extern "C" int akv_linear_adds_rows(const void* x, const void* wp, float* stream_out, float* sums_out, float* pieces,
+                                    unsigned int* arrivals, int exchange_tiles, int rows, int outs, int k, int n_tiles,
+                                    int k_tiles, const float* bias, void* rows_out, const float* gain, hipStream_t stream) {
+  if (rows_out == nullptr || gain == nullptr) return -2;
+  return linear_adds(x, wp, stream_out, sums_out, pieces, arrivals, exchange_tiles, rows, outs, k, n_tiles, k_tiles, bias,
+                     rows_out, gain, stream);
+}
+
+// y [rows, outs] = (x W^T) with every row scaled by rsqrt(its mean of squares + eps), plus `bias` (gated: silu of
+// the scaled gate times the scaled up): x [rows, k] bfloat16 are the rows akv_linear_adds_rows left - the residual
+// sum times the norm's weight -, `sums` [sum_tiles][16] the partial sums of squares of the residual rows it left
+// (sum_tiles = ceil(k / 16)).  Sizes, `pieces`, `arrivals`, `row_tiles`: as for akv_linear_scaled, without its limit
+// on the rows' bytes.
+extern "C" int akv_linear_rowscaled(const void* x, const float* sums, int sum_tiles, float eps, const void* wp, void* y,
+                                    float* pieces, unsigned int* arrivals, int exchange_tiles, int rows, int outs, int k,
+                                    int n_tiles, int k_tiles, int gated, int row_tiles, const float* bias,
+                                    hipStream_t stream) {
+  if (rows <= 0 || outs <= 0) return 0;
+  if (rows > 16 || (k & 7) != 0 || k_tiles * 32 < k || sum_tiles != (k + 15) / 16) return -2;
+  if (row_tiles < 0 || row_tiles > 2 || (gated && (row_tiles == 1 || bias != nullptr))) return -2;
+  if (gated ? ((outs & 15) != 0 || n_tiles * 8 != outs) : n_tiles * 16 < outs) return -2;
+  DecodeArgs a{};
+  a.x = static_cast<const bf16_t*>(x);
+  a.sums = sums;
+  a.sum_tiles = sum_tiles;
+  a.eps = eps;
+  a.wp = static_cast<const uintx4*>(wp);
+  a.y = static_cast<bf16_t*>(y);
+  a.bias = bias;
+  if (pieces != nullptr && arrivals != nullptr && exchange_tiles >= n_tiles + 1) a.pieces = pieces, a.arrivals = arrivals;
+  const bool may = a.pieces != nullptr;
+  a.rows = rows, a.outs = outs, a.k = k, a.k_tiles = k_tiles, a.n_tiles = n_tiles;
+  if (gated) return launch_decode<2, true, false, false, true>(a, stream);
+  // (rows from memory: two row tiles a wave share the rows' loads, as in the plain product)
+  if (row_tiles == 0)
+    row_tiles = n_tiles >= 2 && plan_decode(2, n_tiles, k_tiles, k, 0, may).work < plan_decode(1, n_tiles, k_tiles, k, 0, may).work ? 2 : 1;
+  if (row_tiles == 2) return launch_decode<2, false, false, false, true>(a, stream);
+  return launch_decode<1, false, false, false, true>(a, stream);
 }
 
 // y [rows, outs] = norm(stream) W^T (gated: y [rows, inter] = silu(. Wgate^T) * (. Wup^T), wp as for

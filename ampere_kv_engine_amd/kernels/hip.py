@@ -143,7 +143,8 @@ class HipKernels(KernelSet):
                      "akv_linear_tiled", "akv_linear_packed", "akv_linear_packed_swiglu", "akv_linear_packed_normed",
                      "akv_pack_rows", "akv_linear_packed_static", "akv_linear_mid", "akv_linear_mid_workspace",
                      "akv_linear_mid_adds", "akv_linear_mid_rowscaled", "akv_linear_mid_bands", "akv_linear_mid_most_groups",
-                     "akv_linear_adds", "akv_linear_scaled", "akv_linear_decode_plan", "akv_read_probe",
+                     "akv_linear_adds", "akv_linear_scaled", "akv_linear_adds_rows", "akv_linear_rowscaled",
+                     "akv_linear_decode_plan", "akv_read_probe",
                      "akv_attention_rows", "akv_decode_plan", "akv_sample", "akv_sample_slots", "akv_step_prologue"):
             getattr(self.lib, name).restype = ctypes.c_int
         self._check_slot_layout()
@@ -533,6 +534,8 @@ class HipKernels(KernelSet):
                                     # (measured from 1 to 16 rows at Qwen3-8B sizes: 5 to 14 us less per layer)
     FOLD_NORM_BYTES = 160 * 1024 - 832   # ... while the normed rows fit into a compute unit's LDS beside the scales
     fold_norms = True
+    fold_rows_left = True           # ... the adding product leaving the rows times the next norm's weight, so that
+                                    # the reading one only scales its sums (`linear_rowscaled`) instead of norming rows
     FOLD_MID_ROWS = 512             # ... and steps of up to this many, where the mid-size kernel takes the products:
     fold_mid = True                 # (a layer launches two norm kernels less: 5 us each and the gaps around them)
 
@@ -543,8 +546,8 @@ class HipKernels(KernelSet):
         norm's weight and divides its results by the rows' root mean square (`linear_rowscaled`)."""
         if dtype != torch.bfloat16 or hidden % 8 != 0:
             return False
-        if 0 < rows <= self.FOLD_NORM_ROWS:
-            return self.fold_norms and rows * hidden * 2 <= self.FOLD_NORM_BYTES
+        if 0 < rows <= self.FOLD_NORM_ROWS:     # (a product that norms its rows itself keeps them in LDS)
+            return self.fold_norms and (self.fold_rows_left or rows * hidden * 2 <= self.FOLD_NORM_BYTES)
         return self.fold_mid and rows <= self.FOLD_MID_ROWS
 
     def _reserve_exchange(self, n_tiles: int) -> None:
@@ -592,8 +595,12 @@ class HipKernels(KernelSet):
         rows = x.shape[0]
         if rows <= self.FOLD_NORM_ROWS:
             sums = arena.take(((weight.outs + 15) // 16, 16), torch.float32)
-            self.linear_adds(x, weight, stream, sums, bias=bias)
-            return StreamSums(sums)
+            if gain is None or not self.fold_rows_left:
+                self.linear_adds(x, weight, stream, sums, bias=bias)
+                return StreamSums(sums)
+            left = arena.take((rows, weight.outs), torch.bfloat16)
+            self.linear_adds(x, weight, stream, sums, bias=bias, rows_out=left, gain=gain)
+            return StreamSums(sums, rows=left, gain=gain)
         self._dense(x, "x", torch.bfloat16, (rows, weight.k))
         self._dense(stream, "stream", torch.float32, (rows, weight.outs))
         self._dense(gain, "norm weight", torch.float32, (weight.outs,))
@@ -608,14 +615,17 @@ class HipKernels(KernelSet):
     def scales_rows_in_product(self, rows: int, weight, dtype, sums) -> bool:
         gated = isinstance(weight, GatedWeight)
         packed = weight.packed if gated else weight
-        if (not isinstance(packed, PackedWeight) or sums.rows is None or not self.FOLD_NORM_ROWS < rows <= self.FOLD_MID_ROWS
-                or dtype != torch.bfloat16 or sums.sums.shape[0] > self.lib.akv_linear_mid_most_groups(rows)):
+        if not isinstance(packed, PackedWeight) or sums.rows is None or dtype != torch.bfloat16:
+            return False
+        if rows <= self.FOLD_NORM_ROWS:         # the decode products
+            return self.fold_norms and rows > 0 and packed.k % 8 == 0 and tuple(sums.sums.shape) == ((packed.k + 15) // 16, 16)
+        if rows > self.FOLD_MID_ROWS or sums.sums.shape[0] > self.lib.akv_linear_mid_most_groups(rows):
             return False
         if gated:
             return self._route("gated", weight.inter, packed.k, rows, weight.stacked is not None, dtype) == "mid"
         return self._route("linear", packed.outs, packed.k, rows, packed.row_major is not None, dtype) == "mid"
 
-    def linear_rowscaled(self, x, sums, eps, weight, out, bias=None) -> None:
+    def linear_rowscaled(self, x, sums, eps, weight, out, bias=None, row_tiles: int = 0) -> None:
         """out = (x W^T) with every row divided by sqrt(mean of squares + eps), plus `bias` (a `GatedWeight`: silu of
         the scaled gate times the scaled up): x [rows, k] are rows that `add_to_stream` left - the residual sum times
         the norm's weight -, sums [groups, rows rounded up to 16] the partial sums of squares of the residual rows."""
@@ -624,21 +634,32 @@ class HipKernels(KernelSet):
         rows = x.shape[0]
         outs = weight.inter if gated else packed.outs
         self._dense(x, "x", torch.bfloat16, (rows, packed.k))
-        self._dense(sums, "sums", torch.float32, (sums.shape[0], (rows + 15) // 16 * 16))
         self._dense(out, "out", torch.bfloat16, (rows, outs))
         self._dense(packed.data, "packed weight", torch.bfloat16)
         if bias is not None and gated:
             raise KernelError("the gated product takes no bias")
         self._bias(bias, outs)
+        if rows <= self.FOLD_NORM_ROWS:         # a decode step: sums per (16 values of a row, row), as `linear_adds` leaves them
+            self._dense(sums, "sums", torch.float32, ((packed.k + 15) // 16, 16))
+            pieces, arrivals = self._exchange(packed.n_tiles)
+            self._check(self.lib.akv_linear_rowscaled(_ptr(x), _ptr(sums), (packed.k + 15) // 16, ctypes.c_float(eps),
+                                                      _ptr(packed.data), _ptr(out), _ptr(pieces), _ptr(arrivals),
+                                                      self._exchange_tiles if pieces is not None else 0, rows, outs,
+                                                      packed.k, packed.n_tiles, packed.k_tiles, 1 if gated else 0,
+                                                      row_tiles, _ptr(bias), self._stream()), "linear_rowscaled")
+            return
+        self._dense(sums, "sums", torch.float32, (sums.shape[0], (rows + 15) // 16 * 16))
         self._mid(x, packed, out, rows, outs, gated, bias, scaled=(sums, eps))
 
     def norms_rows_in_product(self, rows: int, weight, dtype) -> bool:
         packed = weight.packed if isinstance(weight, GatedWeight) else weight
-        return isinstance(packed, PackedWeight) and rows <= self.FOLD_NORM_ROWS and self.folds_norm(rows, packed.k, dtype)
+        return (isinstance(packed, PackedWeight) and 0 < rows <= self.FOLD_NORM_ROWS and self.fold_norms
+                and dtype == torch.bfloat16 and packed.k % 8 == 0 and rows * packed.k * 2 <= self.FOLD_NORM_BYTES)
 
-    def linear_adds(self, x, weight: PackedWeight, stream, sums, bias=None) -> None:
+    def linear_adds(self, x, weight: PackedWeight, stream, sums, bias=None, rows_out=None, gain=None) -> None:
         """stream [rows, outs] (float32) += bfloat16(x W^T (+ bias)), in place; sums [ceil(outs / 16), 16] (float32) receives
-        per tile of 16 outputs and row the sum of squares of the new values."""
+        per tile of 16 outputs and row the sum of squares of the new values; `rows_out` [rows, outs] bfloat16, if
+        given, the new sum times `gain` [outs] (the weight of the norm that follows: what `linear_rowscaled` reads)."""
         rows = x.shape[0]
         if not isinstance(weight, PackedWeight) or rows > 16:
             raise KernelError("the product that adds to the residual sum takes a packed matrix and up to 16 rows")
@@ -647,6 +668,15 @@ class HipKernels(KernelSet):
         self._dense(sums, "sums", torch.float32, ((weight.outs + 15) // 16, 16))
         self._dense(weight.data, "packed weight", torch.bfloat16)
         pieces, arrivals = self._exchange(weight.n_tiles)
+        if rows_out is not None:
+            self._dense(rows_out, "rows_out", torch.bfloat16, (rows, weight.outs))
+            self._dense(gain, "norm weight", torch.float32, (weight.outs,))
+            self._check(self.lib.akv_linear_adds_rows(_ptr(x), _ptr(weight.data), _ptr(stream), _ptr(sums), _ptr(pieces),
+                                                      _ptr(arrivals), self._exchange_tiles if pieces is not None else 0,
+                                                      rows, weight.outs, weight.k, weight.n_tiles, weight.k_tiles,
+                                                      _ptr(self._bias(bias, weight.outs)), _ptr(rows_out), _ptr(gain),
+                                                      self._stream()), "linear_adds")
+            return
         self._check(self.lib.akv_linear_adds(_ptr(x), _ptr(weight.data), _ptr(stream), _ptr(sums), _ptr(pieces),
                                              _ptr(arrivals), self._exchange_tiles if pieces is not None else 0,
                                              rows, weight.outs, weight.k, weight.n_tiles,

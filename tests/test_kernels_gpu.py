@@ -367,8 +367,12 @@ def test_a_product_adds_itself_to_the_residual_sum_and_leaves_its_rows_sums_of_s
     y = torch.empty(rows, outs, dtype=torch.bfloat16)
     ref.linear(x, w, y)
     packed = hip.prepare_linear(w.cuda())
-    # (the engine folds only where the next product can hold the normed rows in LDS; the kernel takes any 16 rows)
+    # (any 16 rows; with `fold_rows_left` off the engine folds only where the next product, which then norms the rows
+    # itself, can hold them in LDS)
+    assert hip.adds_to_stream(rows, packed, torch.bfloat16)
+    monkeypatch.setattr(hip, "fold_rows_left", False)
     assert hip.adds_to_stream(rows, packed, torch.bfloat16) == (rows * outs * 2 <= hip.FOLD_NORM_BYTES)
+    monkeypatch.setattr(hip, "fold_rows_left", True)
     assert not hip.adds_to_stream(17, packed, torch.bfloat16)
     got = stream.cuda()
     tiles = (outs + 15) // 16
@@ -826,6 +830,66 @@ def test_mid_size_products_keep_the_residual_sum_and_the_norm(hip_own, ref, rows
     hip_own.linear_rowscaled(left.rows, left.sums, eps, gated, got)
     assert torch.equal(first, got)
     assert int(hip_own._mid_counters.abs().sum()) == 0 if hip_own._mid_counters is not None else True
+
+
+@pytest.mark.parametrize("rows,hidden,k,inter", [(1, 96, 72, 64), (3, 304, 520, 208), (8, 4096, 4096, 1024), (16, 4096, 512, 512),
+                                                 (5, 1000, 2048, 256), (16, 5120, 256, 64), (8, 104, 64, 32), (2, 8192, 1024, 128)])
+def test_decode_products_leave_rows_for_a_product_that_scales_its_sums(hip, ref, rows, hidden, k, inter, monkeypatch):
+    """Steps of up to 16 rows: `linear_adds(..., rows_out=, gain=)` adds to the residual sum exactly as without the
+    two (the same bits, sums of squares included) and leaves the new rows times the next norm's weight;
+    `linear_rowscaled` multiplies such rows and scales every sum by its row's 1 / rms - plain with and without a bias,
+    with one and two row tiles a wave, and gated - against its formula and against the product that norms its rows
+    itself (`linear_scaled`)."""
+    monkeypatch.setattr(hip, "fold_norms", True)
+    eps = 1e-5
+    w = rand(hidden, k, dtype=torch.bfloat16, seed=401, scale=0.05)
+    x = rand(rows, k, dtype=torch.bfloat16, seed=402)
+    bias = rand(hidden, seed=403, scale=0.5)
+    before = rand(rows, hidden, seed=404, scale=2.0)
+    gain = rand(hidden, seed=405).abs() + 0.5
+    packed = hip.prepare_linear(w.cuda())
+    tiles = (hidden + 15) // 16
+    plain_stream, plain_sums = before.clone().cuda(), torch.full((tiles, 16), float("nan"), device="cuda")
+    hip.linear_adds(x.cuda(), packed, plain_stream, plain_sums, bias=bias.cuda())
+    stream, sums = before.clone().cuda(), torch.full((tiles, 16), float("nan"), device="cuda")
+    left = torch.full((rows, hidden), float("nan"), dtype=torch.bfloat16, device="cuda")
+    hip.linear_adds(x.cuda(), packed, stream, sums, bias=bias.cuda(), rows_out=left, gain=gain.cuda())
+    assert torch.equal(stream, plain_stream) and torch.equal(sums, plain_sums)
+    now = stream.cpu()
+    assert torch.equal(left.cpu(), (now * gain).bfloat16())
+    from ampere_kv_engine_amd.parts.base import StreamSums
+    handed = StreamSums(sums, rows=left, gain=gain)
+    totals = sums.sum(0).cpu()
+    scale = torch.rsqrt(totals[:rows, None] / hidden + eps)
+    rows_left = left.cpu().float()
+    second = rand(inter, hidden, dtype=torch.bfloat16, seed=406, scale=0.05)
+    second_bias = rand(inter, seed=407, scale=0.5)
+    plain = hip.prepare_linear(second.cuda())
+    assert hip.scales_rows_in_product(rows, plain, torch.bfloat16, handed)
+    for with_bias in (False, True):
+        b = second_bias.cuda() if with_bias else None
+        norming = None
+        if hip.norms_rows_in_product(rows, plain, torch.bfloat16):     # (its normed rows must fit a compute unit's LDS)
+            norming = torch.empty((rows, inter), dtype=torch.bfloat16, device="cuda")
+            hip.linear_scaled(stream, sums, gain.cuda(), eps, plain, norming, bias=b)
+        want = rows_left @ second.float().T * scale + (second_bias if with_bias else 0.0)
+        for row_tiles in (0, 1, 2):
+            got = torch.full((rows, inter), float("nan"), dtype=torch.bfloat16, device="cuda")
+            hip.linear_rowscaled(left, sums, eps, plain, got, bias=b, row_tiles=row_tiles)
+            torch.testing.assert_close(got.cpu().float(), want.bfloat16().float(), **tol(torch.bfloat16))
+            if norming is not None:
+                apart = got.float() - norming.float()      # operands rounded elsewhere: little over all outputs
+                assert float(apart.pow(2).mean().sqrt()) <= 2.0 ** -7 * float(norming.float().pow(2).mean().sqrt())
+    gate, up = (rand(inter, hidden, dtype=torch.bfloat16, seed=408 + i, scale=0.05) for i in range(2))
+    gated = hip.prepare_gated_linear(gate.cuda(), up.cuda())
+    assert hip.scales_rows_in_product(rows, gated, torch.bfloat16, handed)
+    got = torch.full((rows, inter), float("nan"), dtype=torch.bfloat16, device="cuda")
+    hip.linear_rowscaled(left, sums, eps, gated, got)
+    g, u = rows_left @ gate.float().T * scale, rows_left @ up.float().T * scale
+    torch.testing.assert_close(got.cpu().float(), (g * torch.sigmoid(g) * u).bfloat16().float(), **tol(torch.bfloat16))
+    again = torch.empty_like(got)
+    hip.linear_rowscaled(left, sums, eps, gated, again)
+    assert torch.equal(got, again)
 
 
 def test_linear_keeps_other_weights_row_major(hip):
