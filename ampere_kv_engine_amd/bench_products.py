@@ -99,7 +99,12 @@ def main(argv=None) -> int:
                 sums = torch.empty((outs + 15) // 16, 16, dtype=torch.float32, device=device)
                 record["adds_to_stream_us"] = timed([(lambda i=i: kernels.linear_adds(x, weights[turn(i)], stream, sums))
                                                      for i in range(args.repeats)])
-            elif rows * k * 2 <= kernels.FOLD_NORM_BYTES:   # the product norms the residual rows itself
+                # ... and leaves the new rows times the next norm's weight for a product that scales its sums
+                left, gain = torch.empty(rows, outs, dtype=torch.bfloat16, device=device), torch.ones(outs, device=device)
+                record["adds_and_leaves_rows_us"] = timed([(lambda i=i: kernels.linear_adds(x, weights[turn(i)], stream, sums,
+                                                                                            rows_out=left, gain=gain))
+                                                           for i in range(args.repeats)])
+            else:
                 stream = torch.randn(rows, k, device=device, generator=generator)
                 sums = torch.zeros((k + 15) // 16, 16, dtype=torch.float32, device=device)
                 sums[:, :rows] = (stream * stream).view(rows, -1, 16).sum(-1).T if k % 16 == 0 else 1.0
@@ -107,8 +112,14 @@ def main(argv=None) -> int:
                 normed = torch.empty(rows, k, dtype=torch.bfloat16, device=device)
                 record["norm_kernel_us"] = timed([(lambda: kernels.add_rmsnorm(stream, None, gain, 1e-6, normed))
                                                   for _ in range(args.repeats)])
-                record["norms_its_rows_us"] = timed([(lambda i=i: kernels.linear_scaled(stream, sums, gain, 1e-6, weights[turn(i)], out))
-                                                     for i in range(args.repeats)])
+                if rows * k * 2 <= kernels.FOLD_NORM_BYTES:   # the product norms the residual rows itself
+                    record["norms_its_rows_us"] = timed([(lambda i=i: kernels.linear_scaled(stream, sums, gain, 1e-6, weights[turn(i)], out))
+                                                         for i in range(args.repeats)])
+                # the product reads rows that were left times the norm's weight and scales its sums by their 1 / rms
+                for tiles in ((0,) if kind == "gated" else (0, 1, 2)):
+                    name_of = "scales_its_sums_us" if tiles == 0 else f"scales_its_sums_{tiles}_row_tiles_us"
+                    record[name_of] = timed([(lambda i=i: kernels.linear_rowscaled(x, sums, 1e-6, weights[turn(i)], out, row_tiles=tiles))
+                                             for i in range(args.repeats)])
             print(json.dumps(record), flush=True)
         del weights, data
     return 0
