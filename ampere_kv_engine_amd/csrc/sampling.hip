@@ -71,7 +71,8 @@ __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ 
   float value = -INFINITY;
   int index = vocab;  // "none yet"; any real index is lower
   // eight loads of a thread are on their way before the first is looked at; ids still ascend per thread, so the
-  // first maximum stays
+  // first maximum stays.  (Every load is issued whatever its place - beyond the row it asks for the row's last piece,
+  // which is then not looked at -: behind a test each, the eight would be waited for one by one.)
   constexpr int kAhead = 8;
   auto look_at = [&](int i, float score) {
     saw_nan |= score != score;
@@ -90,10 +91,10 @@ __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ 
       float4 fetched[kAhead];
 #pragma unroll
       for (int u = 0; u < kAhead; ++u) {
-        const int p = p0 + u * blockDim.x;
-        fetched[u] = p < pieces ? *reinterpret_cast<const float4*>(x + 4 * static_cast<size_t>(p))
-                                : float4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+        const int p = min(p0 + u * static_cast<int>(blockDim.x), pieces - 1);
+        fetched[u] = *reinterpret_cast<const float4*>(x + 4 * static_cast<size_t>(p));
       }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int u = 0; u < kAhead; ++u) {
         const int i = 4 * (p0 + u * blockDim.x);
@@ -110,9 +111,9 @@ __global__ __launch_bounds__(1024) void sample_kernel(const float* __restrict__ 
       float fetched[kAhead];
 #pragma unroll
       for (int u = 0; u < kAhead; ++u) {
-        const int i = i0 + u * blockDim.x;
-        fetched[u] = i < vocab ? x[i] : -INFINITY;
+        fetched[u] = x[min(i0 + u * static_cast<int>(blockDim.x), vocab - 1)];
       }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int u = 0; u < kAhead; ++u) look_at(i0 + u * blockDim.x, fetched[u]);
     }
