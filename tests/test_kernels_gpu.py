@@ -832,6 +832,30 @@ def test_mid_size_products_keep_the_residual_sum_and_the_norm(hip_own, ref, rows
     assert int(hip_own._mid_counters.abs().sum()) == 0 if hip_own._mid_counters is not None else True
 
 
+@pytest.mark.parametrize("rows", [5, 16, 40, 130])
+@pytest.mark.parametrize("outs", [100, 90, 35])
+def test_adding_products_at_widths_that_are_no_multiple_of_four(hip_own, rows, outs, monkeypatch):
+    """The adding products' epilogues element by element (the engine never asks for such widths - a product that
+    reads the rows needs a width that is a multiple of 8 - but the entry points take them): the residual sum, the
+    rows left and the sums of squares, at up to 16 rows and beyond."""
+    from ampere_kv_engine_amd.engine.batch import Arena
+    monkeypatch.setattr(hip_own, "fold_norms", True)
+    k = 264
+    w = rand(outs, k, dtype=torch.bfloat16, seed=501, scale=0.05)
+    x = rand(rows, k, dtype=torch.bfloat16, seed=502)
+    bias = rand(outs, seed=503, scale=0.5)
+    before = rand(rows, outs, seed=504, scale=2.0)
+    gain = rand(outs, seed=505).abs() + 0.5
+    stream = before.clone().cuda()
+    left = hip_own.add_to_stream(x.cuda(), hip_own.prepare_linear(w.cuda()), stream, Arena("cuda:0"), bias=bias.cuda(), gain=gain.cuda())
+    product = (x.float() @ w.float().T + bias).bfloat16().float()
+    torch.testing.assert_close(stream.cpu() - before, product, rtol=1.6e-2, atol=2e-3)
+    now = stream.cpu()
+    assert torch.equal(left.rows.cpu(), (now * gain).bfloat16())
+    totals = left.sums.sum(0).cpu()
+    torch.testing.assert_close(totals[:rows], (now * now).sum(-1), rtol=1e-5, atol=1e-6)
+
+
 @pytest.mark.parametrize("rows,hidden,k,inter", [(1, 96, 72, 64), (3, 304, 520, 208), (8, 4096, 4096, 1024), (16, 4096, 512, 512),
                                                  (5, 1000, 2048, 256), (16, 5120, 256, 64), (8, 104, 64, 32), (2, 8192, 1024, 128)])
 def test_decode_products_leave_rows_for_a_product_that_scales_its_sums(hip, ref, rows, hidden, k, inter, monkeypatch):
