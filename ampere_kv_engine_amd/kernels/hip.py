@@ -137,6 +137,7 @@ class HipKernels(KernelSet):
         self.pair_launch = True         # a step of single tokens and short portions: their attention as one launch,
         self.portions_beside_single_tokens = True   # or, where that does not fit, the portions' on a second stream
         self._beside_stream = None
+        self._sample_workspace = None   # where a row's blocks leave their parts' best logits (see `_sample_parts`)
         self.compute_units = torch.cuda.get_device_properties(self.device).multi_processor_count
         for name in ("akv_embed", "akv_add_rmsnorm", "akv_rmsnorm_rows", "akv_copy_rows", "akv_gather_rows",
                      "akv_swiglu", "akv_rope_table", "akv_rope", "akv_kv_write", "akv_qk_norm_rope_write",
@@ -145,7 +146,8 @@ class HipKernels(KernelSet):
                      "akv_linear_mid_adds", "akv_linear_mid_rowscaled", "akv_linear_mid_bands", "akv_linear_mid_most_groups",
                      "akv_linear_adds", "akv_linear_scaled", "akv_linear_adds_rows", "akv_linear_rowscaled",
                      "akv_linear_decode_plan", "akv_read_probe",
-                     "akv_attention_rows", "akv_decode_plan", "akv_sample", "akv_sample_slots", "akv_step_prologue"):
+                     "akv_attention_rows", "akv_decode_plan", "akv_sample", "akv_sample_slots", "akv_sample_parts",
+                     "akv_step_prologue"):
             getattr(self.lib, name).restype = ctypes.c_int
         self._check_slot_layout()
 
@@ -1230,6 +1232,25 @@ class HipKernels(KernelSet):
             int(window) if window is not None else 0, self._stream()), "attention")
 
     # ---- sampling ----------------------------------------------------------------------------------------
+    # A row of logits is cut over several blocks where the rows are few (one block on one compute unit takes 18 us
+    # for 151,936 logits): enough parts for some 256 blocks, each of at least 2,048 logits.
+    SAMPLE_PART_ROWS = 1024         # rows the parts' workspace serves; more rows have a block each anyway
+    sample_in_parts = True
+
+    def _sample_parts(self, rows: int, vocab: int) -> int:
+        if not self.sample_in_parts or rows > self.SAMPLE_PART_ROWS:
+            return 1
+        parts = min(64, max(1, 256 // rows), vocab // 2048)
+        if parts < 2:
+            return 1
+        if self._sample_workspace is None:
+            if torch.cuda.is_current_stream_capturing():
+                return 1
+            self._sample_workspace = (torch.empty(self.SAMPLE_PART_ROWS * 64, dtype=torch.float32, device=self.device),
+                                      torch.empty(self.SAMPLE_PART_ROWS * 64, dtype=torch.int32, device=self.device),
+                                      torch.zeros(self.SAMPLE_PART_ROWS, dtype=torch.int32, device=self.device))
+        return parts
+
     def sample(self, logits, temperature, seeds, draws, out):
         rows, vocab = logits.shape
         self._dense(logits, "logits", torch.float32)
@@ -1238,6 +1259,13 @@ class HipKernels(KernelSet):
             self._dense(temperature, "temperature", torch.float32, (rows,))
             self._dense(seeds, "seeds", torch.int64, (rows,))
             self._dense(draws, "draws", torch.int32, (rows,))
+        parts = self._sample_parts(rows, vocab)
+        if parts > 1:
+            values, ids, arrivals = self._sample_workspace
+            self._check(self.lib.akv_sample_parts(_ptr(logits), _ptr(temperature), _ptr(seeds), _ptr(draws), None, None, None,
+                                                  None, _ptr(out), rows, vocab, parts, _ptr(values), _ptr(ids),
+                                                  _ptr(arrivals), self._stream()), "sample")
+            return
         self._check(self.lib.akv_sample(_ptr(logits), _ptr(temperature), _ptr(seeds), _ptr(draws), _ptr(out), rows,
                                         vocab, self._stream()), "sample")
 
@@ -1253,6 +1281,13 @@ class HipKernels(KernelSet):
         self._dense(ctx.slot_words, "slot_words", torch.int32)
         if max(ctx.host_seq_slots) >= ctx.slot_words.shape[0]:
             raise KernelError("a request's slot lies outside the slot words")
+        parts = self._sample_parts(rows, vocab)
+        if parts > 1:
+            values, ids, arrivals = self._sample_workspace
+            self._check(self.lib.akv_sample_parts(_ptr(logits), None, None, None, _ptr(ctx.logit_rows), _ptr(ctx.seq_of_token),
+                                                  _ptr(ctx.seq_slots), _ptr(ctx.slot_words), _ptr(out), rows, vocab, parts,
+                                                  _ptr(values), _ptr(ids), _ptr(arrivals), self._stream()), "sample_slots")
+            return
         self._check(self.lib.akv_sample_slots(_ptr(logits), _ptr(ctx.logit_rows), _ptr(ctx.seq_of_token),
                                               _ptr(ctx.seq_slots), _ptr(ctx.slot_words), _ptr(out), rows, vocab,
                                               self._stream()), "sample_slots")

@@ -1451,6 +1451,51 @@ def test_sample(hip, vocab):
     assert greedy.cpu().tolist() == [int(r.argmax()) if i != 1 else 100 for i, r in enumerate(logits)]
 
 
+@pytest.mark.parametrize("rows,vocab", [(1, 151936), (3, 40004), (8, 151936), (64, 32768), (5, 8197), (300, 4096)])
+def test_a_row_cut_over_several_blocks_chooses_what_one_block_chooses(hip, rows, vocab, monkeypatch):
+    """Few rows of many logits are cut over several blocks a row, whose bests the last block of the row compares:
+    greedy and with temperatures, ties within and across parts, a row with a NaN, a row of -inf - the tokens are
+    those of the one-block kernel, twice in a row (the arrival counters are left at zero), handed in and from slots."""
+    import struct
+    generator = torch.Generator().manual_seed(rows * 7 + vocab)
+    logits = torch.randn(rows, vocab, generator=generator) * 2
+    logits[0, vocab - 1] = logits[0, 17] = 60.0                  # a tie across the row's ends: the lowest id
+    if rows > 2:
+        logits[1, vocab // 3] = float("nan")
+        logits[2] = float("-inf")
+    temperature = torch.tensor([0.0 if r % 2 == 0 else 0.5 + 0.1 * (r % 7) for r in range(rows)])
+    seeds = torch.arange(rows, dtype=torch.int64) * 977 + (3 << 34)
+    draws = torch.arange(rows, dtype=torch.int32) % 5
+    on = [t.cuda() for t in (logits, temperature, seeds, draws)]
+    monkeypatch.setattr(hip, "sample_in_parts", False)
+    want = torch.empty(rows, dtype=torch.int32, device="cuda")
+    hip.sample(*on, want)
+    monkeypatch.setattr(hip, "sample_in_parts", True)
+    assert (hip._sample_parts(rows, vocab) > 1) == (rows <= 128 and vocab >= 4096)
+    for _ in range(2):
+        got = torch.full((rows,), -7, dtype=torch.int32, device="cuda")
+        hip.sample(*on, got)
+        assert torch.equal(got, want)
+    assert want[0] == 17 and (rows <= 2 or (want[1] == -1 and want[2] == -1))
+    if hip._sample_workspace is not None:
+        assert int(hip._sample_workspace[2].abs().sum()) == 0
+    # from slots: request r in slot rows - 1 - r, one token row each
+    words = torch.zeros(rows, 8, dtype=torch.int32)
+    for r in range(rows):
+        seed = int(seeds[r])
+        words[rows - 1 - r] = torch.tensor([1, -1, struct.unpack("<i", struct.pack("<f", float(temperature[r])))[0],
+                                            seed & 0xFFFFFFFF, seed >> 32, int(draws[r]), 1, 0])
+    ctx = SimpleNamespace(num_tokens=rows, num_seqs=rows, logit_rows=torch.arange(rows, dtype=torch.int32).cuda(),
+                          seq_of_token=torch.arange(rows, dtype=torch.int32).cuda(),
+                          seq_slots=torch.arange(rows - 1, -1, -1, dtype=torch.int32).cuda(),
+                          host_seq_slots=list(range(rows - 1, -1, -1)), slot_words=words.cuda())
+    got = torch.empty(rows, dtype=torch.int32, device="cuda")
+    hip.sample_slots(on[0], ctx, got)
+    assert torch.equal(got, want)
+    after = ctx.slot_words.cpu()
+    assert after[:, 1].flip(0).tolist() == want.cpu().tolist() and after[:, 5].flip(0).tolist() == (draws + 1).tolist()
+
+
 def test_sampling_follows_the_distribution(hip):
     probs = torch.tensor([0.5, 0.25, 0.125, 0.125])
     rows = 4000
