@@ -44,6 +44,28 @@ __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ 
     return;
   }
   const T* src = table + static_cast<size_t>(id) * hidden;
+  if constexpr (std::is_same<T, bf16_t>::value) {
+    if ((hidden & 7) == 0) {     // 16 bytes of the row a thread and turn, all of a thread's loads on their way at once
+      constexpr int kTurns = 4;
+      for (int d0 = threadIdx.x * 8; d0 < hidden; d0 += kTurns * blockDim.x * 8) {
+        uint4 raw[kTurns];
+#pragma unroll
+        for (int u = 0; u < kTurns; ++u)
+          raw[u] = *reinterpret_cast<const uint4*>(src + min(d0 + u * static_cast<int>(blockDim.x) * 8, hidden - 8));
+#pragma unroll
+        for (int u = 0; u < kTurns; ++u) {
+          const int d = d0 + u * blockDim.x * 8;
+          if (d >= hidden) break;
+          const uint32_t w[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+          *reinterpret_cast<float4*>(dst + d) = make_float4(__uint_as_float(w[0] << 16), __uint_as_float(w[0] & 0xffff0000u),
+                                                            __uint_as_float(w[1] << 16), __uint_as_float(w[1] & 0xffff0000u));
+          *reinterpret_cast<float4*>(dst + d + 4) = make_float4(__uint_as_float(w[2] << 16), __uint_as_float(w[2] & 0xffff0000u),
+                                                                __uint_as_float(w[3] << 16), __uint_as_float(w[3] & 0xffff0000u));
+        }
+      }
+      return;
+    }
+  }
   for (int d = threadIdx.x; d < hidden; d += blockDim.x) dst[d] = to_float(src[d]);
 }
 
