@@ -90,7 +90,7 @@ def check(engine, case, schedule):
         what = f"{case['name']}/{dtype} request {name} (page size {case['page_size']})"
         worst = max(worst, *assert_logits_close(got[name], want, dtype, "plain", what))
     if dtype == "bfloat16" and engine.device.type == "cuda":
-        same, _ = schedules.run(double_engine(case), case["requests"], schedule)
+        same, _ = schedules.run(double_engine(case, like=engine.kernels), case["requests"], schedule)
         for name in case["expected"]:
             what = f"{case['name']}/{dtype} request {name} (page size {case['page_size']})"
             worst = max(worst, *assert_logits_close(got[name], same[name], dtype, "double", what))
@@ -103,13 +103,18 @@ def check(engine, case, schedule):
 _DOUBLES = {}
 
 
-def double_engine(case, dtype="bfloat16"):
-    """The engine of `case` with the torch double of the kernel set, on the CPU (kept between tests)."""
+def double_engine(case, dtype="bfloat16", like=None):
+    """The engine of `case` with the torch double of the kernel set, on the CPU (kept between tests).  `like`: a HIP
+    kernel set whose roundings the double is to share - where that one's products keep the residual sum and leave the
+    rows times the next norm's weight for a product that scales its results, the double's do."""
     from torch_kernels import TorchKernels
     pages = max(POOL_TOKENS // case["page_size"], 4, case.get("pool_pages", 0))    # (room for every schedule of the case)
-    key = (case["name"], case["folder"], dtype, case["page_size"], pages)
+    few = 16 if like is not None and like.fold_norms and like.fold_rows_left else 0
+    many = like.FOLD_MID_ROWS if like is not None and like.fold_mid else 0
+    key = (case["name"], case["folder"], dtype, case["page_size"], pages, few, many)
     if key not in _DOUBLES:
-        _DOUBLES[key] = make_engine(case, dtype, "cpu", kernels=TorchKernels(), num_pages=pages)
+        kernels = TorchKernels(fold_rows=few, fold_many_rows=many, rows_left=few > 0)
+        _DOUBLES[key] = make_engine(case, dtype, "cpu", kernels=kernels, num_pages=pages)
     return _DOUBLES[key]
 
 

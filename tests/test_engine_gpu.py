@@ -265,7 +265,8 @@ def test_a_wrong_page_is_seen_in_bfloat16(case, fault):
     with the wrong page must leave the limits that every cutting is held to; its neighbour must stay inside them."""
     from ampere_kv_engine_amd.engine import StepEntry
     ids = {"c": case["requests"]["c"], "d": case["requests"]["d"]}
-    engine, double = cases.make_engine(case, "bfloat16", "cuda:0"), cases.double_engine(case)
+    engine = cases.make_engine(case, "bfloat16", "cuda:0")
+    double = cases.double_engine(case, like=engine.kernels)
     logits = {}
     for name, eng in (("engine", engine), ("double", double)):
         seqs = {n: eng.open(n) for n in ids}

@@ -23,7 +23,7 @@ def _round(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
 class TorchKernels(KernelSet):
     name = "torch-double"
 
-    def __init__(self, fold_rows: int = 0, fold_many_rows: int = 0):
+    def __init__(self, fold_rows: int = 0, fold_many_rows: int = 0, rows_left: bool = False):
         """`fold_rows`: steps of up to this many rows let a branch's last product add itself to the residual sum and
         the next product norm its rows from the sums of squares left there, as the HIP kernel set does in decode
         steps (0: never).  `fold_many_rows`: steps of more rows, up to this many, do the same the way the HIP
@@ -31,6 +31,9 @@ class TorchKernels(KernelSet):
         the reading product divides its results by the rows' root mean square."""
         self.fold_rows = fold_rows
         self.fold_many_rows = fold_many_rows
+        # steps of up to `fold_rows` rows too: the adding product leaves the rows times the next norm's weight where it
+        # is told that weight, and the reader scales its results (what the HIP kernel set's decode products do)
+        self.rows_left = rows_left
 
     def check_attention_sizes(self, q_heads, kv_heads, head_dim, page_size):
         if q_heads % kv_heads:
@@ -104,7 +107,11 @@ class TorchKernels(KernelSet):
         if rows <= self.fold_rows:
             sums = arena.take(((outs + 15) // 16, 16), torch.float32)
             self.linear_adds(x, weight, stream, sums, bias=bias)
-            return StreamSums(sums)
+            if not self.rows_left or gain is None:
+                return StreamSums(sums)
+            left = arena.take((rows, outs), x.dtype)
+            left.copy_((stream * gain).to(x.dtype))
+            return StreamSums(sums, rows=left, gain=gain)
         # many rows: the new rows times the next norm's weight, and three groups of partial sums per row
         y = torch.empty(rows, outs, dtype=x.dtype)
         self.linear(x, weight, y, bias)
@@ -118,7 +125,7 @@ class TorchKernels(KernelSet):
         return StreamSums(sums, rows=left, gain=gain)
 
     def scales_rows_in_product(self, rows, weight, dtype, sums):
-        return sums.rows is not None and self.fold_rows < rows <= self.fold_many_rows and dtype == torch.bfloat16
+        return sums.rows is not None and 0 < rows <= max(self.fold_rows, self.fold_many_rows) and dtype == torch.bfloat16
 
     def linear_rowscaled(self, x, sums, eps, weight, out, bias=None):
         rows, k = x.shape
