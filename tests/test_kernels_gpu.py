@@ -1472,7 +1472,7 @@ def test_a_row_cut_over_several_blocks_chooses_what_one_block_chooses(hip, rows,
     hip.sample(*on, want)
     monkeypatch.setattr(hip, "sample_in_parts", True)
     assert (hip._sample_parts(rows, vocab) > 1) == (rows <= 128 and vocab >= 4096)
-    for _ in range(2):
+    for _ in range(200 if rows == 8 else 2):      # (back to back: whichever block of a row is last, the same token)
         got = torch.full((rows,), -7, dtype=torch.int32, device="cuda")
         hip.sample(*on, got)
         assert torch.equal(got, want)
