@@ -1173,8 +1173,15 @@ template <int NQ>
 __global__ __launch_bounds__(64 * kMergeWaves) void attention_merge_kernel(const Args a) {
   constexpr int PER = (D + 63) / 64;
   __shared__ float sums[kMergeWaves][PER * 64 + 1];  // per wave: the weighted sum per dim, then the denominator
-  const Tile t = find_tile(a, blockIdx.x, a.tokens_per_tile);
-  if (!t.found) return;
+  Tile t{};
+  if (a.plan != nullptr) {   // single tokens cut by a plan: block x is request seq_first + x, one row each
+    t.found = true;
+    t.tokens = 1;
+    t.first_row = a.q_start[a.seq_first] + static_cast<int>(blockIdx.x);
+  } else {
+    t = find_tile(a, blockIdx.x, a.tokens_per_tile);
+    if (!t.found) return;
+  }
   const int kvh = blockIdx.y / a.head_groups, hg = blockIdx.y % a.head_groups;
   const int c = blockIdx.z, lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int token = c / a.heads_per_tile, head_in_group = hg * a.heads_per_tile + c % a.heads_per_tile;
